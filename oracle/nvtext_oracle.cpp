@@ -1,0 +1,564 @@
+// nvtext_oracle.cpp -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// Scalar host restatement of libcudf's nvtext::minhash / minhash64 /
+// wordpiece_tokenize (+ wordpiece_vocabulary) semantics.  It exists only to
+// check the HIP implementation (tests, the smoke check and the bench's
+// cpu_baseline leg); the product library never links or loads it.
+//
+// Every function cites the reference file:line it restates (paths relative to
+// the cudf source tree).  The arithmetic of MurmurHash3 lives in the
+// un-vendored dependency NVIDIA/cuCollections (cuco::murmurhash3_32 and
+// cuco::murmurhash3_x64_128, pinned by rapids-cmake for cudf 26.10); it is
+// Austin Appleby's published MurmurHash3 and is restated here from the
+// published algorithm.
+//
+// Parity status: every function below is pinned by the reference's own test
+// vectors (tests/test_oracle_golden.py); two behaviours are pinned by code
+// reading only -- the size_bytes/2 word cap and validity being ignored when
+// max_words_per_row == 0 -- and one reference behaviour is racy and therefore
+// unpinnable: rows ending in >= 2 spaces with max_words_per_row > 0.  For that
+// class this file uses the plain "first N space-delimited words" definition.
+//
+// Build: make -C oracle   (g++ -O2 -std=c++17 -shared -fPIC -pthread)
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <string>
+#include <string_view>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// status codes shared with the C ABI of the product (include/nvtext_amd.h)
+// ---------------------------------------------------------------------------
+enum : int { OK = 0, INVALID_ARGUMENT = 1, OVERFLOW_ERROR = 2, LOGIC_ERROR = 3 };
+
+// ---------------------------------------------------------------------------
+// MurmurHash3_x86_32 -- cpp/include/cudf/hashing/detail/murmurhash3_x86_32.cuh:21-46,69-76
+// (forwards to cuco::murmurhash3_32<Key>::compute_hash; published algorithm)
+// ---------------------------------------------------------------------------
+inline uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
+inline uint64_t rotl64(uint64_t x, int r) { return (x << r) | (x >> (64 - r)); }
+
+uint32_t murmur3_x86_32(uint8_t const* data, int64_t len, uint32_t seed)
+{
+  uint32_t const c1 = 0xcc9e2d51u, c2 = 0x1b873593u;
+  uint32_t h1       = seed;
+  int64_t nblocks   = len / 4;
+  for (int64_t i = 0; i < nblocks; ++i) {
+    uint32_t k1;
+    std::memcpy(&k1, data + 4 * i, 4);  // little-endian host
+    k1 *= c1;
+    k1 = rotl32(k1, 15);
+    k1 *= c2;
+    h1 ^= k1;
+    h1 = rotl32(h1, 13);
+    h1 = h1 * 5 + 0xe6546b64u;
+  }
+  uint8_t const* tail = data + 4 * nblocks;
+  uint32_t k1         = 0;
+  switch (len & 3) {
+    case 3: k1 ^= uint32_t(tail[2]) << 16; [[fallthrough]];
+    case 2: k1 ^= uint32_t(tail[1]) << 8; [[fallthrough]];
+    case 1:
+      k1 ^= uint32_t(tail[0]);
+      k1 *= c1;
+      k1 = rotl32(k1, 15);
+      k1 *= c2;
+      h1 ^= k1;
+  }
+  h1 ^= uint32_t(len);
+  h1 ^= h1 >> 16;
+  h1 *= 0x85ebca6bu;
+  h1 ^= h1 >> 13;
+  h1 *= 0xc2b2ae35u;
+  h1 ^= h1 >> 16;
+  return h1;
+}
+
+// ---------------------------------------------------------------------------
+// MurmurHash3_x64_128 -- cpp/include/cudf/hashing/detail/murmurhash3_x64_128.cuh:18-43,66-73
+// (forwards to cuco::murmurhash3_x64_128; h1 = h2 = seed; published algorithm)
+// ---------------------------------------------------------------------------
+inline uint64_t fmix64(uint64_t k)
+{
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  k *= 0xc4ceb9fe1a85ec53ull;
+  k ^= k >> 33;
+  return k;
+}
+
+void murmur3_x64_128(uint8_t const* data, int64_t len, uint64_t seed, uint64_t out[2])
+{
+  uint64_t const c1 = 0x87c37b91114253d5ull, c2 = 0x4cf5ad432745937full;
+  uint64_t h1 = seed, h2 = seed;
+  int64_t nblocks = len / 16;
+  for (int64_t i = 0; i < nblocks; ++i) {
+    uint64_t k1, k2;
+    std::memcpy(&k1, data + 16 * i, 8);
+    std::memcpy(&k2, data + 16 * i + 8, 8);
+    k1 *= c1;
+    k1 = rotl64(k1, 31);
+    k1 *= c2;
+    h1 ^= k1;
+    h1 = rotl64(h1, 27);
+    h1 += h2;
+    h1 = h1 * 5 + 0x52dce729;
+    k2 *= c2;
+    k2 = rotl64(k2, 33);
+    k2 *= c1;
+    h2 ^= k2;
+    h2 = rotl64(h2, 31);
+    h2 += h1;
+    h2 = h2 * 5 + 0x38495ab5;
+  }
+  uint8_t const* tail = data + 16 * nblocks;
+  uint64_t k1 = 0, k2 = 0;
+  switch (len & 15) {
+    case 15: k2 ^= uint64_t(tail[14]) << 48; [[fallthrough]];
+    case 14: k2 ^= uint64_t(tail[13]) << 40; [[fallthrough]];
+    case 13: k2 ^= uint64_t(tail[12]) << 32; [[fallthrough]];
+    case 12: k2 ^= uint64_t(tail[11]) << 24; [[fallthrough]];
+    case 11: k2 ^= uint64_t(tail[10]) << 16; [[fallthrough]];
+    case 10: k2 ^= uint64_t(tail[9]) << 8; [[fallthrough]];
+    case 9:
+      k2 ^= uint64_t(tail[8]);
+      k2 *= c2;
+      k2 = rotl64(k2, 33);
+      k2 *= c1;
+      h2 ^= k2;
+      [[fallthrough]];
+    case 8: k1 ^= uint64_t(tail[7]) << 56; [[fallthrough]];
+    case 7: k1 ^= uint64_t(tail[6]) << 48; [[fallthrough]];
+    case 6: k1 ^= uint64_t(tail[5]) << 40; [[fallthrough]];
+    case 5: k1 ^= uint64_t(tail[4]) << 32; [[fallthrough]];
+    case 4: k1 ^= uint64_t(tail[3]) << 24; [[fallthrough]];
+    case 3: k1 ^= uint64_t(tail[2]) << 16; [[fallthrough]];
+    case 2: k1 ^= uint64_t(tail[1]) << 8; [[fallthrough]];
+    case 1:
+      k1 ^= uint64_t(tail[0]);
+      k1 *= c1;
+      k1 = rotl64(k1, 31);
+      k1 *= c2;
+      h1 ^= k1;
+  }
+  h1 ^= uint64_t(len);
+  h2 ^= uint64_t(len);
+  h1 += h2;
+  h2 += h1;
+  h1 = fmix64(h1);
+  h2 = fmix64(h2);
+  h1 += h2;
+  h2 += h1;
+  out[0] = h1;
+  out[1] = h2;
+}
+
+// ---------------------------------------------------------------------------
+// UTF-8 helpers -- cpp/include/cudf/strings/detail/utf8.hpp:23-27 and 84-90
+// ---------------------------------------------------------------------------
+inline bool is_utf8_continuation_char(uint8_t b) { return (b & 0xC0) == 0x80; }
+
+inline int bytes_in_utf8_byte(uint8_t b)
+{
+  return 1 + int((b & 0xF0) == 0xF0) + int((b & 0xE0) == 0xE0) + int((b & 0xC0) == 0xC0) -
+         int((b & 0xC0) == 0x80);
+}
+
+// cpp/include/cudf/strings/string_view.cuh:67-80: walks BYTES, adds the declared
+// width of every lead byte, stops once `pos` lead bytes were seen or input ends.
+inline void bytes_to_character_position(uint8_t const* p, int64_t n, int pos, int64_t& bytes, int& left)
+{
+  bytes = 0;
+  int64_t i = 0;
+  while (pos > 0 && i < n) {
+    int const w = bytes_in_utf8_byte(p[i]);
+    if (w) { --pos; }
+    bytes += w;
+    ++i;
+  }
+  left = pos;
+}
+
+// ---------------------------------------------------------------------------
+// Arrow-layout strings column on the host
+// (cpp/include/cudf/strings/strings_column_view.hpp:27-114; row i of a sliced view
+// is chars[off[i+offset] .. off[i+offset+1]), bit i+offset of the mask is its validity)
+// ---------------------------------------------------------------------------
+struct StringsCol {
+  uint8_t const* chars;
+  void const* offsets;
+  int offsets_is_int64;
+  uint32_t const* mask;  // may be null
+  int32_t size;
+  int32_t offset;
+  int32_t null_count;
+
+  int64_t off(int64_t i) const
+  {
+    return offsets_is_int64 ? static_cast<int64_t const*>(offsets)[i + offset]
+                            : static_cast<int32_t const*>(offsets)[i + offset];
+  }
+  bool valid(int64_t i) const
+  {
+    if (!mask) return true;
+    int64_t const b = i + offset;
+    return (mask[b >> 5] >> (b & 31)) & 1u;
+  }
+};
+
+template <typename F>
+void parallel_rows(int32_t rows, int nthreads, F f)
+{
+  if (nthreads <= 1 || rows < 2 * nthreads) {
+    f(0, 0, rows);
+    return;
+  }
+  std::vector<std::thread> ts;
+  for (int t = 0; t < nthreads; ++t) {
+    int32_t const lo = int64_t(rows) * t / nthreads;
+    int32_t const hi = int64_t(rows) * (t + 1) / nthreads;
+    ts.emplace_back([=] { f(t, lo, hi); });
+  }
+  for (auto& t : ts) t.join();
+}
+
+// ---------------------------------------------------------------------------
+// minhash / minhash64 -- cpp/src/text/minhash.cu:87-157 (window hashing),
+// 281-376 (permutation + min), 426-513 (argument checks), 605-630 (list assembly)
+// ---------------------------------------------------------------------------
+template <typename T>
+struct HashOf;
+template <>
+struct HashOf<uint32_t> {
+  static uint32_t hash(uint8_t const* p, int64_t n, uint32_t seed) { return murmur3_x86_32(p, n, seed); }
+};
+template <>
+struct HashOf<uint64_t> {
+  // minhash.cu:138 -- first 64-bit word of the 128-bit result
+  static uint64_t hash(uint8_t const* p, int64_t n, uint64_t seed)
+  {
+    uint64_t o[2];
+    murmur3_x64_128(p, n, seed, o);
+    return o[0];
+  }
+};
+
+template <typename T>
+inline T permute(T hv, T a, T b)
+{
+  // minhash.cu:350-351: arithmetic is in hash_value_type, so the product and the
+  // sum wrap modulo 2^32 / 2^64 BEFORE the % (2^61-1); for 32-bit values the
+  // modulus and the "& max" are no-ops.
+  constexpr uint64_t mersenne_prime = (1ull << 61) - 1;
+  T const x = static_cast<T>(hv * a + b);
+  return static_cast<T>((static_cast<uint64_t>(x) % mersenne_prime) &
+                        static_cast<uint64_t>(std::numeric_limits<T>::max()));
+}
+
+template <typename T>
+void minhash_row(uint8_t const* s, int64_t n, T seed, T const* a, T const* b, int32_t P, int32_t width, T* out)
+{
+  if (n == 0) {  // minhash.cu:318 -- init = 0 for an empty (valid) row
+    std::fill(out, out + P, T{0});
+    return;
+  }
+  std::fill(out, out + P, std::numeric_limits<T>::max());
+  for (int64_t i = 0; i < n; ++i) {
+    if (is_utf8_continuation_char(s[i])) continue;  // minhash.cu:120-123
+    int64_t bytes;
+    int left;
+    bytes_to_character_position(s + i, n - i, width, bytes, left);
+    if (i != 0 && left > 0) continue;  // minhash.cu:127-131
+    // A malformed trailing lead byte may declare more bytes than the row holds;
+    // the window is clamped to the row (well-formed UTF-8 never needs the clamp).
+    bytes  = std::min<int64_t>(bytes, n - i);
+    T hv   = HashOf<T>::hash(s + i, bytes, seed);
+    hv     = std::max<T>(hv, T{1});  // minhash.cu:141
+    for (int32_t j = 0; j < P; ++j) {
+      T const v = permute<T>(hv, a[j], b[j]);
+      if (v < out[j]) out[j] = v;
+    }
+  }
+}
+
+template <typename T>
+int minhash_impl(StringsCol const& col, T seed, T const* a, T const* b, int32_t P, int32_t width,
+                 int nthreads, int32_t* out_offsets, T* out_child, int64_t* out_child_len)
+{
+  // minhash.cu:435-446, in this order
+  if (width < 2) return INVALID_ARGUMENT;
+  if (P <= 0) return INVALID_ARGUMENT;
+  if (static_cast<uint64_t>(col.size) * static_cast<uint64_t>(P) >=
+      static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
+    return OVERFLOW_ERROR;
+  if (col.size == 0) {  // minhash.cu:449 + 616: offsets = [0], empty child
+    if (out_offsets) out_offsets[0] = 0;
+    *out_child_len = 0;
+    return OK;
+  }
+  // minhash.cu:626-628: with nulls present the identity gather of
+  // purge_nonempty_nulls drops the P slots of every null row
+  // (cpp/src/copying/purge_nonempty_nulls.cu:79-94); offsets follow.
+  bool const purge = col.null_count > 0;
+  int64_t pos      = 0;
+  for (int32_t r = 0; r < col.size; ++r) {
+    out_offsets[r] = static_cast<int32_t>(pos);
+    if (!(purge && !col.valid(r))) pos += P;
+  }
+  out_offsets[col.size] = static_cast<int32_t>(pos);
+  *out_child_len        = pos;
+  parallel_rows(col.size, nthreads, [&](int, int32_t lo, int32_t hi) {
+    for (int32_t r = lo; r < hi; ++r) {
+      if (purge && !col.valid(r)) continue;
+      int64_t const o = col.off(r);
+      int64_t n       = col.off(r + 1) - o;
+      // a null row reached here only when null_count == 0 was (wrongly) declared;
+      // treat it as the reference's seed kernel does: no hashes -> it is not defined.
+      minhash_row<T>(col.chars + o, n, seed, a, b, P, width, out_child + out_offsets[r]);
+    }
+  });
+  return OK;
+}
+
+// ---------------------------------------------------------------------------
+// wordpiece vocabulary -- cpp/src/text/wordpiece_tokenize.cu:184-209, 213-282
+// ---------------------------------------------------------------------------
+struct Vocab {
+  std::string chars;             // deep copy (wordpiece_tokenize.cu:221)
+  std::vector<int64_t> offsets;  // V + 1
+  std::unordered_map<std::string_view, int32_t> full;  // every row, keyed by its text
+  std::unordered_map<std::string_view, int32_t> sub;   // "##x" rows keyed by "x" (92-120, 184-192)
+  int32_t unk_id = -1;                                 // 199-209, 273-275
+};
+
+// wordpiece_tokenize.cu:307-317
+inline int64_t remove_last_char(uint8_t const* p, int64_t n)
+{
+  if (n < 2) return 0;
+  int64_t e = n - 1;
+  while (e > 0 && is_utf8_continuation_char(p[e])) --e;
+  return e;
+}
+
+constexpr int32_t no_token      = std::numeric_limits<int32_t>::max();
+constexpr int64_t max_word_size = 200;  // wordpiece_tokenize.cu:300
+
+// wordpiece_tokenize.cu:349-407.  Returns the token count; tokens appended to `out`.
+inline void wp_tokenize(Vocab const& v, uint8_t const* w, int64_t n, std::vector<int32_t>& out)
+{
+  auto sv = [](uint8_t const* p, int64_t n) { return std::string_view(reinterpret_cast<char const*>(p), size_t(n)); };
+  auto it = v.full.find(sv(w, n));
+  if (it != v.full.end()) {
+    out.push_back(it->second);
+    return;
+  }
+  size_t const first = out.size();
+  int64_t piece      = remove_last_char(w, n);
+  while (piece > 0) {
+    it = v.full.find(sv(w, piece));
+    if (it == v.full.end()) {
+      piece = remove_last_char(w, piece);
+      continue;
+    }
+    out.push_back(it->second);
+    break;
+  }
+  if (piece == 0) {
+    out.push_back(v.unk_id);
+    return;
+  }
+  uint8_t const* rest = w + piece;
+  int64_t rest_n      = n - piece;
+  piece               = rest_n;
+  while (piece > 0) {
+    auto is = v.sub.find(sv(rest, piece));
+    if (is == v.sub.end()) {
+      piece = remove_last_char(rest, piece);
+      continue;
+    }
+    out.push_back(is->second);
+    rest += piece;
+    rest_n -= piece;
+    piece = rest_n;
+  }
+  if (rest_n > 0) {  // 396-404: the whole word collapses to one unknown token
+    out.resize(first);
+    out.push_back(v.unk_id);
+  }
+}
+
+// Tokens of one row.  max_words == 0: wordpiece_tokenize.cu:503-568 + 426-448
+// (every maximal run of non-space bytes, validity not consulted).
+// max_words > 0: 757-835 (null -> none; cap = min(max_words, size_bytes / 2) at :780).
+inline void tokenize_row(Vocab const& v, uint8_t const* s, int64_t n, bool valid, int32_t max_words,
+                         std::vector<int32_t>& out)
+{
+  int64_t cap = std::numeric_limits<int64_t>::max();
+  if (max_words > 0) {
+    if (!valid) return;
+    cap = std::min<int64_t>(max_words, n / 2);
+  }
+  int64_t words = 0;
+  int64_t i     = 0;
+  while (i < n && words < cap) {
+    while (i < n && s[i] == ' ') ++i;
+    if (i >= n) break;
+    int64_t const b = i;
+    while (i < n && s[i] != ' ') ++i;
+    int64_t const len = i - b;
+    ++words;
+    if (len >= max_word_size) {  // 442-445, 738-741
+      out.push_back(v.unk_id);
+    } else {
+      wp_tokenize(v, s + b, len, out);
+    }
+  }
+}
+
+}  // namespace
+
+// ===========================================================================
+// C entry points (ctypes)
+// ===========================================================================
+extern "C" {
+
+uint32_t oracle_murmur3_x86_32(uint8_t const* data, int64_t len, uint32_t seed)
+{
+  return murmur3_x86_32(data, len, seed);
+}
+
+void oracle_murmur3_x64_128(uint8_t const* data, int64_t len, uint64_t seed, uint64_t* out2)
+{
+  murmur3_x64_128(data, len, seed, out2);
+}
+
+int oracle_minhash(uint8_t const* chars, void const* offsets, int offsets_is_int64, uint32_t const* mask,
+                   int32_t size, int32_t offset, int32_t null_count, uint32_t seed, uint32_t const* a,
+                   uint32_t const* b, int32_t P, int32_t width, int nthreads, int32_t* out_offsets,
+                   uint32_t* out_child, int64_t* out_child_len)
+{
+  StringsCol c{chars, offsets, offsets_is_int64, mask, size, offset, null_count};
+  return minhash_impl<uint32_t>(c, seed, a, b, P, width, nthreads, out_offsets, out_child, out_child_len);
+}
+
+int oracle_minhash64(uint8_t const* chars, void const* offsets, int offsets_is_int64, uint32_t const* mask,
+                     int32_t size, int32_t offset, int32_t null_count, uint64_t seed, uint64_t const* a,
+                     uint64_t const* b, int32_t P, int32_t width, int nthreads, int32_t* out_offsets,
+                     uint64_t* out_child, int64_t* out_child_len)
+{
+  StringsCol c{chars, offsets, offsets_is_int64, mask, size, offset, null_count};
+  return minhash_impl<uint64_t>(c, seed, a, b, P, width, nthreads, out_offsets, out_child, out_child_len);
+}
+
+// wordpiece_tokenize.cu:213-282.  Returns INVALID_ARGUMENT for an empty vocabulary
+// or one with nulls (217-218).
+int oracle_vocab_create(uint8_t const* chars, void const* offsets, int offsets_is_int64, int32_t size,
+                        int32_t offset, int32_t null_count, void** handle)
+{
+  *handle = nullptr;
+  if (size == 0) return INVALID_ARGUMENT;
+  if (null_count > 0) return INVALID_ARGUMENT;
+  StringsCol c{chars, offsets, offsets_is_int64, nullptr, size, offset, 0};
+  auto* v          = new Vocab;
+  int64_t const o0 = c.off(0);
+  v->chars.assign(reinterpret_cast<char const*>(chars) + o0, size_t(c.off(size) - o0));
+  v->offsets.resize(size_t(size) + 1);
+  for (int32_t i = 0; i <= size; ++i) v->offsets[i] = c.off(i) - o0;
+  v->full.reserve(size_t(size) * 2);
+  for (int32_t i = 0; i < size; ++i) {
+    std::string_view s(v->chars.data() + v->offsets[i], size_t(v->offsets[i + 1] - v->offsets[i]));
+    v->full.emplace(s, i);  // duplicates are undefined in the reference (wordpiece_tokenize.hpp:30-31)
+    if (s.size() >= 2 && s[0] == '#' && s[1] == '#') v->sub.emplace(s.substr(2), i);
+  }
+  auto u = v->full.find(std::string_view("[UNK]"));
+  if (u == v->full.end()) u = v->full.find(std::string_view("[unk]"));
+  v->unk_id = (u == v->full.end()) ? -1 : u->second;
+  *handle   = v;
+  return OK;
+}
+
+void oracle_vocab_destroy(void* handle) { delete static_cast<Vocab*>(handle); }
+
+int32_t oracle_vocab_unk_id(void const* handle) { return static_cast<Vocab const*>(handle)->unk_id; }
+
+// wordpiece_tokenize.cu:839-888.  `out_offsets` has size+1 entries (caller-owned);
+// `*out_tokens` is malloc'ed here and released with oracle_free.
+// *out_kind: 0 = ordinary result, 1 = all-null list (849-851), 2 = empty list (852).
+int oracle_wordpiece_tokenize(void const* handle, uint8_t const* chars, void const* offsets,
+                              int offsets_is_int64, uint32_t const* mask, int32_t size, int32_t offset,
+                              int32_t null_count, int32_t max_words_per_row, int nthreads,
+                              int32_t* out_offsets, int32_t** out_tokens, int64_t* out_ntokens,
+                              int32_t* out_kind)
+{
+  *out_tokens  = nullptr;
+  *out_ntokens = 0;
+  *out_kind    = 0;
+  if (max_words_per_row < 0) return INVALID_ARGUMENT;
+  Vocab const& v = *static_cast<Vocab const*>(handle);
+  StringsCol c{chars, offsets, offsets_is_int64, mask, size, offset, null_count};
+  if (size == null_count) {
+    if (null_count > 0) {
+      *out_kind = 1;
+      std::fill(out_offsets, out_offsets + size + 1, 0);
+    } else {
+      *out_kind = 2;
+    }
+    return OK;
+  }
+  int const nt = std::max(1, nthreads);
+  std::vector<std::vector<int32_t>> parts(static_cast<size_t>(nt));
+  std::vector<int32_t> counts(static_cast<size_t>(size));
+  parallel_rows(size, nt, [&](int t, int32_t lo, int32_t hi) {
+    auto& out = parts[size_t(t)];
+    for (int32_t r = lo; r < hi; ++r) {
+      size_t const before = out.size();
+      int64_t const o     = c.off(r);
+      tokenize_row(v, chars + o, c.off(r + 1) - o, c.valid(r), max_words_per_row, out);
+      counts[size_t(r)] = static_cast<int32_t>(out.size() - before);
+    }
+  });
+  // cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339
+  int64_t total = 0;
+  for (int32_t r = 0; r < size; ++r) {
+    out_offsets[r] = static_cast<int32_t>(total);
+    total += counts[size_t(r)];
+  }
+  if (total > std::numeric_limits<int32_t>::max()) return OVERFLOW_ERROR;
+  out_offsets[size] = static_cast<int32_t>(total);
+  auto* toks        = static_cast<int32_t*>(std::malloc(std::max<size_t>(size_t(total) * 4, 4)));
+  int64_t w         = 0;
+  for (auto const& p : parts) {
+    if (!p.empty()) std::memcpy(toks + w, p.data(), p.size() * 4);
+    w += int64_t(p.size());
+  }
+  *out_tokens  = toks;
+  *out_ntokens = total;
+  return OK;
+}
+
+void oracle_free(void* p) { std::free(p); }
+
+// cpp/src/bitmask/null_mask.cu:332-347,357-391: bit i of the result = bit i+offset of the source.
+// `out` has ceil(size/32) words; bits past `size` are cleared.
+void oracle_copy_bitmask(uint32_t const* mask, int32_t offset, int32_t size, uint32_t* out)
+{
+  int32_t const words = (size + 31) / 32;
+  for (int32_t w = 0; w < words; ++w) out[w] = 0;
+  for (int32_t i = 0; i < size; ++i) {
+    int64_t const b = int64_t(i) + offset;
+    if ((mask[b >> 5] >> (b & 31)) & 1u) out[i >> 5] |= 1u << (i & 31);
+  }
+}
+
+int oracle_hardware_threads() { return int(std::thread::hardware_concurrency()); }
+
+}  // extern "C"

@@ -1,0 +1,231 @@
+"""Pins the host oracle to every known-answer vector the reference holds for this path,
+to published MurmurHash3 values, to an independent library (HF `tokenizers` WordPiece)
+and to closed forms a plausible mistake would break.  CPU only."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from oracle.pyoracle import OracleError
+from tests import golden_cases as gc
+from tests.golden_cases import strings
+
+
+# ----------------------------------------------------------------------------- hashes
+def test_murmur32_public_vectors():
+    for v in gc.murmur32_vectors():
+        assert orc.murmur3_x86_32(bytes.fromhex(v["hex"]), v["seed"]) == v["hash"], v
+
+
+def test_murmur64_reference_vectors():
+    v = gc.murmur64_vectors()
+    for s, e0, e7 in zip(v["strings"], v["seed0"], v["seed7"]):
+        b = s.encode("utf-8")
+        assert orc.murmur3_x64_128(b, 0)[0] == e0, s
+        assert orc.murmur3_x64_128(b, 7)[0] == e7, s
+
+
+def test_murmur64_tail_lengths_change_hash():
+    # every tail length 0..31 goes through a different switch arm; all distinct
+    seen = {orc.murmur3_x64_128(b"q" * n, 7) for n in range(32)}
+    assert len(seen) == 32
+
+
+# ----------------------------------------------------------------------------- minhash
+@pytest.mark.parametrize("case", gc.minhash_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_minhash_golden(case, dtype):
+    col = strings(case["rows"], dtype)
+    if "expected32" in case:
+        got = orc.minhash(col, case["seed"], case["a"], case["b"], case["width"], nthreads=2)
+        assert gc.expected_list_equal(got.to_pylist(), case["expected32"])
+        assert got.child.dtype == np.uint32 and got.offsets.dtype == np.int32
+    if "expected64" in case:
+        got = orc.minhash64(col, case["seed"], case["a"], case["b"], case["width"], nthreads=2)
+        assert gc.expected_list_equal(got.to_pylist(), case["expected64"])
+        assert got.child.dtype == np.uint64
+
+
+def test_minhash_single_window_closed_form():
+    # a row shorter than width contributes exactly one hash: out[j] = max(h,1)*a_j + b_j
+    a = np.array([10, 0xFFFFFFFF, 3], np.uint32)
+    b = np.array([10, 7, 0xFFFFFFF0], np.uint32)
+    for s in ["d", "ab", "xyz", "é"]:
+        h = max(orc.murmur3_x86_32(s.encode(), 0), 1)
+        got = orc.minhash(strings([s]), 0, a, b, 4).to_pylist()[0]
+        assert got == [(h * int(x) + int(y)) % 2**32 for x, y in zip(a, b)]
+        h64 = max(orc.murmur3_x64_128(s.encode(), 7)[0], 1)
+        a64 = np.array([2, 2**63 + 5], np.uint64)
+        b64 = np.array([5, 2**64 - 1], np.uint64)
+        got = orc.minhash64(strings([s]), 7, a64, b64, 4).to_pylist()[0]
+        assert got == [((h64 * int(x) + int(y)) % 2**64) % (2**61 - 1) for x, y in zip(a64, b64)]
+
+
+def test_minhash_invariants():
+    rng = np.random.default_rng(3)
+    a = rng.integers(1, 2**32, 17, dtype=np.uint64).astype(np.uint32)
+    b = rng.integers(0, 2**32, 17, dtype=np.uint64).astype(np.uint32)
+    # a run of one repeated character has one distinct window -> equals the single-window row
+    one = orc.minhash(strings(["zzzzz"]), 42, a, b, 5).to_pylist()[0]
+    many = orc.minhash(strings(["z" * 300]), 42, a, b, 5).to_pylist()[0]
+    assert one == many
+    # appending a copy of the text that re-creates only existing windows does not change the result
+    base = orc.minhash(strings(["abcabc"]), 42, a, b, 3).to_pylist()[0]
+    more = orc.minhash(strings(["abcabcabcabc"]), 42, a, b, 3).to_pylist()[0]
+    assert base == more
+    # the minimum over a union of window sets is the element-wise minimum
+    x = orc.minhash(strings(["hello world"]), 1, a, b, 4).to_pylist()[0]
+    y = orc.minhash(strings(["world hello"]), 1, a, b, 4).to_pylist()[0]
+    xy = orc.minhash(strings(["hello world hello"]), 1, a, b, 4).to_pylist()[0]
+    assert xy == [min(p, q) for p, q in zip(x, y)]
+
+
+def test_minhash_utf8_windows_are_characters():
+    # width counts characters: "ééé" (6 bytes) with width 3 is ONE window = whole row
+    a = np.array([1], np.uint32)
+    b = np.array([0], np.uint32)
+    h = max(orc.murmur3_x86_32("ééé".encode(), 0), 1)
+    assert orc.minhash(strings(["ééé"]), 0, a, b, 3).to_pylist()[0] == [h]
+    # "éaé" + "b": width 3 -> windows "éaé", "aéb"; continuation bytes never start a window
+    hs = [max(orc.murmur3_x86_32(w.encode(), 0), 1) for w in ["éaé", "aéb"]]
+    assert orc.minhash(strings(["éaéb"]), 0, a, b, 3).to_pylist()[0] == [min(hs)]
+
+
+def test_minhash_nulls_empty_sliced():
+    rows = ["abcdef", None, "", "xyzuvw", None, "k"]
+    a = np.array([3, 5], np.uint32)
+    col = strings(rows)
+    got = orc.minhash(col, 0, a, a, 4)
+    assert got.null_count == 2 and got.size == 6
+    assert got.offsets.tolist() == [0, 2, 2, 4, 6, 6, 8]
+    pl = got.to_pylist()
+    assert pl[1] is None and pl[4] is None and pl[2] == [0, 0]
+    sl = col.slice(2, 5)
+    got_s = orc.minhash(sl, 0, a, a, 4)
+    assert got_s.to_pylist() == pl[2:5]
+    assert got_s.offsets.tolist() == [0, 2, 4, 4]
+
+
+def test_minhash_errors_and_empty():
+    col = strings(["this string intentionally left blank"])
+    e = np.zeros(0, np.uint32)
+    with pytest.raises(OracleError) as ei:
+        orc.minhash(col, 0, e, e, 0)
+    assert ei.value.code == orc.INVALID_ARGUMENT
+    with pytest.raises(OracleError):
+        orc.minhash(col, 0, e, e, 4)
+    with pytest.raises(OracleError):
+        orc.minhash(col, 0, np.ones(2, np.uint32), np.ones(2, np.uint32), 1)
+    big = strings([""] * 50000)
+    z = np.zeros(50000, np.uint32)
+    with pytest.raises(OracleError) as ei:
+        orc.minhash(big, 0, z, z, 4)
+    assert ei.value.code == orc.OVERFLOW_ERROR
+    empty = strings([])
+    got = orc.minhash(empty, 0, np.ones(3, np.uint32), np.ones(3, np.uint32), 4)
+    assert got.size == 0 and got.child.size == 0
+
+
+# ----------------------------------------------------------------------------- wordpiece
+@pytest.mark.parametrize("case", gc.wordpiece_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_wordpiece_golden(case, dtype):
+    vocab = orc.Vocabulary(strings(case["vocab"]))
+    col = strings(case["rows"], dtype)
+    if "slice" in case:
+        col = col.slice(*case["slice"])
+    for run in case["runs"]:
+        got = orc.wordpiece_tokenize(col, vocab, run["max_words"], nthreads=2)
+        assert gc.expected_list_equal(got.to_pylist(), run["expected"]), (case["name"], run["max_words"])
+        assert got.child.dtype == np.int32
+
+
+def test_wordpiece_bert_sentences():
+    d = gc.bert_case()
+    vocab = orc.Vocabulary(strings(d["vocab"]))
+    assert vocab.unk_id == 100
+    col = strings(d["rows"])
+    for mw, exp in d["expected"].items():
+        got = orc.wordpiece_tokenize(col, vocab, int(mw))
+        assert gc.expected_list_equal(got.to_pylist(), exp), mw
+
+
+def test_wordpiece_errors_and_empty():
+    with pytest.raises(OracleError):
+        orc.Vocabulary(strings([]))
+    with pytest.raises(OracleError):
+        orc.Vocabulary(strings([None, None, None]))
+    v = orc.Vocabulary(strings(["x"]))
+    with pytest.raises(OracleError):
+        orc.wordpiece_tokenize(strings(["  "]), v, -1)
+    v2 = orc.Vocabulary(strings([""]))
+    for mw in (0, 10):
+        got = orc.wordpiece_tokenize(strings([]), v2, mw)
+        assert got.size == 0 and got.offsets.size == 0
+
+
+def test_wordpiece_long_word_and_cap_rules():
+    v = orc.Vocabulary(strings(["[UNK]", "a", "##a", "b"]))
+    # 199 bytes tokenizes piece by piece, 200 bytes is a single unknown token
+    got = orc.wordpiece_tokenize(strings(["a" * 199, "a" * 200, "a" * 250 + " b"]), v, 0).to_pylist()
+    assert got[0] == [1] + [2] * 198 and got[1] == [0] and got[2] == [0, 3]
+    # cap = min(max_words, size_bytes // 2): "a b a" has 5 bytes -> 2 words, a 1-byte row -> none
+    got = orc.wordpiece_tokenize(strings(["a b a", "a", "a b"]), v, 100).to_pylist()
+    assert got == [[1, 3], [], [1]]
+    # a null row with max_words > 0 has no tokens and stays null
+    got = orc.wordpiece_tokenize(strings(["a b", None, "b"]), v, 3)
+    assert got.to_pylist() == [[1], None, []] and got.null_count == 1
+
+
+def test_wordpiece_matches_hf_tokenizers():
+    """Independent implementation of the same greedy longest-match-first rule."""
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers.models import WordPiece
+    rng = np.random.default_rng(11)
+    letters = "abcdefgh"
+    vocab = ["[PAD]", "[UNK]"] + list(letters) + ["##" + c for c in letters[:5]]
+    seen = set(vocab)
+    while len(vocab) < 400:
+        n = int(rng.integers(2, 6))
+        s = "".join(rng.choice(list(letters), n))
+        if rng.random() < 0.4:
+            s = "##" + s
+        if s not in seen:
+            seen.add(s)
+            vocab.append(s)
+    model = WordPiece({t: i for i, t in enumerate(vocab)}, unk_token="[UNK]", max_input_chars_per_word=100)
+    words = ["".join(rng.choice(list(letters), int(rng.integers(1, 12)))) for _ in range(3000)]
+    rows = [" ".join(words[i:i + 30]) for i in range(0, 3000, 30)]
+    v = orc.Vocabulary(strings(vocab))
+    got = orc.wordpiece_tokenize(strings(rows), v, 0).to_pylist()
+    multi = 0
+    for row, g in zip(rows, got):
+        exp = []
+        for w in row.split(" "):
+            ids = [t.id for t in model.tokenize(w)]
+            multi += len(ids) > 1
+            exp.extend(ids)
+        assert g == exp
+    assert multi > 100  # the comparison exercised real sub-word splits
+
+
+def test_wordpiece_concatenation_and_cap_equivalence():
+    d = gc.bert_case()
+    v = orc.Vocabulary(strings(d["vocab"]))
+    rows = d["rows"]
+    full = orc.wordpiece_tokenize(strings(rows), v, 0).to_pylist()
+    # tokens of a row = concatenation of the tokens of its words
+    for row, toks in zip(rows, full):
+        words = [w for w in row.split(" ") if w]
+        per_word = orc.wordpiece_tokenize(strings(words), v, 0).to_pylist()
+        assert sum(per_word, []) == toks
+    # a cap above the word count (and below size/2) changes nothing
+    capped = orc.wordpiece_tokenize(strings(rows), v, 150).to_pylist()
+    assert capped == full
+
+
+def test_copy_bitmask_shift():
+    col = strings(["a", None, "b", None, None, "c"] * 20)
+    sl = col.slice(7, 101)
+    m = orc.copy_bitmask(sl)
+    from cudf_amd.arrow_host import unpack_validity
+    assert np.array_equal(unpack_validity(m, sl.size), col.validity()[7:101])
