@@ -1,0 +1,101 @@
+"""ctypes declarations for the C ABI in include/nvtext_amd.h (libnvtext_amd.so)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnvtext_amd.so")
+
+SUCCESS, INVALID_ARGUMENT, OVERFLOW, LOGIC_ERROR, DEVICE_ERROR, ALLOC_FAILED = range(6)
+TYPE_INT32, TYPE_UINT32, TYPE_UINT64 = 3, 7, 8
+
+EXPORTS = [
+    "nvtext_amd_version",
+    "nvtext_amd_last_error",
+    "nvtext_amd_minhash",
+    "nvtext_amd_minhash64",
+    "nvtext_amd_wordpiece_vocabulary_create",
+    "nvtext_amd_wordpiece_vocabulary_destroy",
+    "nvtext_amd_wordpiece_vocabulary_unk_id",
+    "nvtext_amd_wordpiece_tokenize",
+    "nvtext_amd_list_column_free",
+]
+
+
+class StringsColumn(C.Structure):
+    _fields_ = [
+        ("chars", C.c_void_p),
+        ("offsets", C.c_void_p),
+        ("offsets_is_int64", C.c_int32),
+        ("null_mask", C.c_void_p),
+        ("size", C.c_int32),
+        ("offset", C.c_int32),
+        ("null_count", C.c_int32),
+    ]
+
+
+ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p)
+DEALLOC_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p)
+
+
+class Allocator(C.Structure):
+    _fields_ = [("ctx", C.c_void_p), ("allocate", ALLOC_FN), ("deallocate", DEALLOC_FN)]
+
+
+class ListColumn(C.Structure):
+    _fields_ = [
+        ("size", C.c_int32),
+        ("null_count", C.c_int32),
+        ("child_type", C.c_int32),
+        ("offsets_size", C.c_int32),
+        ("offsets", C.c_void_p),
+        ("child", C.c_void_p),
+        ("child_size", C.c_int64),
+        ("null_mask", C.c_void_p),
+        ("offsets_bytes", C.c_size_t),
+        ("child_bytes", C.c_size_t),
+        ("null_mask_bytes", C.c_size_t),
+    ]
+
+
+_lib = None
+
+
+class ExtensionMissing(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the HIP library.  There is no fallback: without it the package cannot compute."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ExtensionMissing(
+            f"{LIB_PATH} is missing: build it with `make -C cudf_amd/csrc` (or __graft_entry__.build())")
+    L = C.CDLL(LIB_PATH)
+    L.nvtext_amd_version.restype = C.c_int32
+    L.nvtext_amd_version.argtypes = []
+    L.nvtext_amd_last_error.restype = C.c_char_p
+    L.nvtext_amd_last_error.argtypes = []
+    common_tail = [C.c_int32, C.c_void_p, C.POINTER(Allocator), C.POINTER(ListColumn)]
+    L.nvtext_amd_minhash.restype = C.c_int
+    L.nvtext_amd_minhash.argtypes = [C.POINTER(StringsColumn), C.c_uint32, C.c_void_p, C.c_void_p,
+                                     C.c_int64, C.c_int64] + common_tail
+    L.nvtext_amd_minhash64.restype = C.c_int
+    L.nvtext_amd_minhash64.argtypes = [C.POINTER(StringsColumn), C.c_uint64, C.c_void_p, C.c_void_p,
+                                       C.c_int64, C.c_int64] + common_tail
+    L.nvtext_amd_wordpiece_vocabulary_create.restype = C.c_int
+    L.nvtext_amd_wordpiece_vocabulary_create.argtypes = [C.POINTER(StringsColumn), C.c_void_p,
+                                                         C.POINTER(Allocator), C.POINTER(C.c_void_p)]
+    L.nvtext_amd_wordpiece_vocabulary_destroy.restype = None
+    L.nvtext_amd_wordpiece_vocabulary_destroy.argtypes = [C.c_void_p]
+    L.nvtext_amd_wordpiece_vocabulary_unk_id.restype = C.c_int32
+    L.nvtext_amd_wordpiece_vocabulary_unk_id.argtypes = [C.c_void_p]
+    L.nvtext_amd_wordpiece_tokenize.restype = C.c_int
+    L.nvtext_amd_wordpiece_tokenize.argtypes = [C.POINTER(StringsColumn), C.c_void_p] + common_tail
+    L.nvtext_amd_list_column_free.restype = None
+    L.nvtext_amd_list_column_free.argtypes = [C.POINTER(ListColumn), C.c_void_p, C.POINTER(Allocator)]
+    _lib = L
+    return L

@@ -1,0 +1,284 @@
+// Shared host/device helpers for the gfx950 nvtext kernels: status reporting,
+// stream-ordered temporaries, the device view of an Arrow strings column,
+// wavefront (64-lane) DPP scans, workgroup scans and a device-wide exclusive scan.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/nvtext_amd.h"
+
+namespace nvtext_amd {
+
+constexpr int kWave = 64;
+
+// ------------------------------------------------------------------ status
+void set_last_error(const char* msg);
+nvtext_amd_status fail(nvtext_amd_status st, const char* msg);
+
+#define NVTEXT_HIP_TRY(expr)                                                          \
+  do {                                                                                \
+    hipError_t _e = (expr);                                                           \
+    if (_e != hipSuccess) {                                                           \
+      std::string _m = std::string(#expr) + ": " + hipGetErrorString(_e);             \
+      return ::nvtext_amd::fail(NVTEXT_AMD_DEVICE_ERROR, _m.c_str());                 \
+    }                                                                                 \
+  } while (0)
+
+// ------------------------------------------------------------------ memory
+// Stream-ordered allocation through the caller's allocator (or hipMallocAsync).
+struct Mr {
+  const nvtext_amd_allocator* a;
+  hipStream_t stream;
+  void* allocate(size_t bytes) const;
+  void deallocate(void* p, size_t bytes) const;
+};
+
+// Temporary released (stream-ordered) when it goes out of scope.
+struct Temp {
+  Mr mr;
+  void* ptr   = nullptr;
+  size_t size = 0;
+  Temp(Mr m, size_t bytes) : mr(m), size(bytes)
+  {
+    if (bytes) ptr = mr.allocate(bytes);
+  }
+  ~Temp()
+  {
+    if (ptr) mr.deallocate(ptr, size);
+  }
+  Temp(const Temp&)            = delete;
+  Temp& operator=(const Temp&) = delete;
+  bool ok() const { return size == 0 || ptr != nullptr; }
+  template <typename T>
+  T* as() const
+  {
+    return static_cast<T*>(ptr);
+  }
+};
+
+inline size_t mask_alloc_bytes(int64_t bits)
+{
+  // libcudf pads bitmask allocations to 64 bytes (cpp/include/cudf/null_mask.hpp:56-57)
+  size_t const bytes = static_cast<size_t>((bits + 7) / 8);
+  return (bytes + 63) / 64 * 64;
+}
+
+// ------------------------------------------------------------------ column view on the device
+struct ColView {
+  const uint8_t* chars;
+  const void* offsets;
+  const uint32_t* mask;
+  int32_t size;
+  int32_t offset;
+  int32_t is64;
+  int32_t use_mask;  // 1 when validity must be consulted (mask present and null_count > 0)
+
+  __device__ __forceinline__ int64_t off(int64_t i) const
+  {
+    return is64 ? static_cast<const int64_t*>(offsets)[i + offset]
+                : static_cast<int64_t>(static_cast<const int32_t*>(offsets)[i + offset]);
+  }
+  __device__ __forceinline__ bool valid(int64_t i) const
+  {
+    if (!use_mask) return true;
+    int64_t const b = i + offset;
+    return (mask[b >> 5] >> (b & 31)) & 1u;
+  }
+};
+
+inline ColView make_view(const nvtext_amd_strings_column& c)
+{
+  ColView v;
+  v.chars    = reinterpret_cast<const uint8_t*>(c.chars);
+  v.offsets  = c.offsets;
+  v.mask     = c.null_mask;
+  v.size     = c.size;
+  v.offset   = c.offset;
+  v.is64     = c.offsets_is_int64 ? 1 : 0;
+  v.use_mask = (c.null_mask != nullptr && c.null_count > 0) ? 1 : 0;
+  return v;
+}
+
+// ------------------------------------------------------------------ UTF-8
+// cpp/include/cudf/strings/detail/utf8.hpp:23-27, 84-90
+__device__ __forceinline__ bool is_utf8_continuation(uint32_t b) { return (b & 0xC0u) == 0x80u; }
+__device__ __forceinline__ int bytes_in_utf8_byte(uint32_t b)
+{
+  return 1 + int((b & 0xF0u) == 0xF0u) + int((b & 0xE0u) == 0xE0u) + int((b & 0xC0u) == 0xC0u) -
+         int((b & 0xC0u) == 0x80u);
+}
+
+// ------------------------------------------------------------------ wavefront primitives (wave64, DPP)
+__device__ __forceinline__ int lane_id() { return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_zero(uint32_t v)
+{
+  // lanes without a source (or masked-out rows) read 0
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Inclusive prefix sum across the 64 lanes: four row_shr steps inside each row of 16,
+// then row_bcast:15 / row_bcast:31 carry the row totals forward.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
+{
+  v += dpp_zero<0x111, 0xf>(v);  // row_shr:1
+  v += dpp_zero<0x112, 0xf>(v);  // row_shr:2
+  v += dpp_zero<0x114, 0xf>(v);  // row_shr:4
+  v += dpp_zero<0x118, 0xf>(v);  // row_shr:8
+  v += dpp_zero<0x142, 0xa>(v);  // row_bcast:15 -> rows 1,3
+  v += dpp_zero<0x143, 0xc>(v);  // row_bcast:31 -> rows 2,3
+  return v;
+}
+
+__device__ __forceinline__ uint64_t wave_inclusive_scan64(uint64_t v)
+{
+#define NVTEXT_DPP64(CTRL, RM)                                                                  \
+  {                                                                                             \
+    uint32_t lo = dpp_zero<CTRL, RM>(static_cast<uint32_t>(v));                                 \
+    uint32_t hi = dpp_zero<CTRL, RM>(static_cast<uint32_t>(v >> 32));                           \
+    v += (static_cast<uint64_t>(hi) << 32) | lo;                                                \
+  }
+  NVTEXT_DPP64(0x111, 0xf)
+  NVTEXT_DPP64(0x112, 0xf)
+  NVTEXT_DPP64(0x114, 0xf)
+  NVTEXT_DPP64(0x118, 0xf)
+  NVTEXT_DPP64(0x142, 0xa)
+  NVTEXT_DPP64(0x143, 0xc)
+#undef NVTEXT_DPP64
+  return v;
+}
+
+__device__ __forceinline__ uint32_t wave_bcast(uint32_t v, int lane) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane)); }
+__device__ __forceinline__ uint64_t wave_bcast64(uint64_t v, int lane)
+{
+  uint32_t lo = wave_bcast(static_cast<uint32_t>(v), lane);
+  uint32_t hi = wave_bcast(static_cast<uint32_t>(v >> 32), lane);
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+__device__ __forceinline__ uint64_t ballot64(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask)
+{
+  return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+// Workgroup exclusive scan of one uint32 per thread.  `lds` needs (blockDim/64 + 1) words.
+// Returns the exclusive prefix; *total receives the workgroup sum (same value on every thread).
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* lds, uint32_t* total)
+{
+  constexpr int W  = THREADS / kWave;
+  int const lane   = lane_id();
+  int const wave   = threadIdx.x / kWave;
+  uint32_t const i = wave_inclusive_scan(v);
+  __syncthreads();  // protect lds reuse between calls
+  if (lane == kWave - 1) lds[wave] = i;
+  __syncthreads();
+  uint32_t base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    uint32_t const t = lds[w];
+    if (w < wave) base += t;
+    sum += t;
+  }
+  *total = sum;
+  return base + i - v;
+}
+
+template <int THREADS>
+__device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t v, uint64_t* lds, uint64_t* total)
+{
+  constexpr int W  = THREADS / kWave;
+  int const lane   = lane_id();
+  int const wave   = threadIdx.x / kWave;
+  uint64_t const i = wave_inclusive_scan64(v);
+  __syncthreads();
+  if (lane == kWave - 1) lds[wave] = i;
+  __syncthreads();
+  uint64_t base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    uint64_t const t = lds[w];
+    if (w < wave) base += t;
+    sum += t;
+  }
+  *total = sum;
+  return base + i - v;
+}
+
+// ------------------------------------------------------------------ device-wide exclusive scan
+// out[i] = sum_{j<i} f(j) for i in [0, n]  (n+1 entries; out[n] is the total).
+// Three launches: per-tile sums, scan of the tile sums (one workgroup), rescan + add.
+constexpr int kScanThreads = 256;
+constexpr int kScanItems   = 8;
+constexpr int kScanTile    = kScanThreads * kScanItems;
+
+template <typename F>
+__global__ void __launch_bounds__(kScanThreads) scan_tile_sums_kernel(F f, int64_t n, uint64_t* tile_sums)
+{
+  __shared__ uint64_t lds[kScanThreads / kWave + 1];
+  int64_t const base = static_cast<int64_t>(blockIdx.x) * kScanTile + static_cast<int64_t>(threadIdx.x) * kScanItems;
+  uint64_t s         = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t const i = base + k;
+    if (i < n) s += f(i);
+  }
+  uint64_t total;
+  block_exclusive_scan64<kScanThreads>(s, lds, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// exclusive scan of tile_sums in place; tile_sums[ntiles] = grand total
+__global__ void __launch_bounds__(kScanThreads) scan_tile_offsets_kernel(uint64_t* tile_sums, int64_t ntiles);
+
+template <typename F, typename OutT>
+__global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n, const uint64_t* tile_offsets, OutT* out)
+{
+  __shared__ uint64_t lds[kScanThreads / kWave + 1];
+  int64_t const base = static_cast<int64_t>(blockIdx.x) * kScanTile + static_cast<int64_t>(threadIdx.x) * kScanItems;
+  uint64_t vals[kScanItems];
+  uint64_t s = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t const i = base + k;
+    vals[k]         = (i < n) ? static_cast<uint64_t>(f(i)) : 0;
+    s += vals[k];
+  }
+  uint64_t total;
+  uint64_t run = block_exclusive_scan64<kScanThreads>(s, lds, &total) + tile_offsets[blockIdx.x];
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t const i = base + k;
+    if (i < n) out[i] = static_cast<OutT>(run);
+    run += vals[k];
+    if (i == n - 1) out[n] = static_cast<OutT>(run);
+  }
+}
+
+inline int64_t scan_tiles(int64_t n) { return (n + kScanTile - 1) / kScanTile; }
+inline size_t scan_temp_bytes(int64_t n) { return static_cast<size_t>(scan_tiles(n) + 1) * sizeof(uint64_t); }
+
+// `temp` holds scan_temp_bytes(n) bytes; temp[ntiles] receives the grand total (uint64).
+// n must be > 0.
+template <typename F, typename OutT>
+void device_exclusive_scan(F f, int64_t n, OutT* out, uint64_t* temp, hipStream_t stream)
+{
+  int64_t const tiles = scan_tiles(n);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(scan_tile_sums_kernel<F>), dim3(static_cast<unsigned>(tiles)), dim3(kScanThreads), 0, stream, f, n, temp);
+  hipLaunchKernelGGL(scan_tile_offsets_kernel, dim3(1), dim3(kScanThreads), 0, stream, temp, tiles);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(scan_apply_kernel<F, OutT>), dim3(static_cast<unsigned>(tiles)), dim3(kScanThreads), 0, stream, f, n, temp, out);
+}
+
+// ------------------------------------------------------------------ bitmask copy
+// dst bit i = src bit (i + begin_bit); bits past `bits` are cleared
+// (cpp/src/bitmask/null_mask.cu:332-347).
+void launch_copy_bitmask(uint32_t* dst, const uint32_t* src, int32_t begin_bit, int32_t bits, hipStream_t stream);
+
+void launch_fill_u32(uint32_t* dst, uint32_t value, int64_t count, hipStream_t stream);
+
+}  // namespace nvtext_amd

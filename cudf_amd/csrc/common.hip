@@ -1,0 +1,112 @@
+// Host-side plumbing shared by the entry points: status text, allocator adaptor,
+// bitmask copy, fills, the middle stage of the device-wide scan and the small
+// C-ABI utilities (version, last error, result release).
+#include "common.cuh"
+
+#include <cstring>
+
+namespace nvtext_amd {
+
+namespace {
+thread_local std::string g_last_error;
+}
+
+void set_last_error(const char* msg) { g_last_error = msg ? msg : ""; }
+
+nvtext_amd_status fail(nvtext_amd_status st, const char* msg)
+{
+  set_last_error(msg);
+  return st;
+}
+
+void* Mr::allocate(size_t bytes) const
+{
+  if (bytes == 0) return nullptr;
+  if (a && a->allocate) return a->allocate(a->ctx, bytes, stream);
+  void* p = nullptr;
+  if (hipMallocAsync(&p, bytes, stream) != hipSuccess) return nullptr;
+  return p;
+}
+
+void Mr::deallocate(void* p, size_t bytes) const
+{
+  if (!p) return;
+  if (a && a->deallocate) {
+    a->deallocate(a->ctx, p, bytes, stream);
+    return;
+  }
+  (void)hipFreeAsync(p, stream);
+}
+
+__global__ void __launch_bounds__(kScanThreads) scan_tile_offsets_kernel(uint64_t* tile_sums, int64_t ntiles)
+{
+  __shared__ uint64_t lds[kScanThreads / kWave + 1];
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < ntiles; base += kScanThreads) {
+    int64_t const i  = base + threadIdx.x;
+    uint64_t const v = (i < ntiles) ? tile_sums[i] : 0;
+    uint64_t total;
+    uint64_t const ex = block_exclusive_scan64<kScanThreads>(v, lds, &total);
+    if (i < ntiles) tile_sums[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) tile_sums[ntiles] = carry;
+}
+
+namespace {
+__global__ void copy_bitmask_kernel(uint32_t* dst, const uint32_t* src, int32_t begin_bit, int32_t bits, int32_t words)
+{
+  int32_t const w = blockIdx.x * blockDim.x + threadIdx.x;
+  if (w >= words) return;
+  int64_t const first = static_cast<int64_t>(begin_bit) + static_cast<int64_t>(w) * 32;
+  int64_t const sw    = first >> 5;
+  int const sh        = static_cast<int>(first & 31);
+  int64_t const last_src_word = (static_cast<int64_t>(begin_bit) + bits - 1) >> 5;
+  uint32_t v = src[sw] >> sh;
+  if (sh != 0 && sw + 1 <= last_src_word) v |= src[sw + 1] << (32 - sh);
+  int32_t const remaining = bits - w * 32;
+  if (remaining < 32) v &= (1u << remaining) - 1u;
+  dst[w] = v;
+}
+
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, int64_t count)
+{
+  int64_t const stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) dst[i] = value;
+}
+}  // namespace
+
+void launch_copy_bitmask(uint32_t* dst, const uint32_t* src, int32_t begin_bit, int32_t bits, hipStream_t stream)
+{
+  int32_t const words = (bits + 31) / 32;
+  if (words == 0) return;
+  hipLaunchKernelGGL(copy_bitmask_kernel, dim3((words + 255) / 256), dim3(256), 0, stream, dst, src, begin_bit, bits, words);
+}
+
+void launch_fill_u32(uint32_t* dst, uint32_t value, int64_t count, hipStream_t stream)
+{
+  if (count <= 0) return;
+  int64_t blocks = (count + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, value, count);
+}
+
+}  // namespace nvtext_amd
+
+extern "C" {
+
+int32_t nvtext_amd_version(void) { return 100; }
+
+const char* nvtext_amd_last_error(void) { return nvtext_amd::g_last_error.c_str(); }
+
+void nvtext_amd_list_column_free(nvtext_amd_list_column* col, void* stream, const nvtext_amd_allocator* mr)
+{
+  if (!col) return;
+  nvtext_amd::Mr m{mr, static_cast<hipStream_t>(stream)};
+  m.deallocate(col->offsets, col->offsets_bytes);
+  m.deallocate(col->child, col->child_bytes);
+  m.deallocate(col->null_mask, col->null_mask_bytes);
+  std::memset(col, 0, sizeof(*col));
+}
+
+}  // extern "C"

@@ -1,0 +1,445 @@
+// minhash / minhash64 for gfx950.
+//
+// Replaces the reference's three-kernel pipeline (cpp/src/text/minhash.cu:87-157 seed
+// hashes into a chars-sized temporary, 281-376 permutation kernel re-reading it,
+// 390-424 size partitioning) with one fused pass and no chars-sized temporary:
+//
+//   * a wavefront owns a section of a row.  Per 256-position tile it stages the bytes
+//     in LDS (coalesced aligned dword loads), hashes the windows with lanes <-> window
+//     starts, and compacts the hashes into LDS;
+//   * it then switches to lanes <-> parameters: every lane keeps K (a, b) pairs and
+//     K running minima in registers and streams the tile's hashes through LDS
+//     broadcast reads, so the inner loop is v_mad_u64_u32 + v_min only;
+//   * the 4 wavefronts of a workgroup split the first 16 KiB of a row and combine in
+//     LDS (plain store); the rest of a longer row is covered by extra workgroups that
+//     merge with atomic min, so no output pre-initialisation is needed.
+//
+// Null rows get no output slot (the reference drops them with purge_nonempty_nulls,
+// minhash.cu:626-628), empty rows are all zeros (minhash.cu:318).
+#include "common.cuh"
+#include "murmur.cuh"
+
+#include <limits>
+
+namespace nvtext_amd {
+namespace {
+
+constexpr int kWaves     = 4;                  // wavefronts per workgroup
+constexpr int kThreads   = kWaves * kWave;     // 256
+constexpr int kTile      = 256;                // window starts per wavefront tile
+constexpr int kHalo      = 128;                // bytes staged past the tile (windows up to 32 4-byte chars)
+constexpr int kTileWords = (kTile + kHalo + 4 + 24) / 4;  // +4 misalignment, +24 over-read of the hash tail
+constexpr int kSpan      = 16384;              // bytes of a row handled by one workgroup
+
+template <typename T>
+struct HashTraits;
+template <>
+struct HashTraits<uint32_t> {
+  template <typename Src>
+  static __device__ __forceinline__ uint32_t hash(Src const& src, uint32_t len, uint32_t seed)
+  {
+    return murmur3_x86_32(src, len, seed);
+  }
+  // minhash.cu:350-351 in uint32 arithmetic: the product and sum wrap mod 2^32, after
+  // which "% (2^61-1)" and "& max" change nothing.
+  static __device__ __forceinline__ uint32_t permute(uint32_t hv, uint32_t a, uint32_t b) { return hv * a + b; }
+};
+template <>
+struct HashTraits<uint64_t> {
+  template <typename Src>
+  static __device__ __forceinline__ uint64_t hash(Src const& src, uint32_t len, uint64_t seed)
+  {
+    return murmur3_x64_128_lo(src, len, seed);  // minhash.cu:138: first word of the 128-bit hash
+  }
+  // ((hv*a + b) mod 2^64) % (2^61-1): x = q*2^61 + r with q <= 7, so r + q <= p + 7 and one
+  // conditional subtraction finishes the reduction.
+  static __device__ __forceinline__ uint64_t permute(uint64_t hv, uint64_t a, uint64_t b)
+  {
+    constexpr uint64_t p = (1ull << 61) - 1;
+    uint64_t const x     = hv * a + b;
+    uint64_t const y     = (x & p) + (x >> 61);
+    return y >= p ? y - p : y;
+  }
+};
+
+template <typename T>
+struct WaveLds {
+  uint32_t bytes[kTileWords];
+  alignas(16) T hashes[kTile + 4];
+};
+
+// Stage row bytes [base, base+len) into dst; returns the byte offset of `base` inside it.
+// Only aligned dwords that overlap the range are read.  *all_ascii: no byte of the range
+// has its top bit set (wave-uniform).
+__device__ __forceinline__ uint32_t stage_bytes(const uint8_t* row, int64_t base, uint32_t len, uint32_t* dst, int lane, bool* all_ascii)
+{
+  const uint8_t* g   = row + base;
+  uint32_t const mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(g) & 3u);
+  const uint32_t* ap = reinterpret_cast<const uint32_t*>(g - mis);
+  uint32_t const end = mis + len;  // exclusive byte offset inside dst
+  uint32_t const nw  = (end + 3u) >> 2;
+  uint32_t hibits    = 0;
+  for (uint32_t i = lane; i < nw; i += kWave) {
+    uint32_t const v = ap[i];
+    dst[i]           = v;
+    uint32_t keep    = 0xffffffffu;
+    if (i == 0) keep <<= 8 * mis;                                    // bytes before the range
+    if (4 * i + 4 > end) keep &= (1u << (8 * (end - 4 * i))) - 1u;    // bytes after the range
+    hibits |= v & keep & 0x80808080u;
+  }
+  *all_ascii = ballot64(hibits != 0) == 0;
+  return mis;
+}
+
+// Decides whether a window starts at this position and how many bytes it hashes
+// (cpp/src/text/minhash.cu:120-133 with cpp/include/cudf/strings/string_view.cuh:67-80).
+// `remaining` = row bytes from this position on; `readable` = bytes of them reachable through src.
+template <typename Src>
+__device__ __forceinline__ bool window_at(Src const& src, int64_t remaining, uint32_t readable, bool first, bool all_ascii, int32_t width,
+                                          uint32_t* hlen)
+{
+  if (all_ascii) {
+    if (remaining >= width) {
+      *hlen = static_cast<uint32_t>(width);
+      return true;
+    }
+    *hlen = static_cast<uint32_t>(remaining);
+    return first;
+  }
+  if (is_utf8_continuation(src.byte(0))) return false;
+  uint32_t bytes = 0, j = 0;
+  int32_t left = width;
+  while (left > 0 && j < readable) {  // byte-wise, as the reference walks
+    int const w = bytes_in_utf8_byte(src.byte(j));
+    left -= (w != 0);
+    bytes += w;
+    ++j;
+  }
+  // a malformed trailing lead byte may declare more bytes than the row holds: clamp to the row
+  *hlen = static_cast<uint32_t>(min(static_cast<int64_t>(bytes), remaining));
+  return first || left <= 0;
+}
+
+// Folds `count` compacted hashes (padded here to a multiple of 4) into m[K]; lanes <-> parameters.
+template <typename T, int K>
+__device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane)
+{
+  using H = HashTraits<T>;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (count == 0) return;
+  // a duplicate never changes a minimum
+  uint32_t const padded = (count + 3u) & ~3u;
+  if (lane < static_cast<int>(padded - count)) lds.hashes[count + lane] = lds.hashes[0];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (uint32_t i = 0; i < padded; i += 4) {
+    T const h0 = lds.hashes[i], h1 = lds.hashes[i + 1], h2 = lds.hashes[i + 2], h3 = lds.hashes[i + 3];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      T const r0 = H::permute(h0, a[k], b[k]);
+      T const r1 = H::permute(h1, a[k], b[k]);
+      T const r2 = H::permute(h2, a[k], b[k]);
+      T const r3 = H::permute(h3, a[k], b[k]);
+      m[k]       = min(min(min(m[k], r0), min(r1, r2)), r3);
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Processes the window starts [s_begin, s_end) of one row with one wavefront and folds the
+// permuted hashes into m[K].  Lane l owns parameters chunk_base + l + 64*k.
+template <typename T, int K>
+__device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, int64_t s_begin, int64_t s_end, T seed, int32_t width,
+                                                const T (&a)[K], const T (&b)[K], T (&m)[K], WaveLds<T>& lds, int lane)
+{
+  using H = HashTraits<T>;
+  if (static_cast<int64_t>(width) * 4 <= kHalo) {
+    // usual case: a window (<= 4*width bytes) fits the halo staged behind every tile
+    uint32_t const halo = static_cast<uint32_t>(width) * 4u;
+    for (int64_t base = s_begin; base < s_end; base += kTile) {
+      uint32_t const cnt = static_cast<uint32_t>(min(static_cast<int64_t>(kTile), s_end - base));
+      uint32_t const len = static_cast<uint32_t>(min(n - base, static_cast<int64_t>(cnt + halo)));
+      bool all_ascii;
+      uint32_t const mis = stage_bytes(row, base, len, lds.bytes, lane, &all_ascii);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      uint32_t count = 0;  // compacted hashes so far (wave-uniform)
+      for (uint32_t q = 0; q < cnt; q += kWave) {
+        uint32_t const p = q + lane;
+        bool valid       = false;
+        T hv             = 0;
+        if (p < cnt) {
+          int64_t const gpos = base + p;
+          WordSrc const src{lds.bytes, mis + p};
+          uint32_t hlen;
+          valid = window_at(src, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen);
+          if (valid) {
+            hv = H::hash(src, hlen, seed);
+            hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
+          }
+        }
+        uint64_t const vm = ballot64(valid);
+        if (valid) lds.hashes[count + lanes_below(vm)] = hv;
+        count += static_cast<uint32_t>(__builtin_popcountll(vm));
+      }
+      fold_hashes<T, K>(lds, count, a, b, m, lane);
+    }
+  } else {
+    // very wide windows: 64 starts at a time, bytes read straight from global memory
+    for (int64_t base = s_begin; base < s_end; base += kWave) {
+      int64_t const gpos = base + lane;
+      bool valid         = false;
+      T hv               = 0;
+      if (gpos < s_end) {
+        int64_t const remaining = n - gpos;
+        BoundedSrc const src{row + gpos, remaining};
+        uint32_t hlen;
+        uint32_t const readable = static_cast<uint32_t>(min(remaining, static_cast<int64_t>(width) * 4));
+        valid = window_at(src, remaining, readable, gpos == 0, false, width, &hlen);
+        if (valid) {
+          hv = H::hash(src, hlen, seed);
+          hv = hv < 1 ? T{1} : hv;
+        }
+      }
+      uint64_t const vm = ballot64(valid);
+      if (valid) lds.hashes[lanes_below(vm)] = hv;
+      fold_hashes<T, K>(lds, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
+    }
+  }
+}
+
+template <typename T, int K>
+__device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P, int32_t chunk_base, int lane, T (&a)[K], T (&b)[K], T (&m)[K])
+{
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    int32_t const j = chunk_base + lane + kWave * k;
+    a[k]            = j < P ? pa[j] : T{0};
+    b[k]            = j < P ? pb[j] : T{0};
+    m[k]            = std::numeric_limits<T>::max();
+  }
+}
+
+// One workgroup per (row, parameter chunk): the first kSpan bytes of the row.
+template <typename T, int K>
+__global__ void __launch_bounds__(kThreads) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
+                                                                int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out)
+{
+  __shared__ WaveLds<T> lds[kWaves];
+  __shared__ T red[kWaves][K * kWave];
+
+  int64_t const r = blockIdx.x;
+  if (!col.valid(r)) return;
+  int32_t const chunk_base = blockIdx.y * (K * kWave);
+  int64_t const o          = col.off(r);
+  int64_t const n          = col.off(r + 1) - o;
+  T* dst                   = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
+  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
+  if (n == 0) {
+    for (int j = threadIdx.x; j < in_chunk; j += kThreads) dst[j] = T{0};
+    return;
+  }
+  int const lane = lane_id();
+  int const wave = threadIdx.x / kWave;
+  T a[K], b[K], m[K];
+  load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
+
+  int64_t const span = min(n, static_cast<int64_t>(kSpan));
+  int64_t sec        = (span + kWaves - 1) / kWaves;
+  sec                = (sec + kWave - 1) / kWave * kWave;
+  int64_t const sb   = min(span, wave * sec);
+  int64_t const se   = min(span, sb + sec);
+  if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane);
+
+#pragma unroll
+  for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+  __syncthreads();
+  for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
+    T v = red[0][j];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
+    dst[j] = v;
+  }
+}
+
+// Extra parts of rows longer than kSpan: task t covers bytes [part*kSpan, (part+1)*kSpan) of its row.
+// extra_prefix[r] = number of extra parts in rows < r (rows+1 entries).
+template <typename T, int K>
+__global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
+                                                                 int32_t width, const int32_t* __restrict__ out_offsets,
+                                                                 const uint32_t* __restrict__ extra_prefix, T* __restrict__ out)
+{
+  __shared__ WaveLds<T> lds[kWaves];
+  __shared__ T red[kWaves][K * kWave];
+  uint32_t const total     = extra_prefix[col.size];
+  int32_t const chunk_base = blockIdx.y * (K * kWave);
+  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
+  int const lane           = lane_id();
+  int const wave           = threadIdx.x / kWave;
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+    // last row r with extra_prefix[r] <= t
+    int64_t lo = 0, hi = col.size;
+    while (hi - lo > 1) {
+      int64_t const mid = (lo + hi) >> 1;
+      if (extra_prefix[mid] <= t) lo = mid; else hi = mid;
+    }
+    int64_t const r    = lo;
+    int64_t const part = static_cast<int64_t>(t - extra_prefix[r]) + 1;
+    int64_t const o    = col.off(r);
+    int64_t const n    = col.off(r + 1) - o;
+    T a[K], b[K], m[K];
+    load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
+    int64_t const pb0  = part * kSpan;
+    int64_t const pe0  = min(n, pb0 + kSpan);
+    int64_t const sec  = kSpan / kWaves;
+    int64_t const sb   = min(pe0, pb0 + wave * sec);
+    int64_t const se   = min(pe0, sb + sec);
+    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+    __syncthreads();
+    T* dst = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
+    for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
+      T v = red[0][j];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
+      if (v != std::numeric_limits<T>::max()) atomicMin(&dst[j], v);
+    }
+  }
+}
+
+struct ValidTimesP {
+  ColView col;
+  int32_t P;
+  __device__ uint64_t operator()(int64_t i) const { return col.valid(i) ? static_cast<uint64_t>(P) : 0; }
+};
+
+struct ExtraParts {
+  ColView col;
+  __device__ uint64_t operator()(int64_t i) const
+  {
+    if (!col.valid(i)) return 0;
+    int64_t const n = col.off(i + 1) - col.off(i);
+    return n > kSpan ? static_cast<uint64_t>((n + kSpan - 1) / kSpan - 1) : 0;
+  }
+};
+
+__global__ void uniform_offsets_kernel(int32_t* out, int32_t rows, int32_t P)
+{
+  int64_t const i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i <= rows) out[i] = static_cast<int32_t>(i * P);
+}
+
+template <typename T, int K>
+void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, const int32_t* offsets,
+                    const uint32_t* extra_prefix, T* child, hipStream_t stream)
+{
+  int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
+  dim3 grid(static_cast<unsigned>(v.size), static_cast<unsigned>(chunks));
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
+  dim3 grid2(4096, static_cast<unsigned>(chunks));
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_extra_kernel<T, K>), grid2, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets,
+                     extra_prefix, child);
+}
+
+template <typename T>
+nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, const T* a, const T* b, int64_t a_count, int64_t b_count,
+                               int32_t width, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out, int32_t type_id)
+{
+  if (!input || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  *out = nvtext_amd_list_column{};
+  // cpp/src/text/minhash.cu:435-446, same order and messages
+  if (width < 2) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameter width should be an integer value of 2 or greater");
+  if (a_count <= 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B cannot be empty");
+  if (a_count != b_count) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B should have the same number of elements");
+  if (static_cast<uint64_t>(input->size) * static_cast<uint64_t>(a_count) >= static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
+    return fail(NVTEXT_AMD_OVERFLOW, "The number of parameters times the number of input rows exceeds the column size limit");
+  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
+  if (input->null_count > 0 && !input->null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
+
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Mr mr{mr_, stream};
+  int32_t const rows = input->size;
+  int32_t const P    = static_cast<int32_t>(a_count);
+  out->child_type    = type_id;
+  out->size          = rows;
+  out->null_count    = input->null_count;
+  out->offsets_size  = rows + 1;
+  out->offsets_bytes = static_cast<size_t>(rows + 1) * sizeof(int32_t);
+  out->offsets       = static_cast<int32_t*>(mr.allocate(out->offsets_bytes));
+  if (!out->offsets) return fail(NVTEXT_AMD_ALLOC_FAILED, "offsets allocation failed");
+  if (rows == 0) {  // minhash.cu:449 then 616: zero rows, offsets = [0], empty child
+    launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, 1, stream);
+    NVTEXT_HIP_TRY(hipGetLastError());
+    return NVTEXT_AMD_SUCCESS;
+  }
+  out->child_size  = static_cast<int64_t>(rows - input->null_count) * P;
+  out->child_bytes = static_cast<size_t>(out->child_size) * sizeof(T);
+  if (out->child_bytes) {
+    out->child = mr.allocate(out->child_bytes);
+    if (!out->child) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
+    }
+  }
+  if (input->null_mask) {  // copy_bitmask(input): cpp/src/bitmask/null_mask.cu:381-391
+    out->null_mask_bytes = mask_alloc_bytes(rows);
+    out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
+    if (!out->null_mask) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
+    }
+    launch_copy_bitmask(out->null_mask, input->null_mask, input->offset, rows, stream);
+  }
+
+  ColView const v = make_view(*input);
+  Temp scan_tmp(mr, scan_temp_bytes(rows));
+  Temp extra(mr, static_cast<size_t>(rows + 1) * sizeof(uint32_t));
+  if (!scan_tmp.ok() || !extra.ok()) {
+    nvtext_amd_list_column_free(out, stream_, mr_);
+    return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+  }
+  if (v.use_mask) {
+    device_exclusive_scan(ValidTimesP{v, P}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
+  } else {
+    hipLaunchKernelGGL(uniform_offsets_kernel, dim3((rows + 1 + 255) / 256), dim3(256), 0, stream, out->offsets, rows, P);
+  }
+  device_exclusive_scan(ExtraParts{v}, static_cast<int64_t>(rows), extra.as<uint32_t>(), scan_tmp.as<uint64_t>(), stream);
+
+  T* child = static_cast<T*>(out->child);
+  if (out->child_size > 0) {
+    if (P > 2 * kWave)
+      launch_kernels<T, 4>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
+    else if (P > kWave)
+      launch_kernels<T, 2>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
+    else
+      launch_kernels<T, 1>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
+  }
+  NVTEXT_HIP_TRY(hipGetLastError());
+  return NVTEXT_AMD_SUCCESS;
+}
+
+}  // namespace
+}  // namespace nvtext_amd
+
+extern "C" {
+
+nvtext_amd_status nvtext_amd_minhash(const nvtext_amd_strings_column* input, uint32_t seed, const uint32_t* a, const uint32_t* b, int64_t a_count,
+                                     int64_t b_count, int32_t width, void* stream, const nvtext_amd_allocator* mr, nvtext_amd_list_column* out)
+{
+  return nvtext_amd::minhash_impl<uint32_t>(input, seed, a, b, a_count, b_count, width, stream, mr, out, NVTEXT_AMD_TYPE_UINT32);
+}
+
+nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input, uint64_t seed, const uint64_t* a, const uint64_t* b, int64_t a_count,
+                                       int64_t b_count, int32_t width, void* stream, const nvtext_amd_allocator* mr, nvtext_amd_list_column* out)
+{
+  return nvtext_amd::minhash_impl<uint64_t>(input, seed, a, b, a_count, b_count, width, stream, mr, out, NVTEXT_AMD_TYPE_UINT64);
+}
+
+}  // extern "C"

@@ -1,0 +1,237 @@
+"""Python host side of the nvtext hot path, over the C ABI.
+
+Mirrors the call contract of pylibcudf's bindings for this path
+(python/pylibcudf/pylibcudf/nvtext/minhash.pyx:33-141,
+ python/pylibcudf/pylibcudf/nvtext/wordpiece_tokenize.pyx:22-97): same function names,
+argument order and error behaviour (std::invalid_argument -> ValueError,
+std::overflow_error -> OverflowError, as libcudf_exception_handler maps them).
+
+PyTorch is used only as the owner of device memory and the provider of the HIP stream;
+every computation happens in libnvtext_amd.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Dict, Optional
+
+import numpy as np
+
+from . import _capi
+from .arrow_host import HostListColumn, HostStringsColumn
+
+
+def _torch():
+    import torch
+    return torch
+
+
+class _TorchAllocator:
+    """nvtext_amd_allocator backed by torch's caching allocator (stream-ordered on the
+    current stream).  Buffers handed back in a result stay alive in `take()`n tensors."""
+
+    def __init__(self):
+        self.live: Dict[int, object] = {}
+        torch = _torch()
+
+        def _alloc(ctx, nbytes, stream):
+            try:
+                t = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda")
+            except Exception:  # out of memory -> NULL, reported as ALLOC_FAILED
+                return None
+            self.live[t.data_ptr()] = t
+            return t.data_ptr()
+
+        def _free(ctx, ptr, nbytes, stream):
+            self.live.pop(int(ptr) if ptr else 0, None)
+
+        self._alloc_cb = _capi.ALLOC_FN(_alloc)
+        self._free_cb = _capi.DEALLOC_FN(_free)
+        self.struct = _capi.Allocator(None, self._alloc_cb, self._free_cb)
+
+    def take(self, ptr):
+        return self.live.pop(int(ptr), None) if ptr else None
+
+
+_allocator: Optional[_TorchAllocator] = None
+
+
+def _mr() -> _TorchAllocator:
+    global _allocator
+    if _allocator is None:
+        _allocator = _TorchAllocator()
+    return _allocator
+
+
+def _stream_handle() -> int:
+    return int(_torch().cuda.current_stream().cuda_stream)
+
+
+def _raise(status: int):
+    msg = _capi.load().nvtext_amd_last_error().decode("utf-8", "replace")
+    if status == _capi.INVALID_ARGUMENT:
+        raise ValueError(msg)
+    if status == _capi.OVERFLOW:
+        raise OverflowError(msg)
+    if status == _capi.ALLOC_FAILED:
+        raise MemoryError(msg)
+    raise RuntimeError(msg)
+
+
+@dataclass
+class DeviceStringsColumn:
+    """Arrow-layout strings column in HBM (torch tensors own the buffers)."""
+    chars: object            # uint8 tensor
+    offsets: object          # int32 / int64 tensor (parent_size + 1 entries) or None
+    mask: object             # int32 tensor holding the uint32 validity words, or None
+    size: int
+    offset: int = 0
+    null_count: int = 0
+
+    @staticmethod
+    def from_host(h: HostStringsColumn, device: str = "cuda") -> "DeviceStringsColumn":
+        torch = _torch()
+        chars = torch.from_numpy(np.ascontiguousarray(h.chars)).to(device)
+        offsets = torch.from_numpy(np.ascontiguousarray(h.offsets)).to(device) if h.offsets.size else None
+        mask = None
+        if h.mask is not None:
+            mask = torch.from_numpy(np.ascontiguousarray(h.mask).view(np.int32)).to(device)
+        return DeviceStringsColumn(chars, offsets, mask, int(h.size), int(h.offset), int(h.null_count))
+
+    def slice(self, lo: int, hi: int, null_count: int) -> "DeviceStringsColumn":
+        return DeviceStringsColumn(self.chars, self.offsets, self.mask, hi - lo, self.offset + lo, null_count)
+
+    def _c(self) -> _capi.StringsColumn:
+        torch = _torch()
+        is64 = 0
+        if self.offsets is not None:
+            if self.offsets.dtype == torch.int64:
+                is64 = 1
+            elif self.offsets.dtype != torch.int32:
+                raise TypeError("offsets must be int32 or int64")
+        return _capi.StringsColumn(
+            self.chars.data_ptr() if self.chars is not None and self.chars.numel() else None,
+            self.offsets.data_ptr() if self.offsets is not None else None,
+            is64,
+            self.mask.data_ptr() if self.mask is not None else None,
+            self.size, self.offset, self.null_count)
+
+
+@dataclass
+class DeviceListColumn:
+    """LIST result in HBM.  offsets: int32 tensor; child: raw tensor viewed as child_dtype."""
+    offsets: object
+    child: object
+    mask: object
+    size: int
+    null_count: int
+    child_dtype: np.dtype
+    child_size: int
+
+    def to_host(self) -> HostListColumn:
+        torch = _torch()
+        torch.cuda.current_stream().synchronize()
+        offsets = (self.offsets.cpu().numpy().view(np.int32)[: self.size + 1].copy()
+                   if self.offsets is not None else np.zeros(0, np.int32))
+        if self.child is not None:
+            child = self.child.cpu().numpy().view(self.child_dtype)[: self.child_size].copy()
+        else:
+            child = np.zeros(0, self.child_dtype)
+        mask = None
+        if self.mask is not None:
+            mask = self.mask.cpu().numpy().view(np.uint32)[: (self.size + 31) // 32].copy()
+        return HostListColumn(offsets, child, mask, self.size, self.null_count)
+
+
+_DTYPES = {_capi.TYPE_INT32: np.dtype(np.int32), _capi.TYPE_UINT32: np.dtype(np.uint32),
+           _capi.TYPE_UINT64: np.dtype(np.uint64)}
+
+
+def _wrap(out: _capi.ListColumn) -> DeviceListColumn:
+    mr = _mr()
+    return DeviceListColumn(mr.take(out.offsets), mr.take(out.child), mr.take(out.null_mask),
+                            int(out.size), int(out.null_count), _DTYPES[int(out.child_type)], int(out.child_size))
+
+
+def _param_tensor(x, np_dtype):
+    """a/b parameters: a device tensor (raw bits of uint32/uint64) or anything numpy can read."""
+    torch = _torch()
+    if isinstance(x, torch.Tensor):
+        want = 4 if np_dtype == np.uint32 else 8
+        if x.element_size() != want:
+            raise TypeError(f"parameter tensor must have {want}-byte elements")
+        return x.contiguous()
+    arr = np.ascontiguousarray(x)
+    if arr.dtype != np_dtype:
+        raise TypeError(f"parameters must be {np.dtype(np_dtype).name}")
+    signed = np.int32 if np_dtype == np.uint32 else np.int64
+    return torch.from_numpy(arr.view(signed)).to("cuda")
+
+
+def minhash(input: DeviceStringsColumn, seed: int, a, b, width: int) -> DeviceListColumn:
+    """nvtext::minhash (cpp/include/nvtext/minhash.hpp:62-69); pylibcudf minhash.pyx:33-84."""
+    L = _capi.load()
+    if not (0 <= int(seed) < 2**32):
+        raise ValueError("seed must fit uint32")
+    ta, tb = _param_tensor(a, np.uint32), _param_tensor(b, np.uint32)
+    out = _capi.ListColumn()
+    col = input._c()
+    st = L.nvtext_amd_minhash(C.byref(col), int(seed), ta.data_ptr() if ta.numel() else None,
+                              tb.data_ptr() if tb.numel() else None, ta.numel(), tb.numel(), int(width),
+                              _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    return _wrap(out)
+
+
+def minhash64(input: DeviceStringsColumn, seed: int, a, b, width: int) -> DeviceListColumn:
+    """nvtext::minhash64 (cpp/include/nvtext/minhash.hpp:109-116); pylibcudf minhash.pyx:88-141."""
+    L = _capi.load()
+    if not (0 <= int(seed) < 2**64):
+        raise ValueError("seed must fit uint64")
+    ta, tb = _param_tensor(a, np.uint64), _param_tensor(b, np.uint64)
+    out = _capi.ListColumn()
+    col = input._c()
+    st = L.nvtext_amd_minhash64(C.byref(col), int(seed), ta.data_ptr() if ta.numel() else None,
+                                tb.data_ptr() if tb.numel() else None, ta.numel(), tb.numel(), int(width),
+                                _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    return _wrap(out)
+
+
+class WordPieceVocabulary:
+    """nvtext::wordpiece_vocabulary (cpp/include/nvtext/wordpiece_tokenize.hpp:26-66);
+    pylibcudf wordpiece_tokenize.pyx:22-47."""
+
+    def __init__(self, vocab: DeviceStringsColumn):
+        L = _capi.load()
+        h = C.c_void_p()
+        col = vocab._c()
+        st = L.nvtext_amd_wordpiece_vocabulary_create(C.byref(col), _stream_handle(), C.byref(_mr().struct), C.byref(h))
+        if st != _capi.SUCCESS:
+            _raise(st)
+        self._h = h
+        self.unk_id = int(L.nvtext_amd_wordpiece_vocabulary_unk_id(h))
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            try:
+                _capi.load().nvtext_amd_wordpiece_vocabulary_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+
+def wordpiece_tokenize(input: DeviceStringsColumn, vocabulary: WordPieceVocabulary, max_words_per_row: int = 0) -> DeviceListColumn:
+    """nvtext::wordpiece_tokenize (cpp/include/nvtext/wordpiece_tokenize.hpp:68-111);
+    pylibcudf wordpiece_tokenize.pyx:51-97."""
+    L = _capi.load()
+    out = _capi.ListColumn()
+    col = input._c()
+    st = L.nvtext_amd_wordpiece_tokenize(C.byref(col), vocabulary._h, int(max_words_per_row), _stream_handle(),
+                                         C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    return _wrap(out)

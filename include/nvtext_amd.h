@@ -1,0 +1,153 @@
+/*
+ * nvtext_amd.h -- C ABI of the MI355X (gfx950) implementation of libcudf's nvtext
+ * text-dedup hot path: minhash / minhash64 over character windows and
+ * wordpiece_tokenize with its wordpiece_vocabulary.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" is HIP device memory
+ * that must stay valid until the work queued on `stream` has completed.  All work is
+ * queued on the caller's stream; results are valid once that stream is synchronised
+ * (wordpiece_tokenize synchronises it once internally to learn the token total).
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the
+ * cudf source tree).
+ */
+#ifndef NVTEXT_AMD_H
+#define NVTEXT_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  The C++ shim rethrows them as the reference's exception types
+ * (cpp/include/cudf/utilities/error.hpp:35-103,182-199,280-284). */
+typedef enum nvtext_amd_status {
+  NVTEXT_AMD_SUCCESS          = 0,
+  NVTEXT_AMD_INVALID_ARGUMENT = 1, /* std::invalid_argument */
+  NVTEXT_AMD_OVERFLOW         = 2, /* std::overflow_error   */
+  NVTEXT_AMD_LOGIC_ERROR      = 3, /* cudf::logic_error     */
+  NVTEXT_AMD_DEVICE_ERROR     = 4, /* cudf::cuda_error      */
+  NVTEXT_AMD_ALLOC_FAILED     = 5  /* std::bad_alloc        */
+} nvtext_amd_status;
+
+/* cudf::type_id values used by this path (cpp/include/cudf/types.hpp:185-217). */
+enum {
+  NVTEXT_AMD_TYPE_INT32  = 3,
+  NVTEXT_AMD_TYPE_UINT32 = 7,
+  NVTEXT_AMD_TYPE_UINT64 = 8
+};
+
+/* Non-owning view of an Arrow-layout strings column as libcudf lays it out
+ * (cudf::strings_column_view, cpp/include/cudf/strings/strings_column_view.hpp:27-114;
+ *  cudf::column_view, cpp/include/cudf/column/column_view.hpp:44-293).
+ * Row i is chars[offsets[i+offset] .. offsets[i+offset+1]); bit (i+offset) of
+ * null_mask (uint32 words, LSB first) is its validity. */
+typedef struct nvtext_amd_strings_column {
+  const char*     chars;            /* device; may be NULL when there are no bytes            */
+  const void*     offsets;          /* device; element 0 of the offsets child; NULL if size 0 */
+  int32_t         offsets_is_int64; /* 0: int32 offsets, 1: int64 offsets                     */
+  const uint32_t* null_mask;        /* device or NULL                                         */
+  int32_t         size;             /* rows in this view                                      */
+  int32_t         offset;           /* first row of the view inside the parent buffers        */
+  int32_t         null_count;       /* nulls in the view (>= 0)                               */
+} nvtext_amd_strings_column;
+
+/* Stream-ordered allocator for results and temporaries; the counterpart of
+ * rmm::device_async_resource_ref in the reference signatures.  A NULL allocator (or
+ * NULL members) selects hipMallocAsync / hipFreeAsync on `stream`. */
+typedef struct nvtext_amd_allocator {
+  void* ctx;
+  void* (*allocate)(void* ctx, size_t bytes, void* stream);
+  void  (*deallocate)(void* ctx, void* ptr, size_t bytes, void* stream);
+} nvtext_amd_allocator;
+
+/* Owning result: a LIST column (cudf::make_lists_column,
+ * cpp/src/lists/lists_column_factories.cu:106-129).  Buffers come from the allocator
+ * given to the call and belong to the caller afterwards. */
+typedef struct nvtext_amd_list_column {
+  int32_t   size;            /* rows                                                        */
+  int32_t   null_count;
+  int32_t   child_type;      /* NVTEXT_AMD_TYPE_*                                           */
+  int32_t   offsets_size;    /* size+1, or 0 for the canonical empty list column            */
+  int32_t*  offsets;         /* device, offsets_size entries (NULL if 0)                    */
+  void*     child;           /* device, child_size elements of child_type (NULL if 0)       */
+  int64_t   child_size;
+  uint32_t* null_mask;       /* device or NULL; bit i = row i                               */
+  size_t    offsets_bytes;   /* allocation sizes, for deallocate()                          */
+  size_t    child_bytes;
+  size_t    null_mask_bytes;
+} nvtext_amd_list_column;
+
+typedef struct nvtext_amd_wordpiece_vocabulary nvtext_amd_wordpiece_vocabulary;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int32_t nvtext_amd_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* nvtext_amd_last_error(void);
+
+/* Replaces nvtext::minhash (cpp/include/nvtext/minhash.hpp:62-69; cpp/src/text/minhash.cu:691-701).
+ * MurmurHash3_x86_32(seed) of every `width`-character window, permuted by
+ * (hash*a[j]+b[j]) in uint32 arithmetic, minimum per j.  Result: LIST<UINT32>,
+ * param_count values per valid row, none for a null row, zeros for an empty row.
+ * a, b: device arrays of param_count values. */
+nvtext_amd_status nvtext_amd_minhash(const nvtext_amd_strings_column* input,
+                                     uint32_t seed,
+                                     const uint32_t* a,
+                                     const uint32_t* b,
+                                     int64_t a_count,
+                                     int64_t b_count,
+                                     int32_t width,
+                                     void* stream,
+                                     const nvtext_amd_allocator* mr,
+                                     nvtext_amd_list_column* out);
+
+/* Replaces nvtext::minhash64 (cpp/include/nvtext/minhash.hpp:109-116; cpp/src/text/minhash.cu:716-726).
+ * MurmurHash3_x64_128(seed) word 0; permutation ((hash*a+b) mod 2^64) % (2^61-1).  Result: LIST<UINT64>. */
+nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input,
+                                       uint64_t seed,
+                                       const uint64_t* a,
+                                       const uint64_t* b,
+                                       int64_t a_count,
+                                       int64_t b_count,
+                                       int32_t width,
+                                       void* stream,
+                                       const nvtext_amd_allocator* mr,
+                                       nvtext_amd_list_column* out);
+
+/* Replaces nvtext::load_wordpiece_vocabulary / wordpiece_vocabulary::wordpiece_vocabulary
+ * (cpp/include/nvtext/wordpiece_tokenize.hpp:26-66; cpp/src/text/wordpiece_tokenize.cu:213-293).
+ * Token id = row index.  Fails with INVALID_ARGUMENT for an empty vocabulary or one with nulls.
+ * The object owns a device copy of the entries and its lookup tables; it is immutable and
+ * may be shared by concurrent calls. */
+nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_strings_column* vocabulary,
+                                                         void* stream,
+                                                         const nvtext_amd_allocator* mr,
+                                                         nvtext_amd_wordpiece_vocabulary** out);
+
+/* Replaces wordpiece_vocabulary::~wordpiece_vocabulary (cpp/src/text/wordpiece_tokenize.cu:284). */
+void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* vocabulary);
+
+/* Id of "[UNK]" (else "[unk]", else -1): cpp/src/text/wordpiece_tokenize.cu:199-209,273-275. */
+int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* vocabulary);
+
+/* Replaces nvtext::wordpiece_tokenize (cpp/include/nvtext/wordpiece_tokenize.hpp:68-111;
+ * cpp/src/text/wordpiece_tokenize.cu:839-899).  Result: LIST<INT32> of token ids per row.
+ * max_words_per_row == 0 tokenizes every word; > 0 only the first
+ * min(max_words_per_row, row_bytes/2) words of each valid row; < 0 is INVALID_ARGUMENT. */
+nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column* input,
+                                                const nvtext_amd_wordpiece_vocabulary* vocabulary,
+                                                int32_t max_words_per_row,
+                                                void* stream,
+                                                const nvtext_amd_allocator* mr,
+                                                nvtext_amd_list_column* out);
+
+/* Releases the buffers of a result through the allocator that produced them. */
+void nvtext_amd_list_column_free(nvtext_amd_list_column* col, void* stream, const nvtext_amd_allocator* mr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NVTEXT_AMD_H */

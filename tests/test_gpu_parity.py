@@ -1,0 +1,325 @@
+"""GPU parity: the HIP path, called through the C ABI, against the reference's known-answer
+vectors and against the host oracle on seeded inputs.  Bit-exact (integer work)."""
+import numpy as np
+import pytest
+
+from tests import golden_cases as gc
+from tests.golden_cases import strings
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from cudf_amd import nvtext
+    from cudf_amd import _capi
+    _capi.load()  # fails loudly if the HIP library is missing
+    return nvtext
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import pyoracle
+    return pyoracle
+
+
+def dev(nv, host):
+    return nv.DeviceStringsColumn.from_host(host)
+
+
+def assert_same(got, exp, what=""):
+    assert got.size == exp.size, what
+    assert got.null_count == exp.null_count, what
+    assert got.child.dtype == exp.child.dtype, what
+    assert np.array_equal(got.validity(), exp.validity()), what
+    assert got.offsets.size == exp.offsets.size, what
+    assert np.array_equal(got.offsets, exp.offsets), what
+    if not np.array_equal(got.child, exp.child):
+        bad = np.flatnonzero(got.child != exp.child)
+        raise AssertionError(f"{what}: {bad.size} child values differ, first at {bad[:5]}: "
+                             f"got {got.child[bad[:5]]} expected {exp.child[bad[:5]]}")
+
+
+# ----------------------------------------------------------------------------- minhash golden
+@pytest.mark.parametrize("case", gc.minhash_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_minhash_golden(nv, case, dtype):
+    col = dev(nv, strings(case["rows"], dtype))
+    if "expected32" in case:
+        got = nv.minhash(col, case["seed"], np.array(case["a"], np.uint32), np.array(case["b"], np.uint32), case["width"]).to_host()
+        assert gc.expected_list_equal(got.to_pylist(), case["expected32"])
+    if "expected64" in case:
+        got = nv.minhash64(col, case["seed"], np.array(case["a"], np.uint64), np.array(case["b"], np.uint64), case["width"]).to_host()
+        assert gc.expected_list_equal(got.to_pylist(), case["expected64"])
+
+
+def random_rows(rng, n, max_len, utf8=False, p_null=0.05, p_empty=0.05):
+    ascii_alpha = list("abcdefghijklmnopqrstuvwxyz      .,")
+    wide = list("éüñßçøå") + list("漢字仮名日本語中文") + ["😀", "𝄞"]
+    rows = []
+    for _ in range(n):
+        u = rng.random()
+        if u < p_null:
+            rows.append(None)
+            continue
+        if u < p_null + p_empty:
+            rows.append("")
+            continue
+        ln = int(rng.integers(1, max_len))
+        if utf8:
+            pool = ascii_alpha + wide
+            rows.append("".join(rng.choice(pool, ln)))
+        else:
+            rows.append("".join(rng.choice(ascii_alpha, ln)))
+    return rows
+
+
+@pytest.mark.parametrize("utf8", [False, True], ids=["ascii", "utf8"])
+@pytest.mark.parametrize("P,width", [(3, 4), (64, 5), (100, 2), (128, 8), (256, 5), (260, 12)])
+def test_minhash_random_vs_oracle(nv, orc, utf8, P, width):
+    rng = np.random.default_rng(1000 + P + width + int(utf8))
+    rows = random_rows(rng, 300, 700, utf8=utf8)
+    rows += ["a", "ab", "é", "abcde" * 1000, "x" * 255, "y" * 256, "z" * 257, "w" * 1023, "v" * 1025]
+    host = strings(rows)
+    col = dev(nv, host)
+    a32 = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+    b32 = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+    assert_same(nv.minhash(col, 42, a32, b32, width).to_host(), orc.minhash(host, 42, a32, b32, width, nthreads=8), "minhash")
+    a64 = rng.integers(1, 2**64, P, dtype=np.uint64)
+    b64 = rng.integers(0, 2**64, P, dtype=np.uint64)
+    assert_same(nv.minhash64(col, 7, a64, b64, width).to_host(), orc.minhash64(host, 7, a64, b64, width, nthreads=8), "minhash64")
+
+
+def test_minhash_long_rows_cross_workgroups(nv, orc):
+    """Rows longer than one workgroup span (16 KiB) take the multi-workgroup + atomic-min route."""
+    rng = np.random.default_rng(5)
+    words = ["".join(rng.choice(list("abcdefghij"), int(rng.integers(1, 9)))) for _ in range(500)]
+
+    def doc(nbytes):
+        out, ln = [], 0
+        while ln < nbytes:
+            w = words[int(rng.integers(0, len(words)))]
+            out.append(w)
+            ln += len(w) + 1
+        return " ".join(out)[:nbytes]
+
+    rows = [doc(16384), doc(16385), doc(40000), None, "", doc(300000), doc(100), doc(16383), doc(70000) + "é漢" * 3000]
+    host = strings(rows, np.int64)
+    col = dev(nv, host)
+    a32 = rng.integers(1, 2**32, 128, dtype=np.uint64).astype(np.uint32)
+    b32 = rng.integers(0, 2**32, 128, dtype=np.uint64).astype(np.uint32)
+    assert_same(nv.minhash(col, 9, a32, b32, 5).to_host(), orc.minhash(host, 9, a32, b32, 5, nthreads=8), "minhash long")
+    a64 = rng.integers(1, 2**64, 128, dtype=np.uint64)
+    b64 = rng.integers(0, 2**64, 128, dtype=np.uint64)
+    assert_same(nv.minhash64(col, 7, a64, b64, 5).to_host(), orc.minhash64(host, 7, a64, b64, 5, nthreads=8), "minhash64 long")
+
+
+def test_minhash_very_wide_window(nv, orc):
+    """width*4 bytes beyond the staged halo: bytes are read straight from global memory."""
+    rng = np.random.default_rng(6)
+    rows = random_rows(rng, 40, 900, utf8=True) + ["q" * 50, "ab" * 300]
+    host = strings(rows)
+    col = dev(nv, host)
+    a = rng.integers(1, 2**32, 5, dtype=np.uint64).astype(np.uint32)
+    assert_same(nv.minhash(col, 1, a, a, 40).to_host(), orc.minhash(host, 1, a, a, 40), "wide window")
+    a64 = rng.integers(1, 2**64, 5, dtype=np.uint64)
+    assert_same(nv.minhash64(col, 1, a64, a64, 100).to_host(), orc.minhash64(host, 1, a64, a64, 100), "wide window 64")
+
+
+def test_minhash64_reduction_edge(nv, orc):
+    """Parameters that drive (h*a+b) mod 2^64 onto p, p+1.. and 2^64-1 exercise the final subtraction."""
+    p = 2**61 - 1
+    host = strings(["hello world", "abc", "x" * 600])
+    col = dev(nv, host)
+    a = np.array([0, 0, 0, 0, 0, 1, 2**63], np.uint64)
+    b = np.array([p, p + 1, p + 7, 2**64 - 1, p - 1, 0, 2**64 - 1], np.uint64)
+    assert_same(nv.minhash64(col, 0, a, b, 4).to_host(), orc.minhash64(host, 0, a, b, 4), "mod edge")
+
+
+def test_minhash_sliced_and_nulls(nv, orc):
+    rng = np.random.default_rng(8)
+    rows = random_rows(rng, 200, 300, p_null=0.2, p_empty=0.1)
+    host = strings(rows)
+    a = rng.integers(1, 2**32, 64, dtype=np.uint64).astype(np.uint32)
+    for lo, hi in [(0, 200), (3, 150), (33, 97), (64, 128), (199, 200)]:
+        hs = host.slice(lo, hi)
+        ds = dev(nv, host).slice(lo, hi, hs.null_count)
+        assert_same(nv.minhash(ds, 3, a, a, 4).to_host(), orc.minhash(hs, 3, a, a, 4), f"slice {lo}:{hi}")
+
+
+def test_minhash_errors_and_empty(nv):
+    col = dev(nv, strings(["this string intentionally left blank"]))
+    e32, e64 = np.zeros(0, np.uint32), np.zeros(0, np.uint64)
+    with pytest.raises(ValueError):
+        nv.minhash(col, 0, e32, e32, 0)
+    with pytest.raises(ValueError):
+        nv.minhash64(col, 0, e64, e64, 0)
+    with pytest.raises(ValueError):
+        nv.minhash(col, 0, e32, e32, 4)
+    with pytest.raises(ValueError):
+        nv.minhash64(col, 0, e64, e64, 4)
+    with pytest.raises(ValueError):
+        nv.minhash(col, 0, np.ones(3, np.uint32), np.ones(2, np.uint32), 4)
+    big = dev(nv, strings([""] * 50000))
+    with pytest.raises(OverflowError):
+        nv.minhash(big, 0, np.zeros(50000, np.uint32), np.zeros(50000, np.uint32), 4)
+    with pytest.raises(OverflowError):
+        nv.minhash64(big, 0, np.zeros(50000, np.uint64), np.zeros(50000, np.uint64), 4)
+    empty = dev(nv, strings([]))
+    got = nv.minhash(empty, 0, np.ones(3, np.uint32), np.ones(3, np.uint32), 4).to_host()
+    assert got.size == 0 and got.child.size == 0
+    got = nv.minhash64(empty, 0, np.ones(3, np.uint64), np.ones(3, np.uint64), 4).to_host()
+    assert got.size == 0 and got.child.size == 0
+
+
+# ----------------------------------------------------------------------------- wordpiece
+@pytest.mark.parametrize("case", gc.wordpiece_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_wordpiece_golden(nv, case, dtype):
+    vocab = nv.WordPieceVocabulary(dev(nv, strings(case["vocab"])))
+    host = strings(case["rows"], dtype)
+    col = dev(nv, host)
+    if "slice" in case:
+        lo, hi = case["slice"]
+        col = col.slice(lo, hi, host.slice(lo, hi).null_count)
+    for run in case["runs"]:
+        got = nv.wordpiece_tokenize(col, vocab, run["max_words"]).to_host()
+        assert gc.expected_list_equal(got.to_pylist(), run["expected"]), (case["name"], run["max_words"])
+        assert got.child.dtype == np.int32
+
+
+def test_wordpiece_bert_sentences(nv):
+    d = gc.bert_case()
+    vocab = nv.WordPieceVocabulary(dev(nv, strings(d["vocab"])))
+    assert vocab.unk_id == 100
+    col = dev(nv, strings(d["rows"]))
+    for mw, exp in d["expected"].items():
+        got = nv.wordpiece_tokenize(col, vocab, int(mw)).to_host()
+        assert gc.expected_list_equal(got.to_pylist(), exp), mw
+
+
+def test_wordpiece_errors_and_empty(nv):
+    with pytest.raises(ValueError):
+        nv.WordPieceVocabulary(dev(nv, strings([])))
+    with pytest.raises(ValueError):
+        nv.WordPieceVocabulary(dev(nv, strings([None, None, None])))
+    v = nv.WordPieceVocabulary(dev(nv, strings(["x"])))
+    assert v.unk_id == -1
+    with pytest.raises(ValueError):
+        nv.wordpiece_tokenize(dev(nv, strings(["  "])), v, -1)
+    v2 = nv.WordPieceVocabulary(dev(nv, strings([""])))
+    for mw in (0, 10):
+        got = nv.wordpiece_tokenize(dev(nv, strings([])), v2, mw).to_host()
+        assert got.size == 0 and got.offsets.size == 0
+
+
+def make_vocab(rng, n, letters, with_unk=True):
+    vocab = (["[PAD]", "[UNK]"] if with_unk else ["[PAD]"]) + list(letters) + ["##" + c for c in letters]
+    seen = set(vocab)
+    while len(vocab) < n:
+        ln = int(rng.integers(2, 14))
+        s = "".join(rng.choice(list(letters), ln))
+        if rng.random() < 0.4:
+            s = "##" + s
+        if s not in seen:
+            seen.add(s)
+            vocab.append(s)
+    return vocab
+
+
+@pytest.mark.parametrize("max_words", [0, 7, 1000])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_wordpiece_random_vs_oracle(nv, orc, max_words, dtype):
+    rng = np.random.default_rng(77 + max_words)
+    letters = "abcdefghijkl"
+    vocab = make_vocab(rng, 3000, letters)
+    stems = [v for v in vocab[2:] if not v.startswith("##")]
+    rows = []
+    for _ in range(1500):
+        u = rng.random()
+        if u < 0.03:
+            rows.append(None)
+            continue
+        if u < 0.06:
+            rows.append("")
+            continue
+        nw = int(rng.integers(1, 120))
+        ws = []
+        for _ in range(nw):
+            t = rng.random()
+            if t < 0.7:
+                ws.append(stems[int(rng.integers(0, len(stems)))])
+            elif t < 0.97:
+                ws.append("".join(rng.choice(list(letters + "xyz"), int(rng.integers(1, 20)))))
+            else:
+                ws.append("".join(rng.choice(list(letters), int(rng.integers(150, 260)))))
+        sep = " " if max_words else ("  " if rng.random() < 0.1 else " ")
+        s = sep.join(ws)
+        if rng.random() < 0.2:
+            s = " " + s
+        if rng.random() < 0.2:
+            s = s + " "  # a single trailing space is well defined in both paths
+        rows.append(s)
+    rows += ["a", " ", "a b", "ab", "  a", "a" * 199, "a" * 200, "a" * 600 + " b"]
+    host = strings(rows, dtype)
+    hv = strings(vocab)
+    got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), max_words).to_host()
+    exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), max_words, nthreads=8)
+    assert_same(got, exp, f"wordpiece mw={max_words}")
+    assert exp.child.size > (5000 if max_words == 7 else 50000)
+
+
+def test_wordpiece_utf8_vs_oracle(nv, orc):
+    rng = np.random.default_rng(99)
+    base = list("abcdeé漢字ñ語😀")
+    vocab = ["[unk]"] + base + ["##" + c for c in base[:8]]
+    seen = set(vocab)
+    while len(vocab) < 1500:
+        s = "".join(rng.choice(base, int(rng.integers(2, 6))))
+        if rng.random() < 0.4:
+            s = "##" + s
+        if s not in seen:
+            seen.add(s)
+            vocab.append(s)
+    rows = [" ".join("".join(rng.choice(base + ["z"], int(rng.integers(1, 9)))) for _ in range(int(rng.integers(1, 60))))
+            for _ in range(800)]
+    host = strings(rows, np.int64)
+    hv = strings(vocab)
+    for mw in (0, 16):
+        got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
+        assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4), f"utf8 mw={mw}")
+
+
+def test_wordpiece_sliced_nulls_vs_oracle(nv, orc):
+    rng = np.random.default_rng(123)
+    vocab = make_vocab(rng, 500, "abcdef")
+    rows = []
+    for _ in range(400):
+        if rng.random() < 0.25:
+            rows.append(None)
+        else:
+            rows.append(" ".join("".join(rng.choice(list("abcdefg"), int(rng.integers(1, 8)))) for _ in range(int(rng.integers(0, 30)))))
+    host = strings(rows)
+    hv = strings(vocab)
+    dv = nv.WordPieceVocabulary(dev(nv, hv))
+    ov = orc.Vocabulary(hv)
+    for lo, hi in [(0, 400), (5, 390), (33, 65), (100, 101)]:
+        hs = host.slice(lo, hi)
+        ds = dev(nv, host).slice(lo, hi, hs.null_count)
+        for mw in (0, 5):
+            assert_same(nv.wordpiece_tokenize(ds, dv, mw).to_host(), orc.wordpiece_tokenize(hs, ov, mw), f"slice {lo}:{hi} mw={mw}")
+
+
+def test_wordpiece_row_longer_than_chunks(nv, orc):
+    """One row spanning many 256-byte chunks, with words straddling chunk boundaries."""
+    rng = np.random.default_rng(321)
+    vocab = make_vocab(rng, 2000, "abcdefgh")
+    words = ["".join(rng.choice(list("abcdefghz"), int(rng.integers(1, 30)))) for _ in range(20000)]
+    rows = [" ".join(words), " ".join(words[:7000]), "x", " ".join(words[100:5000])]
+    host = strings(rows)
+    hv = strings(vocab)
+    for mw in (0, 3000):
+        got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
+        assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4), f"long row mw={mw}")
