@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the nvtext hot path on one MI355X.
+
+A step is one wordpiece_tokenize call over the whole synthetic batch of configuration C2
+(4M rows, lognormal mean 256 B, Zipf(1.1) words over a 30,522-entry vocabulary, 15 % OOV,
+int32 offsets, max_words_per_row=128), inputs resident in HBM, output allocation included.
+Prints one JSON line: input GB/s as `value`, plus Mrows/s, the roofline of the dominant
+kernel, the host-oracle baseline on a bounded sample, and the minhash / minhash64 figures
+(configurations C3 / C4 at a stated scale).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def median(xs):
+    s = sorted(xs)
+    n = len(s)
+    return s[n // 2] if n % 2 else 0.5 * (s[n // 2 - 1] + s[n // 2])
+
+
+def input_bytes(col):
+    """chars + (rows+1) offsets + validity mask (the input term of the algorithmic bytes)."""
+    ow = col.offsets.dtype.itemsize
+    return col.chars_bytes + (col.size + 1) * ow + ((col.size + 7) // 8 if col.mask is not None else 0)
+
+
+def timed_steps(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_times(fn, reps, capi, torch):
+    """Average duration of each library kernel, from HIP events recorded by the library on the
+    stream it launches on."""
+    capi.profile_enable(True)
+    capi.profile_read()
+    acc = {}
+    for _ in range(reps):
+        fn()
+        torch.cuda.synchronize()
+        for name, ms in capi.profile_read():
+            acc.setdefault(name, []).append(ms)
+    capi.profile_enable(False)
+    return {k: sum(v) / len(v) for k, v in acc.items()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--scale", type=float, default=1.0, help="row-count multiplier of the headline workload (1.0 = 4M rows)")
+    ap.add_argument("--minhash-scale", type=float, default=0.25, help="row-count multiplier of the C3/C4 minhash legs (0 = skip)")
+    ap.add_argument("--cpu-sample-rows", type=int, default=400_000, help="rows of the workload given to the host oracle")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; the path shards by row ranges with no exchange step, "
+              "run one process per GPU on disjoint row ranges instead (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from cudf_amd import _capi, datagen, nvtext
+    _capi.load()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+
+    # ------------------------------------------------------------------ headline: wordpiece_tokenize on C2
+    t0 = time.time()
+    wl = datagen.config2(args.scale)
+    host = wl.rows
+    log(f"[bench] C2 generated: rows={host.size} chars={host.chars_bytes / 1e9:.3f} GB in {time.time() - t0:.1f}s")
+    dcol = nvtext.DeviceStringsColumn.from_host(host)
+    dvoc = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(wl.vocab))
+    mw = wl.params["max_words_per_row"]
+    result = {}
+
+    def step():
+        result["out"] = nvtext.wordpiece_tokenize(dcol, dvoc, mw)
+
+    sec = timed_steps(step, args.steps, args.warmup, torch)
+    out = result["out"]
+    tokens = out.child_size
+    in_b = input_bytes(host)
+    out_b = 4 * tokens + 4 * (host.size + 1) + ((host.size + 7) // 8 if host.mask is not None else 0)
+    kt = kernel_times(step, 3, _capi, torch)
+    log(f"[bench] tokenize: {sec * 1e3:.3f} ms/step, tokens={tokens}, kernels={ {k: round(v, 3) for k, v in kt.items()} }")
+    dom = "wordpiece_rows_kernel<fill>"
+    dom_ms = kt.get(dom, float("nan"))
+    achieved = (in_b + out_b) / (dom_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes": in_b + out_b, "kernel_ms": round(dom_ms, 4),
+                "all_kernels_ms": {k: round(v, 4) for k, v in kt.items()},
+                "frac_whole_op": round((in_b + out_b) / sec / 1e9 / HBM_PEAK_GBS, 4)}
+
+    # ------------------------------------------------------------------ host oracle on a bounded sample (also the parity check)
+    cpu = None
+    parity = "skipped"
+    if not args.no_cpu:
+        from oracle import pyoracle as orc
+        n = min(args.cpu_sample_rows, host.size)
+        sample = host.slice(0, n)
+        ovoc = orc.Vocabulary(wl.vocab)
+        threads = max(1, min(orc.hardware_threads(), 16))
+        t0 = time.perf_counter()
+        exp = orc.wordpiece_tokenize(sample, ovoc, mw, nthreads=threads)
+        cpu_s = time.perf_counter() - t0
+        cpu = {"value": round(input_bytes(sample) / cpu_s / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": f"first {n} rows of the same workload ({sample.chars_bytes / 1e6:.0f} MB), {cpu_s:.2f} s",
+               "mrows_per_s": round(n / cpu_s / 1e6, 3)}
+        got = nvtext.wordpiece_tokenize(dcol.slice(0, n, 0), dvoc, mw).to_host()
+        parity = "PASS" if got.equals(exp) else "FAIL"
+        log(f"[bench] oracle: {cpu_s:.2f}s on {threads} threads; parity {parity}")
+    del dcol, out, result
+
+    # ------------------------------------------------------------------ minhash legs (C3 uint32, C4 uint64)
+    extra = {}
+    if args.minhash_scale > 0:
+        for name, fn in (("C3", nvtext.minhash), ("C4", nvtext.minhash64)):
+            torch.cuda.empty_cache()
+            t0 = time.time()
+            w = datagen.CONFIGS[name](args.minhash_scale)
+            p = w.params
+            a, b = datagen.make_params(p["P"], p["hash_bits"], p["param_seed"])
+            signed = np.int32 if p["hash_bits"] == 32 else np.int64
+            da = torch.from_numpy(a.view(signed)).cuda()
+            db = torch.from_numpy(b.view(signed)).cuda()
+            log(f"[bench] {name} generated: rows={w.rows.size} chars={w.rows.chars_bytes / 1e9:.3f} GB in {time.time() - t0:.1f}s")
+            dc = nvtext.DeviceStringsColumn.from_host(w.rows)
+            keep = {}
+
+            def mstep():
+                keep["o"] = fn(dc, p["seed"], da, db, p["width"])
+
+            msec = timed_steps(mstep, max(3, args.steps // 2), 1, torch)
+            mk = kernel_times(mstep, 2, _capi, torch)
+            ib = input_bytes(w.rows)
+            valid = w.rows.size - w.rows.null_count
+            windows = int(w.rows.chars_bytes - valid * (p["width"] - 1))  # ASCII rows longer than width
+            leg = {"workload": f"{name} x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes,
+                   "ms_per_step": round(msec * 1e3, 3), "input_GBps": round(ib / msec / 1e9, 2),
+                   "mrows_per_s": round(w.rows.size / msec / 1e6, 3),
+                   "gperm_per_s": round(windows * p["P"] / msec / 1e9, 1),
+                   "kernels_ms": {k: round(v, 3) for k, v in mk.items()}}
+            if not args.no_cpu:
+                from oracle import pyoracle as orc
+                n = min(w.rows.size, 20000 if name == "C3" else 2000)
+                smp = w.rows.slice(0, n)
+                ofn = orc.minhash if name == "C3" else orc.minhash64
+                threads = max(1, min(orc.hardware_threads(), 16))
+                t0 = time.perf_counter()
+                exp = ofn(smp, p["seed"], a, b, p["width"], nthreads=threads)
+                cs = time.perf_counter() - t0
+                got = fn(dc.slice(0, n, smp.null_count), p["seed"], da, db, p["width"]).to_host()
+                leg["cpu_baseline"] = {"value": round(input_bytes(smp) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
+                                       "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+                leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
+            log(f"[bench] {name}: {leg}")
+            extra["minhash" if name == "C3" else "minhash64"] = leg
+            del dc, keep
+
+    line = {
+        "metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline",
+        "value": round(in_b / sec / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8/int32", "data": "synthetic",
+        "config": {"workload": f"C2 wordpiece_tokenize x{args.scale}", "rows": host.size, "chars_bytes": host.chars_bytes,
+                   "vocab_entries": wl.vocab.size, "max_words_per_row": mw, "tokens_out": tokens, "offsets": "int32"},
+        "mrows_per_s": round(host.size / sec / 1e6, 3),
+        "roofline": roofline, "cpu_baseline": cpu, "parity_vs_oracle": parity,
+    }
+    line.update(extra)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

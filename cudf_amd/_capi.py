@@ -20,6 +20,8 @@ EXPORTS = [
     "nvtext_amd_wordpiece_vocabulary_unk_id",
     "nvtext_amd_wordpiece_tokenize",
     "nvtext_amd_list_column_free",
+    "nvtext_amd_profile_enable",
+    "nvtext_amd_profile_read",
 ]
 
 
@@ -97,5 +99,21 @@ def load():
     L.nvtext_amd_wordpiece_tokenize.argtypes = [C.POINTER(StringsColumn), C.c_void_p] + common_tail
     L.nvtext_amd_list_column_free.restype = None
     L.nvtext_amd_list_column_free.argtypes = [C.POINTER(ListColumn), C.c_void_p, C.POINTER(Allocator)]
+    L.nvtext_amd_profile_enable.restype = None
+    L.nvtext_amd_profile_enable.argtypes = [C.c_int32]
+    L.nvtext_amd_profile_read.restype = C.c_int32
+    L.nvtext_amd_profile_read.argtypes = [C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.c_int32]
     _lib = L
     return L
+
+
+def profile_enable(on: bool) -> None:
+    load().nvtext_amd_profile_enable(1 if on else 0)
+
+
+def profile_read(capacity: int = 4096):
+    """[(kernel name, milliseconds)] in launch order since the last read."""
+    names = (C.c_char_p * capacity)()
+    ms = (C.c_float * capacity)()
+    n = load().nvtext_amd_profile_read(names, ms, capacity)
+    return [(names[i].decode(), float(ms[i])) for i in range(n)]

@@ -27,6 +27,25 @@ nvtext_amd_status fail(nvtext_amd_status st, const char* msg);
     }                                                                                 \
   } while (0)
 
+// ------------------------------------------------------------------ kernel timing (benchmarks)
+bool profiling_on();
+void profile_mark_begin(const char* name, hipStream_t stream);
+void profile_mark_end(hipStream_t stream);
+
+// Brackets one kernel launch with HIP events when profiling is enabled.
+struct ProfileScope {
+  hipStream_t stream;
+  bool on;
+  ProfileScope(const char* name, hipStream_t s) : stream(s), on(profiling_on())
+  {
+    if (on) profile_mark_begin(name, stream);
+  }
+  ~ProfileScope()
+  {
+    if (on) profile_mark_end(stream);
+  }
+};
+
 // ------------------------------------------------------------------ memory
 // Stream-ordered allocation through the caller's allocator (or hipMallocAsync).
 struct Mr {

@@ -4,11 +4,35 @@
 #include "common.cuh"
 
 #include <cstring>
+#include <vector>
 
 namespace nvtext_amd {
 
 namespace {
 thread_local std::string g_last_error;
+
+struct ProfileRecord {
+  const char* name;
+  hipEvent_t begin;
+  hipEvent_t end;
+};
+bool g_profile_on = false;
+std::vector<ProfileRecord> g_profile;
+}  // namespace
+
+bool profiling_on() { return g_profile_on; }
+
+void profile_mark_begin(const char* name, hipStream_t stream)
+{
+  ProfileRecord r{name, nullptr, nullptr};
+  if (hipEventCreate(&r.begin) != hipSuccess || hipEventCreate(&r.end) != hipSuccess) return;
+  (void)hipEventRecord(r.begin, stream);
+  g_profile.push_back(r);
+}
+
+void profile_mark_end(hipStream_t stream)
+{
+  if (!g_profile.empty()) (void)hipEventRecord(g_profile.back().end, stream);
 }
 
 void set_last_error(const char* msg) { g_last_error = msg ? msg : ""; }
@@ -96,6 +120,29 @@ void launch_fill_u32(uint32_t* dst, uint32_t value, int64_t count, hipStream_t s
 extern "C" {
 
 int32_t nvtext_amd_version(void) { return 100; }
+
+void nvtext_amd_profile_enable(int32_t on)
+{
+  nvtext_amd::g_profile_on = on != 0;
+}
+
+int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t capacity)
+{
+  int32_t n = 0;
+  for (auto& r : nvtext_amd::g_profile) {
+    float ms = 0.f;
+    if (r.begin && r.end && hipEventSynchronize(r.end) == hipSuccess && hipEventElapsedTime(&ms, r.begin, r.end) == hipSuccess &&
+        n < capacity) {
+      names[n]        = r.name;
+      milliseconds[n] = ms;
+      ++n;
+    }
+    if (r.begin) (void)hipEventDestroy(r.begin);
+    if (r.end) (void)hipEventDestroy(r.end);
+  }
+  nvtext_amd::g_profile.clear();
+  return n;
+}
 
 const char* nvtext_amd_last_error(void) { return nvtext_amd::g_last_error.c_str(); }
 

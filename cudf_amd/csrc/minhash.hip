@@ -342,10 +342,16 @@ void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P,
 {
   int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
   dim3 grid(static_cast<unsigned>(v.size), static_cast<unsigned>(chunks));
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
+  {
+    ProfileScope ps("minhash_rows_kernel", stream);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
+  }
   dim3 grid2(4096, static_cast<unsigned>(chunks));
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_extra_kernel<T, K>), grid2, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets,
-                     extra_prefix, child);
+  {
+    ProfileScope ps("minhash_extra_kernel", stream);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_extra_kernel<T, K>), grid2, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets,
+                       extra_prefix, child);
+  }
 }
 
 template <typename T>

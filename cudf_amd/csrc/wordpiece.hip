@@ -563,8 +563,11 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
   unsigned const blocks = static_cast<unsigned>((static_cast<int64_t>(rows) + kTokWaves - 1) / kTokWaves);
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(wordpiece_rows_kernel<false>), dim3(blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table,
-                     max_words_per_row, counts.as<int32_t>(), static_cast<const int32_t*>(nullptr), static_cast<int32_t*>(nullptr));
+  {
+    ProfileScope ps("wordpiece_rows_kernel<count>", stream);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(wordpiece_rows_kernel<false>), dim3(blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table,
+                       max_words_per_row, counts.as<int32_t>(), static_cast<const int32_t*>(nullptr), static_cast<int32_t*>(nullptr));
+  }
   // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
   device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
   uint64_t total = 0;
@@ -586,6 +589,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       nvtext_amd_list_column_free(out, stream_, mr_);
       return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
     }
+    ProfileScope ps("wordpiece_rows_kernel<fill>", stream);
     hipLaunchKernelGGL(HIP_KERNEL_NAME(wordpiece_rows_kernel<true>), dim3(blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table,
                        max_words_per_row, static_cast<int32_t*>(nullptr), out->offsets, static_cast<int32_t*>(out->child));
   }

@@ -144,6 +144,16 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
                                                 const nvtext_amd_allocator* mr,
                                                 nvtext_amd_list_column* out);
 
+/* Kernel timing for benchmarks.  The reference marks these entry points with NVTX ranges
+ * (CUDF_FUNC_RANGE, cpp/src/text/minhash.cu:699, cpp/src/text/wordpiece_tokenize.cu:897) and is
+ * timed from outside with Nsight; here the library itself brackets each of its kernels with HIP
+ * events on the caller's stream while profiling is on.  nvtext_amd_profile_read synchronises the
+ * recorded events, returns up to `capacity` (name, milliseconds) pairs in launch order and clears
+ * the record; the names are static strings.  Off by default; not thread-safe against concurrent
+ * entry-point calls. */
+void    nvtext_amd_profile_enable(int32_t on);
+int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t capacity);
+
 /* Releases the buffers of a result through the allocator that produced them. */
 void nvtext_amd_list_column_free(nvtext_amd_list_column* col, void* stream, const nvtext_amd_allocator* mr);
 
