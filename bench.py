@@ -105,7 +105,7 @@ def main():
     out_b = 4 * tokens + 4 * (host.size + 1) + ((host.size + 7) // 8 if host.mask is not None else 0)
     kt = kernel_times(step, 3, _capi, torch)
     log(f"[bench] tokenize: {sec * 1e3:.3f} ms/step, tokens={tokens}, kernels={ {k: round(v, 3) for k, v in kt.items()} }")
-    dom = "wordpiece_tokenize_kernel"
+    dom = "wordpiece_probe_kernel"
     dom_ms = kt.get(dom, float("nan"))
     achieved = (in_b + out_b) / (dom_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

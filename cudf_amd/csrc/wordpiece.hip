@@ -11,20 +11,23 @@
 //     spaces: whole entries (kind 0) and "##" entries without their prefix (kind 1).  Keys of
 //     up to 8 bytes sit inside the slot, so a probe is one 32-byte read; the table for a
 //     30k-entry vocabulary is 2 MiB and stays in L2.
-//   * the key hash is polynomial (H <- H*B + byte mod 2^32).  A wavefront owns a row and walks
-//     it in 256-byte chunks with lanes <-> bytes: a segmented DPP scan over (multiplier, value)
-//     pairs gives the hash of every word prefix at once, so no lane ever loops over the bytes of
-//     its word, and the hash of any inner piece is P[e] - P[p] * B^(e-p).
-//   * words are handled in the chunk where they END; the previous chunk stays in a 512-byte LDS
-//     ring so a word (< 200 bytes) is always whole.  Then lanes <-> words: one probe settles an
-//     in-vocabulary word, the rest follow the greedy longest-match rule with O(1) hashes.
-//     Tokens are written over the word's own prefix-hash slots (a word never has more tokens than
-//     bytes) and copied out after a DPP scan of the per-word counts.
-//   * pass 1 tokenizes every row once into an arena with floor(bytes/2)+1 slots per row and
-//     records the counts; a device-wide scan makes the int32 list offsets; pass 2 copies the
-//     arena rows into place (a row that overflowed its arena slots is tokenized again, directly).
+//   * the key hash is polynomial (H <- H*B + byte mod 2^32): dropping the last byte of a
+//     candidate is one subtract and one multiply by B^-1, and an inner piece is
+//     P[e] - P[p] * B^(e-p), so no candidate is ever re-hashed.
+//   * probe pass: a wavefront walks rows in 256-byte chunks with lanes <-> bytes; a segmented
+//     DPP scan over (multiplier, value) pairs yields the hash of every word at its last byte,
+//     a max-scan yields its start.  Then lanes <-> words: ONE probe per word.  A hit stores the
+//     token in the row's word arena (one slot per word, floor(bytes/2)+1 slots per row); a miss
+//     stores a marker and appends the word to a queue.
+//   * out-of-vocabulary pass: one lane per queued word, all lanes busy, runs the greedy
+//     longest-match rule with O(1) hash updates and stores count + tokens per queue entry.
+//     (Doing this inside the probe pass leaves 90 % of the lanes idle behind a chain of
+//     dependent L2 probes.)
+//   * a device-wide scan of the per-row token counts makes the int32 list offsets; the emit pass
+//     expands each row's word arena into its tokens.  No chars-sized temporary is written.
 #include "common.cuh"
 
+#include <algorithm>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -35,6 +38,15 @@ namespace {
 
 constexpr uint32_t kMaxWord = 200;  // wordpiece_tokenize.cu:300: words this long become one [UNK]
 constexpr uint32_t kHashB   = 0x01000193u;
+
+constexpr uint32_t inv_mod_2_32(uint32_t a)
+{
+  uint32_t x = a;  // Newton iteration: correct to 3 bits, doubles every step
+  for (int i = 0; i < 5; ++i) x *= 2u - a * x;
+  return x;
+}
+constexpr uint32_t kHashBInv = inv_mod_2_32(kHashB);
+static_assert(kHashB * kHashBInv == 1u, "B^-1 mod 2^32");
 
 __host__ __device__ __forceinline__ uint32_t mix32(uint32_t h)
 {
@@ -85,28 +97,31 @@ constexpr int kTokThreads = kTokWaves * kWave;
 constexpr int kChunk      = 256;  // bytes per wavefront step (4 per lane)
 constexpr int kRing       = 512;  // two chunks: the current one and the one before it
 constexpr int32_t kNone   = std::numeric_limits<int32_t>::min();
+constexpr int kOovKeep    = 8;    // tokens stored per queued word; longer results are redone at emit time
+constexpr uint32_t kOovMark = 0x80000000u;  // word-arena value 0x80000000 | queue index (never 0xFFFFFFFF = id -1)
 
-struct TokLds {
-  uint32_t bytes[kRing / 4];       // row bytes (everything outside the row is ' ')
-  uint32_t pt[kRing];              // prefix hash of each byte's word up to that byte; later the word's tokens
-  uint16_t wend[kChunk / 2 + 2];   // ring index of the last byte of each word ending in the chunk
-  uint16_t wlen[kChunk / 2 + 2];   // its length in bytes (clamped to kMaxWord)
+struct OovEntry {
+  int32_t row;     // -1: unused entry
+  uint32_t delta;  // byte offset of the word inside its row
+  uint32_t widx;   // index of the word inside its row (its word-arena slot)
+  uint32_t pad;
+};
+struct OovResult {
+  int32_t tok[kOovKeep];
 };
 
-// One word inside the ring: byte k of the word is ring byte (start + k) & 511.
-struct Word {
-  const TokLds* lds;
+// ------------------------------------------------------------------ keys in the LDS ring / in global memory
+// A word inside the 512-byte ring: byte k of the word is ring byte (start + k) & 511.
+struct RingWord {
+  const uint32_t* ring;
   uint32_t start;
-  __device__ __forceinline__ uint32_t byte(uint32_t k) const { return reinterpret_cast<const uint8_t*>(lds->bytes)[(start + k) & (kRing - 1)]; }
-  // hash of word bytes [0, k]
-  __device__ __forceinline__ uint32_t prefix_hash(uint32_t k) const { return lds->pt[(start + k) & (kRing - 1)]; }
-  // word bytes [p, p+8) as two dwords, zero padded past len
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const { return reinterpret_cast<const uint8_t*>(ring)[(start + k) & (kRing - 1)]; }
   __device__ __forceinline__ void key8(uint32_t p, uint32_t len, uint32_t* k0, uint32_t* k1) const
   {
     uint32_t const o  = (start + p) & (kRing - 1);
     uint32_t const i  = o >> 2;
     uint32_t const sh = (o & 3u) * 8u;
-    uint32_t const d0 = lds->bytes[i], d1 = lds->bytes[(i + 1) & (kRing / 4 - 1)], d2 = lds->bytes[(i + 2) & (kRing / 4 - 1)];
+    uint32_t const d0 = ring[i], d1 = ring[(i + 1) & (kRing / 4 - 1)], d2 = ring[(i + 2) & (kRing / 4 - 1)];
     uint32_t lo       = __builtin_amdgcn_alignbit(d1, d0, sh);
     uint32_t hi       = __builtin_amdgcn_alignbit(d2, d1, sh);
     if (len < 4) lo &= (1u << (8 * len)) - 1u;
@@ -117,7 +132,32 @@ struct Word {
   }
 };
 
-__device__ __forceinline__ bool slot_matches(VocabTable const& t, uint4 const& s, uint32_t want, uint32_t len, uint32_t k0, uint32_t k1, Word const& w,
+// A word in global memory (bytes p[0 .. )).  key8 reads only aligned dwords that overlap the key.
+struct GlobalWord {
+  const uint8_t* p;
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const { return p[k]; }
+  __device__ __forceinline__ void key8(uint32_t off, uint32_t len, uint32_t* k0, uint32_t* k1) const
+  {
+    const uint8_t* q    = p + off;
+    uint32_t const mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(q) & 3u);
+    const uint32_t* a   = reinterpret_cast<const uint32_t*>(q - mis);
+    uint32_t const sh   = mis * 8u;
+    uint32_t const need = mis + (len < 8 ? len : 8);  // bytes from the aligned base
+    uint32_t const d0   = a[0];
+    uint32_t const d1   = need > 4 ? a[1] : 0u;
+    uint32_t const d2   = need > 8 ? a[2] : 0u;
+    uint32_t lo         = __builtin_amdgcn_alignbit(d1, d0, sh);
+    uint32_t hi         = __builtin_amdgcn_alignbit(d2, d1, sh);
+    if (len < 4) lo &= (1u << (8 * len)) - 1u;
+    if (len <= 4) hi = 0;
+    else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+    *k0 = lo;
+    *k1 = hi;
+  }
+};
+
+template <typename W>
+__device__ __forceinline__ bool slot_matches(VocabTable const& t, uint4 const& s, uint32_t want, uint32_t len, uint32_t k0, uint32_t k1, W const& w,
                                              uint32_t p)
 {
   if (s.x != want) return false;
@@ -129,7 +169,8 @@ __device__ __forceinline__ bool slot_matches(VocabTable const& t, uint4 const& s
 }
 
 // Token id of word bytes [p, p+len) in key space `kind` (hash h), or kNone.
-__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, uint32_t h, Word const& w, uint32_t p, uint32_t len)
+template <typename W>
+__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, uint32_t h, W const& w, uint32_t p, uint32_t len)
 {
   uint32_t b;
   uint32_t const want = slot_word0(h, kind, len, &b);
@@ -147,70 +188,7 @@ __device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, ui
   }
 }
 
-// cpp/src/text/wordpiece_tokenize.cu:307-317 on word bytes [p, e): the end after dropping the last
-// UTF-8 character; returns p when nothing is left.
-__device__ __forceinline__ uint32_t drop_last_char(Word const& w, uint32_t p, uint32_t e)
-{
-  if (e - p < 2) return p;
-  uint32_t x = e - 1;
-  while (x > p && is_utf8_continuation(w.byte(x))) --x;
-  return x;
-}
-
-// Greedy longest-match-first tokenization of one word of `len` bytes (1..199)
-// (cpp/src/text/wordpiece_tokenize.cu:349-407).  Tokens go to tok[(start + j) & 511]; returns the count.
-// `pw[k]` = B^k.
-__device__ __forceinline__ uint32_t wp_tokenize(VocabTable const& t, TokLds& lds, const uint32_t* pw, uint32_t start, uint32_t len)
-{
-  Word const w{&lds, start};
-  uint32_t* const tok = lds.pt;
-  auto put            = [&](uint32_t j, int32_t id) { tok[(start + j) & (kRing - 1)] = static_cast<uint32_t>(id); };
-  // whole word, then ever shorter prefixes, in the full key space
-  int32_t id = len <= t.max_len[0] ? lookup(t, 0, w.prefix_hash(len - 1), w, 0, len) : kNone;
-  if (id != kNone) {
-    put(0, id);
-    return 1;
-  }
-  uint32_t e = len;
-  for (;;) {
-    e = drop_last_char(w, 0, e);
-    if (e == 0) {  // nothing matched: one unknown token (375-379)
-      put(0, t.unk_id);
-      return 1;
-    }
-    if (e > t.max_len[0]) continue;
-    id = lookup(t, 0, w.prefix_hash(e - 1), w, 0, e);
-    if (id != kNone) break;
-  }
-  uint32_t hp = w.prefix_hash(e - 1);  // hash of bytes [0, p)
-  put(0, id);
-  uint32_t count = 1;
-  uint32_t p     = e;
-  // the rest, piece by piece, in the "##" key space (381-395)
-  while (p < len) {
-    e = len;
-    for (;;) {
-      uint32_t const pl = e - p;
-      if (pl <= t.max_len[1]) {
-        uint32_t const he = w.prefix_hash(e - 1);
-        id                = lookup(t, 1, he - hp * pw[pl], w, p, pl);
-        if (id != kNone) {
-          hp = he;  // read before the token below may overwrite that slot
-          break;
-        }
-      }
-      e = drop_last_char(w, p, e);
-      if (e == p) {  // 396-404: the word collapses to a single unknown token
-        put(0, t.unk_id);
-        return 1;
-      }
-    }
-    put(count++, id);
-    p = e;
-  }
-  return count;
-}
-
+// ------------------------------------------------------------------ wavefront scans used by the probe pass
 template <int CTRL, int ROW_MASK, int OLD>
 __device__ __forceinline__ uint32_t dpp_old(uint32_t v)
 {
@@ -248,32 +226,34 @@ __device__ __forceinline__ uint32_t wave_scan_max(uint32_t v)
   return v;
 }
 
-// value of the lane below (lane 0 gets `first`)
+// value of the lane below (lane 0 gets FIRST)
 template <int FIRST>
 __device__ __forceinline__ uint32_t from_lane_below(uint32_t v)
 {
   return dpp_old<0x138, 0xf, FIRST>(v);  // wave_shr:1
 }
 
-// Tokenizes row r with one wavefront.  Tokens are delivered in order to dst[0 .. ) but only while
-// the running index is below `slots`; returns the row's token count (which may exceed slots).
-__device__ __forceinline__ uint32_t tokenize_row(ColView const& col, VocabTable const& table, int32_t max_words, int64_t r, TokLds& lds,
-                                                 const uint32_t* pw, int32_t* dst, int64_t slots, int lane)
-{
-  int64_t const o = col.off(r);
-  int64_t const n = col.off(r + 1) - o;
-  // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
-  // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
-  int64_t cap = std::numeric_limits<int64_t>::max();
-  if (max_words > 0) cap = col.valid(r) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
+// Row r owns the word-arena slots [arena_pos(r), arena_pos(r+1)): at least floor(bytes/2) + 1, and a
+// row cannot hold more words than that.
+__device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
 
-  const uint8_t* row   = col.chars + o;
-  uint32_t const mis   = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 3u);
-  const uint32_t* arow = reinterpret_cast<const uint32_t*>(row - mis);
-  int64_t const aend   = static_cast<int64_t>(mis) + n;  // row end in aligned coordinates
+struct ProbeLds {
+  uint32_t bytes[kRing / 4];        // row bytes (everything outside the row is ' ')
+  uint32_t wstart[kChunk / 2 + 2];  // per word ending in the chunk: 1-based aligned coordinate of its first byte,
+  uint32_t wend[kChunk / 2 + 2];    // of its last byte,
+  uint32_t whash[kChunk / 2 + 2];   // and its hash
+};
 
+// ------------------------------------------------------------------ probe pass
+// Where a row sits relative to 4-byte aligned memory.
+struct RowCtx {
+  const uint32_t* arow;  // aligned base at or below the row's first byte
+  uint32_t mis;          // row start inside that dword
+  int64_t n;             // row bytes
+  int64_t aend;          // row end in aligned coordinates (mis + n)
   // aligned dword at coordinate a0 with every byte outside the row replaced by ' '
-  auto load_clean = [&](int64_t a0) -> uint32_t {
+  __device__ __forceinline__ uint32_t load_clean(int64_t a0) const
+  {
     uint32_t v = 0x20202020u;
     if (a0 < aend && a0 + 4 > static_cast<int64_t>(mis)) {
       v = arow[a0 >> 2];
@@ -287,165 +267,451 @@ __device__ __forceinline__ uint32_t tokenize_row(ColView const& col, VocabTable 
       }
     }
     return v;
-  };
+  }
+};
 
-  int64_t words_done   = 0;
-  uint32_t tokens_done = 0;
-  uint32_t carry_hash  = 0;     // hash of the word running into the chunk (0 after a space)
-  uint32_t carry_start = 0;     // 1 + aligned coordinate of the start of that word
-  uint32_t prev_last   = 0x20;  // byte before the chunk
-  for (int64_t cbase = 0; cbase < aend && words_done < cap; cbase += kChunk) {
-    int64_t const a0    = cbase + 4 * lane;
-    uint32_t const mine = load_clean(a0);
-    uint32_t const ring0 = static_cast<uint32_t>(a0) & (kRing - 1);
-    lds.bytes[ring0 >> 2] = mine;
-    // neighbours: the byte before my four and the byte after them
-    uint32_t before = from_lane_below<0>(mine >> 24);
-    if (lane == 0) before = prev_last;
-    uint32_t after = static_cast<uint32_t>(__shfl_down(static_cast<int>(mine & 0xffu), 1));
-    if (lane == kWave - 1) after = load_clean(a0 + 4) & 0xffu;
-    prev_last = wave_bcast(mine >> 24, kWave - 1);
+__device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, int64_t n)
+{
+  const uint8_t* row = col.chars + o;
+  RowCtx c;
+  c.mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 3u);
+  c.arow = reinterpret_cast<const uint32_t*>(row - c.mis);
+  c.n    = n;
+  c.aend = static_cast<int64_t>(c.mis) + n;
+  return c;
+}
 
-    // per byte: hash block of my bytes so far, word starts and word ends
-    uint32_t bm[4], bv[4];
-    uint32_t m = 1, v = 0, smax = 0, ends = 0;
-    uint32_t prevb = before;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      uint32_t const b    = (mine >> (8 * j)) & 0xffu;
-      uint32_t const next = j < 3 ? (mine >> (8 * (j + 1))) & 0xffu : after;
-      bool const sp       = b == 0x20u;
-      uint32_t const em   = sp ? 0u : kHashB;
-      uint32_t const ev   = sp ? 0u : b;
-      v                   = v * em + ev;
-      m                   = m * em;
-      bm[j]               = m;
-      bv[j]               = v;
-      if (!sp && prevb == 0x20u) smax = static_cast<uint32_t>(a0) + j + 1;  // word start (1-based coordinate)
-      if (!sp && next == 0x20u) ends |= 1u << j;
-      prevb = b;
+
+// Persistent wavefronts, one row at a time, with the next row's offsets and the next chunk already in
+// flight.  For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an
+// out-of-vocabulary marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass
+// overwrites it with the word's token count); nwords[r] = words kept; counts[r] = one per hit.
+__global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
+                                                                      uint32_t* __restrict__ arena, uint8_t* __restrict__ arena_cnt,
+                                                                      int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
+                                                                      OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
+                                                                      uint32_t* __restrict__ queue_size)
+{
+  __shared__ ProbeLds lds_all[kTokWaves];
+  int const lane      = lane_id();
+  int const wave      = threadIdx.x / kWave;
+  ProbeLds& lds       = lds_all[wave];
+  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
+  int64_t const rows  = col.size;
+  uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
+
+  int64_t r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
+  // software pipeline: offsets two rows ahead, first chunk one row ahead
+  int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
+  if (r < rows) {
+    o_cur = col.off(r);
+    e_cur = col.off(r + 1);
+  }
+  if (r + nwave < rows) {
+    o_nxt = col.off(r + nwave);
+    e_nxt = col.off(r + nwave + 1);
+  }
+  RowCtx ctx = make_row_ctx(col, o_cur, e_cur - o_cur);
+  // the chunk about to be processed: my four bytes and (lane 63) the byte that follows the chunk
+  uint32_t mine_cur = r < rows ? ctx.load_clean(4 * lane) : 0x20202020u;
+  uint32_t tail_cur = (r < rows && lane == kWave - 1) ? ctx.load_clean(kChunk) : 0x20202020u;
+
+  for (; r < rows; r += nwave) {
+    // issue the loads of the rows to come before touching this row's data
+    RowCtx const ctx_nxt = make_row_ctx(col, o_nxt, e_nxt - o_nxt);
+    bool const have_nxt  = r + nwave < rows;
+    int64_t o_nn = 0, e_nn = 0;
+    if (r + 2 * nwave < rows) {
+      o_nn = col.off(r + 2 * nwave);
+      e_nn = col.off(r + 2 * nwave + 1);
     }
-    // prefix over the lanes below (exclusive), seeded with the carry from the previous chunk
-    uint32_t im = m, iv = v;
-    wave_scan_hash(im, iv);
-    uint32_t xm = from_lane_below<1>(im);
-    uint32_t xv = from_lane_below<0>(iv);
-    xv          = carry_hash * xm + xv;
-    uint32_t const is   = wave_scan_max(smax);
-    uint32_t xs         = max(from_lane_below<0>(is), carry_start);
-    carry_hash          = carry_hash * wave_bcast(im, kWave - 1) + wave_bcast(iv, kWave - 1);
-    carry_start         = max(carry_start, wave_bcast(is, kWave - 1));
 
-    uint32_t const ne   = __builtin_popcount(ends);
-    uint32_t const incl = wave_inclusive_scan(ne);
-    uint32_t const total = wave_bcast(incl, kWave - 1);
-    uint32_t slot        = incl - ne;
-    uint32_t prevb2      = before;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      uint32_t const b = (mine >> (8 * j)) & 0xffu;
-      lds.pt[ring0 + j] = xv * bm[j] + bv[j];
-      if (b != 0x20u && prevb2 == 0x20u) xs = static_cast<uint32_t>(a0) + j + 1;
-      if (ends & (1u << j)) {
-        uint32_t const wl = static_cast<uint32_t>(a0) + j + 1 - xs + 1;
-        lds.wend[slot]    = static_cast<uint16_t>(ring0 + j);
-        lds.wlen[slot]    = static_cast<uint16_t>(min(wl, kMaxWord));
-        ++slot;
+    int64_t const n = ctx.n;
+    // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
+    // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
+    int64_t cap = std::numeric_limits<int64_t>::max();
+    if (max_words > 0) cap = col.valid(r) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
+    int64_t const slot0   = ((o_cur - first_offset) >> 1) + r;
+    uint32_t* const slots = arena + slot0;
+    uint8_t* const scnt   = arena_cnt + slot0;
+
+    int64_t words_done   = 0;
+    uint32_t hits        = 0;
+    uint32_t carry_hash  = 0;     // hash of the word running into the chunk (0 after a space)
+    uint32_t carry_start = 0;     // 1-based aligned coordinate of the start of that word
+    uint32_t prev_last   = 0x20;  // byte before the chunk
+    bool next_is_row = false;  // whether the prefetched chunk is the next row's first one
+    for (int64_t cbase = 0; cbase < ctx.aend && words_done < cap; cbase += kChunk) {
+      int64_t const a0    = cbase + 4 * lane;
+      uint32_t const mine = mine_cur;
+      uint32_t const tail = tail_cur;
+      // prefetch the chunk that follows: the rest of this row, else the start of the next row
+      bool const more = cbase + kChunk < ctx.aend;
+      next_is_row     = !more;
+      if (more || have_nxt) {
+        RowCtx const& pc    = more ? ctx : ctx_nxt;
+        int64_t const pbase = more ? cbase + kChunk : 0;
+        mine_cur            = pc.load_clean(pbase + 4 * lane);
+        tail_cur            = lane == kWave - 1 ? pc.load_clean(pbase + kChunk) : 0x20202020u;
       }
-      prevb2 = b;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      uint32_t const ring0 = static_cast<uint32_t>(a0) & (kRing - 1);
+      lds.bytes[ring0 >> 2] = mine;
+      // neighbours: the byte before my four and the byte after them
+      uint32_t before = from_lane_below<0>(mine >> 24);
+      if (lane == 0) before = prev_last;
+      uint32_t after = static_cast<uint32_t>(__shfl_down(static_cast<int>(mine & 0xffu), 1));
+      if (lane == kWave - 1) after = tail & 0xffu;
+      prev_last = wave_bcast(mine >> 24, kWave - 1);
 
-    int64_t const allowed = min(static_cast<int64_t>(total), cap - words_done);
-    for (uint32_t w0 = 0; w0 < allowed; w0 += kWave) {
-      uint32_t const wi = w0 + lane;
-      bool const active = wi < allowed;
-      uint32_t cnt = 0, wstart = 0;
+      // hash block of my bytes, last word start among them, word ends
+      uint32_t bm[4], bv[4];
+      uint32_t m = 1, v = 0, smax = 0, ends = 0;
+      uint32_t prevb = before;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t const b    = (mine >> (8 * j)) & 0xffu;
+        uint32_t const next = j < 3 ? (mine >> (8 * (j + 1))) & 0xffu : after;
+        bool const sp       = b == 0x20u;
+        uint32_t const em   = sp ? 0u : kHashB;
+        uint32_t const ev   = sp ? 0u : b;
+        v                   = v * em + ev;
+        m                   = m * em;
+        bm[j]               = m;
+        bv[j]               = v;
+        if (!sp && prevb == 0x20u) smax = static_cast<uint32_t>(a0) + j + 1;
+        if (!sp && next == 0x20u) ends |= 1u << j;
+        prevb = b;
+      }
+      // state entering my bytes: lanes below (exclusive) seeded with the carry from the previous chunk
+      uint32_t im = m, iv = v;
+      wave_scan_hash(im, iv);
+      uint32_t const xm = from_lane_below<1>(im);
+      uint32_t const xv = carry_hash * xm + from_lane_below<0>(iv);
+      uint32_t const is = wave_scan_max(smax);
+      uint32_t xs       = max(from_lane_below<0>(is), carry_start);
+      carry_hash        = carry_hash * wave_bcast(im, kWave - 1) + wave_bcast(iv, kWave - 1);
+      carry_start       = max(carry_start, wave_bcast(is, kWave - 1));
+
+      uint32_t const ne    = __builtin_popcount(ends);
+      uint32_t const incl  = wave_inclusive_scan(ne);
+      uint32_t const total = wave_bcast(incl, kWave - 1);
+      uint32_t slot        = incl - ne;
+      prevb                = before;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t const b = (mine >> (8 * j)) & 0xffu;
+        if (b != 0x20u && prevb == 0x20u) xs = static_cast<uint32_t>(a0) + j + 1;
+        if (ends & (1u << j)) {
+          lds.wstart[slot] = xs;
+          lds.wend[slot]   = static_cast<uint32_t>(a0) + j + 1;
+          lds.whash[slot]  = xv * bm[j] + bv[j];
+          ++slot;
+        }
+        prevb = b;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      int64_t const allowed = min(static_cast<int64_t>(total), cap - words_done);
+      for (uint32_t w0 = 0; w0 < allowed; w0 += kWave) {
+        uint32_t const wi = w0 + lane;
+        bool const active = wi < allowed;
+        bool miss         = false;
+        uint32_t value    = 0, ws = 0;
+        if (active) {
+          ws                = lds.wstart[wi];
+          uint32_t const wl = lds.wend[wi] - ws + 1;
+          if (wl >= kMaxWord) {
+            value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+          } else {
+            int32_t id = kNone;
+            if (wl <= table.max_len[0]) id = lookup(table, 0, lds.whash[wi], RingWord{lds.bytes, (ws - 1) & (kRing - 1)}, 0, wl);
+            miss  = id == kNone;
+            value = static_cast<uint32_t>(id);
+          }
+        }
+        uint64_t const mm = ballot64(miss);
+        if (mm) {
+          uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
+          if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
+            // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
+            for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+              if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(queue_size, queue_block);
+            q_pos = wave_bcast(base, 0);
+            q_lim = q_pos + queue_block;
+          }
+          if (miss) {
+            uint32_t const q = q_pos + lanes_below(mm);
+            if (q < queue_capacity) queue[q] = OovEntry{static_cast<int32_t>(r), ws - 1 - ctx.mis, static_cast<uint32_t>(words_done) + wi, 0u};
+            value = kOovMark | q;
+          }
+          q_pos += nm;
+        }
+        if (active) {
+          slots[words_done + wi] = value;
+          scnt[words_done + wi]  = 1;
+        }
+        hits += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && !miss)));
+      }
+      words_done += allowed;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0) {
+      nwords[r] = static_cast<int32_t>(words_done);
+      counts[r] = static_cast<int32_t>(hits);
+    }
+    // rotate the pipeline.  The prefetched chunk is the next row's first one unless the row was left
+    // early (word limit reached, or an empty row whose loop never ran): then fetch it now.
+    if (!next_is_row && have_nxt) {
+      mine_cur = ctx_nxt.load_clean(4 * lane);
+      tail_cur = lane == kWave - 1 ? ctx_nxt.load_clean(kChunk) : 0x20202020u;
+    }
+    ctx   = ctx_nxt;
+    o_cur = o_nxt;
+    o_nxt    = o_nn;
+    e_nxt    = e_nn;
+  }
+  for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+}
+
+// ------------------------------------------------------------------ out-of-vocabulary pass
+constexpr uint32_t kStage = 64;  // bytes of each queued word kept in LDS (from a 16-byte aligned base)
+
+// A queued word whose first kStage - mis bytes sit in this lane's LDS window; later bytes come from memory.
+struct StagedWord {
+  const uint32_t* win;  // this lane's kStage-byte window
+  const uint8_t* p;     // the word in global memory
+  uint32_t mis;         // offset of the word inside the window
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const
+  {
+    uint32_t const o = mis + k;
+    return o < kStage ? reinterpret_cast<const uint8_t*>(win)[o] : p[k];
+  }
+  __device__ __forceinline__ void key8(uint32_t off, uint32_t len, uint32_t* k0, uint32_t* k1) const
+  {
+    uint32_t const o = mis + off;
+    uint32_t lo, hi;
+    if (o + 12 <= kStage) {
+      uint32_t const i  = o >> 2;
+      uint32_t const sh = (o & 3u) * 8u;
+      uint32_t const d0 = win[i], d1 = win[i + 1], d2 = win[i + 2];
+      lo                = __builtin_amdgcn_alignbit(d1, d0, sh);
+      hi                = __builtin_amdgcn_alignbit(d2, d1, sh);
+    } else {
+      lo = hi = 0;
+      for (uint32_t k = 0; k < 8 && k < len; ++k) {
+        uint32_t const b = byte(off + k);
+        if (k < 4) lo |= b << (8 * k); else hi |= b << (8 * (k - 4));
+      }
+    }
+    if (len < 4) lo &= (1u << (8 * len)) - 1u;
+    if (len <= 4) hi = 0;
+    else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+    *k0 = lo;
+    *k1 = hi;
+  }
+};
+
+// Greedy longest-match-first tokenization (cpp/src/text/wordpiece_tokenize.cu:349-407) of a word of
+// `len` bytes, 1 <= len < 200, whose whole-word lookup has already failed.  `emit(j, id)` receives token j;
+// returns the token count (a collapse to one unknown token re-emits token 0).
+//
+// One flat loop with one table probe per trip, so that the lanes of a wavefront, each at a different
+// stage of its own word, share trips instead of serialising nested loops.  The state is the piece
+// being searched: bytes [start, e) with `he` = hash of [0, e), `hs` = hash of [0, start) and
+// pwe = B^(e - start); its hash is he - hs * pwe.  The first piece (start 0) lives in the full key
+// space, later ones in the "##" space.
+template <typename W, typename Emit>
+__device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
+{
+  uint32_t hfull = 0, pwr = 1;  // pwr = B^(len - start)
+  for (uint32_t i = 0; i < len; ++i) {
+    hfull = hfull * kHashB + w.byte(i);
+    pwr *= kHashB;
+  }
+  uint32_t start = 0, hs = 0, e = len, he = hfull, pwe = pwr, count = 0;
+  bool fresh = false;  // the whole word is known to be absent: begin by shortening it
+  for (;;) {
+    if (!fresh) {
+      // wordpiece_tokenize.cu:307-317: drop the last UTF-8 character of the candidate
+      uint32_t x = (e - start) < 2 ? start : e - 1;
+      while (x > start && is_utf8_continuation(w.byte(x))) --x;
+      if (x == start) {
+        // no prefix of the word matched (375-379), or a later piece has no match and the word
+        // collapses (396-404): either way a single unknown token
+        emit(0u, t.unk_id);
+        return 1;
+      }
+      for (uint32_t i = e; i > x; --i) {
+        he = (he - w.byte(i - 1)) * kHashBInv;
+        pwe *= kHashBInv;
+      }
+      e = x;
+    }
+    fresh                = false;
+    uint32_t const kind = count ? 1u : 0u;
+    uint32_t const pl   = e - start;
+    if (pl > t.max_len[kind]) continue;
+    int32_t const id = lookup(t, kind, he - hs * pwe, w, start, pl);
+    if (id == kNone) continue;
+    emit(count++, id);
+    if (e == len) return count;
+    // next piece: the rest of the word (381-395)
+    for (uint32_t i = start; i < e; ++i) pwr *= kHashBInv;
+    start = e;
+    hs    = he;
+    e     = len;
+    he    = hfull;
+    pwe   = pwr;
+    fresh = true;
+  }
+}
+
+// Brings the first bytes of the word at p (row bytes end at row_end) into this lane's LDS window with
+// 16-byte aligned loads that stay inside [p & ~15, row_end rounded up to 16), and returns its length.
+__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, int64_t avail, uint32_t* win, uint32_t* mis_out)
+{
+  uint32_t const mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
+  const uint4* a     = reinterpret_cast<const uint4*>(p - mis);
+  // 16-byte blocks that hold row bytes (never a block wholly past the row)
+  uint32_t const blocks = static_cast<uint32_t>(min(static_cast<int64_t>(kStage / 16), (static_cast<int64_t>(mis) + avail + 15) >> 4));
+  uint4* w4             = reinterpret_cast<uint4*>(win);
+  for (uint32_t i = 0; i < blocks; ++i) w4[i] = a[i];
+  *mis_out = mis;
+  // the word ends at the first space or at the end of the row
+  uint32_t const lim = static_cast<uint32_t>(min(avail, static_cast<int64_t>(kMaxWord)));
+  uint32_t len       = 0;
+  const uint8_t* wb  = reinterpret_cast<const uint8_t*>(win) + mis;
+  uint32_t const in_window = min(lim, kStage - mis);
+  while (len < in_window && wb[len] != 0x20u) ++len;
+  if (len == in_window)
+    while (len < lim && p[len] != 0x20u) ++len;
+  return len;
+}
+
+// One lane per queued word.  results[q] = its first kOovKeep tokens; arena_cnt[slot] = its token count;
+// counts[row] += count.
+__global__ void __launch_bounds__(256) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
+                                                            const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
+                                                            int64_t first_offset, OovResult* __restrict__ results,
+                                                            uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts)
+{
+  __shared__ __align__(16) uint32_t windows[256][kStage / 4];
+  uint32_t const total  = min(*queue_size, queue_capacity);
+  uint32_t const stride = gridDim.x * blockDim.x;
+  uint32_t* const win   = windows[threadIdx.x];
+  for (uint32_t q = blockIdx.x * blockDim.x + threadIdx.x; q < total; q += stride) {
+    OovEntry const e = queue[q];
+    if (e.row < 0) continue;  // unused tail of a reserved range
+    int64_t const o  = col.off(e.row);
+    int64_t const n  = col.off(e.row + 1) - o;
+    const uint8_t* p = col.chars + o + e.delta;
+    uint32_t mis;
+    uint32_t const len = stage_word(p, n - static_cast<int64_t>(e.delta), win, &mis);
+    StagedWord const w{win, p, mis};
+    int32_t tok[kOovKeep];
+    uint32_t const cnt = tokenize_oov_word(table, w, len, [&](uint32_t j, int32_t id) {
+#pragma unroll
+      for (int k = 0; k < kOovKeep; ++k)
+        if (j == static_cast<uint32_t>(k)) tok[k] = id;
+    });
+    OovResult res;
+#pragma unroll
+    for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
+    results[q] = res;
+    arena_cnt[((o - first_offset) >> 1) + e.row + e.widx] = static_cast<uint8_t>(cnt);  // cnt <= len < 200
+    atomicAdd(&counts[e.row], static_cast<int32_t>(cnt));
+  }
+}
+
+// ------------------------------------------------------------------ emit pass
+// Persistent wavefronts, one row at a time: expands the row's word arena into out + offsets[r].
+// Row descriptors are loaded two rows ahead and the first 64 word slots one row ahead.
+__global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
+                                                                     const uint32_t* __restrict__ arena, const uint8_t* __restrict__ arena_cnt,
+                                                                     const int32_t* __restrict__ nwords, const OovEntry* __restrict__ queue,
+                                                                     const OovResult* __restrict__ results, const int32_t* __restrict__ offsets,
+                                                                     int32_t* __restrict__ out)
+{
+  int const lane      = lane_id();
+  int const wave      = threadIdx.x / kWave;
+  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
+  int64_t const rows  = col.size;
+  int64_t r           = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
+
+  struct Desc {
+    int32_t W;
+    int32_t begin;
+    int64_t slot0;
+  };
+  auto load_desc = [&](int64_t row) -> Desc {
+    Desc d{0, 0, 0};
+    if (row < rows) {
+      d.W     = nwords[row];
+      d.begin = offsets[row];
+      d.slot0 = arena_pos(col, first_offset, row);
+    }
+    return d;
+  };
+  Desc cur = load_desc(r);
+  Desc nxt = load_desc(r + nwave);
+  uint32_t v_cur = 0, c_cur = 0;
+  if (lane < cur.W) {
+    v_cur = arena[cur.slot0 + lane];
+    c_cur = arena_cnt[cur.slot0 + lane];
+  }
+  for (; r < rows; r += nwave) {
+    Desc const nn = load_desc(r + 2 * nwave);
+    uint32_t v_nxt = 0, c_nxt = 0;
+    if (lane < nxt.W) {
+      v_nxt = arena[nxt.slot0 + lane];
+      c_nxt = arena_cnt[nxt.slot0 + lane];
+    }
+    int32_t* const dst = out + cur.begin;
+    uint32_t done      = 0;
+    for (int32_t w0 = 0; w0 < cur.W; w0 += kWave) {
+      int32_t const wi  = w0 + lane;
+      bool const active = wi < cur.W;
+      uint32_t value = v_cur, cnt = c_cur;
+      if (w0 > 0) {
+        value = active ? arena[cur.slot0 + wi] : 0u;
+        cnt   = active ? arena_cnt[cur.slot0 + wi] : 0u;
+      }
+      if (!active) cnt = 0;
+      bool const oov      = active && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
+      uint32_t const incl = wave_inclusive_scan(cnt);
       if (active) {
-        uint32_t const wl = lds.wlen[wi];
-        wstart            = (static_cast<uint32_t>(lds.wend[wi]) + kRing + 1 - wl) & (kRing - 1);
-        if (wl >= kMaxWord) {
-          // wordpiece_tokenize.cu:442-445, 738-741.  The clamped length no longer locates the word start,
-          // so the single token is parked on the word's last byte.
-          wstart         = lds.wend[wi];
-          lds.pt[wstart] = static_cast<uint32_t>(table.unk_id);
-          cnt            = 1;
+        int32_t* d = dst + done + (incl - cnt);
+        if (!oov) {
+          d[0] = static_cast<int32_t>(value);
         } else {
-          cnt = wp_tokenize(table, lds, pw, wstart, wl);
+          uint32_t const q = value & ~kOovMark;
+          if (cnt <= kOovKeep) {
+            for (uint32_t k = 0; k < cnt; ++k) d[k] = results[q].tok[k];
+          } else {
+            // more pieces than a queue entry keeps: tokenize the word again, straight into place
+            OovEntry const e = queue[q];
+            int64_t const o  = col.off(e.row);
+            int64_t const n  = col.off(e.row + 1) - o;
+            const uint8_t* p = col.chars + o + e.delta;
+            uint32_t const avail = static_cast<uint32_t>(min(n - static_cast<int64_t>(e.delta), static_cast<int64_t>(kMaxWord)));
+            uint32_t len         = 0;
+            while (len < avail && p[len] != 0x20u) ++len;
+            tokenize_oov_word(table, GlobalWord{p}, len, [&](uint32_t j, int32_t id) { d[j] = id; });
+          }
         }
       }
-      uint32_t const inc2 = wave_inclusive_scan(cnt);
-      if (active) {
-        int64_t at = static_cast<int64_t>(tokens_done) + (inc2 - cnt);
-        for (uint32_t k = 0; k < cnt; ++k, ++at)
-          if (at < slots) dst[at] = static_cast<int32_t>(lds.pt[(wstart + k) & (kRing - 1)]);
-      }
-      tokens_done += wave_bcast(inc2, kWave - 1);
+      done += wave_bcast(incl, kWave - 1);
     }
-    words_done += allowed;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-  }
-  return tokens_done;
-}
-
-// Arena layout: row r owns the slots [arena_pos(r), arena_pos(r+1)), at least floor(bytes/2) + 1 of them.
-__device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
-
-__device__ __forceinline__ void init_powers(uint32_t* pw)
-{
-  // pw[k] = B^k mod 2^32 for k < kMaxWord, by square-and-multiply
-  for (uint32_t k = threadIdx.x; k < kMaxWord; k += blockDim.x) {
-    uint32_t r = 1, b = kHashB;
-    for (uint32_t e = k; e; e >>= 1) {
-      if (e & 1u) r *= b;
-      b *= b;
-    }
-    pw[k] = r;
-  }
-  __syncthreads();
-}
-
-// Pass 1: one wavefront per row tokenizes into the arena; counts[r] = tokens of row r.
-__global__ void __launch_bounds__(kTokThreads) wordpiece_tokenize_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                         int32_t* __restrict__ arena, int32_t* __restrict__ counts)
-{
-  __shared__ TokLds lds_all[kTokWaves];
-  __shared__ uint32_t pw[kMaxWord];
-  init_powers(pw);
-  int const lane  = lane_id();
-  int const wave  = threadIdx.x / kWave;
-  int64_t const r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
-  if (r >= col.size) return;
-  int64_t const ap    = arena_pos(col, first_offset, r);
-  int64_t const slots = arena_pos(col, first_offset, r + 1) - ap;
-  uint32_t const n    = tokenize_row(col, table, max_words, r, lds_all[wave], pw, arena + ap, slots, lane);
-  if (lane == 0) counts[r] = static_cast<int32_t>(n);
-}
-
-// Pass 2: copy each row's tokens from the arena to out + offsets[r]; a row with more tokens than
-// arena slots is tokenized again straight into place.
-__global__ void __launch_bounds__(kTokThreads) wordpiece_gather_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                       const int32_t* __restrict__ arena, const int32_t* __restrict__ offsets,
-                                                                       int32_t* __restrict__ out)
-{
-  __shared__ TokLds lds_all[kTokWaves];
-  __shared__ uint32_t pw[kMaxWord];
-  init_powers(pw);
-  int const lane  = lane_id();
-  int const wave  = threadIdx.x / kWave;
-  int64_t const r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
-  if (r >= col.size) return;
-  int32_t const begin = offsets[r];
-  int32_t const n     = offsets[r + 1] - begin;
-  int64_t const ap    = arena_pos(col, first_offset, r);
-  int64_t const slots = arena_pos(col, first_offset, r + 1) - ap;
-  if (n <= slots) {
-    for (int32_t k = lane; k < n; k += kWave) out[begin + k] = arena[ap + k];
-  } else {
-    tokenize_row(col, table, max_words, r, lds_all[wave], pw, out + begin, std::numeric_limits<int64_t>::max(), lane);
+    cur   = nxt;
+    nxt   = nn;
+    v_cur = v_nxt;
+    c_cur = c_nxt;
   }
 }
 
@@ -716,44 +982,90 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_INVALID_ARGUMENT, "offsets are not monotone");
   }
+  // word arena: one slot per possible word; row r gets floor(bytes/2) + 1 slots
   size_t const arena_slots = static_cast<size_t>((last_offset - first_offset) >> 1) + static_cast<size_t>(rows) + 1;
-  Temp arena(mr, arena_slots * sizeof(int32_t));
+  // queue of words whose whole-word probe missed.  Sized for a generous share of the input; if a run
+  // overflows it the exact size is known afterwards and the passes are repeated once.
+  int device = 0, cus = 256;
+  (void)hipGetDevice(&device);
+  (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+  unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves - 1) / kTokWaves,
+                                                                      static_cast<int64_t>(cus) * 8));
+  // Each wavefront reserves queue entries `queue_block` at a time (one atomic per block).
+  uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
+  uint32_t queue_block = 64;
+  while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
+  uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
+  Temp arena(mr, arena_slots * sizeof(uint32_t));
+  Temp arena_cnt(mr, arena_slots);
+  Temp nwords(mr, static_cast<size_t>(rows) * sizeof(int32_t));
   Temp counts(mr, static_cast<size_t>(rows) * sizeof(int32_t));
   Temp scan_tmp(mr, scan_temp_bytes(rows));
-  if (!arena.ok() || !counts.ok() || !scan_tmp.ok()) {
+  Temp qsize(mr, 256);
+  if (!arena.ok() || !arena_cnt.ok() || !nwords.ok() || !counts.ok() || !scan_tmp.ok() || !qsize.ok()) {
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
-  unsigned const blocks = static_cast<unsigned>((static_cast<int64_t>(rows) + kTokWaves - 1) / kTokWaves);
-  {
-    ProfileScope ps("wordpiece_tokenize_kernel", stream);
-    hipLaunchKernelGGL(wordpiece_tokenize_kernel, dim3(blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
-                       first_offset, arena.as<int32_t>(), counts.as<int32_t>());
-  }
-  // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
-  device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
   uint64_t total = 0;
-  hipError_t e   = hipMemcpyAsync(&total, scan_tmp.as<uint64_t>() + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-  if (e == hipSuccess) e = hipStreamSynchronize(stream);
-  if (e != hipSuccess) {
-    nvtext_amd_list_column_free(out, stream_, mr_);
-    return fail(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
-  }
-  if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
-    nvtext_amd_list_column_free(out, stream_, mr_);
-    return fail(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
-  }
-  out->child_size  = static_cast<int64_t>(total);
-  out->child_bytes = static_cast<size_t>(total) * sizeof(int32_t);
-  if (total) {
-    out->child = mr.allocate(out->child_bytes);
-    if (!out->child) {
+  for (int attempt = 0;; ++attempt) {
+    if (queue_capacity > 0x7FFFFFFEull) queue_capacity = 0x7FFFFFFEull;
+    uint32_t const qcap = static_cast<uint32_t>(queue_capacity);
+    Temp queue(mr, static_cast<size_t>(qcap) * sizeof(OovEntry));
+    Temp results(mr, static_cast<size_t>(qcap) * sizeof(OovResult));
+    if (!queue.ok() || !results.ok()) {
       nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
     }
-    ProfileScope ps("wordpiece_gather_kernel", stream);
-    hipLaunchKernelGGL(wordpiece_gather_kernel, dim3(blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row, first_offset,
-                       arena.as<int32_t>(), out->offsets, static_cast<int32_t*>(out->child));
+    launch_fill_u32(qsize.as<uint32_t>(), 0u, 1, stream);
+    {
+      ProfileScope ps("wordpiece_probe_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
+                         first_offset, arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
+                         queue_block, qsize.as<uint32_t>());
+    }
+    {
+      ProfileScope ps("wordpiece_oov_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(cus) * 8), dim3(256), 0, stream, v, vocabulary->table,
+                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, first_offset, results.as<OovResult>(), arena_cnt.as<uint8_t>(),
+                         counts.as<int32_t>());
+    }
+    // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
+    device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
+    uint32_t queued = 0;
+    hipError_t e    = hipMemcpyAsync(&total, scan_tmp.as<uint64_t>() + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(&queued, qsize.as<uint32_t>(), sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+    }
+    if (queued > qcap) {  // the queue was too small: repeat once with the exact size
+      if (attempt > 0 || queued > 0x7FFFFFFEu) {
+        nvtext_amd_list_column_free(out, stream_, mr_);
+        return fail(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+      }
+      queue_capacity = queued;
+      continue;
+    }
+    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
+    }
+    out->child_size  = static_cast<int64_t>(total);
+    out->child_bytes = static_cast<size_t>(total) * sizeof(int32_t);
+    if (total) {
+      out->child = mr.allocate(out->child_bytes);
+      if (!out->child) {
+        nvtext_amd_list_column_free(out, stream_, mr_);
+        return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
+      }
+      ProfileScope ps("wordpiece_emit_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
+                         arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
+                         out->offsets,
+                         static_cast<int32_t*>(out->child));
+    }
+    break;
   }
   NVTEXT_HIP_TRY(hipGetLastError());
   return NVTEXT_AMD_SUCCESS;
