@@ -1,28 +1,23 @@
 // wordpiece_vocabulary + wordpiece_tokenize for gfx950.
 //
 // The reference (cpp/src/text/wordpiece_tokenize.cu) keeps two cuco hash maps keyed by
-// MurmurHash3 of the candidate substring and re-hashes every shrinking prefix (O(L^2) per
-// out-of-vocabulary word, 349-407), marks word starts with a copy_if over all bytes, merges
-// them with the row offsets and writes tokens into a 4-byte-per-input-byte temporary that is
-// then counted and compacted (503-568, 462-491, 877-881).
+// MurmurHash3 of the candidate substring, marks word starts with a copy_if over all bytes,
+// merges them with the row offsets and writes tokens into a 4-byte-per-input-byte temporary
+// that is then counted and compacted (503-568, 462-491, 877-881).
 //
 // Here:
 //   * one open-addressing table of 2-slot buckets (16-byte slots, load <= 0.5) holds both key
 //     spaces: whole entries (kind 0) and "##" entries without their prefix (kind 1).  Keys of
-//     up to 8 bytes sit inside the slot, so a probe is one 32-byte read; the table for a
-//     30k-entry vocabulary is 2 MiB and stays in L2.
-//   * the key hash is polynomial (H <- H*B + byte mod 2^32): dropping the last byte of a
-//     candidate is one subtract and one multiply by B^-1, and an inner piece is
-//     P[e] - P[p] * B^(e-p), so no candidate is ever re-hashed.
-//   * probe pass: a wavefront walks rows in 256-byte chunks with lanes <-> bytes; a segmented
-//     DPP scan over (multiplier, value) pairs yields the hash of every word at its last byte,
-//     a max-scan yields its start.  Then lanes <-> words: ONE probe per word.  A hit stores the
-//     token in the row's word arena (one slot per word, floor(bytes/2)+1 slots per row); a miss
-//     stores a marker and appends the word to a queue.
+//     up to 8 bytes sit inside the slot, so a probe is one 32-byte read and the key's two dwords
+//     are also what gets hashed; the table for a 30k-entry vocabulary is 2 MiB and stays in L2.
+//   * probe pass: a wavefront walks a row in 1 KiB chunks, 16 bytes per lane.  Spaces become a
+//     16-bit mask per lane with four SWAR operations per dword; word starts and ends are bit
+//     operations on that mask; DPP scans place the words of the chunk in an LDS list.  Then
+//     lanes <-> words: ONE probe per word.  A hit stores the token in the row's word arena (one
+//     slot per word, floor(bytes/2)+1 slots per row); a miss stores a marker and queues the word.
 //   * out-of-vocabulary pass: one lane per queued word, all lanes busy, runs the greedy
-//     longest-match rule with O(1) hash updates and stores count + tokens per queue entry.
-//     (Doing this inside the probe pass leaves 90 % of the lanes idle behind a chain of
-//     dependent L2 probes.)
+//     longest-match rule as a flat loop with one probe per trip and stores the tokens per queue
+//     entry.  (Inside the probe pass this chain of dependent probes would idle 90 % of the lanes.)
 //   * a device-wide scan of the per-row token counts makes the int32 list offsets; the emit pass
 //     expands each row's word arena into its tokens.  No chars-sized temporary is written.
 #include "common.cuh"
@@ -37,16 +32,6 @@ namespace nvtext_amd {
 namespace {
 
 constexpr uint32_t kMaxWord = 200;  // wordpiece_tokenize.cu:300: words this long become one [UNK]
-constexpr uint32_t kHashB   = 0x01000193u;
-
-constexpr uint32_t inv_mod_2_32(uint32_t a)
-{
-  uint32_t x = a;  // Newton iteration: correct to 3 bits, doubles every step
-  for (int i = 0; i < 5; ++i) x *= 2u - a * x;
-  return x;
-}
-constexpr uint32_t kHashBInv = inv_mod_2_32(kHashB);
-static_assert(kHashB * kHashBInv == 1u, "B^-1 mod 2^32");
 
 __host__ __device__ __forceinline__ uint32_t mix32(uint32_t h)
 {
@@ -56,6 +41,15 @@ __host__ __device__ __forceinline__ uint32_t mix32(uint32_t h)
   h *= 0xc2b2ae35u;
   h ^= h >> 16;
   return h;
+}
+
+// Key hash: the key is consumed in 8-byte blocks (two little-endian dwords, zero padded).
+__host__ __device__ __forceinline__ uint32_t key_hash_init(uint32_t len) { return len * 0xC2B2AE3Du; }
+__host__ __device__ __forceinline__ uint32_t key_hash_block(uint32_t h, uint32_t lo, uint32_t hi)
+{
+  h = (h ^ lo) * 0x9E3779B1u;
+  h = (h ^ hi) * 0x85EBCA77u;
+  return h ^ (h >> 15);
 }
 
 // slot.x = (tag23 << 9) | (kind << 8) | len   (0 = empty; len in 1..199)
@@ -72,7 +66,7 @@ struct VocabTable {
 
 __host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t h, uint32_t kind, uint32_t len, uint32_t* bucket)
 {
-  uint32_t const x = mix32(h + len * 0x9E3779B9u + kind * 0x7F4A7C15u);
+  uint32_t const x = mix32(h + kind * 0x7F4A7C15u);
   *bucket          = x;
   return (x & 0xFFFFFE00u) | (kind << 8) | len;
 }
@@ -92,12 +86,12 @@ struct nvtext_amd_wordpiece_vocabulary {
 namespace nvtext_amd {
 namespace {
 
-constexpr int kTokWaves   = 4;
-constexpr int kTokThreads = kTokWaves * kWave;
-constexpr int kChunk      = 256;  // bytes per wavefront step (4 per lane)
-constexpr int kRing       = 512;  // two chunks: the current one and the one before it
-constexpr int32_t kNone   = std::numeric_limits<int32_t>::min();
-constexpr int kOovKeep    = 8;    // tokens stored per queued word; longer results are redone at emit time
+constexpr int kTokWaves     = 4;
+constexpr int kTokThreads   = kTokWaves * kWave;
+constexpr int kChunk        = 1024;  // bytes per wavefront step (16 per lane)
+constexpr int kRing         = 2048;  // two chunks: the current one and the one before it
+constexpr int32_t kNone     = std::numeric_limits<int32_t>::min();
+constexpr int kOovKeep      = 8;     // tokens stored per queued word; longer results are redone at emit time
 constexpr uint32_t kOovMark = 0x80000000u;  // word-arena value 0x80000000 | queue index (never 0xFFFFFFFF = id -1)
 
 struct OovEntry {
@@ -110,8 +104,16 @@ struct OovResult {
   int32_t tok[kOovKeep];
 };
 
-// ------------------------------------------------------------------ keys in the LDS ring / in global memory
-// A word inside the 512-byte ring: byte k of the word is ring byte (start + k) & 511.
+// ------------------------------------------------------------------ where candidate keys live
+// Each source offers byte(k) and key8(p, len, &k0, &k1): bytes [p, p+8) as two dwords, zero padded past len.
+__device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& hi)
+{
+  if (len < 4) lo &= (1u << (8 * len)) - 1u;
+  if (len <= 4) hi = 0;
+  else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+}
+
+// A word inside the 2 KiB LDS ring of the probe pass: byte k of the word is ring byte (start + k) & 2047.
 struct RingWord {
   const uint32_t* ring;
   uint32_t start;
@@ -124,15 +126,13 @@ struct RingWord {
     uint32_t const d0 = ring[i], d1 = ring[(i + 1) & (kRing / 4 - 1)], d2 = ring[(i + 2) & (kRing / 4 - 1)];
     uint32_t lo       = __builtin_amdgcn_alignbit(d1, d0, sh);
     uint32_t hi       = __builtin_amdgcn_alignbit(d2, d1, sh);
-    if (len < 4) lo &= (1u << (8 * len)) - 1u;
-    if (len <= 4) hi = 0;
-    else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+    trim_key8(len, lo, hi);
     *k0 = lo;
     *k1 = hi;
   }
 };
 
-// A word in global memory (bytes p[0 .. )).  key8 reads only aligned dwords that overlap the key.
+// A word in global memory (emit pass, rare path).  key8 reads only aligned dwords that overlap the key.
 struct GlobalWord {
   const uint8_t* p;
   __device__ __forceinline__ uint32_t byte(uint32_t k) const { return p[k]; }
@@ -141,348 +141,21 @@ struct GlobalWord {
     const uint8_t* q    = p + off;
     uint32_t const mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(q) & 3u);
     const uint32_t* a   = reinterpret_cast<const uint32_t*>(q - mis);
-    uint32_t const sh   = mis * 8u;
     uint32_t const need = mis + (len < 8 ? len : 8);  // bytes from the aligned base
     uint32_t const d0   = a[0];
     uint32_t const d1   = need > 4 ? a[1] : 0u;
     uint32_t const d2   = need > 8 ? a[2] : 0u;
-    uint32_t lo         = __builtin_amdgcn_alignbit(d1, d0, sh);
-    uint32_t hi         = __builtin_amdgcn_alignbit(d2, d1, sh);
-    if (len < 4) lo &= (1u << (8 * len)) - 1u;
-    if (len <= 4) hi = 0;
-    else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+    uint32_t lo         = __builtin_amdgcn_alignbit(d1, d0, mis * 8u);
+    uint32_t hi         = __builtin_amdgcn_alignbit(d2, d1, mis * 8u);
+    trim_key8(len, lo, hi);
     *k0 = lo;
     *k1 = hi;
   }
 };
 
-template <typename W>
-__device__ __forceinline__ bool slot_matches(VocabTable const& t, uint4 const& s, uint32_t want, uint32_t len, uint32_t k0, uint32_t k1, W const& w,
-                                             uint32_t p)
-{
-  if (s.x != want) return false;
-  if (len <= 8) return s.z == k0 && s.w == k1;
-  const uint8_t* e = t.pool + s.z;
-  uint32_t i       = 0;
-  while (i < len && e[i] == w.byte(p + i)) ++i;
-  return i == len;
-}
-
-// Token id of word bytes [p, p+len) in key space `kind` (hash h), or kNone.
-template <typename W>
-__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, uint32_t h, W const& w, uint32_t p, uint32_t len)
-{
-  uint32_t b;
-  uint32_t const want = slot_word0(h, kind, len, &b);
-  uint32_t k0 = 0, k1 = 0;
-  if (len <= 8) w.key8(p, len, &k0, &k1);
-  for (;;) {
-    b &= t.bucket_mask;
-    uint4 const s0 = t.slots[2 * b];
-    uint4 const s1 = t.slots[2 * b + 1];
-    if (slot_matches(t, s0, want, len, k0, k1, w, p)) return static_cast<int32_t>(s0.y);
-    if (s0.x == 0) return kNone;
-    if (slot_matches(t, s1, want, len, k0, k1, w, p)) return static_cast<int32_t>(s1.y);
-    if (s1.x == 0) return kNone;
-    ++b;
-  }
-}
-
-// ------------------------------------------------------------------ wavefront scans used by the probe pass
-template <int CTRL, int ROW_MASK, int OLD>
-__device__ __forceinline__ uint32_t dpp_old(uint32_t v)
-{
-  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(OLD, static_cast<int>(v), CTRL, ROW_MASK, 0xf, false));
-}
-
-// Inclusive scan across the wavefront of hash blocks (m, v) under (m1,v1).(m2,v2) = (m1*m2, v1*m2 + v2):
-// appending block 2 to a prefix of hash v1 gives v1*m2 + v2.  Lanes without a source compose with (1, 0).
-__device__ __forceinline__ void wave_scan_hash(uint32_t& m, uint32_t& v)
-{
-#define NVTEXT_HASH_STEP(CTRL, RM)                          \
-  {                                                         \
-    uint32_t const ms = dpp_old<CTRL, RM, 1>(m);            \
-    uint32_t const vs = dpp_old<CTRL, RM, 0>(v);            \
-    v                 = vs * m + v;                         \
-    m                 = ms * m;                             \
-  }
-  NVTEXT_HASH_STEP(0x111, 0xf)
-  NVTEXT_HASH_STEP(0x112, 0xf)
-  NVTEXT_HASH_STEP(0x114, 0xf)
-  NVTEXT_HASH_STEP(0x118, 0xf)
-  NVTEXT_HASH_STEP(0x142, 0xa)
-  NVTEXT_HASH_STEP(0x143, 0xc)
-#undef NVTEXT_HASH_STEP
-}
-
-__device__ __forceinline__ uint32_t wave_scan_max(uint32_t v)
-{
-  v = max(v, dpp_zero<0x111, 0xf>(v));
-  v = max(v, dpp_zero<0x112, 0xf>(v));
-  v = max(v, dpp_zero<0x114, 0xf>(v));
-  v = max(v, dpp_zero<0x118, 0xf>(v));
-  v = max(v, dpp_zero<0x142, 0xa>(v));
-  v = max(v, dpp_zero<0x143, 0xc>(v));
-  return v;
-}
-
-// value of the lane below (lane 0 gets FIRST)
-template <int FIRST>
-__device__ __forceinline__ uint32_t from_lane_below(uint32_t v)
-{
-  return dpp_old<0x138, 0xf, FIRST>(v);  // wave_shr:1
-}
-
-// Row r owns the word-arena slots [arena_pos(r), arena_pos(r+1)): at least floor(bytes/2) + 1, and a
-// row cannot hold more words than that.
-__device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
-
-struct ProbeLds {
-  uint32_t bytes[kRing / 4];        // row bytes (everything outside the row is ' ')
-  uint32_t wstart[kChunk / 2 + 2];  // per word ending in the chunk: 1-based aligned coordinate of its first byte,
-  uint32_t wend[kChunk / 2 + 2];    // of its last byte,
-  uint32_t whash[kChunk / 2 + 2];   // and its hash
-};
-
-// ------------------------------------------------------------------ probe pass
-// Where a row sits relative to 4-byte aligned memory.
-struct RowCtx {
-  const uint32_t* arow;  // aligned base at or below the row's first byte
-  uint32_t mis;          // row start inside that dword
-  int64_t n;             // row bytes
-  int64_t aend;          // row end in aligned coordinates (mis + n)
-  // aligned dword at coordinate a0 with every byte outside the row replaced by ' '
-  __device__ __forceinline__ uint32_t load_clean(int64_t a0) const
-  {
-    uint32_t v = 0x20202020u;
-    if (a0 < aend && a0 + 4 > static_cast<int64_t>(mis)) {
-      v = arow[a0 >> 2];
-      if (a0 < static_cast<int64_t>(mis)) {
-        uint32_t const m = (1u << (8 * static_cast<uint32_t>(mis - a0))) - 1u;
-        v                = (v & ~m) | (0x20202020u & m);
-      }
-      if (a0 + 4 > aend) {
-        uint32_t const m = (1u << (8 * static_cast<uint32_t>(aend - a0))) - 1u;
-        v                = (v & m) | (0x20202020u & ~m);
-      }
-    }
-    return v;
-  }
-};
-
-__device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, int64_t n)
-{
-  const uint8_t* row = col.chars + o;
-  RowCtx c;
-  c.mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 3u);
-  c.arow = reinterpret_cast<const uint32_t*>(row - c.mis);
-  c.n    = n;
-  c.aend = static_cast<int64_t>(c.mis) + n;
-  return c;
-}
-
-
-// Persistent wavefronts, one row at a time, with the next row's offsets and the next chunk already in
-// flight.  For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an
-// out-of-vocabulary marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass
-// overwrites it with the word's token count); nwords[r] = words kept; counts[r] = one per hit.
-__global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                      uint32_t* __restrict__ arena, uint8_t* __restrict__ arena_cnt,
-                                                                      int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
-                                                                      OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
-                                                                      uint32_t* __restrict__ queue_size)
-{
-  __shared__ ProbeLds lds_all[kTokWaves];
-  int const lane      = lane_id();
-  int const wave      = threadIdx.x / kWave;
-  ProbeLds& lds       = lds_all[wave];
-  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
-  int64_t const rows  = col.size;
-  uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
-
-  int64_t r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
-  // software pipeline: offsets two rows ahead, first chunk one row ahead
-  int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
-  if (r < rows) {
-    o_cur = col.off(r);
-    e_cur = col.off(r + 1);
-  }
-  if (r + nwave < rows) {
-    o_nxt = col.off(r + nwave);
-    e_nxt = col.off(r + nwave + 1);
-  }
-  RowCtx ctx = make_row_ctx(col, o_cur, e_cur - o_cur);
-  // the chunk about to be processed: my four bytes and (lane 63) the byte that follows the chunk
-  uint32_t mine_cur = r < rows ? ctx.load_clean(4 * lane) : 0x20202020u;
-  uint32_t tail_cur = (r < rows && lane == kWave - 1) ? ctx.load_clean(kChunk) : 0x20202020u;
-
-  for (; r < rows; r += nwave) {
-    // issue the loads of the rows to come before touching this row's data
-    RowCtx const ctx_nxt = make_row_ctx(col, o_nxt, e_nxt - o_nxt);
-    bool const have_nxt  = r + nwave < rows;
-    int64_t o_nn = 0, e_nn = 0;
-    if (r + 2 * nwave < rows) {
-      o_nn = col.off(r + 2 * nwave);
-      e_nn = col.off(r + 2 * nwave + 1);
-    }
-
-    int64_t const n = ctx.n;
-    // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
-    // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
-    int64_t cap = std::numeric_limits<int64_t>::max();
-    if (max_words > 0) cap = col.valid(r) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
-    int64_t const slot0   = ((o_cur - first_offset) >> 1) + r;
-    uint32_t* const slots = arena + slot0;
-    uint8_t* const scnt   = arena_cnt + slot0;
-
-    int64_t words_done   = 0;
-    uint32_t hits        = 0;
-    uint32_t carry_hash  = 0;     // hash of the word running into the chunk (0 after a space)
-    uint32_t carry_start = 0;     // 1-based aligned coordinate of the start of that word
-    uint32_t prev_last   = 0x20;  // byte before the chunk
-    bool next_is_row = false;  // whether the prefetched chunk is the next row's first one
-    for (int64_t cbase = 0; cbase < ctx.aend && words_done < cap; cbase += kChunk) {
-      int64_t const a0    = cbase + 4 * lane;
-      uint32_t const mine = mine_cur;
-      uint32_t const tail = tail_cur;
-      // prefetch the chunk that follows: the rest of this row, else the start of the next row
-      bool const more = cbase + kChunk < ctx.aend;
-      next_is_row     = !more;
-      if (more || have_nxt) {
-        RowCtx const& pc    = more ? ctx : ctx_nxt;
-        int64_t const pbase = more ? cbase + kChunk : 0;
-        mine_cur            = pc.load_clean(pbase + 4 * lane);
-        tail_cur            = lane == kWave - 1 ? pc.load_clean(pbase + kChunk) : 0x20202020u;
-      }
-      uint32_t const ring0 = static_cast<uint32_t>(a0) & (kRing - 1);
-      lds.bytes[ring0 >> 2] = mine;
-      // neighbours: the byte before my four and the byte after them
-      uint32_t before = from_lane_below<0>(mine >> 24);
-      if (lane == 0) before = prev_last;
-      uint32_t after = static_cast<uint32_t>(__shfl_down(static_cast<int>(mine & 0xffu), 1));
-      if (lane == kWave - 1) after = tail & 0xffu;
-      prev_last = wave_bcast(mine >> 24, kWave - 1);
-
-      // hash block of my bytes, last word start among them, word ends
-      uint32_t bm[4], bv[4];
-      uint32_t m = 1, v = 0, smax = 0, ends = 0;
-      uint32_t prevb = before;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t const b    = (mine >> (8 * j)) & 0xffu;
-        uint32_t const next = j < 3 ? (mine >> (8 * (j + 1))) & 0xffu : after;
-        bool const sp       = b == 0x20u;
-        uint32_t const em   = sp ? 0u : kHashB;
-        uint32_t const ev   = sp ? 0u : b;
-        v                   = v * em + ev;
-        m                   = m * em;
-        bm[j]               = m;
-        bv[j]               = v;
-        if (!sp && prevb == 0x20u) smax = static_cast<uint32_t>(a0) + j + 1;
-        if (!sp && next == 0x20u) ends |= 1u << j;
-        prevb = b;
-      }
-      // state entering my bytes: lanes below (exclusive) seeded with the carry from the previous chunk
-      uint32_t im = m, iv = v;
-      wave_scan_hash(im, iv);
-      uint32_t const xm = from_lane_below<1>(im);
-      uint32_t const xv = carry_hash * xm + from_lane_below<0>(iv);
-      uint32_t const is = wave_scan_max(smax);
-      uint32_t xs       = max(from_lane_below<0>(is), carry_start);
-      carry_hash        = carry_hash * wave_bcast(im, kWave - 1) + wave_bcast(iv, kWave - 1);
-      carry_start       = max(carry_start, wave_bcast(is, kWave - 1));
-
-      uint32_t const ne    = __builtin_popcount(ends);
-      uint32_t const incl  = wave_inclusive_scan(ne);
-      uint32_t const total = wave_bcast(incl, kWave - 1);
-      uint32_t slot        = incl - ne;
-      prevb                = before;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t const b = (mine >> (8 * j)) & 0xffu;
-        if (b != 0x20u && prevb == 0x20u) xs = static_cast<uint32_t>(a0) + j + 1;
-        if (ends & (1u << j)) {
-          lds.wstart[slot] = xs;
-          lds.wend[slot]   = static_cast<uint32_t>(a0) + j + 1;
-          lds.whash[slot]  = xv * bm[j] + bv[j];
-          ++slot;
-        }
-        prevb = b;
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-      int64_t const allowed = min(static_cast<int64_t>(total), cap - words_done);
-      for (uint32_t w0 = 0; w0 < allowed; w0 += kWave) {
-        uint32_t const wi = w0 + lane;
-        bool const active = wi < allowed;
-        bool miss         = false;
-        uint32_t value    = 0, ws = 0;
-        if (active) {
-          ws                = lds.wstart[wi];
-          uint32_t const wl = lds.wend[wi] - ws + 1;
-          if (wl >= kMaxWord) {
-            value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
-          } else {
-            int32_t id = kNone;
-            if (wl <= table.max_len[0]) id = lookup(table, 0, lds.whash[wi], RingWord{lds.bytes, (ws - 1) & (kRing - 1)}, 0, wl);
-            miss  = id == kNone;
-            value = static_cast<uint32_t>(id);
-          }
-        }
-        uint64_t const mm = ballot64(miss);
-        if (mm) {
-          uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
-          if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
-            // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
-            for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-              if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(queue_size, queue_block);
-            q_pos = wave_bcast(base, 0);
-            q_lim = q_pos + queue_block;
-          }
-          if (miss) {
-            uint32_t const q = q_pos + lanes_below(mm);
-            if (q < queue_capacity) queue[q] = OovEntry{static_cast<int32_t>(r), ws - 1 - ctx.mis, static_cast<uint32_t>(words_done) + wi, 0u};
-            value = kOovMark | q;
-          }
-          q_pos += nm;
-        }
-        if (active) {
-          slots[words_done + wi] = value;
-          scnt[words_done + wi]  = 1;
-        }
-        hits += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && !miss)));
-      }
-      words_done += allowed;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    }
-    if (lane == 0) {
-      nwords[r] = static_cast<int32_t>(words_done);
-      counts[r] = static_cast<int32_t>(hits);
-    }
-    // rotate the pipeline.  The prefetched chunk is the next row's first one unless the row was left
-    // early (word limit reached, or an empty row whose loop never ran): then fetch it now.
-    if (!next_is_row && have_nxt) {
-      mine_cur = ctx_nxt.load_clean(4 * lane);
-      tail_cur = lane == kWave - 1 ? ctx_nxt.load_clean(kChunk) : 0x20202020u;
-    }
-    ctx   = ctx_nxt;
-    o_cur = o_nxt;
-    o_nxt    = o_nn;
-    e_nxt    = e_nn;
-  }
-  for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
-}
-
-// ------------------------------------------------------------------ out-of-vocabulary pass
 constexpr uint32_t kStage = 64;  // bytes of each queued word kept in LDS (from a 16-byte aligned base)
 
-// A queued word whose first kStage - mis bytes sit in this lane's LDS window; later bytes come from memory.
+// A queued word whose first kStage - mis bytes sit in its lane's LDS window; later bytes come from memory.
 struct StagedWord {
   const uint32_t* win;  // this lane's kStage-byte window
   const uint8_t* p;     // the word in global memory
@@ -509,32 +182,333 @@ struct StagedWord {
         if (k < 4) lo |= b << (8 * k); else hi |= b << (8 * (k - 4));
       }
     }
-    if (len < 4) lo &= (1u << (8 * len)) - 1u;
-    if (len <= 4) hi = 0;
-    else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+    trim_key8(len, lo, hi);
     *k0 = lo;
     *k1 = hi;
   }
 };
 
+// Token id of key bytes [p, p+len) of `w` in key space `kind`, or kNone.  1 <= len < 200.
+template <typename W>
+__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len)
+{
+  uint32_t k0, k1;
+  w.key8(p, len, &k0, &k1);
+  uint32_t h = key_hash_block(key_hash_init(len), k0, k1);
+  for (uint32_t done = 8; done < len; done += 8) {  // keys longer than one block (not kept inside the slot)
+    uint32_t b0, b1;
+    w.key8(p + done, len - done, &b0, &b1);
+    h = key_hash_block(h, b0, b1);
+  }
+  uint32_t b;
+  uint32_t const want = slot_word0(h, kind, len, &b);
+  for (;;) {
+    b &= t.bucket_mask;
+    uint4 const s0 = t.slots[2 * b];
+    uint4 const s1 = t.slots[2 * b + 1];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      uint4 const& s = j ? s1 : s0;
+      if (s.x == want) {
+        if (len <= 8) {
+          if (s.z == k0 && s.w == k1) return static_cast<int32_t>(s.y);
+        } else {
+          const uint8_t* e = t.pool + s.z;
+          uint32_t i       = 0;
+          while (i < len && e[i] == w.byte(p + i)) ++i;
+          if (i == len) return static_cast<int32_t>(s.y);
+        }
+      }
+      if (s.x == 0) return kNone;
+    }
+    ++b;
+  }
+}
+
+// ------------------------------------------------------------------ wavefront helpers of the probe pass
+template <int CTRL, int ROW_MASK, int OLD>
+__device__ __forceinline__ uint32_t dpp_old(uint32_t v)
+{
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(OLD, static_cast<int>(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+__device__ __forceinline__ uint32_t wave_scan_max(uint32_t v)
+{
+  v = max(v, dpp_zero<0x111, 0xf>(v));
+  v = max(v, dpp_zero<0x112, 0xf>(v));
+  v = max(v, dpp_zero<0x114, 0xf>(v));
+  v = max(v, dpp_zero<0x118, 0xf>(v));
+  v = max(v, dpp_zero<0x142, 0xa>(v));
+  v = max(v, dpp_zero<0x143, 0xc>(v));
+  return v;
+}
+
+// value of the lane below (lane 0 gets FIRST)
+template <int FIRST>
+__device__ __forceinline__ uint32_t from_lane_below(uint32_t v)
+{
+  return dpp_old<0x138, 0xf, FIRST>(v);  // wave_shr:1
+}
+
+// Bit 7 of every byte of x that equals ' ' (exact: no carries cross bytes).
+__device__ __forceinline__ uint32_t space_bytes(uint32_t x)
+{
+  uint32_t const t = x ^ 0x20202020u;
+  return ~(((t & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | t) & 0x80808080u;
+}
+// Gathers bits 7, 15, 23, 31 into bits 0..3.
+__device__ __forceinline__ uint32_t gather_byte_flags(uint32_t z) { return (((z >> 7) * 0x00204081u) >> 21) & 0xFu; }
+
+// Row r owns the word-arena slots [arena_pos(r), arena_pos(r+1)): at least floor(bytes/2) + 1, and a
+// row cannot hold more words than that.
+__device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
+
+struct ProbeLds {
+  uint32_t bytes[kRing / 4];       // row bytes (everything outside the row is ' ')
+  uint16_t wend[kChunk / 2 + 2];   // per word ending in the chunk: offset of its last byte inside the chunk
+  uint16_t wlen[kChunk / 2 + 2];   // and its length in bytes, clamped to kMaxWord
+};
+
+// Where a row sits relative to 16-byte aligned memory.  Coordinates count bytes from `base`.
+struct RowCtx {
+  const uint4* base;  // aligned address at or below the row's first byte
+  uint32_t mis;       // row start inside that block
+  int64_t aend;       // row end (mis + row bytes)
+  // 16 bytes at coordinate a0 (a multiple of 16) with every byte outside the row replaced by ' '
+  __device__ __forceinline__ uint4 load_clean(int64_t a0) const
+  {
+    uint4 v = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
+    if (a0 < aend && a0 + 16 > static_cast<int64_t>(mis)) {
+      v = base[a0 >> 4];
+      if (a0 < static_cast<int64_t>(mis) || a0 + 16 > aend) {
+        uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          int64_t const b0 = a0 + 4 * j;
+          uint32_t keep    = 0xFFFFFFFFu;
+          if (b0 < static_cast<int64_t>(mis)) keep = b0 + 4 <= static_cast<int64_t>(mis) ? 0u : keep << (8 * static_cast<uint32_t>(mis - b0));
+          if (b0 + 4 > aend) keep = b0 >= aend ? 0u : keep & ((1u << (8 * static_cast<uint32_t>(aend - b0))) - 1u);
+          d[j] = (d[j] & keep) | (0x20202020u & ~keep);
+        }
+        v = make_uint4(d[0], d[1], d[2], d[3]);
+      }
+    }
+    return v;
+  }
+  // the byte at coordinate a (any alignment); ' ' outside the row
+  __device__ __forceinline__ uint32_t byte_at(int64_t a) const
+  {
+    if (a < static_cast<int64_t>(mis) || a >= aend) return 0x20u;
+    return reinterpret_cast<const uint8_t*>(base)[a];
+  }
+};
+
+__device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, int64_t n)
+{
+  const uint8_t* row = col.chars + o;
+  RowCtx c;
+  c.mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u);
+  c.base = reinterpret_cast<const uint4*>(row - c.mis);
+  c.aend = static_cast<int64_t>(c.mis) + n;
+  return c;
+}
+
+// ------------------------------------------------------------------ probe pass
+// Persistent wavefronts, one row at a time, with the next row's offsets and the next chunk already in
+// flight.  For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an
+// out-of-vocabulary marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass
+// overwrites it with the word's token count); nwords[r] = words kept; counts[r] = one per hit.
+__global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
+                                                                      uint32_t* __restrict__ arena, uint8_t* __restrict__ arena_cnt,
+                                                                      int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
+                                                                      OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
+                                                                      uint32_t* __restrict__ queue_size)
+{
+  __shared__ ProbeLds lds_all[kTokWaves];
+  int const lane      = lane_id();
+  int const wave      = threadIdx.x / kWave;
+  ProbeLds& lds       = lds_all[wave];
+  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
+  int64_t const rows  = col.size;
+  uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
+
+  int64_t r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
+  // software pipeline: offsets two rows ahead, the next chunk one step ahead
+  int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
+  if (r < rows) {
+    o_cur = col.off(r);
+    e_cur = col.off(r + 1);
+  }
+  if (r + nwave < rows) {
+    o_nxt = col.off(r + nwave);
+    e_nxt = col.off(r + nwave + 1);
+  }
+  RowCtx ctx = make_row_ctx(col, o_cur, e_cur - o_cur);
+  // the chunk about to be processed: my sixteen bytes and (lane 63) the byte after the chunk
+  uint4 mine_cur    = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
+  uint32_t tail_cur = 0x20u;
+  if (r < rows) {
+    mine_cur = ctx.load_clean(16 * lane);
+    if (lane == kWave - 1) tail_cur = ctx.byte_at(kChunk);
+  }
+
+  for (; r < rows; r += nwave) {
+    RowCtx const ctx_nxt = make_row_ctx(col, o_nxt, e_nxt - o_nxt);
+    bool const have_nxt  = r + nwave < rows;
+    int64_t o_nn = 0, e_nn = 0;
+    if (r + 2 * nwave < rows) {
+      o_nn = col.off(r + 2 * nwave);
+      e_nn = col.off(r + 2 * nwave + 1);
+    }
+
+    int64_t const n = e_cur - o_cur;
+    // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
+    // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
+    int64_t cap = std::numeric_limits<int64_t>::max();
+    if (max_words > 0) cap = col.valid(r) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
+    int64_t const slot0   = ((o_cur - first_offset) >> 1) + r;
+    uint32_t* const slots = arena + slot0;
+    uint8_t* const scnt   = arena_cnt + slot0;
+
+    int64_t words_done   = 0;
+    uint32_t hits        = 0;
+    uint32_t carry_start = 0;     // 1-based coordinate of the start of the word running into the chunk
+    bool prev_space      = true;  // the byte before the chunk is a space (or the row starts here)
+    bool next_is_row     = false; // whether the prefetched chunk is the next row's first one
+    for (int64_t cbase = 0; cbase < ctx.aend && words_done < cap; cbase += kChunk) {
+      int64_t const a0      = cbase + 16 * lane;
+      uint4 const mine    = mine_cur;
+      uint32_t const tail = tail_cur;
+      // prefetch the chunk that follows: the rest of this row, else the start of the next row
+      bool const more = cbase + kChunk < ctx.aend;
+      next_is_row     = !more;
+      if (more || have_nxt) {
+        RowCtx const& pc    = more ? ctx : ctx_nxt;
+        int64_t const pbase = more ? cbase + kChunk : 0;
+        mine_cur            = pc.load_clean(pbase + 16 * lane);
+        if (lane == kWave - 1) tail_cur = pc.byte_at(pbase + kChunk);
+      }
+      uint32_t const ring0 = static_cast<uint32_t>(a0) & (kRing - 1);
+      *reinterpret_cast<uint4*>(&lds.bytes[ring0 >> 2]) = mine;
+
+      // bit i of sp: my byte i is a space
+      uint32_t const sp = gather_byte_flags(space_bytes(mine.x)) | (gather_byte_flags(space_bytes(mine.y)) << 4) |
+                          (gather_byte_flags(space_bytes(mine.z)) << 8) | (gather_byte_flags(space_bytes(mine.w)) << 12);
+      // neighbours: is the byte before my sixteen a space, and the byte after them
+      uint32_t before = from_lane_below<1>(sp >> 15);
+      if (lane == 0) before = prev_space ? 1u : 0u;
+      uint32_t after = static_cast<uint32_t>(__shfl_down(static_cast<int>(sp & 1u), 1));
+      if (lane == kWave - 1) after = tail == 0x20u ? 1u : 0u;
+      prev_space = wave_bcast(sp >> 15, kWave - 1) != 0;
+
+      uint32_t const word   = ~sp & 0xFFFFu;
+      uint32_t const starts = word & ((sp << 1) | before);            // a word byte after a space
+      uint32_t const ends   = word & ((sp >> 1) | (after << 15));     // a word byte before a space
+      // start of the word that runs into my bytes: the last start in the lanes below, else the carry
+      uint32_t const my_last = starts ? static_cast<uint32_t>(a0) + (32u - __builtin_clz(starts)) : 0u;
+      uint32_t const is      = wave_scan_max(my_last);
+      uint32_t const xs      = max(from_lane_below<0>(is), carry_start);
+      carry_start            = max(carry_start, wave_bcast(is, kWave - 1));
+
+      uint32_t const ne    = __builtin_popcount(ends);
+      uint32_t const incl  = wave_inclusive_scan(ne);
+      uint32_t const total = wave_bcast(incl, kWave - 1);
+      uint32_t slot        = incl - ne;
+      for (uint32_t em = ends; em; em &= em - 1) {
+        uint32_t const p  = __builtin_ctz(em);
+        uint32_t const sb = starts & ((2u << p) - 1u);
+        uint32_t const st = sb ? static_cast<uint32_t>(a0) + (32u - __builtin_clz(sb)) : xs;  // 1-based
+        uint32_t const wl = static_cast<uint32_t>(a0) + p + 1u - st + 1u;
+        lds.wend[slot]    = static_cast<uint16_t>(16u * lane + p);
+        lds.wlen[slot]    = static_cast<uint16_t>(min(wl, kMaxWord));
+        ++slot;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      int64_t const allowed = min(static_cast<int64_t>(total), cap - words_done);
+      for (uint32_t w0 = 0; w0 < allowed; w0 += kWave) {
+        uint32_t const wi = w0 + lane;
+        bool const active = wi < allowed;
+        bool miss         = false;
+        uint32_t value    = 0;
+        int64_t wstart    = 0;  // coordinate of the word's first byte
+        if (active) {
+          uint32_t const wl = lds.wlen[wi];
+          wstart            = cbase + lds.wend[wi] + 1 - static_cast<int64_t>(wl);
+          if (wl >= kMaxWord) {
+            value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+          } else {
+            int32_t id = kNone;
+            if (wl <= table.max_len[0]) id = lookup(table, 0, RingWord{lds.bytes, static_cast<uint32_t>(wstart) & (kRing - 1)}, 0, wl);
+            miss  = id == kNone;
+            value = static_cast<uint32_t>(id);
+          }
+        }
+        uint64_t const mm = ballot64(miss);
+        if (mm) {
+          uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
+          if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
+            // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
+            for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+              if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(queue_size, queue_block);
+            q_pos = wave_bcast(base, 0);
+            q_lim = q_pos + queue_block;
+          }
+          if (miss) {
+            uint32_t const q = q_pos + lanes_below(mm);
+            if (q < queue_capacity)
+              queue[q] = OovEntry{static_cast<int32_t>(r), static_cast<uint32_t>(wstart - ctx.mis), static_cast<uint32_t>(words_done) + wi, 0u};
+            value = kOovMark | q;
+          }
+          q_pos += nm;
+        }
+        if (active) {
+          slots[words_done + wi] = value;
+          scnt[words_done + wi]  = 1;
+        }
+        hits += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && !miss)));
+      }
+      words_done += allowed;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0) {
+      nwords[r] = static_cast<int32_t>(words_done);
+      counts[r] = static_cast<int32_t>(hits);
+    }
+    // rotate the pipeline.  The prefetched chunk is the next row's first one unless the row was left
+    // early (word limit reached, or a row whose loop never ran): then fetch it now.
+    if (!next_is_row && have_nxt) {
+      mine_cur = ctx_nxt.load_clean(16 * lane);
+      if (lane == kWave - 1) tail_cur = ctx_nxt.byte_at(kChunk);
+    }
+    ctx   = ctx_nxt;
+    o_cur = o_nxt;
+    e_cur = e_nxt;
+    o_nxt = o_nn;
+    e_nxt = e_nn;
+  }
+  for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+}
+
+// ------------------------------------------------------------------ out-of-vocabulary pass
 // Greedy longest-match-first tokenization (cpp/src/text/wordpiece_tokenize.cu:349-407) of a word of
 // `len` bytes, 1 <= len < 200, whose whole-word lookup has already failed.  `emit(j, id)` receives token j;
 // returns the token count (a collapse to one unknown token re-emits token 0).
 //
 // One flat loop with one table probe per trip, so that the lanes of a wavefront, each at a different
-// stage of its own word, share trips instead of serialising nested loops.  The state is the piece
-// being searched: bytes [start, e) with `he` = hash of [0, e), `hs` = hash of [0, start) and
-// pwe = B^(e - start); its hash is he - hs * pwe.  The first piece (start 0) lives in the full key
-// space, later ones in the "##" space.
+// stage of its own word, share trips instead of serialising nested loops.  The state is the piece being
+// searched, bytes [start, e): the first piece (start 0) lives in the full key space, later ones in the
+// "##" space.
 template <typename W, typename Emit>
 __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
 {
-  uint32_t hfull = 0, pwr = 1;  // pwr = B^(len - start)
-  for (uint32_t i = 0; i < len; ++i) {
-    hfull = hfull * kHashB + w.byte(i);
-    pwr *= kHashB;
-  }
-  uint32_t start = 0, hs = 0, e = len, he = hfull, pwe = pwr, count = 0;
+  uint32_t start = 0, e = len, count = 0;
   bool fresh = false;  // the whole word is known to be absent: begin by shortening it
   for (;;) {
     if (!fresh) {
@@ -547,46 +521,37 @@ __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W con
         emit(0u, t.unk_id);
         return 1;
       }
-      for (uint32_t i = e; i > x; --i) {
-        he = (he - w.byte(i - 1)) * kHashBInv;
-        pwe *= kHashBInv;
-      }
       e = x;
     }
-    fresh                = false;
+    fresh               = false;
     uint32_t const kind = count ? 1u : 0u;
     uint32_t const pl   = e - start;
-    if (pl > t.max_len[kind]) continue;
-    int32_t const id = lookup(t, kind, he - hs * pwe, w, start, pl);
+    if (pl > t.max_len[kind]) continue;  // no key this long exists: keep shortening
+    int32_t const id = lookup(t, kind, w, start, pl);
     if (id == kNone) continue;
     emit(count++, id);
     if (e == len) return count;
     // next piece: the rest of the word (381-395)
-    for (uint32_t i = start; i < e; ++i) pwr *= kHashBInv;
     start = e;
-    hs    = he;
     e     = len;
-    he    = hfull;
-    pwe   = pwr;
     fresh = true;
   }
 }
 
-// Brings the first bytes of the word at p (row bytes end at row_end) into this lane's LDS window with
-// 16-byte aligned loads that stay inside [p & ~15, row_end rounded up to 16), and returns its length.
+// Brings the first bytes of the word at p (its row has `avail` bytes from p on) into this lane's LDS
+// window with 16-byte aligned loads that never start past the row's last byte, and returns its length.
 __device__ __forceinline__ uint32_t stage_word(const uint8_t* p, int64_t avail, uint32_t* win, uint32_t* mis_out)
 {
-  uint32_t const mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
-  const uint4* a     = reinterpret_cast<const uint4*>(p - mis);
-  // 16-byte blocks that hold row bytes (never a block wholly past the row)
+  uint32_t const mis    = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
+  const uint4* a        = reinterpret_cast<const uint4*>(p - mis);
   uint32_t const blocks = static_cast<uint32_t>(min(static_cast<int64_t>(kStage / 16), (static_cast<int64_t>(mis) + avail + 15) >> 4));
   uint4* w4             = reinterpret_cast<uint4*>(win);
   for (uint32_t i = 0; i < blocks; ++i) w4[i] = a[i];
   *mis_out = mis;
   // the word ends at the first space or at the end of the row
-  uint32_t const lim = static_cast<uint32_t>(min(avail, static_cast<int64_t>(kMaxWord)));
-  uint32_t len       = 0;
-  const uint8_t* wb  = reinterpret_cast<const uint8_t*>(win) + mis;
+  uint32_t const lim       = static_cast<uint32_t>(min(avail, static_cast<int64_t>(kMaxWord)));
+  uint32_t len             = 0;
+  const uint8_t* wb        = reinterpret_cast<const uint8_t*>(win) + mis;
   uint32_t const in_window = min(lim, kStage - mis);
   while (len < in_window && wb[len] != 0x20u) ++len;
   if (len == in_window)
@@ -725,19 +690,23 @@ struct HostSlot {
   uint32_t x, y, z, w;
 };
 
-uint32_t host_hash(const uint8_t* key, uint32_t len)
-{
-  uint32_t h = 0;
-  for (uint32_t i = 0; i < len; ++i) h = h * kHashB + key[i];
-  return h;
-}
-
 void host_key8(const uint8_t* key, uint32_t len, uint32_t* k0, uint32_t* k1)
 {
   uint8_t buf[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   std::memcpy(buf, key, len < 8 ? len : 8);
   std::memcpy(k0, buf, 4);
   std::memcpy(k1, buf + 4, 4);
+}
+
+uint32_t host_hash(const uint8_t* key, uint32_t len)
+{
+  uint32_t h = key_hash_init(len);
+  for (uint32_t done = 0; done < len; done += 8) {
+    uint32_t lo, hi;
+    host_key8(key + done, len - done, &lo, &hi);
+    h = key_hash_block(h, lo, hi);
+  }
+  return h;
 }
 
 bool host_same(HostSlot const& s, uint32_t w0, const std::vector<uint8_t>& pool, const uint8_t* key, uint32_t len, uint32_t k0, uint32_t k1)
