@@ -323,3 +323,14 @@ def test_wordpiece_row_longer_than_chunks(nv, orc):
     for mw in (0, 3000):
         got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
         assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4), f"long row mw={mw}")
+
+
+def test_cpp_api_program():
+    """The C++ mirror of the nvtext API (cudf_amd/include) run on the reference's gtest cases."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "nvtext_api_test")
+    assert os.path.exists(exe), "build it with __graft_entry__.build() or make -C tests/cpp"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "ALL PASSED" in p.stdout
