@@ -40,9 +40,8 @@ struct HashTraits<uint32_t> {
   {
     return murmur3_x86_32(src, len, seed);
   }
-  // minhash.cu:350-351 in uint32 arithmetic: the product and sum wrap mod 2^32, after
-  // which "% (2^61-1)" and "& max" change nothing.
-  static __device__ __forceinline__ uint32_t permute(uint32_t hv, uint32_t a, uint32_t b) { return hv * a + b; }
+  // Permutation (minhash.cu:350-351) in uint32 arithmetic: the product and sum wrap mod 2^32, after
+  // which "% (2^61-1)" and "& max" change nothing: (hv * a + b), see Fold<uint32_t>.
 };
 template <>
 struct HashTraits<uint64_t> {
@@ -51,15 +50,7 @@ struct HashTraits<uint64_t> {
   {
     return murmur3_x64_128_lo(src, len, seed);  // minhash.cu:138: first word of the 128-bit hash
   }
-  // ((hv*a + b) mod 2^64) % (2^61-1): x = q*2^61 + r with q <= 7, so r + q <= p + 7 and one
-  // conditional subtraction finishes the reduction.
-  static __device__ __forceinline__ uint64_t permute(uint64_t hv, uint64_t a, uint64_t b)
-  {
-    constexpr uint64_t p = (1ull << 61) - 1;
-    uint64_t const x     = hv * a + b;
-    uint64_t const y     = (x & p) + (x >> 61);
-    return y >= p ? y - p : y;
-  }
+  // Permutation (minhash.cu:350-351): ((hv*a + b) mod 2^64) % (2^61-1), see Fold<uint64_t>.
 };
 
 template <typename T>
@@ -120,11 +111,95 @@ __device__ __forceinline__ bool window_at(Src const& src, int64_t remaining, uin
   return first || left <= 0;
 }
 
+// (h * a + b) mod 2^64 in three full-rate multiply-adds and one add: lo64 = h.lo*a.lo + b; the two cross
+// products are summed separately (their high halves fall off the end) and added to the high dword.
+__device__ __forceinline__ uint64_t mul_add_u64(uint64_t h, uint64_t a, uint64_t b)
+{
+  uint32_t const hl = static_cast<uint32_t>(h), hh = static_cast<uint32_t>(h >> 32);
+  uint32_t const al = static_cast<uint32_t>(a), ah = static_cast<uint32_t>(a >> 32);
+  uint64_t x, t;
+  asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(x) : "v"(hl), "v"(al), "v"(b) : "vcc");
+  asm("v_mad_u64_u32 %0, vcc, %1, %2, 0" : "=v"(t) : "v"(hl), "v"(ah) : "vcc");
+  asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(t) : "v"(hh), "v"(al), "v"(t) : "vcc");
+  uint32_t const hi = static_cast<uint32_t>(x >> 32) + static_cast<uint32_t>(t);
+  return (static_cast<uint64_t>(hi) << 32) | static_cast<uint32_t>(x);
+}
+
+// min of two values below 2^62 in one instruction: such bit patterns are non-negative finite doubles
+// (or denormals, which this code object keeps: float_denorm_mode_16_64 = 3), and those order like the
+// integers.  An operand that is all ones (the "no hash yet" start value, a NaN pattern) loses to the other.
+__device__ __forceinline__ uint64_t min_below_2_62(uint64_t m, uint64_t y)
+{
+  uint64_t r;
+  asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(m), "v"(y));
+  return r;
+}
+
 // Folds `count` compacted hashes (padded here to a multiple of 4) into m[K]; lanes <-> parameters.
+template <typename T, int K>
+struct Fold;
+
+template <int K>
+struct Fold<uint32_t, K> {
+  static __device__ __forceinline__ void run(const uint32_t* hashes, uint32_t padded, const uint32_t (&a)[K], const uint32_t (&b)[K],
+                                             uint32_t (&m)[K])
+  {
+    for (uint32_t i = 0; i < padded; i += 4) {
+      uint32_t const h0 = hashes[i], h1 = hashes[i + 1], h2 = hashes[i + 2], h3 = hashes[i + 3];
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        // one v_mad_u64_u32 per product, one v_min3_u32 per two products
+        uint32_t const r0 = h0 * a[k] + b[k];
+        uint32_t const r1 = h1 * a[k] + b[k];
+        uint32_t const r2 = h2 * a[k] + b[k];
+        uint32_t const r3 = h3 * a[k] + b[k];
+        m[k]              = min(min(m[k], r0), r1);
+        m[k]              = min(min(m[k], r2), r3);
+      }
+    }
+  }
+};
+
+template <int K>
+struct Fold<uint64_t, K> {
+  static constexpr uint64_t p = (1ull << 61) - 1;
+  // x mod p for x < 2^64: x = q*2^61 + r with q <= 7, so y = r + q <= p + 7.
+  static __device__ __forceinline__ uint64_t fold_once(uint64_t x) { return (x & p) + (x >> 61); }
+
+  static __device__ __forceinline__ void run(const uint64_t* hashes, uint32_t padded, const uint64_t (&a)[K], const uint64_t (&b)[K],
+                                             uint64_t (&m)[K])
+  {
+    // Fast pass: the final "subtract p if y >= p" is left out.  y >= p needs the top dword of y to be
+    // at least 0x1FFFFFFF (one chance in 2^29 per product), which is tracked with a running maximum;
+    // if it ever happens the tile is folded again exactly.  Unreduced values are >= p, above every
+    // reduced value, so they can never displace a correct minimum.
+    uint32_t top = 0;
+    for (uint32_t i = 0; i < padded; i += 2) {
+      uint64_t const h0 = hashes[i], h1 = hashes[i + 1];
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        uint64_t const y0 = fold_once(mul_add_u64(h0, a[k], b[k]));
+        uint64_t const y1 = fold_once(mul_add_u64(h1, a[k], b[k]));
+        top               = max(max(top, static_cast<uint32_t>(y0 >> 32)), static_cast<uint32_t>(y1 >> 32));
+        m[k]              = min_below_2_62(min_below_2_62(m[k], y0), y1);
+      }
+    }
+    if (ballot64(top >= 0x1FFFFFFFu) != 0) {
+      for (uint32_t i = 0; i < padded; ++i) {
+        uint64_t const h = hashes[i];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          uint64_t const y = fold_once(h * a[k] + b[k]);
+          m[k]             = min(m[k], y >= p ? y - p : y);
+        }
+      }
+    }
+  }
+};
+
 template <typename T, int K>
 __device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane)
 {
-  using H = HashTraits<T>;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -135,17 +210,7 @@ __device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, con
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  for (uint32_t i = 0; i < padded; i += 4) {
-    T const h0 = lds.hashes[i], h1 = lds.hashes[i + 1], h2 = lds.hashes[i + 2], h3 = lds.hashes[i + 3];
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-      T const r0 = H::permute(h0, a[k], b[k]);
-      T const r1 = H::permute(h1, a[k], b[k]);
-      T const r2 = H::permute(h2, a[k], b[k]);
-      T const r3 = H::permute(h3, a[k], b[k]);
-      m[k]       = min(min(min(m[k], r0), min(r1, r2)), r3);
-    }
-  }
+  Fold<T, K>::run(lds.hashes, padded, a, b, m);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
 }

@@ -23,6 +23,7 @@
 #include "common.cuh"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -98,7 +99,7 @@ struct OovEntry {
   int32_t row;     // -1: unused entry
   uint32_t delta;  // byte offset of the word inside its row
   uint32_t widx;   // index of the word inside its row (its word-arena slot)
-  uint32_t pad;
+  uint32_t len;    // bytes in the word (1..199)
 };
 struct OovResult {
   int32_t tok[kOovKeep];
@@ -153,17 +154,21 @@ struct GlobalWord {
   }
 };
 
-constexpr uint32_t kStage = 64;  // bytes of each queued word kept in LDS (from a 16-byte aligned base)
+constexpr uint32_t kStage      = 64;   // bytes of each queued word kept in LDS (from a 16-byte aligned base)
+constexpr uint32_t kOovThreads = 256;
 
-// A queued word whose first kStage - mis bytes sit in its lane's LDS window; later bytes come from memory.
+// A queued word whose first kStage - mis bytes sit in LDS; later bytes come from memory.  The windows of
+// the workgroup are interleaved dword by dword (dword j of thread t at [j][t]), so that the lanes of a
+// wavefront reading "their" dword j hit 64 different banks instead of one.
 struct StagedWord {
-  const uint32_t* win;  // this lane's kStage-byte window
+  const uint32_t* win;  // dword 0 of this lane's window; dword j is win[j * kOovThreads]
   const uint8_t* p;     // the word in global memory
   uint32_t mis;         // offset of the word inside the window
+  __device__ __forceinline__ uint32_t dword(uint32_t j) const { return win[j * kOovThreads]; }
   __device__ __forceinline__ uint32_t byte(uint32_t k) const
   {
     uint32_t const o = mis + k;
-    return o < kStage ? reinterpret_cast<const uint8_t*>(win)[o] : p[k];
+    return o < kStage ? (dword(o >> 2) >> (8 * (o & 3u))) & 0xffu : p[k];
   }
   __device__ __forceinline__ void key8(uint32_t off, uint32_t len, uint32_t* k0, uint32_t* k1) const
   {
@@ -172,7 +177,7 @@ struct StagedWord {
     if (o + 12 <= kStage) {
       uint32_t const i  = o >> 2;
       uint32_t const sh = (o & 3u) * 8u;
-      uint32_t const d0 = win[i], d1 = win[i + 1], d2 = win[i + 2];
+      uint32_t const d0 = dword(i), d1 = dword(i + 1), d2 = dword(i + 2);
       lo                = __builtin_amdgcn_alignbit(d1, d0, sh);
       hi                = __builtin_amdgcn_alignbit(d2, d1, sh);
     } else {
@@ -189,11 +194,12 @@ struct StagedWord {
 };
 
 // Token id of key bytes [p, p+len) of `w` in key space `kind`, or kNone.  1 <= len < 200.
+// (raw0, raw1) = bytes [p, p+8) of `w`; whatever lies past the key is trimmed here.
 template <typename W>
-__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len)
+__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len, uint32_t raw0, uint32_t raw1)
 {
-  uint32_t k0, k1;
-  w.key8(p, len, &k0, &k1);
+  uint32_t k0 = raw0, k1 = raw1;
+  trim_key8(len, k0, k1);
   uint32_t h = key_hash_block(key_hash_init(len), k0, k1);
   for (uint32_t done = 8; done < len; done += 8) {  // keys longer than one block (not kept inside the slot)
     uint32_t b0, b1;
@@ -434,14 +440,20 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         bool miss         = false;
         uint32_t value    = 0;
         int64_t wstart    = 0;  // coordinate of the word's first byte
+        uint32_t wl = 0;
         if (active) {
-          uint32_t const wl = lds.wlen[wi];
-          wstart            = cbase + lds.wend[wi] + 1 - static_cast<int64_t>(wl);
+          wl     = lds.wlen[wi];
+          wstart = cbase + lds.wend[wi] + 1 - static_cast<int64_t>(wl);
           if (wl >= kMaxWord) {
             value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
           } else {
             int32_t id = kNone;
-            if (wl <= table.max_len[0]) id = lookup(table, 0, RingWord{lds.bytes, static_cast<uint32_t>(wstart) & (kRing - 1)}, 0, wl);
+            if (wl <= table.max_len[0]) {
+              RingWord const rw{lds.bytes, static_cast<uint32_t>(wstart) & (kRing - 1)};
+              uint32_t r0, r1;
+              rw.key8(0, 8, &r0, &r1);
+              id = lookup(table, 0, rw, 0, wl, r0, r1);
+            }
             miss  = id == kNone;
             value = static_cast<uint32_t>(id);
           }
@@ -461,7 +473,7 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
           if (miss) {
             uint32_t const q = q_pos + lanes_below(mm);
             if (q < queue_capacity)
-              queue[q] = OovEntry{static_cast<int32_t>(r), static_cast<uint32_t>(wstart - ctx.mis), static_cast<uint32_t>(words_done) + wi, 0u};
+              queue[q] = OovEntry{static_cast<int32_t>(r), static_cast<uint32_t>(wstart - ctx.mis), static_cast<uint32_t>(words_done) + wi, wl};
             value = kOovMark | q;
           }
           q_pos += nm;
@@ -510,6 +522,8 @@ __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W con
 {
   uint32_t start = 0, e = len, count = 0;
   bool fresh = false;  // the whole word is known to be absent: begin by shortening it
+  uint32_t raw0, raw1;  // bytes [start, start+8) of the word
+  w.key8(0, min(len, 8u), &raw0, &raw1);
   for (;;) {
     if (!fresh) {
       // wordpiece_tokenize.cu:307-317: drop the last UTF-8 character of the candidate
@@ -527,7 +541,7 @@ __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W con
     uint32_t const kind = count ? 1u : 0u;
     uint32_t const pl   = e - start;
     if (pl > t.max_len[kind]) continue;  // no key this long exists: keep shortening
-    int32_t const id = lookup(t, kind, w, start, pl);
+    int32_t const id = lookup(t, kind, w, start, pl, raw0, raw1);
     if (id == kNone) continue;
     emit(count++, id);
     if (e == len) return count;
@@ -535,52 +549,50 @@ __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W con
     start = e;
     e     = len;
     fresh = true;
+    w.key8(start, min(len - start, 8u), &raw0, &raw1);
   }
 }
 
-// Brings the first bytes of the word at p (its row has `avail` bytes from p on) into this lane's LDS
-// window with 16-byte aligned loads that never start past the row's last byte, and returns its length.
-__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, int64_t avail, uint32_t* win, uint32_t* mis_out)
+// Brings the first bytes of the `len`-byte word at p into this lane's LDS window with 16-byte aligned
+// loads (only blocks that overlap the word).
+__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, uint32_t* win)
 {
   uint32_t const mis    = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
   const uint4* a        = reinterpret_cast<const uint4*>(p - mis);
-  uint32_t const blocks = static_cast<uint32_t>(min(static_cast<int64_t>(kStage / 16), (static_cast<int64_t>(mis) + avail + 15) >> 4));
-  uint4* w4             = reinterpret_cast<uint4*>(win);
-  for (uint32_t i = 0; i < blocks; ++i) w4[i] = a[i];
-  *mis_out = mis;
-  // the word ends at the first space or at the end of the row
-  uint32_t const lim       = static_cast<uint32_t>(min(avail, static_cast<int64_t>(kMaxWord)));
-  uint32_t len             = 0;
-  const uint8_t* wb        = reinterpret_cast<const uint8_t*>(win) + mis;
-  uint32_t const in_window = min(lim, kStage - mis);
-  while (len < in_window && wb[len] != 0x20u) ++len;
-  if (len == in_window)
-    while (len < lim && p[len] != 0x20u) ++len;
-  return len;
+  uint32_t const blocks = min(kStage / 16, (mis + len + 15u) >> 4);
+  for (uint32_t i = 0; i < blocks; ++i) {
+    uint4 const v = a[i];
+    win[(4 * i + 0) * kOovThreads] = v.x;
+    win[(4 * i + 1) * kOovThreads] = v.y;
+    win[(4 * i + 2) * kOovThreads] = v.z;
+    win[(4 * i + 3) * kOovThreads] = v.w;
+  }
+  return mis;
 }
 
 // One lane per queued word.  results[q] = its first kOovKeep tokens; arena_cnt[slot] = its token count;
 // counts[row] += count.
-__global__ void __launch_bounds__(256) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
+__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
                                                             const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
                                                             int64_t first_offset, OovResult* __restrict__ results,
-                                                            uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts)
+                                                            uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts, uint32_t dbg)
 {
-  __shared__ __align__(16) uint32_t windows[256][kStage / 4];
+  __shared__ uint32_t windows[kStage / 4][kOovThreads];
   uint32_t const total  = min(*queue_size, queue_capacity);
   uint32_t const stride = gridDim.x * blockDim.x;
-  uint32_t* const win   = windows[threadIdx.x];
+  uint32_t* const win   = &windows[0][threadIdx.x];
   for (uint32_t q = blockIdx.x * blockDim.x + threadIdx.x; q < total; q += stride) {
     OovEntry const e = queue[q];
     if (e.row < 0) continue;  // unused tail of a reserved range
-    int64_t const o  = col.off(e.row);
-    int64_t const n  = col.off(e.row + 1) - o;
-    const uint8_t* p = col.chars + o + e.delta;
-    uint32_t mis;
-    uint32_t const len = stage_word(p, n - static_cast<int64_t>(e.delta), win, &mis);
+    int64_t const o    = col.off(e.row);
+    const uint8_t* p   = col.chars + o + e.delta;
+    uint32_t const len = e.len;
+    uint32_t const mis = stage_word(p, len, win);
     StagedWord const w{win, p, mis};
     int32_t tok[kOovKeep];
-    uint32_t const cnt = tokenize_oov_word(table, w, len, [&](uint32_t j, int32_t id) {
+    uint32_t cnt = 1;
+    if (dbg & 1u) { tok[0] = static_cast<int32_t>(w.byte(0)); }
+    else cnt = tokenize_oov_word(table, w, len, [&](uint32_t j, int32_t id) {
 #pragma unroll
       for (int k = 0; k < kOovKeep; ++k)
         if (j == static_cast<uint32_t>(k)) tok[k] = id;
@@ -590,68 +602,79 @@ __global__ void __launch_bounds__(256) wordpiece_oov_kernel(ColView col, VocabTa
     for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
     results[q] = res;
     arena_cnt[((o - first_offset) >> 1) + e.row + e.widx] = static_cast<uint8_t>(cnt);  // cnt <= len < 200
-    atomicAdd(&counts[e.row], static_cast<int32_t>(cnt));
+    if (!(dbg & 2u)) atomicAdd(&counts[e.row], static_cast<int32_t>(cnt));
   }
 }
 
 // ------------------------------------------------------------------ emit pass
-// Persistent wavefronts, one row at a time: expands the row's word arena into out + offsets[r].
-// Row descriptors are loaded two rows ahead and the first 64 word slots one row ahead.
+// Expands the word arena into the child column.  A wavefront takes 64 consecutive rows at a time
+// (lanes <-> rows for the descriptors), then walks ALL their words flat, lanes <-> words: because the
+// list offsets are a prefix sum in row order, the tokens of consecutive words are consecutive in the
+// child even across row boundaries, so only the block's first offset is needed.  Each word finds its
+// row by binary search in the block's word-count prefix (LDS).
+struct EmitLds {
+  uint32_t word_prefix[kWave + 1];  // words before row k of the block
+  int64_t slot0[kWave];             // arena slot of word 0 of row k
+};
+
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
                                                                      const uint32_t* __restrict__ arena, const uint8_t* __restrict__ arena_cnt,
                                                                      const int32_t* __restrict__ nwords, const OovEntry* __restrict__ queue,
                                                                      const OovResult* __restrict__ results, const int32_t* __restrict__ offsets,
                                                                      int32_t* __restrict__ out)
 {
-  int const lane      = lane_id();
-  int const wave      = threadIdx.x / kWave;
-  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
-  int64_t const rows  = col.size;
-  int64_t r           = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
+  __shared__ EmitLds lds_all[kTokWaves];
+  int const lane        = lane_id();
+  int const wave        = threadIdx.x / kWave;
+  EmitLds& lds          = lds_all[wave];
+  int64_t const rows    = col.size;
+  int64_t const nblocks = (rows + kWave - 1) / kWave;
+  int64_t const nwave   = static_cast<int64_t>(gridDim.x) * kTokWaves;
+  for (int64_t blk = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave; blk < nblocks; blk += nwave) {
+    int64_t const r  = blk * kWave + lane;
+    uint32_t W       = 0;
+    int64_t slot0    = 0;
+    if (r < rows) {
+      W     = static_cast<uint32_t>(nwords[r]);
+      slot0 = arena_pos(col, first_offset, r);
+    }
+    int32_t const base   = offsets[blk * kWave];
+    uint32_t const incl  = wave_inclusive_scan(W);
+    uint32_t const total = wave_bcast(incl, kWave - 1);
+    lds.word_prefix[lane] = incl - W;
+    if (lane == kWave - 1) lds.word_prefix[kWave] = total;
+    lds.slot0[lane] = slot0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-  struct Desc {
-    int32_t W;
-    int32_t begin;
-    int64_t slot0;
-  };
-  auto load_desc = [&](int64_t row) -> Desc {
-    Desc d{0, 0, 0};
-    if (row < rows) {
-      d.W     = nwords[row];
-      d.begin = offsets[row];
-      d.slot0 = arena_pos(col, first_offset, row);
-    }
-    return d;
-  };
-  Desc cur = load_desc(r);
-  Desc nxt = load_desc(r + nwave);
-  uint32_t v_cur = 0, c_cur = 0;
-  if (lane < cur.W) {
-    v_cur = arena[cur.slot0 + lane];
-    c_cur = arena_cnt[cur.slot0 + lane];
-  }
-  for (; r < rows; r += nwave) {
-    Desc const nn = load_desc(r + 2 * nwave);
-    uint32_t v_nxt = 0, c_nxt = 0;
-    if (lane < nxt.W) {
-      v_nxt = arena[nxt.slot0 + lane];
-      c_nxt = arena_cnt[nxt.slot0 + lane];
-    }
-    int32_t* const dst = out + cur.begin;
-    uint32_t done      = 0;
-    for (int32_t w0 = 0; w0 < cur.W; w0 += kWave) {
-      int32_t const wi  = w0 + lane;
-      bool const active = wi < cur.W;
-      uint32_t value = v_cur, cnt = c_cur;
-      if (w0 > 0) {
-        value = active ? arena[cur.slot0 + wi] : 0u;
-        cnt   = active ? arena_cnt[cur.slot0 + wi] : 0u;
+    // the arena entry of flat word j: row k = last row with word_prefix[k] <= j (rows without words are skipped
+    // because their prefix equals the next row's)
+    auto locate = [&](uint32_t j, uint32_t& value, uint32_t& cnt) {
+      value = 0;
+      cnt   = 0;
+      if (j < total) {
+        uint32_t lo = 0;
+#pragma unroll
+        for (uint32_t step = kWave / 2; step > 0; step >>= 1)
+          if (lds.word_prefix[lo + step] <= j) lo += step;
+        int64_t const slot = lds.slot0[lo] + (j - lds.word_prefix[lo]);
+        value              = arena[slot];
+        cnt                = arena_cnt[slot];
       }
-      if (!active) cnt = 0;
+    };
+
+    uint32_t done = 0;  // tokens written so far in this block
+    uint32_t v_nxt, c_nxt;
+    locate(lane, v_nxt, c_nxt);
+    for (uint32_t j0 = 0; j0 < total; j0 += kWave) {
+      uint32_t const value = v_nxt, cnt = c_nxt;
+      locate(j0 + kWave + lane, v_nxt, c_nxt);  // next round's loads are in flight while this one is written
+      bool const active   = j0 + lane < total;
       bool const oov      = active && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
-      uint32_t const incl = wave_inclusive_scan(cnt);
+      uint32_t const incl2 = wave_inclusive_scan(cnt);
       if (active) {
-        int32_t* d = dst + done + (incl - cnt);
+        int32_t* d = out + base + done + (incl2 - cnt);
         if (!oov) {
           d[0] = static_cast<int32_t>(value);
         } else {
@@ -661,22 +684,15 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
           } else {
             // more pieces than a queue entry keeps: tokenize the word again, straight into place
             OovEntry const e = queue[q];
-            int64_t const o  = col.off(e.row);
-            int64_t const n  = col.off(e.row + 1) - o;
-            const uint8_t* p = col.chars + o + e.delta;
-            uint32_t const avail = static_cast<uint32_t>(min(n - static_cast<int64_t>(e.delta), static_cast<int64_t>(kMaxWord)));
-            uint32_t len         = 0;
-            while (len < avail && p[len] != 0x20u) ++len;
-            tokenize_oov_word(table, GlobalWord{p}, len, [&](uint32_t j, int32_t id) { d[j] = id; });
+            const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+            tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t jj, int32_t id) { d[jj] = id; });
           }
         }
       }
-      done += wave_bcast(incl, kWave - 1);
+      done += wave_bcast(incl2, kWave - 1);
     }
-    cur   = nxt;
-    nxt   = nn;
-    v_cur = v_nxt;
-    c_cur = c_nxt;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -994,9 +1010,9 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(cus) * 8), dim3(256), 0, stream, v, vocabulary->table,
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(cus) * 8), dim3(kOovThreads), 0, stream, v, vocabulary->table,
                          queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, first_offset, results.as<OovResult>(), arena_cnt.as<uint8_t>(),
-                         counts.as<int32_t>());
+                         counts.as<int32_t>(), static_cast<uint32_t>(getenv("NVTEXT_DBG") ? atoi(getenv("NVTEXT_DBG")) : 0));
     }
     // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
@@ -1029,7 +1045,9 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
         return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
       }
       ProfileScope ps("wordpiece_emit_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
+      int64_t const emit_blocks = (static_cast<int64_t>(rows) + kWave * kTokWaves - 1) / (kWave * kTokWaves);
+      unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, static_cast<int64_t>(cus) * 8));
+      hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
                          arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
                          out->offsets,
                          static_cast<int32_t*>(out->child));
