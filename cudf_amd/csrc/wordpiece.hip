@@ -23,7 +23,6 @@
 #include "common.cuh"
 
 #include <algorithm>
-#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -193,42 +192,104 @@ struct StagedWord {
   }
 };
 
-// Token id of key bytes [p, p+len) of `w` in key space `kind`, or kNone.  1 <= len < 200.
-// (raw0, raw1) = bytes [p, p+8) of `w`; whatever lies past the key is trimmed here.
+// A candidate key, ready to be probed: its first block (trimmed), tag word and home bucket.
+struct Probe {
+  uint32_t k0, k1;  // key bytes [0, 8), zero padded
+  uint32_t want;    // slot.x of a matching slot
+  uint32_t bucket;  // home bucket (already masked)
+};
+
+// Hash contribution of key bytes [8, len) (keys that do not fit the slot; kept out of line).
 template <typename W>
-__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len, uint32_t raw0, uint32_t raw1)
+__device__ __forceinline__ uint32_t hash_long_key(W const& w, uint32_t p, uint32_t len, uint32_t h)
 {
-  uint32_t k0 = raw0, k1 = raw1;
-  trim_key8(len, k0, k1);
-  uint32_t h = key_hash_block(key_hash_init(len), k0, k1);
-  for (uint32_t done = 8; done < len; done += 8) {  // keys longer than one block (not kept inside the slot)
+  for (uint32_t done = 8; done < len; done += 8) {
     uint32_t b0, b1;
     w.key8(p + done, len - done, &b0, &b1);
     h = key_hash_block(h, b0, b1);
   }
+  return h;
+}
+
+// (raw0, raw1) = bytes [p, p+8) of `w`; whatever lies past the key is trimmed here.  1 <= len < 200.
+template <typename W>
+__device__ __forceinline__ Probe make_probe(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len, uint32_t raw0, uint32_t raw1)
+{
+  Probe pr;
+  pr.k0 = raw0;
+  pr.k1 = raw1;
+  trim_key8(len, pr.k0, pr.k1);
+  uint32_t h = key_hash_block(key_hash_init(len), pr.k0, pr.k1);
+  if (len > 8) h = hash_long_key(w, p, len, h);
   uint32_t b;
-  uint32_t const want = slot_word0(h, kind, len, &b);
-  for (;;) {
-    b &= t.bucket_mask;
-    uint4 const s0 = t.slots[2 * b];
-    uint4 const s1 = t.slots[2 * b + 1];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      uint4 const& s = j ? s1 : s0;
-      if (s.x == want) {
-        if (len <= 8) {
-          if (s.z == k0 && s.w == k1) return static_cast<int32_t>(s.y);
-        } else {
-          const uint8_t* e = t.pool + s.z;
-          uint32_t i       = 0;
-          while (i < len && e[i] == w.byte(p + i)) ++i;
-          if (i == len) return static_cast<int32_t>(s.y);
-        }
-      }
-      if (s.x == 0) return kNone;
+  pr.want   = slot_word0(h, kind, len, &b);
+  pr.bucket = b & t.bucket_mask;
+  return pr;
+}
+
+template <typename W>
+__device__ __forceinline__ bool pool_key_equal(VocabTable const& t, uint32_t pool_off, W const& w, uint32_t p, uint32_t len)
+{
+  const uint8_t* e = t.pool + pool_off;
+  uint32_t i       = 0;
+  while (i < len && e[i] == w.byte(p + i)) ++i;
+  return i == len;
+}
+
+// Examines one slot: 1 = it holds the key (id set), 0 = it is empty (the key is absent), -1 = look further.
+template <typename W>
+__device__ __forceinline__ int check_slot(VocabTable const& t, uint4 const& s, Probe const& pr, W const& w, uint32_t p, uint32_t len, int32_t* id)
+{
+  if (s.x == pr.want) {
+    bool const same = len <= 8 ? (s.z == pr.k0 && s.w == pr.k1) : pool_key_equal(t, s.z, w, p, len);
+    if (same) {
+      *id = static_cast<int32_t>(s.y);
+      return 1;
     }
-    ++b;
   }
+  return s.x == 0 ? 0 : -1;
+}
+
+// Continues a lookup past a full home bucket without a match (rare at load <= 0.5).
+template <typename W>
+__device__ __forceinline__ int32_t lookup_further(VocabTable const& t, Probe const& pr, W const& w, uint32_t p, uint32_t len)
+{
+  uint32_t b = pr.bucket;
+  for (;;) {
+    b = (b + 1) & t.bucket_mask;
+    int32_t id;
+    int r = check_slot(t, t.slots[2 * b], pr, w, p, len, &id);
+    if (r > 0) return id;
+    if (r == 0) return kNone;
+    r = check_slot(t, t.slots[2 * b + 1], pr, w, p, len, &id);
+    if (r > 0) return id;
+    if (r == 0) return kNone;
+  }
+}
+
+// Outcome of a probe whose two home slots s0, s1 have been loaded.
+template <typename W>
+__device__ __forceinline__ int32_t finish_probe(VocabTable const& t, Probe const& pr, uint4 const& s0, uint4 const& s1, W const& w, uint32_t p,
+                                                uint32_t len)
+{
+  int32_t id;
+  int r = check_slot(t, s0, pr, w, p, len, &id);
+  if (r > 0) return id;
+  if (r == 0) return kNone;
+  r = check_slot(t, s1, pr, w, p, len, &id);
+  if (r > 0) return id;
+  if (r == 0) return kNone;
+  return lookup_further(t, pr, w, p, len);
+}
+
+// Token id of key bytes [p, p+len) of `w` in key space `kind`, or kNone.
+template <typename W>
+__device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W const& w, uint32_t p, uint32_t len, uint32_t raw0, uint32_t raw1)
+{
+  Probe const pr = make_probe(t, kind, w, p, len, raw0, raw1);
+  uint4 const s0 = t.slots[2 * pr.bucket];
+  uint4 const s1 = t.slots[2 * pr.bucket + 1];
+  return finish_probe(t, pr, s0, s1, w, p, len);
 }
 
 // ------------------------------------------------------------------ wavefront helpers of the probe pass
@@ -509,48 +570,96 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
 }
 
 // ------------------------------------------------------------------ out-of-vocabulary pass
-// Greedy longest-match-first tokenization (cpp/src/text/wordpiece_tokenize.cu:349-407) of a word of
-// `len` bytes, 1 <= len < 200, whose whole-word lookup has already failed.  `emit(j, id)` receives token j;
-// returns the token count (a collapse to one unknown token re-emits token 0).
-//
-// One flat loop with one table probe per trip, so that the lanes of a wavefront, each at a different
-// stage of its own word, share trips instead of serialising nested loops.  The state is the piece being
-// searched, bytes [start, e): the first piece (start 0) lives in the full key space, later ones in the
-// "##" space.
-template <typename W, typename Emit>
-__device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
-{
-  uint32_t start = 0, e = len, count = 0;
-  bool fresh = false;  // the whole word is known to be absent: begin by shortening it
+// Greedy longest-match-first tokenization (cpp/src/text/wordpiece_tokenize.cu:349-407) of a word whose
+// whole-word lookup has already failed, as a resumable state machine: every step() examines up to two
+// candidates (their table reads are in flight together) and the lanes of a wavefront, each somewhere
+// inside its own word, share the trips.  The state is the piece being searched, bytes [start, e): the
+// first piece (start 0) lives in the full key space, later ones in the "##" space.
+template <typename W>
+struct OovStepper {
+  uint32_t len, start, e, count;
   uint32_t raw0, raw1;  // bytes [start, start+8) of the word
-  w.key8(0, min(len, 8u), &raw0, &raw1);
-  for (;;) {
-    if (!fresh) {
-      // wordpiece_tokenize.cu:307-317: drop the last UTF-8 character of the candidate
-      uint32_t x = (e - start) < 2 ? start : e - 1;
-      while (x > start && is_utf8_continuation(w.byte(x))) --x;
-      if (x == start) {
-        // no prefix of the word matched (375-379), or a later piece has no match and the word
-        // collapses (396-404): either way a single unknown token
-        emit(0u, t.unk_id);
-        return 1;
-      }
-      e = x;
-    }
-    fresh               = false;
+  bool fresh;           // [start, e) itself is still untried
+  bool done;
+
+  // wordpiece_tokenize.cu:307-317: the end after dropping the last UTF-8 character of [start, x); start if none is left
+  static __device__ __forceinline__ uint32_t drop(W const& w, uint32_t start, uint32_t x)
+  {
+    if (x - start < 2) return start;
+    --x;
+    while (x > start && is_utf8_continuation(w.byte(x))) --x;
+    return x;
+  }
+
+  __device__ __forceinline__ void begin(W const& w, uint32_t len_)
+  {
+    len = len_; start = 0; e = len_; count = 0;
+    fresh = false;  // the whole word is known to be absent: begin by shortening it
+    done  = false;
+    w.key8(0, min(len, 8u), &raw0, &raw1);
+  }
+
+  template <typename Emit>
+  __device__ __forceinline__ void step(VocabTable const& t, W const& w, Emit&& emit)
+  {
     uint32_t const kind = count ? 1u : 0u;
-    uint32_t const pl   = e - start;
-    if (pl > t.max_len[kind]) continue;  // no key this long exists: keep shortening
-    int32_t const id = lookup(t, kind, w, start, pl, raw0, raw1);
-    if (id == kNone) continue;
+    uint32_t const maxl = t.max_len[kind];
+    uint32_t ea         = fresh ? e : drop(w, start, e);
+    if (ea - start > maxl) {
+      // no key is this long: go straight to the longest candidate that can exist (on a character boundary)
+      ea = start + maxl;
+      while (ea > start && is_utf8_continuation(w.byte(ea))) --ea;
+    }
+    if (ea == start) {
+      // no prefix of the word matched (375-379), or a later piece has no match and the word collapses
+      // (396-404): either way a single unknown token
+      emit(0u, t.unk_id);
+      count = 1;
+      done  = true;
+      return;
+    }
+    uint32_t const eb = drop(w, start, ea);
+    bool const has_b  = eb > start;
+    Probe const pa    = make_probe(t, kind, w, start, ea - start, raw0, raw1);
+    Probe const pb    = make_probe(t, kind, w, start, has_b ? eb - start : 1u, raw0, raw1);
+    uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
+    uint4 b0 = make_uint4(0, 0, 0, 0), b1 = b0;
+    if (has_b) {
+      b0 = t.slots[2 * pb.bucket];
+      b1 = t.slots[2 * pb.bucket + 1];
+    }
+    uint32_t hit_end = ea;
+    int32_t id       = finish_probe(t, pa, a0, a1, w, start, ea - start);
+    if (id == kNone && has_b) {
+      hit_end = eb;
+      id      = finish_probe(t, pb, b0, b1, w, start, eb - start);
+    }
+    if (id == kNone) {
+      e     = has_b ? eb : ea;
+      fresh = false;
+      return;
+    }
     emit(count++, id);
-    if (e == len) return count;
+    if (hit_end == len) {
+      done = true;
+      return;
+    }
     // next piece: the rest of the word (381-395)
-    start = e;
+    start = hit_end;
     e     = len;
     fresh = true;
     w.key8(start, min(len - start, 8u), &raw0, &raw1);
   }
+};
+
+// Runs one word to completion (used where out-of-vocabulary words are rare).  Returns the token count.
+template <typename W, typename Emit>
+__device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
+{
+  OovStepper<W> st;
+  st.begin(w, len);
+  while (!st.done) st.step(t, w, emit);
+  return st.count;
 }
 
 // Brings the first bytes of the `len`-byte word at p into this lane's LDS window with 16-byte aligned
@@ -570,39 +679,67 @@ __device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, u
   return mis;
 }
 
-// One lane per queued word.  results[q] = its first kOovKeep tokens; arena_cnt[slot] = its token count;
-// counts[row] += count.
+// One lane per queued word, and a lane that finishes its word takes the next one: every wavefront owns a
+// contiguous part of the queue and, every fourth trip, lets its idle lanes store their result and pick up
+// new entries, so lanes with short words do not wait for the longest word of a batch.
+// results[q] = the word's first kOovKeep tokens; arena_cnt[slot] = its token count; counts[row] += count.
 __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
-                                                            const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
-                                                            int64_t first_offset, OovResult* __restrict__ results,
-                                                            uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts, uint32_t dbg)
+                                                                    const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
+                                                                    int64_t first_offset, OovResult* __restrict__ results,
+                                                                    uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts)
 {
   __shared__ uint32_t windows[kStage / 4][kOovThreads];
-  uint32_t const total  = min(*queue_size, queue_capacity);
-  uint32_t const stride = gridDim.x * blockDim.x;
   uint32_t* const win   = &windows[0][threadIdx.x];
-  for (uint32_t q = blockIdx.x * blockDim.x + threadIdx.x; q < total; q += stride) {
-    OovEntry const e = queue[q];
-    if (e.row < 0) continue;  // unused tail of a reserved range
-    int64_t const o    = col.off(e.row);
-    const uint8_t* p   = col.chars + o + e.delta;
-    uint32_t const len = e.len;
-    uint32_t const mis = stage_word(p, len, win);
-    StagedWord const w{win, p, mis};
-    int32_t tok[kOovKeep];
-    uint32_t cnt = 1;
-    if (dbg & 1u) { tok[0] = static_cast<int32_t>(w.byte(0)); }
-    else cnt = tokenize_oov_word(table, w, len, [&](uint32_t j, int32_t id) {
+  uint32_t const total  = min(*queue_size, queue_capacity);
+  uint32_t const nwave  = gridDim.x * (kOovThreads / kWave);
+  uint32_t const wave   = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
+  uint32_t const chunk  = (total + nwave - 1) / nwave;
+  uint32_t next         = min(total, wave * chunk);          // wave-uniform cursor into this wavefront's part
+  uint32_t const q_end  = min(total, next + chunk);
+
+  OovStepper<StagedWord> st;
+  st.done = true;
+  StagedWord w{win, nullptr, 0};
+  bool busy  = false;  // this lane holds a word (finished or not)
+  uint32_t q = 0;
+  OovEntry e{-1, 0, 0, 0};
+  int32_t tok[kOovKeep];
+  for (uint32_t trip = 0;; ++trip) {
+    if ((trip & 3u) == 0) {
+      if (busy && st.done) {  // deliver
+        OovResult res;
 #pragma unroll
-      for (int k = 0; k < kOovKeep; ++k)
-        if (j == static_cast<uint32_t>(k)) tok[k] = id;
-    });
-    OovResult res;
+        for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
+        results[q] = res;
+        arena_cnt[((col.off(e.row) - first_offset) >> 1) + e.row + e.widx] = static_cast<uint8_t>(st.count);  // count <= len < 200
+        atomicAdd(&counts[e.row], static_cast<int32_t>(st.count));
+        busy = false;
+      }
+      uint64_t const idle = ballot64(!busy);
+      if (idle != 0 && next < q_end) {  // refill
+        uint32_t const mine = next + lanes_below(idle);
+        next += static_cast<uint32_t>(__builtin_popcountll(idle));
+        if (!busy && mine < q_end) {
+          e = queue[mine];
+          if (e.row >= 0) {  // (-1 marks the unused tail of a reserved queue range)
+            q                = mine;
+            const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+            w.p              = p;
+            w.mis            = stage_word(p, e.len, win);
+            st.begin(w, e.len);
+            busy = true;
+          }
+        }
+      }
+      if (ballot64(busy) == 0 && next >= q_end) break;
+    }
+    if (busy && !st.done) {
+      st.step(table, w, [&](uint32_t j, int32_t id) {
 #pragma unroll
-    for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
-    results[q] = res;
-    arena_cnt[((o - first_offset) >> 1) + e.row + e.widx] = static_cast<uint8_t>(cnt);  // cnt <= len < 200
-    if (!(dbg & 2u)) atomicAdd(&counts[e.row], static_cast<int32_t>(cnt));
+        for (int k = 0; k < kOovKeep; ++k)
+          if (j == static_cast<uint32_t>(k)) tok[k] = id;
+      });
+    }
   }
 }
 
@@ -974,8 +1111,14 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   int device = 0, cus = 256;
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+  // persistent kernels: as many workgroups as can be resident at once
+  auto resident = [&](const void* kernel, int threads) -> int64_t {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 4;
+    return static_cast<int64_t>(per_cu) * cus;
+  };
   unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves - 1) / kTokWaves,
-                                                                      static_cast<int64_t>(cus) * 8));
+                                                                      resident(reinterpret_cast<const void*>(wordpiece_probe_kernel), kTokThreads)));
   // Each wavefront reserves queue entries `queue_block` at a time (one atomic per block).
   uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
   uint32_t queue_block = 64;
@@ -1010,9 +1153,10 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(cus) * 8), dim3(kOovThreads), 0, stream, v, vocabulary->table,
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads))),
+                         dim3(kOovThreads), 0, stream, v, vocabulary->table,
                          queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, first_offset, results.as<OovResult>(), arena_cnt.as<uint8_t>(),
-                         counts.as<int32_t>(), static_cast<uint32_t>(getenv("NVTEXT_DBG") ? atoi(getenv("NVTEXT_DBG")) : 0));
+                         counts.as<int32_t>());
     }
     // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
@@ -1046,7 +1190,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       }
       ProfileScope ps("wordpiece_emit_kernel", stream);
       int64_t const emit_blocks = (static_cast<int64_t>(rows) + kWave * kTokWaves - 1) / (kWave * kTokWaves);
-      unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, static_cast<int64_t>(cus) * 8));
+      unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
                          arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
                          out->offsets,
