@@ -88,8 +88,10 @@ namespace {
 
 constexpr int kTokWaves     = 4;
 constexpr int kTokThreads   = kTokWaves * kWave;
-constexpr int kChunk        = 1024;  // bytes per wavefront step (16 per lane)
-constexpr int kRing         = 2048;  // two chunks: the current one and the one before it
+constexpr int kGroups       = 4;     // rows a wavefront walks at the same time, 16 lanes each
+constexpr int kGroupLanes   = kWave / kGroups;
+constexpr int kChunk        = 16 * kGroupLanes;  // bytes per group step (16 per lane) = 256
+constexpr int kRing         = 2 * kChunk;        // per group: the current chunk and the one before it
 constexpr int32_t kNone     = std::numeric_limits<int32_t>::min();
 constexpr int kOovKeep      = 8;     // tokens stored per queued word; longer results are redone at emit time
 constexpr uint32_t kOovMark = 0x80000000u;  // word-arena value 0x80000000 | queue index (never 0xFFFFFFFF = id -1)
@@ -113,7 +115,7 @@ __device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& 
   else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
 }
 
-// A word inside the 2 KiB LDS ring of the probe pass: byte k of the word is ring byte (start + k) & 2047.
+// A word inside a group's 512-byte LDS ring of the probe pass: byte k of the word is ring byte (start + k) & 511.
 struct RingWord {
   const uint32_t* ring;
   uint32_t start;
@@ -331,9 +333,9 @@ __device__ __forceinline__ uint32_t gather_byte_flags(uint32_t z) { return (((z 
 __device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
 
 struct ProbeLds {
-  uint32_t bytes[kRing / 4];       // row bytes (everything outside the row is ' ')
-  uint16_t wend[kChunk / 2 + 2];   // per word ending in the chunk: offset of its last byte inside the chunk
-  uint16_t wlen[kChunk / 2 + 2];   // and its length in bytes, clamped to kMaxWord
+  alignas(16) uint32_t bytes[kGroups][kRing / 4];  // per group: row bytes (everything outside the row is ' ')
+  uint16_t wend[kGroups * kChunk / 2 + 2];         // per word ending in this step: offset of its last byte inside its group's chunk
+  uint16_t wlen[kGroups * kChunk / 2 + 2];         // and its length in bytes, clamped to kMaxWord
 };
 
 // Where a row sits relative to 16-byte aligned memory.  Coordinates count bytes from `base`.
@@ -381,10 +383,30 @@ __device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, in
 }
 
 // ------------------------------------------------------------------ probe pass
-// Persistent wavefronts, one row at a time, with the next row's offsets and the next chunk already in
-// flight.  For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an
-// out-of-vocabulary marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass
-// overwrites it with the word's token count); nwords[r] = words kept; counts[r] = one per hit.
+// DPP moves inside a row of 16 lanes; lanes without a source keep `old`.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_row(uint32_t old, uint32_t v)
+{
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(old), static_cast<int>(v), CTRL, 0xf, 0xf, false));
+}
+// inclusive max-scan inside each group of 16 lanes
+__device__ __forceinline__ uint32_t group_scan_max(uint32_t v)
+{
+  v = max(v, dpp_row<0x111>(0u, v));  // row_shr:1
+  v = max(v, dpp_row<0x112>(0u, v));  // row_shr:2
+  v = max(v, dpp_row<0x114>(0u, v));  // row_shr:4
+  v = max(v, dpp_row<0x118>(0u, v));  // row_shr:8
+  return v;
+}
+__device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return static_cast<uint32_t>(__shfl(static_cast<int>(v), src_lane)); }
+
+// Persistent wavefronts.  Each group of 16 lanes walks its own row in 256-byte chunks (16 bytes per lane),
+// so a wavefront has four rows in flight; the words the four groups find in a step are pooled and probed
+// with lanes <-> words.  The next chunk of every group (the rest of its row, else the start of its next
+// row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
+// For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
+// marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass overwrites it with the
+// word's token count); nwords[r] = words kept; counts[r] = one per hit.
 __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
                                                                       uint32_t* __restrict__ arena, uint8_t* __restrict__ arena_cnt,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
@@ -392,178 +414,207 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
                                                                       uint32_t* __restrict__ queue_size)
 {
   __shared__ ProbeLds lds_all[kTokWaves];
-  int const lane      = lane_id();
-  int const wave      = threadIdx.x / kWave;
-  ProbeLds& lds       = lds_all[wave];
-  int64_t const nwave = static_cast<int64_t>(gridDim.x) * kTokWaves;
-  int64_t const rows  = col.size;
+  int const lane       = lane_id();
+  int const wave       = threadIdx.x / kWave;
+  int const g          = lane / kGroupLanes;  // my group
+  int const gl         = lane % kGroupLanes;  // my lane inside it
+  int const g_first    = g * kGroupLanes;
+  int const g_last     = g_first + kGroupLanes - 1;
+  ProbeLds& lds        = lds_all[wave];
+  int64_t const rows   = col.size;
+  int64_t const stride = static_cast<int64_t>(gridDim.x) * kTokWaves * kGroups;  // rows between two rows of a group
   uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
 
-  int64_t r = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave;
-  // software pipeline: offsets two rows ahead, the next chunk one step ahead
+  // ---- per-group state (the same value in all 16 lanes of a group)
+  int64_t r = (static_cast<int64_t>(blockIdx.x) * kTokWaves + wave) * kGroups + g;
   int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
   if (r < rows) {
     o_cur = col.off(r);
     e_cur = col.off(r + 1);
   }
-  if (r + nwave < rows) {
-    o_nxt = col.off(r + nwave);
-    e_nxt = col.off(r + nwave + 1);
+  if (r + stride < rows) {
+    o_nxt = col.off(r + stride);
+    e_nxt = col.off(r + stride + 1);
   }
-  RowCtx ctx = make_row_ctx(col, o_cur, e_cur - o_cur);
-  // the chunk about to be processed: my sixteen bytes and (lane 63) the byte after the chunk
+  RowCtx ctx       = make_row_ctx(col, o_cur, e_cur - o_cur);
+  int64_t cbase    = 0;
+  uint32_t wdone   = 0;     // words kept so far in this row
+  uint32_t hits    = 0;     // of which found in the vocabulary
+  uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
+  uint32_t prev_space  = 1; // the byte before the chunk is a space (or the row starts here)
+  // the chunk about to be processed: my sixteen bytes and (last lane of the group) the byte after the chunk
   uint4 mine_cur    = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
   uint32_t tail_cur = 0x20u;
   if (r < rows) {
-    mine_cur = ctx.load_clean(16 * lane);
-    if (lane == kWave - 1) tail_cur = ctx.byte_at(kChunk);
+    mine_cur = ctx.load_clean(16 * gl);
+    if (gl == kGroupLanes - 1) tail_cur = ctx.byte_at(kChunk);
   }
 
-  for (; r < rows; r += nwave) {
-    RowCtx const ctx_nxt = make_row_ctx(col, o_nxt, e_nxt - o_nxt);
-    bool const have_nxt  = r + nwave < rows;
-    int64_t o_nn = 0, e_nn = 0;
-    if (r + 2 * nwave < rows) {
-      o_nn = col.off(r + 2 * nwave);
-      e_nn = col.off(r + 2 * nwave + 1);
-    }
-
-    int64_t const n = e_cur - o_cur;
+  while (ballot64(r < rows) != 0) {
+    bool const has_row = r < rows;
     // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
     // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
-    int64_t cap = std::numeric_limits<int64_t>::max();
-    if (max_words > 0) cap = col.valid(r) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
-    int64_t const slot0   = ((o_cur - first_offset) >> 1) + r;
-    uint32_t* const slots = arena + slot0;
-    uint8_t* const scnt   = arena_cnt + slot0;
+    int64_t const n = e_cur - o_cur;
+    int64_t cap     = std::numeric_limits<int32_t>::max();
+    if (max_words > 0) cap = (has_row && col.valid(r)) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
+    bool const chunk_ok = has_row && cbase < ctx.aend && static_cast<int64_t>(wdone) < cap;
 
-    int64_t words_done   = 0;
-    uint32_t hits        = 0;
-    uint32_t carry_start = 0;     // 1-based coordinate of the start of the word running into the chunk
-    bool prev_space      = true;  // the byte before the chunk is a space (or the row starts here)
-    bool next_is_row     = false; // whether the prefetched chunk is the next row's first one
-    for (int64_t cbase = 0; cbase < ctx.aend && words_done < cap; cbase += kChunk) {
-      int64_t const a0      = cbase + 16 * lane;
-      uint4 const mine    = mine_cur;
-      uint32_t const tail = tail_cur;
-      // prefetch the chunk that follows: the rest of this row, else the start of the next row
-      bool const more = cbase + kChunk < ctx.aend;
-      next_is_row     = !more;
-      if (more || have_nxt) {
-        RowCtx const& pc    = more ? ctx : ctx_nxt;
-        int64_t const pbase = more ? cbase + kChunk : 0;
-        mine_cur            = pc.load_clean(pbase + 16 * lane);
-        if (lane == kWave - 1) tail_cur = pc.byte_at(pbase + kChunk);
-      }
-      uint32_t const ring0 = static_cast<uint32_t>(a0) & (kRing - 1);
-      *reinterpret_cast<uint4*>(&lds.bytes[ring0 >> 2]) = mine;
-
-      // bit i of sp: my byte i is a space
+    // ---- bytes -> word ends (lanes <-> bytes, per group)
+    uint32_t ends = 0, starts = 0, xs = 0;
+    uint32_t const a0 = static_cast<uint32_t>(cbase) + 16u * gl;  // coordinates fit 32 bits (rows are below 2 GiB)
+    if (chunk_ok) {
+      *reinterpret_cast<uint4*>(&lds.bytes[g][(a0 & (kRing - 1)) >> 2]) = mine_cur;
+    }
+    {
+      uint4 const mine  = mine_cur;
       uint32_t const sp = gather_byte_flags(space_bytes(mine.x)) | (gather_byte_flags(space_bytes(mine.y)) << 4) |
                           (gather_byte_flags(space_bytes(mine.z)) << 8) | (gather_byte_flags(space_bytes(mine.w)) << 12);
-      // neighbours: is the byte before my sixteen a space, and the byte after them
-      uint32_t before = from_lane_below<1>(sp >> 15);
-      if (lane == 0) before = prev_space ? 1u : 0u;
-      uint32_t after = static_cast<uint32_t>(__shfl_down(static_cast<int>(sp & 1u), 1));
-      if (lane == kWave - 1) after = tail == 0x20u ? 1u : 0u;
-      prev_space = wave_bcast(sp >> 15, kWave - 1) != 0;
-
+      // is the byte before my sixteen a space, and the byte after them
+      uint32_t const before = dpp_row<0x111>(prev_space, sp >> 15);                       // row_shr:1
+      uint32_t const after  = dpp_row<0x101>(tail_cur == 0x20u ? 1u : 0u, sp & 1u);        // row_shl:1
       uint32_t const word   = ~sp & 0xFFFFu;
-      uint32_t const starts = word & ((sp << 1) | before);            // a word byte after a space
-      uint32_t const ends   = word & ((sp >> 1) | (after << 15));     // a word byte before a space
+      starts                = word & ((sp << 1) | before);         // a word byte after a space
+      ends                  = word & ((sp >> 1) | (after << 15));  // a word byte before a space
+      if (!chunk_ok) ends = starts = 0;
       // start of the word that runs into my bytes: the last start in the lanes below, else the carry
-      uint32_t const my_last = starts ? static_cast<uint32_t>(a0) + (32u - __builtin_clz(starts)) : 0u;
-      uint32_t const is      = wave_scan_max(my_last);
-      uint32_t const xs      = max(from_lane_below<0>(is), carry_start);
-      carry_start            = max(carry_start, wave_bcast(is, kWave - 1));
-
-      uint32_t const ne    = __builtin_popcount(ends);
-      uint32_t const incl  = wave_inclusive_scan(ne);
-      uint32_t const total = wave_bcast(incl, kWave - 1);
-      uint32_t slot        = incl - ne;
-      for (uint32_t em = ends; em; em &= em - 1) {
-        uint32_t const p  = __builtin_ctz(em);
-        uint32_t const sb = starts & ((2u << p) - 1u);
-        uint32_t const st = sb ? static_cast<uint32_t>(a0) + (32u - __builtin_clz(sb)) : xs;  // 1-based
-        uint32_t const wl = static_cast<uint32_t>(a0) + p + 1u - st + 1u;
-        lds.wend[slot]    = static_cast<uint16_t>(16u * lane + p);
-        lds.wlen[slot]    = static_cast<uint16_t>(min(wl, kMaxWord));
-        ++slot;
+      uint32_t const my_last = starts ? a0 + (32u - __builtin_clz(starts)) : 0u;
+      uint32_t const is      = group_scan_max(my_last);
+      xs                     = max(dpp_row<0x111>(0u, is), carry_start);
+      if (chunk_ok) {
+        carry_start = max(carry_start, shfl_u32(is, g_last));
+        prev_space  = shfl_u32(sp >> 15, g_last);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    uint32_t const ne   = __builtin_popcount(ends);
+    uint32_t const incl = wave_inclusive_scan(ne);
+    // first word slot of every group and the total
+    uint32_t const gb1 = wave_bcast(incl, 15), gb2 = wave_bcast(incl, 31), gb3 = wave_bcast(incl, 47), total = wave_bcast(incl, 63);
+    uint32_t const my_gbase  = g == 0 ? 0u : g == 1 ? gb1 : g == 2 ? gb2 : gb3;
+    uint32_t const my_gtotal = (g == 0 ? gb1 : g == 1 ? gb2 : g == 2 ? gb3 : total) - my_gbase;
+    uint32_t slot            = incl - ne;
+    for (uint32_t em = ends; em; em &= em - 1) {
+      uint32_t const p  = __builtin_ctz(em);
+      uint32_t const sb = starts & ((2u << p) - 1u);
+      uint32_t const st = sb ? a0 + (32u - __builtin_clz(sb)) : xs;  // 1-based
+      uint32_t const wl = a0 + p + 1u - st + 1u;
+      lds.wend[slot]    = static_cast<uint16_t>(16u * gl + p);
+      lds.wlen[slot]    = static_cast<uint16_t>(min(wl, kMaxWord));
+      ++slot;
+    }
+    // words of this chunk that count (the row's word limit may cut them short)
+    uint32_t const allowed = chunk_ok ? static_cast<uint32_t>(min(static_cast<int64_t>(my_gtotal), cap - static_cast<int64_t>(wdone))) : 0u;
 
-      int64_t const allowed = min(static_cast<int64_t>(total), cap - words_done);
-      for (uint32_t w0 = 0; w0 < allowed; w0 += kWave) {
-        uint32_t const wi = w0 + lane;
-        bool const active = wi < allowed;
-        bool miss         = false;
-        uint32_t value    = 0;
-        int64_t wstart    = 0;  // coordinate of the word's first byte
-        uint32_t wl = 0;
-        if (active) {
-          wl     = lds.wlen[wi];
-          wstart = cbase + lds.wend[wi] + 1 - static_cast<int64_t>(wl);
-          if (wl >= kMaxWord) {
-            value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
-          } else {
-            int32_t id = kNone;
-            if (wl <= table.max_len[0]) {
-              RingWord const rw{lds.bytes, static_cast<uint32_t>(wstart) & (kRing - 1)};
-              uint32_t r0, r1;
-              rw.key8(0, 8, &r0, &r1);
-              id = lookup(table, 0, rw, 0, wl, r0, r1);
-            }
-            miss  = id == kNone;
-            value = static_cast<uint32_t>(id);
-          }
+    // ---- what this group looks at next; request it now so it arrives while the probes run
+    int64_t const r_now     = r;
+    int64_t const o_now     = o_cur;
+    uint32_t const mis_now  = ctx.mis;
+    uint32_t const cb_now   = static_cast<uint32_t>(cbase);
+    uint32_t const wd_now   = wdone;
+    uint32_t const wd_after = wdone + allowed;
+    bool const row_done     = has_row && !(chunk_ok && cbase + kChunk < ctx.aend && static_cast<int64_t>(wd_after) < cap);
+    if (has_row) {
+      if (!row_done) {
+        cbase += kChunk;
+        wdone = wd_after;
+      } else {
+        r += stride;
+        o_cur = o_nxt;
+        e_cur = e_nxt;
+        ctx   = make_row_ctx(col, o_cur, e_cur - o_cur);
+        cbase = 0;
+        wdone = 0;
+        carry_start = 0;
+        prev_space  = 1;
+        if (r + stride < rows) {
+          o_nxt = col.off(r + stride);
+          e_nxt = col.off(r + stride + 1);
         }
-        uint64_t const mm = ballot64(miss);
-        if (mm) {
-          uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
-          if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
-            // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
-            for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-              if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
-            uint32_t base = 0;
-            if (lane == 0) base = atomicAdd(queue_size, queue_block);
-            q_pos = wave_bcast(base, 0);
-            q_lim = q_pos + queue_block;
-          }
-          if (miss) {
-            uint32_t const q = q_pos + lanes_below(mm);
-            if (q < queue_capacity)
-              queue[q] = OovEntry{static_cast<int32_t>(r), static_cast<uint32_t>(wstart - ctx.mis), static_cast<uint32_t>(words_done) + wi, wl};
-            value = kOovMark | q;
-          }
-          q_pos += nm;
-        }
-        if (active) {
-          slots[words_done + wi] = value;
-          scnt[words_done + wi]  = 1;
-        }
-        hits += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && !miss)));
       }
-      words_done += allowed;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+      if (r < rows) {
+        mine_cur = ctx.load_clean(cbase + 16 * gl);
+        tail_cur = gl == kGroupLanes - 1 ? ctx.byte_at(cbase + kChunk) : 0x20u;
+      }
     }
-    if (lane == 0) {
-      nwords[r] = static_cast<int32_t>(words_done);
-      counts[r] = static_cast<int32_t>(hits);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // ---- probes (lanes <-> words, all groups pooled)
+    uint32_t my_hits = 0;
+    for (uint32_t w0 = 0; w0 < total; w0 += kWave) {
+      uint32_t const ws = w0 + lane;  // word slot
+      int const gw      = (ws >= gb1) + (ws >= gb2) + (ws >= gb3);
+      int const src     = gw * kGroupLanes;
+      uint32_t const idx = ws - shfl_u32(my_gbase, src);
+      uint32_t const alw = shfl_u32(allowed, src);  // (every lane must take part in a shuffle: keep it out of the && below)
+      bool const active  = ws < total && idx < alw;
+      uint32_t const cbw = shfl_u32(cb_now, src);
+      uint32_t const wdw = shfl_u32(wd_now, src);
+      uint32_t const misw = shfl_u32(mis_now, src);
+      int32_t const rw   = static_cast<int32_t>(shfl_u32(static_cast<uint32_t>(r_now), src));
+      int64_t const ow   = (static_cast<int64_t>(shfl_u32(static_cast<uint32_t>(static_cast<uint64_t>(o_now) >> 32), src)) << 32) |
+                         shfl_u32(static_cast<uint32_t>(o_now), src);
+      bool miss       = false;
+      uint32_t value  = 0, wl = 0, wstart = 0;
+      if (active) {
+        wl     = lds.wlen[ws];
+        wstart = cbw + lds.wend[ws] + 1u - wl;  // coordinate of the word's first byte
+        if (wl >= kMaxWord) {
+          value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+        } else {
+          int32_t id = kNone;
+          if (wl <= table.max_len[0]) {
+            RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
+            uint32_t r0, r1;
+            rw_.key8(0, 8, &r0, &r1);
+            id = lookup(table, 0, rw_, 0, wl, r0, r1);
+          }
+          miss  = id == kNone;
+          value = static_cast<uint32_t>(id);
+        }
+      }
+      uint64_t const mm = ballot64(miss);
+      if (mm) {
+        uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
+        if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
+          // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
+          for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+            if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+          uint32_t base = 0;
+          if (lane == 0) base = atomicAdd(queue_size, queue_block);
+          q_pos = wave_bcast(base, 0);
+          q_lim = q_pos + queue_block;
+        }
+        if (miss) {
+          uint32_t const q = q_pos + lanes_below(mm);
+          if (q < queue_capacity) queue[q] = OovEntry{rw, wstart - misw, wdw + idx, wl};
+          value = kOovMark | q;
+        }
+        q_pos += nm;
+      }
+      if (active) {
+        int64_t const s = ((ow - first_offset) >> 1) + rw + wdw + idx;
+        arena[s]        = value;
+        arena_cnt[s]    = 1;
+      }
+      uint64_t const hit = ballot64(active && !miss);
+      if (hit) {
+        // credit the hits to the groups that own the words
+        uint64_t const in_g0 = ballot64(gw == 0), in_g1 = ballot64(gw == 1), in_g2 = ballot64(gw == 2);
+        uint64_t const mine_mask = g == 0 ? in_g0 : g == 1 ? in_g1 : g == 2 ? in_g2 : ~(in_g0 | in_g1 | in_g2);
+        my_hits += static_cast<uint32_t>(__builtin_popcountll(hit & mine_mask));
+      }
     }
-    // rotate the pipeline.  The prefetched chunk is the next row's first one unless the row was left
-    // early (word limit reached, or a row whose loop never ran): then fetch it now.
-    if (!next_is_row && have_nxt) {
-      mine_cur = ctx_nxt.load_clean(16 * lane);
-      if (lane == kWave - 1) tail_cur = ctx_nxt.byte_at(kChunk);
+    hits += my_hits;
+    if (row_done) {
+      if (gl == 0) {
+        nwords[r_now] = static_cast<int32_t>(wd_after);
+        counts[r_now] = static_cast<int32_t>(hits);
+      }
+      hits = 0;
     }
-    ctx   = ctx_nxt;
-    o_cur = o_nxt;
-    e_cur = e_nxt;
-    o_nxt = o_nn;
-    e_nxt = e_nn;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
   for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
     if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
@@ -1117,7 +1168,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 4;
     return static_cast<int64_t>(per_cu) * cus;
   };
-  unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves - 1) / kTokWaves,
+  unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves * kGroups - 1) / (kTokWaves * kGroups),
                                                                       resident(reinterpret_cast<const void*>(wordpiece_probe_kernel), kTokThreads)));
   // Each wavefront reserves queue entries `queue_block` at a time (one atomic per block).
   uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
