@@ -62,7 +62,21 @@ struct VocabTable {
   uint32_t bucket_mask;  // buckets - 1
   int32_t unk_id;
   uint32_t max_len[2];   // longest key of each key space (longer candidates cannot match)
+  // Length filter: lens[length_filter_index(kind, first three key bytes) & lens_mask] has bit i (i < 31) set
+  // when some key of that key space with those first bytes is i + 3 bytes long, bit 31 for 34 bytes and more.
+  // Entries are shared by hashing, so a set bit promises nothing, a clear bit rules the length out.
+  const uint32_t* lens;
+  uint32_t lens_mask;
 };
+
+__host__ __device__ __forceinline__ uint32_t length_filter_index(uint32_t kind, uint32_t first3)
+{
+  uint32_t x = (first3 | (kind << 24)) * 0x9E3779B1u;
+  x ^= x >> 15;
+  x *= 0x85EBCA77u;
+  return x ^ (x >> 13);
+}
+__host__ __device__ __forceinline__ uint32_t length_filter_bit(uint32_t len) { return len >= 34 ? 31u : len - 3u; }
 
 __host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t h, uint32_t kind, uint32_t len, uint32_t* bucket)
 {
@@ -78,6 +92,7 @@ struct nvtext_amd_wordpiece_vocabulary {
   nvtext_amd::VocabTable table{};
   void* d_slots     = nullptr;
   void* d_pool      = nullptr;
+  void* d_lens      = nullptr;
   size_t slot_bytes = 0;
   size_t pool_bytes = 0;
   int32_t entries   = 0;
@@ -630,24 +645,65 @@ template <typename W>
 struct OovStepper {
   uint32_t len, start, e, count;
   uint32_t raw0, raw1;  // bytes [start, start+8) of the word
+  uint32_t lens;        // length filter word of the piece that starts at `start` (all ones when it is shorter than 3 bytes)
+  bool ascii;           // no byte of the word has bit 7 set: every position is a character boundary
   bool fresh;           // [start, e) itself is still untried
   bool done;
 
+  __device__ __forceinline__ bool inside_character(W const& w, uint32_t x) const { return !ascii && is_utf8_continuation(w.byte(x)); }
+
   // wordpiece_tokenize.cu:307-317: the end after dropping the last UTF-8 character of [start, x); start if none is left
-  static __device__ __forceinline__ uint32_t drop(W const& w, uint32_t start, uint32_t x)
+  __device__ __forceinline__ uint32_t drop(W const& w, uint32_t x) const
   {
     if (x - start < 2) return start;
     --x;
-    while (x > start && is_utf8_continuation(w.byte(x))) --x;
+    while (x > start && inside_character(w, x)) --x;
     return x;
   }
 
-  __device__ __forceinline__ void begin(W const& w, uint32_t len_)
+  // The longest candidate end <= x (x on a character boundary, start < x < len or x == len) that the length
+  // filter does not rule out and that ends on a character boundary; start if there is none.  Only lengths
+  // without a key are skipped, so the candidates that can match are visited in the reference's order.
+  __device__ __forceinline__ uint32_t allowed_end(W const& w, uint32_t x) const
+  {
+    uint32_t l = x - start;
+    bool boundary = true;  // start + l is known to be a character boundary
+    while (l >= 3) {
+      if (l >= 34 && (lens >> 31)) break;
+      uint32_t const top = min(l - 3u, 30u);
+      uint32_t const m   = lens & (0xFFFFFFFFu >> (31u - top));
+      if (m == 0) {
+        l        = 2;
+        boundary = false;
+        break;
+      }
+      uint32_t const best = 34u - static_cast<uint32_t>(__builtin_clz(m));  // 3 + index of the highest set bit
+      boundary            = boundary && best == l;
+      l                   = best;
+      if (boundary || !inside_character(w, start + l)) {
+        boundary = true;
+        break;
+      }
+      --l;
+    }
+    if (!boundary)
+      while (l > 0 && inside_character(w, start + l)) --l;
+    return start + l;
+  }
+
+  __device__ __forceinline__ void load_filter(VocabTable const& t, uint32_t kind)
+  {
+    lens = len - start >= 3 ? t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
+  }
+
+  __device__ __forceinline__ void begin(VocabTable const& t, W const& w, uint32_t len_, bool ascii_)
   {
     len = len_; start = 0; e = len_; count = 0;
+    ascii = ascii_;
     fresh = false;  // the whole word is known to be absent: begin by shortening it
     done  = false;
     w.key8(0, min(len, 8u), &raw0, &raw1);
+    load_filter(t, 0);
   }
 
   template <typename Emit>
@@ -655,12 +711,13 @@ struct OovStepper {
   {
     uint32_t const kind = count ? 1u : 0u;
     uint32_t const maxl = t.max_len[kind];
-    uint32_t ea         = fresh ? e : drop(w, start, e);
+    uint32_t ea         = fresh ? e : drop(w, e);
     if (ea - start > maxl) {
       // no key is this long: go straight to the longest candidate that can exist (on a character boundary)
       ea = start + maxl;
-      while (ea > start && is_utf8_continuation(w.byte(ea))) --ea;
+      while (ea > start && inside_character(w, ea)) --ea;
     }
+    ea = allowed_end(w, ea);
     if (ea == start) {
       // no prefix of the word matched (375-379), or a later piece has no match and the word collapses
       // (396-404): either way a single unknown token
@@ -669,7 +726,7 @@ struct OovStepper {
       done  = true;
       return;
     }
-    uint32_t const eb = drop(w, start, ea);
+    uint32_t const eb = allowed_end(w, drop(w, ea));
     bool const has_b  = eb > start;
     Probe const pa    = make_probe(t, kind, w, start, ea - start, raw0, raw1);
     Probe const pb    = make_probe(t, kind, w, start, has_b ? eb - start : 1u, raw0, raw1);
@@ -700,6 +757,7 @@ struct OovStepper {
     e     = len;
     fresh = true;
     w.key8(start, min(len - start, 8u), &raw0, &raw1);
+    load_filter(t, 1);
   }
 };
 
@@ -708,25 +766,30 @@ template <typename W, typename Emit>
 __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
 {
   OovStepper<W> st;
-  st.begin(w, len);
+  st.begin(t, w, len, false);
   while (!st.done) st.step(t, w, emit);
   return st.count;
 }
 
 // Brings the first bytes of the `len`-byte word at p into this lane's LDS window with 16-byte aligned
-// loads (only blocks that overlap the word).
-__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, uint32_t* win)
+// loads (only blocks that overlap the word).  *ascii = no byte of the word has bit 7 set (judged on the
+// whole blocks, so it may be false for a plain word next to other text; never true wrongly).
+__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, uint32_t* win, bool* ascii)
 {
   uint32_t const mis    = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
   const uint4* a        = reinterpret_cast<const uint4*>(p - mis);
-  uint32_t const blocks = min(kStage / 16, (mis + len + 15u) >> 4);
+  uint32_t const need   = (mis + len + 15u) >> 4;
+  uint32_t const blocks = min(kStage / 16, need);
+  uint32_t seen         = 0;
   for (uint32_t i = 0; i < blocks; ++i) {
     uint4 const v = a[i];
+    seen |= v.x | v.y | v.z | v.w;
     win[(4 * i + 0) * kOovThreads] = v.x;
     win[(4 * i + 1) * kOovThreads] = v.y;
     win[(4 * i + 2) * kOovThreads] = v.z;
     win[(4 * i + 3) * kOovThreads] = v.w;
   }
+  *ascii = (seen & 0x80808080u) == 0 && need <= kStage / 16;
   return mis;
 }
 
@@ -776,8 +839,9 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
             q                = mine;
             const uint8_t* p = col.chars + col.off(e.row) + e.delta;
             w.p              = p;
-            w.mis            = stage_word(p, e.len, win);
-            st.begin(w, e.len);
+            bool ascii;
+            w.mis            = stage_word(p, e.len, win, &ascii);
+            st.begin(table, w, e.len, ascii);
             busy = true;
           }
         }
@@ -803,38 +867,45 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
 struct EmitLds {
   uint32_t word_prefix[kWave + 1];  // words before row k of the block
   int64_t slot0[kWave];             // arena slot of word 0 of row k
+  uint32_t first_token[kWave + 1];  // of the 64 words in flight: (token count << 16) | index of the word's first token
+  uint32_t value[kWave];            // their arena values
 };
 
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
                                                                      const uint32_t* __restrict__ arena, const uint8_t* __restrict__ arena_cnt,
                                                                      const int32_t* __restrict__ nwords, const OovEntry* __restrict__ queue,
                                                                      const OovResult* __restrict__ results, const int32_t* __restrict__ offsets,
-                                                                     int32_t* __restrict__ out)
+                                                                     int32_t* __restrict__ out, int block_rows)
 {
+  // block_rows (1..64) rows per wavefront at a time: fewer when rows are long, so that the walks stay
+  // short and there are enough of them to fill the device
   __shared__ EmitLds lds_all[kTokWaves];
   int const lane        = lane_id();
   int const wave        = threadIdx.x / kWave;
   EmitLds& lds          = lds_all[wave];
   int64_t const rows    = col.size;
-  int64_t const nblocks = (rows + kWave - 1) / kWave;
+  int64_t const nblocks = (rows + block_rows - 1) / block_rows;
   int64_t const nwave   = static_cast<int64_t>(gridDim.x) * kTokWaves;
+  auto lds_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
   for (int64_t blk = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave; blk < nblocks; blk += nwave) {
-    int64_t const r  = blk * kWave + lane;
+    int64_t const r  = blk * block_rows + lane;
     uint32_t W       = 0;
     int64_t slot0    = 0;
-    if (r < rows) {
+    if (lane < block_rows && r < rows) {
       W     = static_cast<uint32_t>(nwords[r]);
       slot0 = arena_pos(col, first_offset, r);
     }
-    int32_t const base   = offsets[blk * kWave];
+    int32_t const base   = offsets[blk * block_rows];
     uint32_t const incl  = wave_inclusive_scan(W);
     uint32_t const total = wave_bcast(incl, kWave - 1);
     lds.word_prefix[lane] = incl - W;
     if (lane == kWave - 1) lds.word_prefix[kWave] = total;
     lds.slot0[lane] = slot0;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    lds_sync();
 
     // the arena entry of flat word j: row k = last row with word_prefix[k] <= j (rows without words are skipped
     // because their prefix equals the next row's)
@@ -852,35 +923,56 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
       }
     };
 
-    uint32_t done = 0;  // tokens written so far in this block
-    uint32_t v_nxt, c_nxt;
+    int32_t* const dst = out + base;
+    uint32_t done      = 0;  // tokens written so far in this block
+    uint32_t v_nxt, c_nxt, v_far, c_far;
     locate(lane, v_nxt, c_nxt);
+    locate(kWave + lane, v_far, c_far);
     for (uint32_t j0 = 0; j0 < total; j0 += kWave) {
       uint32_t const value = v_nxt, cnt = c_nxt;
-      locate(j0 + kWave + lane, v_nxt, c_nxt);  // next round's loads are in flight while this one is written
-      bool const active   = j0 + lane < total;
-      bool const oov      = active && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
-      uint32_t const incl2 = wave_inclusive_scan(cnt);
-      if (active) {
-        int32_t* d = out + base + done + (incl2 - cnt);
-        if (!oov) {
-          d[0] = static_cast<int32_t>(value);
-        } else {
-          uint32_t const q = value & ~kOovMark;
-          if (cnt <= kOovKeep) {
-            for (uint32_t k = 0; k < cnt; ++k) d[k] = results[q].tok[k];
-          } else {
+      v_nxt = v_far;
+      c_nxt = c_far;
+      locate(j0 + 2 * kWave + lane, v_far, c_far);  // the loads of the next two rounds are in flight while this one is written
+      uint32_t const here   = min(total - j0, static_cast<uint32_t>(kWave));  // words of this round (every word has >= 1 token)
+      uint32_t const incl2  = wave_inclusive_scan(cnt);
+      uint32_t const tokens = wave_bcast(incl2, kWave - 1);
+      bool const marked     = static_cast<uint32_t>(lane) < here && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
+      if (tokens == here && ballot64(marked) == 0) {
+        // one token per word and none from the queue: the arena values are the tokens
+        if (static_cast<uint32_t>(lane) < here) dst[done + lane] = static_cast<int32_t>(value);
+      } else {
+        // lanes <-> tokens: each finds its word among the 64 by binary search over the words' first-token indices
+        lds.first_token[lane] = (cnt << 16) | (incl2 - cnt);
+        if (lane == kWave - 1) lds.first_token[kWave] = tokens;
+        lds.value[lane] = value;
+        lds_sync();
+        for (uint32_t t = lane; t < tokens; t += kWave) {
+          uint32_t lo = 0;
+#pragma unroll
+          for (uint32_t step = kWave / 2; step > 0; step >>= 1)
+            if ((lds.first_token[lo + step] & 0xFFFFu) <= t) lo += step;
+          uint32_t const ft = lds.first_token[lo];
+          uint32_t const v  = lds.value[lo];
+          uint32_t const k  = t - (ft & 0xFFFFu);
+          uint32_t const c  = ft >> 16;
+          bool const oov    = (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
+          if (!oov) {
+            dst[done + t] = static_cast<int32_t>(v);
+          } else if (c <= kOovKeep) {
+            dst[done + t] = results[v & ~kOovMark].tok[k];
+          } else if (k == 0) {
             // more pieces than a queue entry keeps: tokenize the word again, straight into place
-            OovEntry const e = queue[q];
+            OovEntry const e = queue[v & ~kOovMark];
             const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+            int32_t* d       = dst + done + t;
             tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t jj, int32_t id) { d[jj] = id; });
           }
         }
+        lds_sync();
       }
-      done += wave_bcast(incl2, kWave - 1);
+      done += tokens;
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    lds_sync();
   }
 }
 
@@ -1035,6 +1127,22 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   }
   if (pool.size() > 0xFFFFFFFFull) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
 
+  // length filter over the first three bytes of every key of three bytes and more
+  size_t lens_size = 1024;
+  while (lens_size < 4 * keys) lens_size <<= 1;
+  std::vector<uint32_t> lens(lens_size, 0u);
+  auto note_length = [&](uint32_t kind, const uint8_t* key, uint32_t len) {
+    if (len < 3) return;
+    uint32_t const first3 = key[0] | (uint32_t{key[1]} << 8) | (uint32_t{key[2]} << 16);
+    lens[length_filter_index(kind, first3) & (lens_size - 1)] |= 1u << length_filter_bit(len);
+  };
+  for (int32_t i = 0; i < V; ++i) {
+    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
+    int64_t const len = e - b;
+    if (len >= 1 && len < kMaxWord) note_length(0, pool.data() + b, static_cast<uint32_t>(len));
+    if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') note_length(1, pool.data() + b + 2, static_cast<uint32_t>(len - 2));
+  }
+
   auto* v = new nvtext_amd_wordpiece_vocabulary;
   v->entries = V;
   // wordpiece_tokenize.cu:199-209, 273-275
@@ -1042,14 +1150,16 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   if (unk < 0) unk = host_find(slots, mask, pool, "[unk]");
   v->slot_bytes = capacity * sizeof(HostSlot);
   v->pool_bytes = pool.size() + 16;
-  if (hipMalloc(&v->d_slots, v->slot_bytes) != hipSuccess || hipMalloc(&v->d_pool, v->pool_bytes) != hipSuccess) {
+  if (hipMalloc(&v->d_slots, v->slot_bytes) != hipSuccess || hipMalloc(&v->d_pool, v->pool_bytes) != hipSuccess ||
+      hipMalloc(&v->d_lens, lens.size() * sizeof(uint32_t)) != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
   hipError_t e1 = hipMemcpyAsync(v->d_slots, slots.data(), v->slot_bytes, hipMemcpyHostToDevice, stream);
   hipError_t e2 = pool.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, pool.data(), pool.size(), hipMemcpyHostToDevice, stream);
+  hipError_t e4 = hipMemcpyAsync(v->d_lens, lens.data(), lens.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
   hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
-  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) {
+  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_DEVICE_ERROR, "vocabulary upload failed");
   }
@@ -1059,6 +1169,8 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.unk_id      = unk;
   v->table.max_len[0]  = max_len[0];
   v->table.max_len[1]  = max_len[1];
+  v->table.lens        = static_cast<const uint32_t*>(v->d_lens);
+  v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
   *out            = v;
   return NVTEXT_AMD_SUCCESS;
 }
@@ -1068,6 +1180,7 @@ void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
   if (!v) return;
   if (v->d_slots) (void)hipFree(v->d_slots);
   if (v->d_pool) (void)hipFree(v->d_pool);
+  if (v->d_lens) (void)hipFree(v->d_lens);
   delete v;
 }
 
@@ -1240,12 +1353,16 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
         return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
       }
       ProfileScope ps("wordpiece_emit_kernel", stream);
-      int64_t const emit_blocks = (static_cast<int64_t>(rows) + kWave * kTokWaves - 1) / (kWave * kTokWaves);
+      // about 4096 words (at 5.6 bytes each) per walk
+      int64_t const mean_bytes = (last_offset - first_offset) / rows + 1;
+      int block_rows           = kWave;
+      while (block_rows > 1 && block_rows * mean_bytes > 4096 * 56 / 10) block_rows >>= 1;
+      int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
                          arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
                          out->offsets,
-                         static_cast<int32_t*>(out->child));
+                         static_cast<int32_t*>(out->child), block_rows);
     }
     break;
   }

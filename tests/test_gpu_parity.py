@@ -325,6 +325,48 @@ def test_wordpiece_row_longer_than_chunks(nv, orc):
         assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4), f"long row mw={mw}")
 
 
+def test_wordpiece_long_keys_and_many_pieces(nv, orc):
+    """Keys of 1..60 bytes that share their first bytes (so the per-prefix length filter has several bits,
+    including the one for 34 bytes and more), multi-byte characters at byte 2 and 3 of keys and words,
+    and words that split into more than eight pieces."""
+    rng = np.random.default_rng(2024)
+    base = list("abcé漢😀")
+    vocab = ["[UNK]"] + base + ["##" + c for c in base]
+    seen = set(vocab)
+    heads = ["ab", "aé", "a漢", "é漢", "漢a", "😀", "abc", "b"]
+    while len(vocab) < 1200:
+        n = int(rng.choice([1, 2, 3, 4, 6, 9, 15, 31, 32, 33, 34, 35, 40, 60]))
+        s = heads[int(rng.integers(0, len(heads)))]
+        while len(s.encode()) < n:
+            s += base[int(rng.integers(0, len(base)))]
+        if rng.random() < 0.5:
+            s = "##" + s
+        if s not in seen and len(s.encode()) < 199:
+            seen.add(s)
+            vocab.append(s)
+    keys = [v[2:] if v.startswith("##") else v for v in vocab[1:]]
+    rows = []
+    for _ in range(600):
+        ws = []
+        for _ in range(int(rng.integers(1, 25))):
+            t = rng.random()
+            if t < 0.5:  # several keys glued together: pieces of every length class
+                ws.append("".join(keys[int(rng.integers(0, len(keys)))] for _ in range(int(rng.integers(1, 5)))))
+            elif t < 0.8:  # single letters: one piece per character, often more than eight
+                ws.append("".join(rng.choice(base, int(rng.integers(1, 30)))))
+            else:  # a key cut short or followed by a letter outside the vocabulary
+                k = keys[int(rng.integers(0, len(keys)))]
+                ws.append(k[: max(1, len(k) - int(rng.integers(0, 3)))] + ("z" if rng.random() < 0.5 else ""))
+        rows.append(" ".join(w for w in ws if w))
+    host = strings(rows, np.int32)
+    hv = strings(vocab)
+    for mw in (0, 10):
+        got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
+        exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4)
+        assert_same(got, exp, f"long keys mw={mw}")
+    assert exp.child.size > 5000
+
+
 def test_cpp_api_program():
     """The C++ mirror of the nvtext API (cudf_amd/include) run on the reference's gtest cases."""
     import os
