@@ -108,7 +108,7 @@ constexpr int kGroupLanes   = kWave / kGroups;
 constexpr int kChunk        = 16 * kGroupLanes;  // bytes per group step (16 per lane) = 256
 constexpr int kRing         = 2 * kChunk;        // per group: the current chunk and the one before it
 constexpr int32_t kNone     = std::numeric_limits<int32_t>::min();
-constexpr int kOovKeep      = 8;     // tokens stored per queued word; longer results are redone at emit time
+constexpr int kOovKeep      = 7;     // tokens stored per queued word; longer results are redone at emit time
 constexpr uint32_t kOovMark = 0x80000000u;  // word-arena value 0x80000000 | queue index (never 0xFFFFFFFF = id -1)
 
 struct OovEntry {
@@ -116,10 +116,13 @@ struct OovEntry {
   uint32_t delta;  // byte offset of the word inside its row
   uint32_t widx;   // index of the word inside its row (its word-arena slot)
   uint32_t len;    // bytes in the word (1..199)
+  uint32_t head[4];  // the word's first 16 bytes, zero padded: most words are tokenized without reading the chars again
 };
 struct OovResult {
   int32_t tok[kOovKeep];
+  uint32_t count;  // tokens of the word (may exceed kOovKeep)
 };
+static_assert(sizeof(OovEntry) == 32 && sizeof(OovResult) == 32, "queue records are two 16-byte stores");
 
 // ------------------------------------------------------------------ where candidate keys live
 // Each source offers byte(k) and key8(p, len, &k0, &k1): bytes [p, p+8) as two dwords, zero padded past len.
@@ -420,10 +423,9 @@ __device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return 
 // with lanes <-> words.  The next chunk of every group (the rest of its row, else the start of its next
 // row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
 // For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
-// marker carrying the queue index; arena_cnt[slot] = 1 (the out-of-vocabulary pass overwrites it with the
-// word's token count); nwords[r] = words kept; counts[r] = one per hit.
+// marker carrying the queue index; nwords[r] = words kept; counts[r] = one per hit.
 __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                      uint32_t* __restrict__ arena, uint8_t* __restrict__ arena_cnt,
+                                                                      uint32_t* __restrict__ arena,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
                                                                       OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
                                                                       uint32_t* __restrict__ queue_size)
@@ -594,7 +596,7 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
           // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
           for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-            if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+            if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
           uint32_t base = 0;
           if (lane == 0) base = atomicAdd(queue_size, queue_block);
           q_pos = wave_bcast(base, 0);
@@ -602,7 +604,13 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         }
         if (miss) {
           uint32_t const q = q_pos + lanes_below(mm);
-          if (q < queue_capacity) queue[q] = OovEntry{rw, wstart - misw, wdw + idx, wl};
+          if (q < queue_capacity) {
+            RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
+            OovEntry e{rw, wstart - misw, wdw + idx, wl, {0u, 0u, 0u, 0u}};
+            rw_.key8(0, min(wl, 8u), &e.head[0], &e.head[1]);
+            if (wl > 8) rw_.key8(8, min(wl - 8u, 8u), &e.head[2], &e.head[3]);
+            queue[q] = e;
+          }
           value = kOovMark | q;
         }
         q_pos += nm;
@@ -610,7 +618,6 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
       if (active) {
         int64_t const s = ((ow - first_offset) >> 1) + rw + wdw + idx;
         arena[s]        = value;
-        arena_cnt[s]    = 1;
       }
       uint64_t const hit = ballot64(active && !miss);
       if (hit) {
@@ -632,7 +639,7 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
     __builtin_amdgcn_wave_barrier();
   }
   for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u};
+    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
 }
 
 // ------------------------------------------------------------------ out-of-vocabulary pass
@@ -796,11 +803,10 @@ __device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, u
 // One lane per queued word, and a lane that finishes its word takes the next one: every wavefront owns a
 // contiguous part of the queue and, every fourth trip, lets its idle lanes store their result and pick up
 // new entries, so lanes with short words do not wait for the longest word of a batch.
-// results[q] = the word's first kOovKeep tokens; arena_cnt[slot] = its token count; counts[row] += count.
+// results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count.
 __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
                                                                     const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
-                                                                    int64_t first_offset, OovResult* __restrict__ results,
-                                                                    uint8_t* __restrict__ arena_cnt, int32_t* __restrict__ counts)
+                                                                    OovResult* __restrict__ results, int32_t* __restrict__ counts)
 {
   __shared__ uint32_t windows[kStage / 4][kOovThreads];
   uint32_t* const win   = &windows[0][threadIdx.x];
@@ -816,7 +822,7 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
   StagedWord w{win, nullptr, 0};
   bool busy  = false;  // this lane holds a word (finished or not)
   uint32_t q = 0;
-  OovEntry e{-1, 0, 0, 0};
+  int32_t row = -1;
   int32_t tok[kOovKeep];
   for (uint32_t trip = 0;; ++trip) {
     if ((trip & 3u) == 0) {
@@ -824,9 +830,9 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
         OovResult res;
 #pragma unroll
         for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
+        res.count  = st.count;
         results[q] = res;
-        arena_cnt[((col.off(e.row) - first_offset) >> 1) + e.row + e.widx] = static_cast<uint8_t>(st.count);  // count <= len < 200
-        atomicAdd(&counts[e.row], static_cast<int32_t>(st.count));
+        atomicAdd(&counts[row], static_cast<int32_t>(st.count));
         busy = false;
       }
       uint64_t const idle = ballot64(!busy);
@@ -834,13 +840,23 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
         uint32_t const mine = next + lanes_below(idle);
         next += static_cast<uint32_t>(__builtin_popcountll(idle));
         if (!busy && mine < q_end) {
-          e = queue[mine];
+          OovEntry const e = queue[mine];
           if (e.row >= 0) {  // (-1 marks the unused tail of a reserved queue range)
-            q                = mine;
-            const uint8_t* p = col.chars + col.off(e.row) + e.delta;
-            w.p              = p;
+            q   = mine;
+            row = e.row;
             bool ascii;
-            w.mis            = stage_word(p, e.len, win, &ascii);
+            if (e.len <= 16) {
+              // the queue entry holds the whole word
+              w.p   = nullptr;
+              w.mis = 0;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) win[k * kOovThreads] = e.head[k];
+              ascii = ((e.head[0] | e.head[1] | e.head[2] | e.head[3]) & 0x80808080u) == 0;
+            } else {
+              const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+              w.p              = p;
+              w.mis            = stage_word(p, e.len, win, &ascii);
+            }
             st.begin(table, w, e.len, ascii);
             busy = true;
           }
@@ -872,7 +888,7 @@ struct EmitLds {
 };
 
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
-                                                                     const uint32_t* __restrict__ arena, const uint8_t* __restrict__ arena_cnt,
+                                                                     const uint32_t* __restrict__ arena,
                                                                      const int32_t* __restrict__ nwords, const OovEntry* __restrict__ queue,
                                                                      const OovResult* __restrict__ results, const int32_t* __restrict__ offsets,
                                                                      int32_t* __restrict__ out, int block_rows)
@@ -909,30 +925,31 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
 
     // the arena entry of flat word j: row k = last row with word_prefix[k] <= j (rows without words are skipped
     // because their prefix equals the next row's)
-    auto locate = [&](uint32_t j, uint32_t& value, uint32_t& cnt) {
-      value = 0;
-      cnt   = 0;
-      if (j < total) {
-        uint32_t lo = 0;
+    auto load_value = [&](uint32_t j) -> uint32_t {
+      if (j >= total) return 0u;
+      uint32_t lo = 0;
 #pragma unroll
-        for (uint32_t step = kWave / 2; step > 0; step >>= 1)
-          if (lds.word_prefix[lo + step] <= j) lo += step;
-        int64_t const slot = lds.slot0[lo] + (j - lds.word_prefix[lo]);
-        value              = arena[slot];
-        cnt                = arena_cnt[slot];
-      }
+      for (uint32_t step = kWave / 2; step > 0; step >>= 1)
+        if (lds.word_prefix[lo + step] <= j) lo += step;
+      return arena[lds.slot0[lo] + (j - lds.word_prefix[lo])];
+    };
+    // tokens of flat word j whose arena value is v: one, or what the out-of-vocabulary pass found
+    auto count_of = [&](uint32_t j, uint32_t v) -> uint32_t {
+      if (j >= total) return 0u;
+      return ((v & kOovMark) != 0 && v != 0xFFFFFFFFu) ? results[v & ~kOovMark].count : 1u;
     };
 
     int32_t* const dst = out + base;
     uint32_t done      = 0;  // tokens written so far in this block
-    uint32_t v_nxt, c_nxt, v_far, c_far;
-    locate(lane, v_nxt, c_nxt);
-    locate(kWave + lane, v_far, c_far);
+    // three stages in flight: arena value two rounds ahead, token count one round ahead, the round being written
+    uint32_t v_nxt = load_value(lane);
+    uint32_t v_far = load_value(kWave + lane);
+    uint32_t c_nxt = count_of(lane, v_nxt);
     for (uint32_t j0 = 0; j0 < total; j0 += kWave) {
       uint32_t const value = v_nxt, cnt = c_nxt;
       v_nxt = v_far;
-      c_nxt = c_far;
-      locate(j0 + 2 * kWave + lane, v_far, c_far);  // the loads of the next two rounds are in flight while this one is written
+      c_nxt = count_of(j0 + kWave + lane, v_nxt);
+      v_far = load_value(j0 + 2 * kWave + lane);
       uint32_t const here   = min(total - j0, static_cast<uint32_t>(kWave));  // words of this round (every word has >= 1 token)
       uint32_t const incl2  = wave_inclusive_scan(cnt);
       uint32_t const tokens = wave_bcast(incl2, kWave - 1);
@@ -1289,12 +1306,11 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
   uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
   Temp arena(mr, arena_slots * sizeof(uint32_t));
-  Temp arena_cnt(mr, arena_slots);
   Temp nwords(mr, static_cast<size_t>(rows) * sizeof(int32_t));
   Temp counts(mr, static_cast<size_t>(rows) * sizeof(int32_t));
   Temp scan_tmp(mr, scan_temp_bytes(rows));
   Temp qsize(mr, 256);
-  if (!arena.ok() || !arena_cnt.ok() || !nwords.ok() || !counts.ok() || !scan_tmp.ok() || !qsize.ok()) {
+  if (!arena.ok() || !nwords.ok() || !counts.ok() || !scan_tmp.ok() || !qsize.ok()) {
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
@@ -1312,15 +1328,14 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     {
       ProfileScope ps("wordpiece_probe_kernel", stream);
       hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
-                         first_offset, arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
+                         first_offset, arena.as<uint32_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
                          queue_block, qsize.as<uint32_t>());
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
       hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads))),
                          dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, first_offset, results.as<OovResult>(), arena_cnt.as<uint8_t>(),
-                         counts.as<int32_t>());
+                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>());
     }
     // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
@@ -1360,7 +1375,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
-                         arena.as<uint32_t>(), arena_cnt.as<uint8_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
+                         arena.as<uint32_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
                          out->offsets,
                          static_cast<int32_t*>(out->child), block_rows);
     }
