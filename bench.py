@@ -19,6 +19,17 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+VALU_PEAK_TOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 lanes x 2.4 GHz: one 32-bit integer operation per lane and cycle
+
+# HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload, from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; the commands and
+# raw readings are in profiles/hbm_traffic_pmc_C2_C3_C4.md.  Counters cannot be read from inside this
+# process, so the line reports these figures only for the workload they were measured on.
+MEASURED_TRAFFIC_C2 = {
+    "wordpiece_probe_kernel": (1735_700_000, 1955_600_000),
+    "wordpiece_oov_kernel": (1515_000_000, 1390_600_000),
+    "wordpiece_emit_kernel": (2179_700_000, 848_000_000),
+}
 
 
 def log(*a):
@@ -109,7 +120,9 @@ def main():
     dom_ms = kt[dom]
     achieved = (in_b + out_b) / (dom_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": sum(MEASURED_TRAFFIC_C2[dom]) if args.scale == 1.0 and dom in MEASURED_TRAFFIC_C2 else None,
+                "traffic_all_kernels": ({k: sum(v) for k, v in MEASURED_TRAFFIC_C2.items()} if args.scale == 1.0 else None),
                 "algorithmic_bytes": in_b + out_b, "kernel_ms": round(dom_ms, 4),
                 "all_kernels_ms": {k: round(v, 4) for k, v in kt.items()},
                 "frac_whole_op": round((in_b + out_b) / sec / 1e9 / HBM_PEAK_GBS, 4)}
@@ -163,6 +176,12 @@ def main():
                    "mrows_per_s": round(w.rows.size / msec / 1e6, 3),
                    "gperm_per_s": round(windows * p["P"] / msec / 1e9, 1),
                    "kernels_ms": {k: round(v, 3) for k, v in mk.items()}}
+            # the bound of minhash is VALU issue: algorithmic lane-operations = windows x P x C_perm (2 for uint32:
+            # multiply-add and min; 12 for uint64: three 32x32 multiply-adds, the fold mod 2^61-1, the 64-bit min)
+            c_perm = 2 if p["hash_bits"] == 32 else 12
+            ops = windows * p["P"] * c_perm
+            leg["valu"] = {"algorithmic_ops": ops, "achieved": round(ops / msec / 1e12, 2), "peak": VALU_PEAK_TOPS,
+                           "unit": "T lane-op/s", "frac": round(ops / msec / 1e12 / VALU_PEAK_TOPS, 3)}
             if not args.no_cpu:
                 from oracle import pyoracle as orc
                 n = min(w.rows.size, 20000 if name == "C3" else 2000)

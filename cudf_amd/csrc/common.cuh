@@ -131,6 +131,24 @@ __device__ __forceinline__ int bytes_in_utf8_byte(uint32_t b)
 }
 
 // ------------------------------------------------------------------ wavefront primitives (wave64, DPP)
+// Loads and stores for data that is touched once: the non-temporal hint lets the caches drop these lines
+// first, so that tables which are probed again and again stay resident.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream(const uint4* p)
+{
+  u32x4_t const v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_stream(uint4* p, uint4 v)
+{
+  u32x4_t w;
+  w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+  __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t*>(p));
+}
+__device__ __forceinline__ uint32_t load_stream(const uint32_t* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void store_stream(uint32_t* p, uint32_t v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void store_stream(int32_t* p, int32_t v) { __builtin_nontemporal_store(v, p); }
+
 __device__ __forceinline__ int lane_id() { return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
 
 template <int CTRL, int ROW_MASK>

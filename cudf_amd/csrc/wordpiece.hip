@@ -366,7 +366,7 @@ struct RowCtx {
   {
     uint4 v = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
     if (a0 < aend && a0 + 16 > static_cast<int64_t>(mis)) {
-      v = base[a0 >> 4];
+      v = load_stream(base + (a0 >> 4));
       if (a0 < static_cast<int64_t>(mis) || a0 + 16 > aend) {
         uint32_t d[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -609,7 +609,9 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
             OovEntry e{rw, wstart - misw, wdw + idx, wl, {0u, 0u, 0u, 0u}};
             rw_.key8(0, min(wl, 8u), &e.head[0], &e.head[1]);
             if (wl > 8) rw_.key8(8, min(wl - 8u, 8u), &e.head[2], &e.head[3]);
-            queue[q] = e;
+            uint4* const dst = reinterpret_cast<uint4*>(queue + q);
+            store_stream(dst, make_uint4(static_cast<uint32_t>(e.row), e.delta, e.widx, e.len));
+            store_stream(dst + 1, make_uint4(e.head[0], e.head[1], e.head[2], e.head[3]));
           }
           value = kOovMark | q;
         }
@@ -617,7 +619,7 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
       }
       if (active) {
         int64_t const s = ((ow - first_offset) >> 1) + rw + wdw + idx;
-        arena[s]        = value;
+        store_stream(arena + s, value);
       }
       uint64_t const hit = ballot64(active && !miss);
       if (hit) {
@@ -840,7 +842,12 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
         uint32_t const mine = next + lanes_below(idle);
         next += static_cast<uint32_t>(__builtin_popcountll(idle));
         if (!busy && mine < q_end) {
-          OovEntry const e = queue[mine];
+          OovEntry e;
+          {
+            const uint4* const src = reinterpret_cast<const uint4*>(queue + mine);
+            uint4 const a = load_stream(src), b = load_stream(src + 1);
+            e = OovEntry{static_cast<int32_t>(a.x), a.y, a.z, a.w, {b.x, b.y, b.z, b.w}};
+          }
           if (e.row >= 0) {  // (-1 marks the unused tail of a reserved queue range)
             q   = mine;
             row = e.row;
