@@ -1,0 +1,201 @@
+"""The five benchmark workloads (cudf_amd.datagen.config1..5) as parity cases.
+
+Host part (no GPU): the generator is deterministic and produces the stated shapes, and the oracle runs
+configuration 1 end to end.  GPU part: every configuration at its full size through the C ABI, compared
+bit for bit with the oracle where the oracle finishes in seconds (all of C1, C2 and C5's tokenization,
+row samples of the minhash workloads, the longest rows of C4) and through size-independent properties on
+the whole output: a slice of the input gives the matching slice of the output, a subset of the (a, b)
+parameters gives the matching columns, null rows have no slots, offsets are the expected arithmetic
+progression.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from cudf_amd import datagen
+
+
+def _crc(col):
+    return zlib.crc32(np.ascontiguousarray(col.offsets).tobytes(), zlib.crc32(np.ascontiguousarray(col.chars).tobytes()))
+
+
+# ----------------------------------------------------------------------------- host
+def test_generator_is_deterministic_and_shaped():
+    a = datagen.config2(0.002)
+    b = datagen.config2(0.002)
+    assert _crc(a.rows) == _crc(b.rows) and _crc(a.vocab) == _crc(b.vocab)
+    assert a.rows.size == 8000 and a.rows.offsets.dtype == np.int32 and a.vocab.size == 30522
+    mean = a.rows.chars_bytes / a.rows.size
+    assert 200 < mean < 320
+    c5 = datagen.config5(0.0005)
+    assert c5.rows.offsets.dtype == np.int64 and c5.vocab.size == 250000
+    assert (np.frombuffer(np.ascontiguousarray(c5.rows.chars), np.uint8) >= 0x80).mean() > 0.05  # multi-byte text
+    c4 = datagen.config4(0.02)
+    assert 0.05 < c4.rows.null_count / c4.rows.size < 0.15
+    lens = np.diff(c4.rows.offsets.astype(np.int64))
+    assert lens.max() <= (1 << 20)
+
+
+def test_config1_on_the_oracle():
+    from oracle import pyoracle as orc
+    w = datagen.config1()
+    p = w.params
+    assert w.rows.size == 10000 and w.rows.null_count > 0
+    tok = orc.wordpiece_tokenize(w.rows, orc.Vocabulary(w.vocab), p["max_words_per_row"], nthreads=4)
+    valid = w.rows.validity()
+    lens = np.diff(w.rows.offsets.astype(np.int64))
+    counts = np.diff(tok.offsets.astype(np.int64))
+    # single spaces, no leading or trailing ones: words = spaces + 1, and every word gives at least one token
+    chars = np.frombuffer(np.ascontiguousarray(w.rows.chars), np.uint8)
+    spaces = np.add.reduceat((chars == 0x20).astype(np.int64), np.minimum(w.rows.offsets[:-1].astype(np.int64), chars.size - 1))
+    words = np.where(lens > 0, spaces + 1, 0)
+    assert np.all(counts >= words) and np.all(counts[lens == 0] == 0)
+    assert tok.null_count == w.rows.null_count
+    a, b = datagen.make_params(p["P"], 32, p["param_seed"])
+    mh = orc.minhash(w.rows, p["seed"], a, b, p["width"], nthreads=4)
+    assert mh.child.size == int(valid.sum()) * p["P"]
+    assert np.array_equal(np.diff(mh.offsets), np.where(valid, p["P"], 0))
+
+
+# ----------------------------------------------------------------------------- GPU
+@pytest.fixture(scope="module")
+def nv():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from cudf_amd import nvtext
+    from cudf_amd import _capi
+    _capi.load()
+    return nvtext
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import pyoracle
+    return pyoracle
+
+
+def _same(got, exp, what):
+    assert got.size == exp.size and got.null_count == exp.null_count, what
+    assert np.array_equal(got.validity(), exp.validity()), what
+    assert np.array_equal(got.offsets, exp.offsets), what
+    assert got.child.dtype == exp.child.dtype and np.array_equal(got.child, exp.child), what
+
+
+def _params(nv, p):
+    import torch
+    a, b = datagen.make_params(p["P"], p["hash_bits"], p["param_seed"])
+    signed = np.int32 if p["hash_bits"] == 32 else np.int64
+    return a, b, torch.from_numpy(a.view(signed)).cuda(), torch.from_numpy(b.view(signed)).cuda()
+
+
+def _child(out):
+    """The child of a device list column as a typed tensor."""
+    import torch
+    t = {4: torch.int32, 8: torch.int64}[out.child_dtype.itemsize]
+    return out.child.view(t)[: out.child_size]
+
+
+def _minhash_properties(nv, fn, ofn, w, dcol, da, db, a, b, sample_rows, what):
+    """Checks on a full-size minhash result `fn(dcol, ...)`; returns the device result."""
+    import torch
+    p = w.params
+    P = p["P"]
+    host = w.rows
+    full = fn(dcol, p["seed"], da, db, p["width"])
+    valid = host.validity()
+    assert full.size == host.size and full.null_count == host.null_count
+    assert full.child_size == int(valid.sum()) * P
+    offs = full.offsets.view(torch.int32)[: host.size + 1].cpu().numpy()
+    assert np.array_equal(np.diff(offs), np.where(valid, P, 0)), what + ": offsets"
+    child = _child(full)
+    # exact on row ranges the oracle finishes in seconds
+    for lo, hi in sample_rows:
+        hs = host.slice(lo, hi)
+        exp = ofn(hs, p["seed"], a, b, p["width"], nthreads=16)
+        got = fn(dcol.slice(lo, hi, hs.null_count), p["seed"], da, db, p["width"])
+        _same(got.to_host(), exp, f"{what}: rows {lo}:{hi} against the oracle")
+        # the slice's output is the matching part of the whole output
+        assert torch.equal(_child(got), child[int(offs[lo]): int(offs[hi])]), f"{what}: slice {lo}:{hi} of the whole"
+    # a subset of the parameters gives the matching columns (only meaningful without null rows in between,
+    # so compare through the valid rows' view)
+    k = P // 2 + 3
+    part = fn(dcol, p["seed"], da[5:5 + k].contiguous(), db[5:5 + k].contiguous(), p["width"])
+    nvalid = int(valid.sum())
+    assert torch.equal(_child(part).view(nvalid, k), child.view(nvalid, P)[:, 5:5 + k]), what + ": parameter subset"
+    return full
+
+
+gpu = pytest.mark.gpu
+
+
+@gpu
+def test_config1_end_to_end(nv, orc):
+    w = datagen.config1()
+    p = w.params
+    d = nv.DeviceStringsColumn.from_host(w.rows)
+    got = nv.wordpiece_tokenize(d, nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(w.vocab)), p["max_words_per_row"]).to_host()
+    _same(got, orc.wordpiece_tokenize(w.rows, orc.Vocabulary(w.vocab), p["max_words_per_row"], nthreads=8), "C1 tokenize")
+    a, b, da, db = _params(nv, p)
+    _same(nv.minhash(d, p["seed"], da, db, p["width"]).to_host(), orc.minhash(w.rows, p["seed"], a, b, p["width"], nthreads=8), "C1 minhash")
+
+
+@gpu
+def test_config2_tokenize_full_size(nv, orc):
+    w = datagen.config2()
+    assert w.rows.size == 4_000_000
+    mw = w.params["max_words_per_row"]
+    d = nv.DeviceStringsColumn.from_host(w.rows)
+    got = nv.wordpiece_tokenize(d, nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(w.vocab)), mw).to_host()
+    exp = orc.wordpiece_tokenize(w.rows, orc.Vocabulary(w.vocab), mw, nthreads=16)
+    _same(got, exp, "C2 tokenize, all 4M rows")
+    assert exp.child.size > 150_000_000
+
+
+@gpu
+def test_config3_minhash_full_size(nv, orc):
+    w = datagen.config3()
+    assert w.rows.size == 2_000_000 and w.rows.offsets.dtype == np.int64
+    a, b, da, db = _params(nv, w.params)
+    d = nv.DeviceStringsColumn.from_host(w.rows)
+    _minhash_properties(nv, nv.minhash, orc.minhash, w, d, da, db, a, b, [(0, 8000), (1_234_567, 1_240_000), (1_999_000, 2_000_000)], "C3")
+
+
+@gpu
+def test_config4_minhash64_full_size(nv, orc):
+    w = datagen.config4()
+    assert w.rows.size == 100_000 and w.rows.null_count > 5000
+    lens = np.diff(w.rows.offsets.astype(np.int64))
+    assert lens.max() >= 256 * 1024, "the workload must hold rows past 256 KiB"
+    a, b, da, db = _params(nv, w.params)
+    d = nv.DeviceStringsColumn.from_host(w.rows)
+    longest = [int(i) for i in np.argsort(lens)[-4:]]
+    ranges = [(0, 600), (50_000, 50_400)] + [(i, i + 1) for i in longest]
+    _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, ranges, "C4")
+
+
+@gpu
+def test_config5_utf8_pipeline_full_size(nv, orc):
+    import torch
+    w = datagen.config5()
+    p = w.params
+    assert w.rows.size == 8_000_000 and w.rows.offsets.dtype == np.int64
+    d = nv.DeviceStringsColumn.from_host(w.rows)
+    dv = nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(w.vocab))
+    ov = orc.Vocabulary(w.vocab)
+    full = nv.wordpiece_tokenize(d, dv, p["max_words_per_row"])
+    offs = full.offsets.view(torch.int32)[: w.rows.size + 1].cpu().numpy()
+    assert np.all(np.diff(offs) >= 0) and int(offs[-1]) == full.child_size
+    child = _child(full)
+    # exact against the oracle on row ranges, each also as a slice of the whole
+    for lo, hi in [(0, 1_000_000), (3_999_999, 4_600_001), (7_400_000, 8_000_000)]:
+        hs = w.rows.slice(lo, hi)
+        exp = orc.wordpiece_tokenize(hs, ov, p["max_words_per_row"], nthreads=16)
+        got = nv.wordpiece_tokenize(d.slice(lo, hi, hs.null_count), dv, p["max_words_per_row"])
+        _same(got.to_host(), exp, f"C5 tokenize rows {lo}:{hi}")
+        assert torch.equal(_child(got), child[int(offs[lo]): int(offs[hi])]), f"C5 tokenize: slice {lo}:{hi} of the whole"
+        assert np.array_equal(exp.offsets.astype(np.int64) + int(offs[lo]), offs[lo: hi + 1].astype(np.int64))
+    del full, child
+    torch.cuda.empty_cache()
+    a, b, da, db = _params(nv, p)
+    _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, [(0, 20_000), (6_000_000, 6_010_000)], "C5 minhash64")
