@@ -80,7 +80,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--scale", type=float, default=1.0, help="row-count multiplier of the headline workload (1.0 = 4M rows)")
-    ap.add_argument("--minhash-scale", type=float, default=0.25, help="row-count multiplier of the C3/C4 minhash legs (0 = skip)")
+    ap.add_argument("--minhash-scale", type=float, default=1.0, help="row-count multiplier of the C3/C4/C5 legs (0 = skip)")
     ap.add_argument("--cpu-sample-rows", type=int, default=4_000_000, help="rows of the workload given to the host oracle")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -198,6 +198,56 @@ def main():
             log(f"[bench] {name}: {leg}")
             extra["minhash" if name == "C3" else "minhash64"] = leg
             del dc, keep
+
+    # ------------------------------------------------------------------ C5: UTF-8 rows, int64 offsets, 250k vocabulary
+    if args.minhash_scale > 0:
+        torch.cuda.empty_cache()
+        t0 = time.time()
+        w = datagen.config5(args.minhash_scale)
+        p = w.params
+        log(f"[bench] C5 generated: rows={w.rows.size} chars={w.rows.chars_bytes / 1e9:.3f} GB in {time.time() - t0:.1f}s")
+        dc = nvtext.DeviceStringsColumn.from_host(w.rows)
+        dv5 = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(w.vocab))
+        keep = {}
+
+        def tstep():
+            keep["o"] = nvtext.wordpiece_tokenize(dc, dv5, p["max_words_per_row"])
+
+        tsec = timed_steps(tstep, max(3, args.steps // 2), 1, torch)
+        tk = kernel_times(tstep, 2, _capi, torch)
+        ib = input_bytes(w.rows)
+        leg = {"workload": f"C5 x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes, "offsets": "int64",
+               "vocab_entries": w.vocab.size,
+               "tokenize": {"ms_per_step": round(tsec * 1e3, 3), "input_GBps": round(ib / tsec / 1e9, 2),
+                            "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": keep["o"].child_size,
+                            "kernels_ms": {k: round(v, 3) for k, v in tk.items()}}}
+        keep.clear()
+        a, b = datagen.make_params(p["P"], 64, p["param_seed"])
+        da = torch.from_numpy(a.view(np.int64)).cuda()
+        db = torch.from_numpy(b.view(np.int64)).cuda()
+
+        def m5step():
+            keep["o"] = nvtext.minhash64(dc, p["seed"], da, db, p["width"])
+
+        msec = timed_steps(m5step, max(3, args.steps // 2), 1, torch)
+        mk = kernel_times(m5step, 2, _capi, torch)
+        leg["minhash64"] = {"ms_per_step": round(msec * 1e3, 3), "input_GBps": round(ib / msec / 1e9, 2),
+                            "mrows_per_s": round(w.rows.size / msec / 1e6, 3), "kernels_ms": {k: round(v, 3) for k, v in mk.items()}}
+        if not args.no_cpu:
+            from oracle import pyoracle as orc
+            n = min(w.rows.size, 400_000)
+            smp = w.rows.slice(0, n)
+            threads = max(1, min(orc.hardware_threads(), 16))
+            t0 = time.perf_counter()
+            exp = orc.wordpiece_tokenize(smp, orc.Vocabulary(w.vocab), p["max_words_per_row"], nthreads=threads)
+            cs = time.perf_counter() - t0
+            got = nvtext.wordpiece_tokenize(dc.slice(0, n, smp.null_count), dv5, p["max_words_per_row"]).to_host()
+            leg["tokenize"]["cpu_baseline"] = {"value": round(input_bytes(smp) / cs / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+                                               "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB), {cs:.2f} s"}
+            leg["tokenize"]["parity"] = "PASS" if got.equals(exp) else "FAIL"
+        log(f"[bench] C5: {leg}")
+        extra["utf8_pipeline"] = leg
+        del dc, keep
 
     line = {
         "metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline",
