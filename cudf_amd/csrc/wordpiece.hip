@@ -802,81 +802,277 @@ __device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, u
   return mis;
 }
 
+// Bit 7 of every byte of x that is a UTF-8 continuation byte (10xxxxxx); exact, no carries cross bytes.
+__device__ __forceinline__ uint32_t continuation_bytes(uint32_t x)
+{
+  uint32_t const t = (x & 0xC0C0C0C0u) ^ 0x80808080u;
+  return ~(((t & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | t) & 0x80808080u;
+}
+
+// The rest of a word of at most 16 bytes, held in registers from the piece being searched on: the whole
+// greedy longest-match-first rule (cpp/src/text/wordpiece_tokenize.cu:349-407) becomes bit operations
+// on a mask of candidate lengths, with no loop over bytes and no memory but the table reads.
+struct ShortWord {
+  uint32_t r[4];   // bytes [start, start + 16) of the word, zero padded
+  uint32_t rem;    // bytes from start to the end of the word
+  uint32_t bnd;    // bit i: start + i is a character boundary (bit rem is set)
+  uint32_t cand;   // lengths still to try for the piece at start (bit l - 1), longest first
+  uint32_t count;  // tokens so far
+  bool done;
+
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const
+  {
+    uint32_t const d = k >> 2;
+    uint32_t const v = d == 0 ? r[0] : d == 1 ? r[1] : d == 2 ? r[2] : r[3];
+    return (v >> (8 * (k & 3u))) & 0xffu;
+  }
+  __device__ __forceinline__ void key8(uint32_t p, uint32_t len, uint32_t* k0, uint32_t* k1) const
+  {
+    // only called with p = 8 by the generic probe code (keys of 9 to 16 bytes)
+    uint32_t lo = p == 0 ? r[0] : r[2], hi = p == 0 ? r[1] : r[3];
+    trim_key8(len, lo, hi);
+    *k0 = lo;
+    *k1 = hi;
+  }
+
+  // Candidate lengths of the piece at start: on a character boundary, no longer than the rest of the word
+  // or the longest key, and not ruled out by the length filter of the piece's first three bytes.
+  __device__ __forceinline__ void open_piece(VocabTable const& t, uint32_t kind)
+  {
+    uint32_t const lens = rem >= 3 ? t.lens[length_filter_index(kind, r[0] & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
+    uint32_t const lim  = min(min(rem, t.max_len[kind]), 16u);
+    cand                = (bnd >> 1) & ((1u << lim) - 1u) & ((lens << 2) | 3u);
+  }
+
+  __device__ __forceinline__ void begin(VocabTable const& t, const uint32_t (&head)[4], uint32_t len)
+  {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = head[k];
+    rem   = len;
+    count = 0;
+    done  = false;
+    uint32_t const cont = gather_byte_flags(continuation_bytes(r[0])) | (gather_byte_flags(continuation_bytes(r[1])) << 4) |
+                          (gather_byte_flags(continuation_bytes(r[2])) << 8) | (gather_byte_flags(continuation_bytes(r[3])) << 12);
+    bnd = (~cont & ((1u << len) - 1u)) | (1u << len);
+    open_piece(t, 0);
+    cand &= ~(1u << (len - 1));  // the whole word is known to be absent
+  }
+
+  __device__ __forceinline__ Probe probe_of(VocabTable const& t, uint32_t kind, uint32_t l) const
+  {
+    Probe pr;
+    pr.k0 = r[0];
+    pr.k1 = r[1];
+    trim_key8(min(l, 8u), pr.k0, pr.k1);
+    uint32_t h  = key_hash_block(key_hash_init(l), pr.k0, pr.k1);
+    uint32_t k2 = r[2], k3 = r[3];
+    trim_key8(l > 8 ? l - 8u : 0u, k2, k3);
+    uint32_t const h2 = key_hash_block(h, k2, k3);
+    h                 = l > 8 ? h2 : h;
+    uint32_t b;
+    pr.want   = slot_word0(h, kind, l, &b);
+    pr.bucket = b & t.bucket_mask;
+    return pr;
+  }
+
+  // Drops the first l bytes (a matched piece).
+  __device__ __forceinline__ void advance(uint32_t l)
+  {
+    uint32_t const d  = l >> 2;
+    uint32_t const sh = (l & 3u) * 8u;
+    uint32_t const t0 = d == 0 ? r[0] : d == 1 ? r[1] : d == 2 ? r[2] : r[3];
+    uint32_t const t1 = d == 0 ? r[1] : d == 1 ? r[2] : d == 2 ? r[3] : 0u;
+    uint32_t const t2 = d == 0 ? r[2] : d == 1 ? r[3] : 0u;
+    uint32_t const t3 = d == 0 ? r[3] : 0u;
+    r[0] = __builtin_amdgcn_alignbit(t1, t0, sh);
+    r[1] = __builtin_amdgcn_alignbit(t2, t1, sh);
+    r[2] = __builtin_amdgcn_alignbit(t3, t2, sh);
+    r[3] = t3 >> sh;
+    rem -= l;
+    bnd >>= l;
+  }
+
+  // What the two home slots say about a candidate of l bytes without any further memory access:
+  // 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or the
+  // bucket is full and the search goes on in the next one: both rare).  Straight-line code.
+  static __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
+  {
+    bool const tag0  = s0.x == pr.want, tag1 = s1.x == pr.want;
+    bool const is0   = tag0 && s0.z == pr.k0 && s0.w == pr.k1;
+    bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
+    bool const small = l <= 8;
+    bool const found = small && (is0 || is1);
+    bool const more  = (!small && (tag0 || tag1)) || (!found && s0.x != 0 && s1.x != 0);
+    *id              = static_cast<int32_t>(is0 ? s0.y : s1.y);
+    return found ? 1u : more ? 2u : 0u;
+  }
+
+  // Examines the two longest remaining candidates (their table reads are in flight together).
+  template <typename Emit>
+  __device__ __forceinline__ void step(VocabTable const& t, Emit&& emit)
+  {
+    uint32_t const kind = count ? 1u : 0u;
+    bool const none     = cand == 0;
+    uint32_t const c1   = none ? 1u : cand;
+    uint32_t const la   = 32u - static_cast<uint32_t>(__builtin_clz(c1));
+    uint32_t const rest = c1 ^ (1u << (la - 1));
+    bool const has_b    = rest != 0;
+    uint32_t const lb   = has_b ? 32u - static_cast<uint32_t>(__builtin_clz(rest)) : 1u;
+    Probe const pa      = probe_of(t, kind, la);
+    Probe const pb      = probe_of(t, kind, lb);
+    uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
+    uint4 const b0 = t.slots[2 * pb.bucket], b1 = t.slots[2 * pb.bucket + 1];
+    int32_t ida, idb;
+    uint32_t va = verdict(pa, a0, a1, la, &ida);
+    uint32_t vb = verdict(pb, b0, b1, lb, &idb);
+    if (va == 2u || (va == 0u && has_b && vb == 2u)) {
+      // the general lookup (keys in the pool, overflowing buckets)
+      if (va == 2u) {
+        ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
+        va  = ida == kNone ? 0u : 1u;
+      }
+      if (va == 0u && vb == 2u) {
+        idb = finish_probe(t, pb, b0, b1, *this, 0u, lb);
+        vb  = idb == kNone ? 0u : 1u;
+      }
+    }
+    bool const hit_a   = !none && va == 1u;
+    bool const hit_b   = !none && !hit_a && has_b && vb == 1u;
+    bool const hit     = hit_a || hit_b;
+    uint32_t const len = hit_a ? la : lb;
+    // no candidate left: no prefix of the word matched (375-379), or a later piece has no match and the word
+    // collapses (396-404): either way a single unknown token
+    bool const unknown = none || (!hit && !has_b) || (!hit && (rest ^ (1u << (lb - 1))) == 0);
+    if (hit || unknown) emit(unknown ? 0u : count, unknown ? t.unk_id : (hit_a ? ida : idb));
+    count = unknown ? 1u : count + (hit ? 1u : 0u);
+    done  = unknown || (hit && len == rem);
+    cand  = has_b ? rest ^ (1u << (lb - 1)) : 0u;  // after two misses
+    if (hit && !done) {
+      advance(len);  // next piece: the rest of the word (381-395)
+      open_piece(t, 1);
+    }
+  }
+};
+
 // One lane per queued word, and a lane that finishes its word takes the next one: every wavefront owns a
 // contiguous part of the queue and, every fourth trip, lets its idle lanes store their result and pick up
-// new entries, so lanes with short words do not wait for the longest word of a batch.
+// new entries, so lanes with short words do not wait for the longest word of a batch.  Words of up to 16
+// bytes (whole in their queue record) run in registers; the few longer ones are set aside for the kernel
+// below: their queue indices go to longer[first entry of the part ...], their number to
+// longer[queue_capacity + wavefront].
 // results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count.
 __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
                                                                     const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
-                                                                    OovResult* __restrict__ results, int32_t* __restrict__ counts)
+                                                                    OovResult* __restrict__ results, int32_t* __restrict__ counts,
+                                                                    uint32_t* __restrict__ longer)
 {
-  __shared__ uint32_t windows[kStage / 4][kOovThreads];
-  uint32_t* const win   = &windows[0][threadIdx.x];
   uint32_t const total  = min(*queue_size, queue_capacity);
   uint32_t const nwave  = gridDim.x * (kOovThreads / kWave);
   uint32_t const wave   = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
   uint32_t const chunk  = (total + nwave - 1) / nwave;
-  uint32_t next         = min(total, wave * chunk);          // wave-uniform cursor into this wavefront's part
-  uint32_t const q_end  = min(total, next + chunk);
+  uint32_t const q_begin = min(total, wave * chunk);
+  uint32_t next          = q_begin;                          // wave-uniform cursor into this wavefront's part
+  uint32_t const q_end   = min(total, next + chunk);
+  uint32_t n_longer      = 0;                                // entries of this part set aside (wave-uniform)
+  int const lane         = lane_id();
 
-  OovStepper<StagedWord> st;
-  st.done = true;
-  StagedWord w{win, nullptr, 0};
-  bool busy  = false;  // this lane holds a word (finished or not)
-  uint32_t q = 0;
-  int32_t row = -1;
   int32_t tok[kOovKeep];
-  for (uint32_t trip = 0;; ++trip) {
-    if ((trip & 3u) == 0) {
-      if (busy && st.done) {  // deliver
-        OovResult res;
+  auto keep_token = [&](uint32_t j, int32_t id) {
 #pragma unroll
-        for (int k = 0; k < kOovKeep; ++k) res.tok[k] = tok[k];
-        res.count  = st.count;
-        results[q] = res;
-        atomicAdd(&counts[row], static_cast<int32_t>(st.count));
-        busy = false;
-      }
-      uint64_t const idle = ballot64(!busy);
-      if (idle != 0 && next < q_end) {  // refill
-        uint32_t const mine = next + lanes_below(idle);
-        next += static_cast<uint32_t>(__builtin_popcountll(idle));
-        if (!busy && mine < q_end) {
-          OovEntry e;
-          {
+    for (int k = 0; k < kOovKeep; ++k)
+      if (j == static_cast<uint32_t>(k)) tok[k] = id;
+  };
+  auto deliver = [&](uint32_t q, int32_t row, uint32_t count) {
+    uint4* const dst = reinterpret_cast<uint4*>(results + q);
+    store_stream(dst, make_uint4(static_cast<uint32_t>(tok[0]), static_cast<uint32_t>(tok[1]), static_cast<uint32_t>(tok[2]), static_cast<uint32_t>(tok[3])));
+    store_stream(dst + 1, make_uint4(static_cast<uint32_t>(tok[4]), static_cast<uint32_t>(tok[5]), static_cast<uint32_t>(tok[6]), count));
+    atomicAdd(&counts[row], static_cast<int32_t>(count));
+  };
+
+  {
+    ShortWord sw;
+    sw.done    = true;
+    bool busy  = false;  // this lane holds a word (finished or not)
+    uint32_t q = 0;
+    int32_t row = -1;
+    for (uint32_t trip = 0;; ++trip) {
+      if ((trip & 3u) == 0) {
+        if (busy && sw.done) {
+          deliver(q, row, sw.count);
+          busy = false;
+        }
+        uint64_t const idle = ballot64(!busy);
+        if (idle != 0 && next < q_end) {  // refill
+          uint32_t const mine = next + lanes_below(idle);
+          next += static_cast<uint32_t>(__builtin_popcountll(idle));
+          bool is_longer = false;
+          if (!busy && mine < q_end) {
             const uint4* const src = reinterpret_cast<const uint4*>(queue + mine);
             uint4 const a = load_stream(src), b = load_stream(src + 1);
-            e = OovEntry{static_cast<int32_t>(a.x), a.y, a.z, a.w, {b.x, b.y, b.z, b.w}};
-          }
-          if (e.row >= 0) {  // (-1 marks the unused tail of a reserved queue range)
-            q   = mine;
-            row = e.row;
-            bool ascii;
-            if (e.len <= 16) {
-              // the queue entry holds the whole word
-              w.p   = nullptr;
-              w.mis = 0;
-#pragma unroll
-              for (int k = 0; k < 4; ++k) win[k * kOovThreads] = e.head[k];
-              ascii = ((e.head[0] | e.head[1] | e.head[2] | e.head[3]) & 0x80808080u) == 0;
-            } else {
-              const uint8_t* p = col.chars + col.off(e.row) + e.delta;
-              w.p              = p;
-              w.mis            = stage_word(p, e.len, win, &ascii);
+            if (static_cast<int32_t>(a.x) >= 0) {  // (-1 marks the unused tail of a reserved queue range)
+              if (a.w <= 16) {
+                q   = mine;
+                row = static_cast<int32_t>(a.x);
+                uint32_t const head[4] = {b.x, b.y, b.z, b.w};
+                sw.begin(table, head, a.w);
+                busy = true;
+              } else {
+                is_longer = true;
+              }
             }
-            st.begin(table, w, e.len, ascii);
-            busy = true;
+          }
+          uint64_t const lm = ballot64(is_longer);
+          if (lm != 0) {
+            if (is_longer) longer[q_begin + n_longer + lanes_below(lm)] = mine;
+            n_longer += static_cast<uint32_t>(__builtin_popcountll(lm));
           }
         }
+        if (ballot64(busy) == 0 && next >= q_end) break;
       }
-      if (ballot64(busy) == 0 && next >= q_end) break;
+      if (busy && !sw.done) sw.step(table, keep_token);
     }
-    if (busy && !st.done) {
-      st.step(table, w, [&](uint32_t j, int32_t id) {
+  }
+
+  if (lane == 0) longer[queue_capacity + wave] = n_longer;
+}
+
+// The queued words of more than 16 bytes, which the kernel above has set aside (same grid, same parts):
+// one lane per word, bytes staged from the chars into the lane's LDS window, the general state machine.
+__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
+                                                                         const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
+                                                                         OovResult* __restrict__ results, int32_t* __restrict__ counts,
+                                                                         const uint32_t* __restrict__ longer)
+{
+  __shared__ uint32_t windows[kStage / 4][kOovThreads];
+  uint32_t* const win    = &windows[0][threadIdx.x];
+  uint32_t const total   = min(*queue_size, queue_capacity);
+  uint32_t const nwave   = gridDim.x * (kOovThreads / kWave);
+  uint32_t const wave    = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
+  uint32_t const chunk   = (total + nwave - 1) / nwave;
+  uint32_t const q_begin = min(total, wave * chunk);
+  uint32_t const n_longer = longer[queue_capacity + wave];
+  uint32_t const lane    = static_cast<uint32_t>(lane_id());
+  for (uint32_t base = 0; base < n_longer; base += kWave) {
+    if (base + lane < n_longer) {
+      uint32_t const q = longer[q_begin + base + lane];
+      OovEntry const e = queue[q];
+      const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+      bool ascii;
+      StagedWord w{win, p, 0};
+      w.mis = stage_word(p, e.len, win, &ascii);
+      OovResult res;
+      OovStepper<StagedWord> st;
+      st.begin(table, w, e.len, ascii);
+      while (!st.done) {
+        st.step(table, w, [&](uint32_t j, int32_t id) {
 #pragma unroll
-        for (int k = 0; k < kOovKeep; ++k)
-          if (j == static_cast<uint32_t>(k)) tok[k] = id;
-      });
+          for (int k = 0; k < kOovKeep; ++k)
+            if (j == static_cast<uint32_t>(k)) res.tok[k] = id;
+        });
+      }
+      res.count  = st.count;
+      results[q] = res;
+      atomicAdd(&counts[e.row], static_cast<int32_t>(st.count));
     }
   }
 }
@@ -1310,6 +1506,8 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   // Each wavefront reserves queue entries `queue_block` at a time (one atomic per block).
   uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
   uint32_t queue_block = 64;
+  // (atomics on one address are slow: about 150 M/s, so blocks are kept large even though the unused tail of
+  // each wavefront's last block, half a block on average, then makes up a tenth or more of the queue)
   while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
   uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
   Temp arena(mr, arena_slots * sizeof(uint32_t));
@@ -1327,7 +1525,10 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     uint32_t const qcap = static_cast<uint32_t>(queue_capacity);
     Temp queue(mr, static_cast<size_t>(qcap) * sizeof(OovEntry));
     Temp results(mr, static_cast<size_t>(qcap) * sizeof(OovResult));
-    if (!queue.ok() || !results.ok()) {
+    // queue indices of the words of more than 16 bytes, then one count per wavefront of the out-of-vocabulary pass
+    int64_t const oov_blocks = resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads);
+    Temp longer(mr, (static_cast<size_t>(qcap) + static_cast<size_t>(oov_blocks) * (kOovThreads / kWave)) * sizeof(uint32_t));
+    if (!queue.ok() || !results.ok() || !longer.ok()) {
       nvtext_amd_list_column_free(out, stream_, mr_);
       return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
     }
@@ -1340,9 +1541,13 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads))),
-                         dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>());
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
+                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>(), longer.as<uint32_t>());
+    }
+    {
+      ProfileScope ps("wordpiece_oov_long_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
+                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>(), longer.as<uint32_t>());
     }
     // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
