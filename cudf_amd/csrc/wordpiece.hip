@@ -54,7 +54,8 @@ __host__ __device__ __forceinline__ uint32_t key_hash_block(uint32_t h, uint32_t
 
 // slot.x = (tag23 << 9) | (kind << 8) | len   (0 = empty; len in 1..199)
 // slot.y = token id
-// slot.z, slot.w = the key itself when len <= 8 (zero padded), else (offset into the pool, 0)
+// slot.z, slot.w = the key itself when len <= 8 (zero padded), else (byte offset of the key in the pool, 0);
+// the pool holds the keys of more than 8 bytes, each zero padded to a multiple of 8 at an 8-byte aligned offset
 // Bucket b = slots[2b], slots[2b+1]; a bucket fills slot 0 first, overflow goes to the next bucket.
 struct VocabTable {
   const uint4* slots;
@@ -128,9 +129,10 @@ static_assert(sizeof(OovEntry) == 32 && sizeof(OovResult) == 32, "queue records 
 // Each source offers byte(k) and key8(p, len, &k0, &k1): bytes [p, p+8) as two dwords, zero padded past len.
 __device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& hi)
 {
-  if (len < 4) lo &= (1u << (8 * len)) - 1u;
-  if (len <= 4) hi = 0;
-  else if (len < 8) hi &= (1u << (8 * (len - 4))) - 1u;
+  // keep bytes [0, len) of the eight (selects, no branches)
+  uint32_t const nlo = min(len, 4u), nhi = max(min(len, 8u), 4u) - 4u;
+  lo &= nlo >= 4 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << (8 * nlo));
+  hi &= nhi >= 4 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << (8 * nhi));
 }
 
 // A word inside a group's 512-byte LDS ring of the probe pass: byte k of the word is ring byte (start + k) & 511.
@@ -149,6 +151,17 @@ struct RingWord {
     trim_key8(len, lo, hi);
     *k0 = lo;
     *k1 = hi;
+  }
+  // bytes [0, 16) of the word, untrimmed
+  __device__ __forceinline__ void head16(uint32_t (&k)[4]) const
+  {
+    uint32_t const i  = start >> 2;
+    uint32_t const sh = (start & 3u) * 8u;
+    uint32_t d[5];
+#pragma unroll
+    for (uint32_t j = 0; j < 5; ++j) d[j] = ring[(i + j) & (kRing / 4 - 1)];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) k[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
   }
 };
 
@@ -250,10 +263,14 @@ __device__ __forceinline__ Probe make_probe(VocabTable const& t, uint32_t kind, 
 template <typename W>
 __device__ __forceinline__ bool pool_key_equal(VocabTable const& t, uint32_t pool_off, W const& w, uint32_t p, uint32_t len)
 {
-  const uint8_t* e = t.pool + pool_off;
-  uint32_t i       = 0;
-  while (i < len && e[i] == w.byte(p + i)) ++i;
-  return i == len;
+  const uint2* e = reinterpret_cast<const uint2*>(t.pool + pool_off);
+  for (uint32_t done = 0; done < len; done += 8) {
+    uint32_t k0, k1;
+    w.key8(p + done, len - done, &k0, &k1);
+    uint2 const v = e[done >> 3];
+    if (v.x != k0 || v.y != k1) return false;
+  }
+  return true;
 }
 
 // Examines one slot: 1 = it holds the key (id set), 0 = it is empty (the key is absent), -1 = look further.
@@ -312,6 +329,21 @@ __device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W 
   return finish_probe(t, pr, s0, s1, w, p, len);
 }
 
+// What the two home slots say about a key of l bytes without any further memory access:
+// 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or the
+// bucket is full and the search goes on in the next one: both rare).  Straight-line code.
+__device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
+{
+  bool const tag0  = s0.x == pr.want, tag1 = s1.x == pr.want;
+  bool const is0   = tag0 && s0.z == pr.k0 && s0.w == pr.k1;
+  bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
+  bool const small = l <= 8;
+  bool const found = small && (is0 || is1);
+  bool const more  = (!small && (tag0 || tag1)) || (!found && s0.x != 0 && s1.x != 0);
+  *id              = static_cast<int32_t>(is0 ? s0.y : s1.y);
+  return found ? 1u : more ? 2u : 0u;
+}
+
 // ------------------------------------------------------------------ wavefront helpers of the probe pass
 template <int CTRL, int ROW_MASK, int OLD>
 __device__ __forceinline__ uint32_t dpp_old(uint32_t v)
@@ -351,41 +383,35 @@ __device__ __forceinline__ uint32_t gather_byte_flags(uint32_t z) { return (((z 
 __device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
 
 struct ProbeLds {
-  alignas(16) uint32_t bytes[kGroups][kRing / 4];  // per group: row bytes (everything outside the row is ' ')
-  uint16_t wend[kGroups * kChunk / 2 + 2];         // per word ending in this step: offset of its last byte inside its group's chunk
-  uint16_t wlen[kGroups * kChunk / 2 + 2];         // and its length in bytes, clamped to kMaxWord
+  alignas(16) uint32_t bytes[kGroups][kRing / 4];  // per group: the bytes of the current chunk and the one before it, as in memory
+  uint32_t word[kGroups * kChunk / 2 + 2];         // per word ending in this step: (length, clamped to kMaxWord) << 16 | offset of its last byte in the chunk
+  alignas(16) uint32_t group[kGroups][8];          // per group: first word slot, words that count, chunk base, words so far, row start in its block, row, arena slot of the row
 };
 
-// Where a row sits relative to 16-byte aligned memory.  Coordinates count bytes from `base`.
+// Where a row sits relative to 16-byte aligned memory.  Coordinates count bytes from `base` and fit 32 bits
+// (a row is below 2 GiB).
 struct RowCtx {
   const uint4* base;  // aligned address at or below the row's first byte
   uint32_t mis;       // row start inside that block
-  int64_t aend;       // row end (mis + row bytes)
-  // 16 bytes at coordinate a0 (a multiple of 16) with every byte outside the row replaced by ' '
-  __device__ __forceinline__ uint4 load_clean(int64_t a0) const
+  uint32_t aend;      // row end (mis + row bytes)
+  // the 16 bytes at coordinate a0 (a multiple of 16) as they are in memory, if any of them belongs to the row
+  __device__ __forceinline__ uint4 load_raw(uint32_t a0) const
   {
-    uint4 v = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
-    if (a0 < aend && a0 + 16 > static_cast<int64_t>(mis)) {
-      v = load_stream(base + (a0 >> 4));
-      if (a0 < static_cast<int64_t>(mis) || a0 + 16 > aend) {
-        uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          int64_t const b0 = a0 + 4 * j;
-          uint32_t keep    = 0xFFFFFFFFu;
-          if (b0 < static_cast<int64_t>(mis)) keep = b0 + 4 <= static_cast<int64_t>(mis) ? 0u : keep << (8 * static_cast<uint32_t>(mis - b0));
-          if (b0 + 4 > aend) keep = b0 >= aend ? 0u : keep & ((1u << (8 * static_cast<uint32_t>(aend - b0))) - 1u);
-          d[j] = (d[j] & keep) | (0x20202020u & ~keep);
-        }
-        v = make_uint4(d[0], d[1], d[2], d[3]);
-      }
-    }
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (a0 < aend && a0 + 16 > mis) v = load_stream(base + (a0 >> 4));
     return v;
   }
-  // the byte at coordinate a (any alignment); ' ' outside the row
-  __device__ __forceinline__ uint32_t byte_at(int64_t a) const
+  // which of the 16 bytes at coordinate a0 belong to the row (bit k = byte a0 + k)
+  __device__ __forceinline__ uint32_t inside(uint32_t a0) const
   {
-    if (a < static_cast<int64_t>(mis) || a >= aend) return 0x20u;
+    uint32_t const lo = mis > a0 ? min(mis - a0, 16u) : 0u;
+    uint32_t const hi = aend > a0 ? min(aend - a0, 16u) : 0u;
+    return ((1u << hi) - 1u) & ~((1u << lo) - 1u);
+  }
+  // the byte at coordinate a (any alignment); ' ' outside the row
+  __device__ __forceinline__ uint32_t byte_at(uint32_t a) const
+  {
+    if (a < mis || a >= aend) return 0x20u;
     return reinterpret_cast<const uint8_t*>(base)[a];
   }
 };
@@ -396,7 +422,7 @@ __device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, in
   RowCtx c;
   c.mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u);
   c.base = reinterpret_cast<const uint4*>(row - c.mis);
-  c.aend = static_cast<int64_t>(c.mis) + n;
+  c.aend = c.mis + static_cast<uint32_t>(n);
   return c;
 }
 
@@ -442,50 +468,54 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
   int64_t const stride = static_cast<int64_t>(gridDim.x) * kTokWaves * kGroups;  // rows between two rows of a group
   uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
 
+  // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
+  // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
+  auto word_cap = [&](int64_t row, int64_t bytes) -> uint32_t {
+    if (max_words <= 0) return static_cast<uint32_t>(std::numeric_limits<int32_t>::max());
+    return col.valid(row) ? static_cast<uint32_t>(min(static_cast<int64_t>(max_words), bytes / 2)) : 0u;
+  };
+
   // ---- per-group state (the same value in all 16 lanes of a group)
   int64_t r = (static_cast<int64_t>(blockIdx.x) * kTokWaves + wave) * kGroups + g;
   int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
+  uint32_t cap = 0;
   if (r < rows) {
     o_cur = col.off(r);
     e_cur = col.off(r + 1);
+    cap   = word_cap(r, e_cur - o_cur);
   }
   if (r + stride < rows) {
     o_nxt = col.off(r + stride);
     e_nxt = col.off(r + stride + 1);
   }
   RowCtx ctx       = make_row_ctx(col, o_cur, e_cur - o_cur);
-  int64_t cbase    = 0;
+  uint32_t cbase   = 0;
   uint32_t wdone   = 0;     // words kept so far in this row
   uint32_t hits    = 0;     // of which found in the vocabulary
   uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
   uint32_t prev_space  = 1; // the byte before the chunk is a space (or the row starts here)
   // the chunk about to be processed: my sixteen bytes and (last lane of the group) the byte after the chunk
-  uint4 mine_cur    = make_uint4(0x20202020u, 0x20202020u, 0x20202020u, 0x20202020u);
+  uint4 mine_cur    = make_uint4(0u, 0u, 0u, 0u);
   uint32_t tail_cur = 0x20u;
   if (r < rows) {
-    mine_cur = ctx.load_clean(16 * gl);
+    mine_cur = ctx.load_raw(16 * gl);
     if (gl == kGroupLanes - 1) tail_cur = ctx.byte_at(kChunk);
   }
 
   while (ballot64(r < rows) != 0) {
-    bool const has_row = r < rows;
-    // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
-    // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
-    int64_t const n = e_cur - o_cur;
-    int64_t cap     = std::numeric_limits<int32_t>::max();
-    if (max_words > 0) cap = (has_row && col.valid(r)) ? min(static_cast<int64_t>(max_words), n / 2) : 0;
-    bool const chunk_ok = has_row && cbase < ctx.aend && static_cast<int64_t>(wdone) < cap;
+    bool const has_row  = r < rows;
+    bool const chunk_ok = has_row && cbase < ctx.aend && wdone < cap;
 
     // ---- bytes -> word ends (lanes <-> bytes, per group)
     uint32_t ends = 0, starts = 0, xs = 0;
-    uint32_t const a0 = static_cast<uint32_t>(cbase) + 16u * gl;  // coordinates fit 32 bits (rows are below 2 GiB)
-    if (chunk_ok) {
-      *reinterpret_cast<uint4*>(&lds.bytes[g][(a0 & (kRing - 1)) >> 2]) = mine_cur;
-    }
+    uint32_t const a0 = cbase + 16u * gl;
+    if (chunk_ok) *reinterpret_cast<uint4*>(&lds.bytes[g][(a0 & (kRing - 1)) >> 2]) = mine_cur;
     {
       uint4 const mine  = mine_cur;
-      uint32_t const sp = gather_byte_flags(space_bytes(mine.x)) | (gather_byte_flags(space_bytes(mine.y)) << 4) |
-                          (gather_byte_flags(space_bytes(mine.z)) << 8) | (gather_byte_flags(space_bytes(mine.w)) << 12);
+      // spaces, and everything outside the row counts as one
+      uint32_t const sp = (gather_byte_flags(space_bytes(mine.x)) | (gather_byte_flags(space_bytes(mine.y)) << 4) |
+                           (gather_byte_flags(space_bytes(mine.z)) << 8) | (gather_byte_flags(space_bytes(mine.w)) << 12) | ~ctx.inside(a0)) &
+                          0xFFFFu;
       // is the byte before my sixteen a space, and the byte after them
       uint32_t const before = dpp_row<0x111>(prev_space, sp >> 15);                       // row_shr:1
       uint32_t const after  = dpp_row<0x101>(tail_cur == 0x20u ? 1u : 0u, sp & 1u);        // row_shl:1
@@ -514,21 +544,22 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
       uint32_t const sb = starts & ((2u << p) - 1u);
       uint32_t const st = sb ? a0 + (32u - __builtin_clz(sb)) : xs;  // 1-based
       uint32_t const wl = a0 + p + 1u - st + 1u;
-      lds.wend[slot]    = static_cast<uint16_t>(16u * gl + p);
-      lds.wlen[slot]    = static_cast<uint16_t>(min(wl, kMaxWord));
+      lds.word[slot]    = (min(wl, kMaxWord) << 16) | (16u * gl + p);
       ++slot;
     }
     // words of this chunk that count (the row's word limit may cut them short)
-    uint32_t const allowed = chunk_ok ? static_cast<uint32_t>(min(static_cast<int64_t>(my_gtotal), cap - static_cast<int64_t>(wdone))) : 0u;
+    uint32_t const allowed = chunk_ok ? min(my_gtotal, cap - wdone) : 0u;
+    uint32_t const wd_after = wdone + allowed;
+    int64_t const r_now     = r;
+    if (gl == 0) {
+      int64_t const row_slot = ((o_cur - first_offset) >> 1) + r;
+      *reinterpret_cast<uint4*>(&lds.group[g][0]) = make_uint4(my_gbase, allowed, cbase, wdone);
+      *reinterpret_cast<uint4*>(&lds.group[g][4]) =
+        make_uint4(ctx.mis, static_cast<uint32_t>(r), static_cast<uint32_t>(row_slot), static_cast<uint32_t>(static_cast<uint64_t>(row_slot) >> 32));
+    }
 
     // ---- what this group looks at next; request it now so it arrives while the probes run
-    int64_t const r_now     = r;
-    int64_t const o_now     = o_cur;
-    uint32_t const mis_now  = ctx.mis;
-    uint32_t const cb_now   = static_cast<uint32_t>(cbase);
-    uint32_t const wd_now   = wdone;
-    uint32_t const wd_after = wdone + allowed;
-    bool const row_done     = has_row && !(chunk_ok && cbase + kChunk < ctx.aend && static_cast<int64_t>(wd_after) < cap);
+    bool const row_done = has_row && !(chunk_ok && cbase + kChunk < ctx.aend && wd_after < cap);
     if (has_row) {
       if (!row_done) {
         cbase += kChunk;
@@ -542,13 +573,14 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         wdone = 0;
         carry_start = 0;
         prev_space  = 1;
+        if (r < rows) cap = word_cap(r, e_cur - o_cur);
         if (r + stride < rows) {
           o_nxt = col.off(r + stride);
           e_nxt = col.off(r + stride + 1);
         }
       }
       if (r < rows) {
-        mine_cur = ctx.load_clean(cbase + 16 * gl);
+        mine_cur = ctx.load_raw(cbase + 16 * gl);
         tail_cur = gl == kGroupLanes - 1 ? ctx.byte_at(cbase + kChunk) : 0x20u;
       }
     }
@@ -561,30 +593,48 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
     for (uint32_t w0 = 0; w0 < total; w0 += kWave) {
       uint32_t const ws = w0 + lane;  // word slot
       int const gw      = (ws >= gb1) + (ws >= gb2) + (ws >= gb3);
-      int const src     = gw * kGroupLanes;
-      uint32_t const idx = ws - shfl_u32(my_gbase, src);
-      uint32_t const alw = shfl_u32(allowed, src);  // (every lane must take part in a shuffle: keep it out of the && below)
-      bool const active  = ws < total && idx < alw;
-      uint32_t const cbw = shfl_u32(cb_now, src);
-      uint32_t const wdw = shfl_u32(wd_now, src);
-      uint32_t const misw = shfl_u32(mis_now, src);
-      int32_t const rw   = static_cast<int32_t>(shfl_u32(static_cast<uint32_t>(r_now), src));
-      int64_t const ow   = (static_cast<int64_t>(shfl_u32(static_cast<uint32_t>(static_cast<uint64_t>(o_now) >> 32), src)) << 32) |
-                         shfl_u32(static_cast<uint32_t>(o_now), src);
+      uint4 const ga    = *reinterpret_cast<const uint4*>(&lds.group[gw][0]);  // first slot, allowed, chunk base, words so far
+      uint4 const gb    = *reinterpret_cast<const uint4*>(&lds.group[gw][4]);  // row start in its block, row, arena slot of the row
+      uint32_t const idx = ws - ga.x;
+      bool const active  = ws < total && idx < ga.y;
       bool miss       = false;
       uint32_t value  = 0, wl = 0, wstart = 0;
+      uint32_t head[4] = {0u, 0u, 0u, 0u};
       if (active) {
-        wl     = lds.wlen[ws];
-        wstart = cbw + lds.wend[ws] + 1u - wl;  // coordinate of the word's first byte
+        uint32_t const rec = lds.word[ws];
+        wl     = rec >> 16;
+        wstart = ga.z + (rec & 0xFFFFu) + 1u - wl;  // coordinate of the word's first byte
         if (wl >= kMaxWord) {
           value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
         } else {
           int32_t id = kNone;
+          RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
+          rw_.head16(head);
+          trim_key8(wl, head[0], head[1]);
+          trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
           if (wl <= table.max_len[0]) {
-            RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
-            uint32_t r0, r1;
-            rw_.key8(0, 8, &r0, &r1);
-            id = lookup(table, 0, rw_, 0, wl, r0, r1);
+            // hash of the first two blocks without a loop; longer words go on from there
+            Probe pr;
+            pr.k0 = head[0];
+            pr.k1 = head[1];
+            uint32_t h        = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
+            uint32_t const h2 = key_hash_block(h, head[2], head[3]);
+            h                 = wl > 8 ? h2 : h;
+            if (wl > 16) {
+              for (uint32_t done = 16; done < wl; done += 8) {
+                uint32_t b0, b1;
+                rw_.key8(done, wl - done, &b0, &b1);
+                h = key_hash_block(h, b0, b1);
+              }
+            }
+            uint32_t b;
+            pr.want   = slot_word0(h, 0, wl, &b);
+            pr.bucket = b & table.bucket_mask;
+            uint4 const s0 = table.slots[2 * pr.bucket];
+            uint4 const s1 = table.slots[2 * pr.bucket + 1];
+            uint32_t const v = verdict(pr, s0, s1, wl, &id);
+            if (v == 2u) id = finish_probe(table, pr, s0, s1, rw_, 0u, wl);
+            else if (v == 0u) id = kNone;
           }
           miss  = id == kNone;
           value = static_cast<uint32_t>(id);
@@ -605,20 +655,16 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         if (miss) {
           uint32_t const q = q_pos + lanes_below(mm);
           if (q < queue_capacity) {
-            RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
-            OovEntry e{rw, wstart - misw, wdw + idx, wl, {0u, 0u, 0u, 0u}};
-            rw_.key8(0, min(wl, 8u), &e.head[0], &e.head[1]);
-            if (wl > 8) rw_.key8(8, min(wl - 8u, 8u), &e.head[2], &e.head[3]);
             uint4* const dst = reinterpret_cast<uint4*>(queue + q);
-            store_stream(dst, make_uint4(static_cast<uint32_t>(e.row), e.delta, e.widx, e.len));
-            store_stream(dst + 1, make_uint4(e.head[0], e.head[1], e.head[2], e.head[3]));
+            store_stream(dst, make_uint4(gb.y, wstart - gb.x, ga.w + idx, wl));
+            store_stream(dst + 1, make_uint4(head[0], head[1], head[2], head[3]));
           }
           value = kOovMark | q;
         }
         q_pos += nm;
       }
       if (active) {
-        int64_t const s = ((ow - first_offset) >> 1) + rw + wdw + idx;
+        int64_t const s = static_cast<int64_t>((static_cast<uint64_t>(gb.w) << 32) | gb.z) + ga.w + idx;
         store_stream(arena + s, value);
       }
       uint64_t const hit = ballot64(active && !miss);
@@ -890,21 +936,6 @@ struct ShortWord {
     r[3] = t3 >> sh;
     rem -= l;
     bnd >>= l;
-  }
-
-  // What the two home slots say about a candidate of l bytes without any further memory access:
-  // 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or the
-  // bucket is full and the search goes on in the next one: both rare).  Straight-line code.
-  static __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
-  {
-    bool const tag0  = s0.x == pr.want, tag1 = s1.x == pr.want;
-    bool const is0   = tag0 && s0.z == pr.k0 && s0.w == pr.k1;
-    bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
-    bool const small = l <= 8;
-    bool const found = small && (is0 || is1);
-    bool const more  = (!small && (tag0 || tag1)) || (!found && s0.x != 0 && s1.x != 0);
-    *id              = static_cast<int32_t>(is0 ? s0.y : s1.y);
-    return found ? 1u : more ? 2u : 0u;
   }
 
   // Examines the two longest remaining candidates (their table reads are in flight together).
@@ -1331,21 +1362,30 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   uint32_t const mask = static_cast<uint32_t>(capacity / 2 - 1);  // buckets of two slots
   std::vector<HostSlot> slots(capacity, HostSlot{0, 0, 0, 0});
   uint32_t max_len[2] = {0, 0};
+  // keys of more than 8 bytes, zero padded to whole 8-byte blocks
+  std::vector<uint8_t> blocks;
+  auto add_blocks = [&](const uint8_t* key, uint32_t len) -> uint32_t {
+    if (len <= 8) return 0u;
+    size_t const at = blocks.size();
+    blocks.resize(at + ((static_cast<size_t>(len) + 7) & ~size_t{7}), 0);
+    std::memcpy(blocks.data() + at, key, len);
+    return static_cast<uint32_t>(at);
+  };
   for (int32_t i = 0; i < V; ++i) {
     int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
     int64_t const len = e - b;
     // entries of 200 bytes or more can never equal a tokenizable word or piece; empty ones are never looked up
     if (len >= 1 && len < kMaxWord) {
-      host_insert(slots, mask, pool, 0, pool.data() + b, static_cast<uint32_t>(len), static_cast<uint32_t>(b), i);
+      host_insert(slots, mask, blocks, 0, pool.data() + b, static_cast<uint32_t>(len), add_blocks(pool.data() + b, static_cast<uint32_t>(len)), i);
       max_len[0] = std::max(max_len[0], static_cast<uint32_t>(len));
     }
     // wordpiece_tokenize.cu:184-192: "##" entries also live, without the prefix, in the second key space
     if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') {
-      host_insert(slots, mask, pool, 1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), static_cast<uint32_t>(b + 2), i);
+      host_insert(slots, mask, blocks, 1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), add_blocks(pool.data() + b + 2, static_cast<uint32_t>(len - 2)), i);
       max_len[1] = std::max(max_len[1], static_cast<uint32_t>(len - 2));
     }
   }
-  if (pool.size() > 0xFFFFFFFFull) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
+  if (blocks.size() > 0xFFFFFFF0ull) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
 
   // length filter over the first three bytes of every key of three bytes and more
   size_t lens_size = 1024;
@@ -1366,17 +1406,17 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   auto* v = new nvtext_amd_wordpiece_vocabulary;
   v->entries = V;
   // wordpiece_tokenize.cu:199-209, 273-275
-  int32_t unk = host_find(slots, mask, pool, "[UNK]");
-  if (unk < 0) unk = host_find(slots, mask, pool, "[unk]");
+  int32_t unk = host_find(slots, mask, blocks, "[UNK]");
+  if (unk < 0) unk = host_find(slots, mask, blocks, "[unk]");
   v->slot_bytes = capacity * sizeof(HostSlot);
-  v->pool_bytes = pool.size() + 16;
+  v->pool_bytes = blocks.size() + 16;
   if (hipMalloc(&v->d_slots, v->slot_bytes) != hipSuccess || hipMalloc(&v->d_pool, v->pool_bytes) != hipSuccess ||
       hipMalloc(&v->d_lens, lens.size() * sizeof(uint32_t)) != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
   hipError_t e1 = hipMemcpyAsync(v->d_slots, slots.data(), v->slot_bytes, hipMemcpyHostToDevice, stream);
-  hipError_t e2 = pool.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, pool.data(), pool.size(), hipMemcpyHostToDevice, stream);
+  hipError_t e2 = blocks.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, blocks.data(), blocks.size(), hipMemcpyHostToDevice, stream);
   hipError_t e4 = hipMemcpyAsync(v->d_lens, lens.data(), lens.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
   hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
   if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess) {
