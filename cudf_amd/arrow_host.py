@@ -97,6 +97,51 @@ class HostStringsColumn:
 
 
 @dataclass
+class HostListStringsColumn:
+    """LIST<STRING> column (cpp/include/cudf/lists/lists_column_view.hpp): int32 list offsets
+    (parent_size + 1 entries, element indices into the child), an optional row validity mask, and a
+    strings child.  A sliced view keeps the buffers and carries ``offset``/``size``."""
+    offsets: np.ndarray          # int32
+    child: HostStringsColumn
+    mask: Optional[np.ndarray]
+    size: int
+    offset: int = 0
+    null_count: int = 0
+
+    @staticmethod
+    def from_pylist(rows, child_offsets_dtype=np.int32) -> "HostListStringsColumn":
+        """rows: list of (list of str/bytes/None) or None.  Null rows are empty lists, as
+        cudf::test::lists_column_wrapper builds them."""
+        flat: List[Text] = []
+        offs = [0]
+        valid = []
+        for r in rows:
+            if r is None:
+                valid.append(False)
+            else:
+                valid.append(True)
+                flat.extend(r)
+            offs.append(len(flat))
+        n = len(valid)
+        nulls = n - int(sum(valid))
+        child = HostStringsColumn.from_pylist(flat, child_offsets_dtype)
+        mask = pack_validity(valid) if nulls and n else None
+        return HostListStringsColumn(np.asarray(offs, dtype=np.int32), child, mask, n, 0, nulls)
+
+    def slice(self, lo: int, hi: int) -> "HostListStringsColumn":
+        assert 0 <= lo <= hi <= self.size
+        nulls = 0
+        if self.mask is not None:
+            nulls = int((~unpack_validity(self.mask, hi - lo, self.offset + lo)).sum())
+        return HostListStringsColumn(self.offsets, self.child, self.mask, hi - lo, self.offset + lo, nulls)
+
+    def validity(self) -> np.ndarray:
+        if self.mask is None:
+            return np.ones(self.size, dtype=bool)
+        return unpack_validity(self.mask, self.size, self.offset)
+
+
+@dataclass
 class HostListColumn:
     """LIST<INT32|UINT32|UINT64> result (cpp/src/lists/lists_column_factories.cu:106-129):
     int32 offsets (size+1 entries, or 0 entries for the canonical empty list column),

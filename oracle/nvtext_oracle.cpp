@@ -330,6 +330,89 @@ int minhash_impl(StringsCol const& col, T seed, T const* a, T const* b, int32_t 
 }
 
 // ---------------------------------------------------------------------------
+// minhash_ngrams / minhash64_ngrams -- cpp/src/text/minhash.cu:182-250 (hashing of
+// runs of list elements), 281-376 (permutation + min with width = ngrams), 515-603
+// ---------------------------------------------------------------------------
+struct ListStringsCol {
+  int32_t const* offsets;  // list offsets (size + offset + 1 entries), element indices into the child view
+  uint32_t const* mask;    // row validity, may be null
+  int32_t size;
+  int32_t offset;
+  int32_t null_count;
+  StringsCol child;
+
+  int32_t off(int64_t i) const { return offsets[i + offset]; }
+  bool valid(int64_t i) const
+  {
+    if (!mask) return true;
+    int64_t const b = i + offset;
+    return (mask[b >> 5] >> (b & 31)) & 1u;
+  }
+};
+
+template <typename T>
+void minhash_ngrams_row(StringsCol const& child, int64_t first, int64_t n, int32_t ngrams, T seed, T const* a, T const* b,
+                        int32_t P, T* out)
+{
+  if (n == 0) {  // minhash.cu:318 -- init = 0 for an empty (valid) row
+    std::fill(out, out + P, T{0});
+    return;
+  }
+  std::fill(out, out + P, std::numeric_limits<T>::max());
+  // minhash.cu:311-314 with width = ngrams: the permutation looks at positions [0, max(1, n - ngrams + 1))
+  int64_t const positions = std::max<int64_t>(1, n - ngrams + 1);
+  for (int64_t idx = 0; idx < positions; ++idx) {
+    if (!child.valid(first + idx)) continue;  // 213-216: hash 0 = skipped (329)
+    // 218-222: the run ends at element idx + ngrams (not idx + ngrams - 1), clamped to the row; a clamped
+    // run is kept only at idx 0
+    int64_t const next = std::min<int64_t>(idx + ngrams, n - 1);
+    if (idx != 0 && (next - idx) < ngrams) continue;
+    // 224-229: one string from the first byte of element idx to the last byte of element next
+    int64_t const bo = child.off(first + idx);
+    int64_t const eo = child.off(first + next + 1);
+    T hv             = HashOf<T>::hash(child.chars + bo, eo - bo, seed);
+    hv               = std::max<T>(hv, T{1});  // 237
+    for (int32_t j = 0; j < P; ++j) {
+      T const v = permute<T>(hv, a[j], b[j]);
+      if (v < out[j]) out[j] = v;
+    }
+  }
+}
+
+template <typename T>
+int minhash_ngrams_impl(ListStringsCol const& col, int32_t ngrams, T seed, T const* a, T const* b, int32_t P, int nthreads,
+                        int32_t* out_offsets, T* out_child, int64_t* out_child_len)
+{
+  // minhash.cu:524-536, in this order
+  if (ngrams < 2) return INVALID_ARGUMENT;
+  if (P <= 0) return INVALID_ARGUMENT;
+  if (static_cast<uint64_t>(col.size) * static_cast<uint64_t>(P) >=
+      static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
+    return OVERFLOW_ERROR;
+  if (col.size == 0) {
+    if (out_offsets) out_offsets[0] = 0;
+    *out_child_len = 0;
+    return OK;
+  }
+  bool const purge = col.null_count > 0;  // minhash.cu:626-628
+  int64_t pos      = 0;
+  for (int32_t r = 0; r < col.size; ++r) {
+    out_offsets[r] = static_cast<int32_t>(pos);
+    if (!(purge && !col.valid(r))) pos += P;
+  }
+  out_offsets[col.size] = static_cast<int32_t>(pos);
+  *out_child_len        = pos;
+  parallel_rows(col.size, nthreads, [&](int, int32_t lo, int32_t hi) {
+    for (int32_t r = lo; r < hi; ++r) {
+      if (purge && !col.valid(r)) continue;
+      int64_t const first = col.off(r);
+      minhash_ngrams_row<T>(col.child, first, col.off(r + 1) - first, ngrams, seed, a, b, P, out_child + out_offsets[r]);
+    }
+  });
+  return OK;
+}
+
+// ---------------------------------------------------------------------------
 // wordpiece vocabulary -- cpp/src/text/wordpiece_tokenize.cu:184-209, 213-282
 // ---------------------------------------------------------------------------
 struct Vocab {
@@ -457,6 +540,29 @@ int oracle_minhash64(uint8_t const* chars, void const* offsets, int offsets_is_i
 {
   StringsCol c{chars, offsets, offsets_is_int64, mask, size, offset, null_count};
   return minhash_impl<uint64_t>(c, seed, a, b, P, width, nthreads, out_offsets, out_child, out_child_len);
+}
+
+// The list column is (list_offsets, list_mask, size, offset, null_count) over a child strings column.
+int oracle_minhash_ngrams(int32_t const* list_offsets, uint32_t const* list_mask, int32_t size, int32_t offset, int32_t null_count,
+                          uint8_t const* chars, void const* child_offsets, int child_offsets_is_int64, uint32_t const* child_mask,
+                          int32_t child_size, int32_t child_offset, int32_t ngrams, uint32_t seed, uint32_t const* a,
+                          uint32_t const* b, int32_t P, int nthreads, int32_t* out_offsets, uint32_t* out_child,
+                          int64_t* out_child_len)
+{
+  ListStringsCol c{list_offsets, list_mask, size, offset, null_count,
+                   StringsCol{chars, child_offsets, child_offsets_is_int64, child_mask, child_size, child_offset, 0}};
+  return minhash_ngrams_impl<uint32_t>(c, ngrams, seed, a, b, P, nthreads, out_offsets, out_child, out_child_len);
+}
+
+int oracle_minhash64_ngrams(int32_t const* list_offsets, uint32_t const* list_mask, int32_t size, int32_t offset, int32_t null_count,
+                            uint8_t const* chars, void const* child_offsets, int child_offsets_is_int64, uint32_t const* child_mask,
+                            int32_t child_size, int32_t child_offset, int32_t ngrams, uint64_t seed, uint64_t const* a,
+                            uint64_t const* b, int32_t P, int nthreads, int32_t* out_offsets, uint64_t* out_child,
+                            int64_t* out_child_len)
+{
+  ListStringsCol c{list_offsets, list_mask, size, offset, null_count,
+                   StringsCol{chars, child_offsets, child_offsets_is_int64, child_mask, child_size, child_offset, 0}};
+  return minhash_ngrams_impl<uint64_t>(c, ngrams, seed, a, b, P, nthreads, out_offsets, out_child, out_child_len);
 }
 
 // wordpiece_tokenize.cu:213-282.  Returns INVALID_ARGUMENT for an empty vocabulary

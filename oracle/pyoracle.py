@@ -50,6 +50,14 @@ def lib():
         L.oracle_minhash64.restype = C.c_int
         L.oracle_minhash64.argtypes = col + [C.c_uint64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int,
                                              C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
+        lcol = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
+                C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int32, C.c_int32]
+        L.oracle_minhash_ngrams.restype = C.c_int
+        L.oracle_minhash_ngrams.argtypes = lcol + [C.c_int32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_int32, C.c_int,
+                                                   C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
+        L.oracle_minhash64_ngrams.restype = C.c_int
+        L.oracle_minhash64_ngrams.argtypes = lcol + [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int,
+                                                     C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
         L.oracle_vocab_create.restype = C.c_int
         L.oracle_vocab_create.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int32, C.c_int32, C.c_int32,
                                           C.POINTER(C.c_void_p)]
@@ -137,6 +145,38 @@ def minhash(col, seed, a, b, width, nthreads: int = 1):
 
 def minhash64(col, seed, a, b, width, nthreads: int = 1):
     return _minhash(col, seed, a, b, width, np.uint64, lib().oracle_minhash64, nthreads)
+
+
+def _minhash_ngrams(col, ngrams, seed, a, b, dtype, fn, nthreads):
+    """col: cudf_amd.arrow_host.HostListStringsColumn."""
+    from cudf_amd.arrow_host import HostListColumn
+    a = np.ascontiguousarray(a, dtype=dtype)
+    b = np.ascontiguousarray(b, dtype=dtype)
+    if a.size != b.size:
+        raise OracleError(INVALID_ARGUMENT)
+    loffs = np.ascontiguousarray(col.offsets, dtype=np.int32)
+    lmask = None if col.mask is None else np.ascontiguousarray(col.mask, dtype=np.uint32)
+    keep, cargs = _col_args(col.child)
+    P = int(a.size)
+    rows = int(col.size)
+    ok_size = ngrams >= 2 and P > 0 and rows * P < 2**31 - 1
+    offsets = np.zeros(rows + 1, dtype=np.int32)
+    child = np.zeros(rows * P if ok_size else 0, dtype=dtype)
+    n = C.c_int64(0)
+    rc = fn(_p(loffs) if loffs.size else None, _p(lmask), rows, int(col.offset), int(col.null_count), *cargs[:6],
+            ngrams, seed, _p(a) if P else None, _p(b) if P else None, P, nthreads,
+            _p(offsets), _p(child) if child.size else None, C.byref(n))
+    if rc != OK:
+        raise OracleError(rc)
+    return HostListColumn(offsets, child[:n.value].copy(), copy_bitmask(col), rows, int(col.null_count))
+
+
+def minhash_ngrams(col, ngrams, seed, a, b, nthreads: int = 1):
+    return _minhash_ngrams(col, ngrams, seed, a, b, np.uint32, lib().oracle_minhash_ngrams, nthreads)
+
+
+def minhash64_ngrams(col, ngrams, seed, a, b, nthreads: int = 1):
+    return _minhash_ngrams(col, ngrams, seed, a, b, np.uint64, lib().oracle_minhash64_ngrams, nthreads)
 
 
 class Vocabulary:

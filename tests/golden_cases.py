@@ -7,7 +7,7 @@ from typing import List, Optional
 
 import numpy as np
 
-from cudf_amd.arrow_host import HostStringsColumn
+from cudf_amd.arrow_host import HostListStringsColumn, HostStringsColumn
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
@@ -27,6 +27,22 @@ def minhash_cases():
         c["rows"] = [_row(r) for r in c["rows"]]
         out.append(c)
     return out
+
+
+def minhash_ngrams_cases():
+    """Each case: rows (list of lists of strings), optional slice, ngrams, seed, a, b, expected32, expected64."""
+    d = json.load(open(os.path.join(GOLDEN, "minhash_ngrams_vectors.json"), encoding="utf-8"))
+    out = []
+    for c in d["cases"]:
+        c = dict(c)
+        if "repeat_rows" in c:
+            c["rows"] = [[s] * n for s, n in c.pop("repeat_rows")]
+        out.append(c)
+    return out
+
+
+def list_strings(rows, child_offsets_dtype=np.int32) -> HostListStringsColumn:
+    return HostListStringsColumn.from_pylist(rows, child_offsets_dtype)
 
 
 def murmur64_vectors():

@@ -126,6 +126,50 @@ def test_minhash_errors_and_empty():
 
 
 # ----------------------------------------------------------------------------- wordpiece
+@pytest.mark.parametrize("case", gc.minhash_ngrams_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_minhash_ngrams_golden(case, dtype):
+    col = gc.list_strings(case["rows"], dtype)
+    if "slice" in case:
+        col = col.slice(*case["slice"])
+    a32, b32 = np.array(case["a"], np.uint32), np.array(case["b"], np.uint32)
+    assert orc.minhash_ngrams(col, case["ngrams"], case["seed"], a32, b32).to_pylist() == case["expected32"]
+    got = orc.minhash64_ngrams(col, case["ngrams"], case["seed"], a32.astype(np.uint64), b32.astype(np.uint64))
+    assert got.to_pylist() == case["expected64"]
+    assert got.child.dtype == np.uint64 and got.null_count == 0
+
+
+def test_minhash_ngrams_rules():
+    """What the vectors do not spell out: a run is ngrams + 1 elements unless the row is shorter (then only the
+    run from element 0 exists); null elements start no run; null rows have no slots; empty rows are zeros; a row
+    whose every run is skipped keeps the all-ones start value."""
+    a, b = np.array([3, 5], np.uint32), np.array([7, 11], np.uint32)
+    words = ["aa", "b", "cc", "ddd", "e", "ff", "g"]
+    col = gc.list_strings([words, None, [], words[:3], [None, "x", "y", "z"]])
+    got = orc.minhash_ngrams(col, 2, 9, a, b)
+    assert got.null_count == 1 and list(np.diff(got.offsets)) == [2, 0, 2, 2, 2]
+    rows = got.to_pylist()
+    # row 0: runs of three elements starting at 0..4 (the run starting at 5 would be clamped and is dropped)
+    hs = [max(orc.murmur3_x86_32("".join(words[i:i + 3]).encode(), 9), 1) for i in range(5)]
+    assert rows[0] == [min((h * int(x) + int(y)) & 0xFFFFFFFF for h in hs) for x, y in zip(a, b)]
+    assert rows[1] is None and rows[2] == [0, 0]
+    # row 3: positions 0 and 1; the run from 0 is whole, the run from 1 is clamped and dropped
+    h = max(orc.murmur3_x86_32(b"aabcc", 9), 1)
+    assert rows[3] == [(h * int(x) + int(y)) & 0xFFFFFFFF for x, y in zip(a, b)]
+    # row 4: positions 0..2: element 0 is null, the run from 1 spans elements 1..3, the run from 2 is clamped
+    h = max(orc.murmur3_x86_32(b"xyz", 9), 1)
+    assert rows[4] == [(h * int(x) + int(y)) & 0xFFFFFFFF for x, y in zip(a, b)]
+    only_null = gc.list_strings([[None, None]])
+    assert orc.minhash_ngrams(only_null, 2, 0, a, b).to_pylist() == [[0xFFFFFFFF, 0xFFFFFFFF]]
+    with pytest.raises(OracleError):
+        orc.minhash_ngrams(col, 1, 0, a, b)
+    with pytest.raises(OracleError):
+        orc.minhash_ngrams(col, 2, 0, a[:0], b[:0])
+    with pytest.raises(OracleError):
+        orc.minhash64_ngrams(col, 2, 0, np.zeros(3, np.uint64), np.zeros(2, np.uint64))
+    assert orc.minhash_ngrams(gc.list_strings([]), 4, 0, a, b).size == 0
+
+
 @pytest.mark.parametrize("case", gc.wordpiece_cases(), ids=lambda c: c["name"])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_wordpiece_golden(case, dtype):
