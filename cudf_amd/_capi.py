@@ -15,6 +15,8 @@ EXPORTS = [
     "nvtext_amd_last_error",
     "nvtext_amd_minhash",
     "nvtext_amd_minhash64",
+    "nvtext_amd_minhash_ngrams",
+    "nvtext_amd_minhash64_ngrams",
     "nvtext_amd_wordpiece_vocabulary_create",
     "nvtext_amd_wordpiece_vocabulary_destroy",
     "nvtext_amd_wordpiece_vocabulary_unk_id",
@@ -34,6 +36,17 @@ class StringsColumn(C.Structure):
         ("size", C.c_int32),
         ("offset", C.c_int32),
         ("null_count", C.c_int32),
+    ]
+
+
+class ListStringsColumn(C.Structure):
+    _fields_ = [
+        ("offsets", C.c_void_p),
+        ("null_mask", C.c_void_p),
+        ("size", C.c_int32),
+        ("offset", C.c_int32),
+        ("null_count", C.c_int32),
+        ("child", StringsColumn),
     ]
 
 
@@ -88,6 +101,12 @@ def load():
     L.nvtext_amd_minhash64.restype = C.c_int
     L.nvtext_amd_minhash64.argtypes = [C.POINTER(StringsColumn), C.c_uint64, C.c_void_p, C.c_void_p,
                                        C.c_int64, C.c_int64] + common_tail
+    L.nvtext_amd_minhash_ngrams.restype = C.c_int
+    L.nvtext_amd_minhash_ngrams.argtypes = [C.POINTER(ListStringsColumn), C.c_int32, C.c_uint32, C.c_void_p, C.c_void_p,
+                                            C.c_int64, C.c_int64] + common_tail[1:]
+    L.nvtext_amd_minhash64_ngrams.restype = C.c_int
+    L.nvtext_amd_minhash64_ngrams.argtypes = [C.POINTER(ListStringsColumn), C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p,
+                                              C.c_int64, C.c_int64] + common_tail[1:]
     L.nvtext_amd_wordpiece_vocabulary_create.restype = C.c_int
     L.nvtext_amd_wordpiece_vocabulary_create.argtypes = [C.POINTER(StringsColumn), C.c_void_p,
                                                          C.POINTER(Allocator), C.POINTER(C.c_void_p)]

@@ -496,6 +496,209 @@ nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, c
   return NVTEXT_AMD_SUCCESS;
 }
 
+
+// ------------------------------------------------------------------ minhash_ngrams / minhash64_ngrams
+// LIST<STRING> rows: the hashed items are runs of consecutive list elements instead of character windows
+// (cpp/src/text/minhash.cu:182-250); the permutation and the minimum are the ones above.
+struct ListView {
+  const int32_t* offsets;  // element index of the first element of row i + offset
+  const uint32_t* mask;
+  int32_t size;
+  int32_t offset;
+  int32_t use_mask;
+  ColView child;           // the elements
+
+  __device__ __forceinline__ int64_t off(int64_t i) const { return offsets[i + offset]; }
+  __device__ __forceinline__ bool valid(int64_t i) const
+  {
+    if (!use_mask) return true;
+    int64_t const b = i + offset;
+    return (mask[b >> 5] >> (b & 31)) & 1u;
+  }
+};
+
+// Byte source over global memory through aligned dword loads that overlap [p, p + len) only.
+struct AlignedSrc {
+  const uint32_t* w;  // aligned address at or below the first byte
+  uint32_t mis;       // first byte inside w[0]
+  uint32_t end;       // mis + len
+  __device__ __forceinline__ AlignedSrc(const uint8_t* p, uint32_t len)
+  {
+    mis = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 3u);
+    w   = reinterpret_cast<const uint32_t*>(p - mis);
+    end = mis + len;
+  }
+  __device__ __forceinline__ uint32_t byte(uint32_t i) const { return reinterpret_cast<const uint8_t*>(w)[mis + i]; }
+  __device__ __forceinline__ uint32_t u32(uint32_t i) const
+  {
+    uint32_t const o  = mis + i;
+    uint32_t const j  = o >> 2;
+    uint32_t const lo = w[j];
+    uint32_t const hi = 4u * (j + 1u) < end ? w[j + 1] : 0u;
+    return __builtin_amdgcn_alignbit(hi, lo, (o & 3u) * 8u);
+  }
+};
+
+// One workgroup per (row, parameter chunk); its wavefronts take the positions of the row 64 at a time.
+template <typename T, int K>
+__global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, int32_t ngrams, T seed, const T* __restrict__ pa,
+                                                                  const T* __restrict__ pb, int32_t P, const int32_t* __restrict__ out_offsets,
+                                                                  T* __restrict__ out)
+{
+  using H = HashTraits<T>;
+  __shared__ WaveLds<T> lds[kWaves];
+  __shared__ T red[kWaves][K * kWave];
+
+  int64_t const r = blockIdx.x;
+  if (!in.valid(r)) return;
+  int32_t const chunk_base = blockIdx.y * (K * kWave);
+  int64_t const first      = in.off(r);
+  int64_t const n          = in.off(r + 1) - first;
+  T* dst                   = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
+  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
+  if (n == 0) {  // minhash.cu:318
+    for (int j = threadIdx.x; j < in_chunk; j += kThreads) dst[j] = T{0};
+    return;
+  }
+  int const lane = lane_id();
+  int const wave = threadIdx.x / kWave;
+  T a[K], b[K], m[K];
+  load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
+
+  // minhash.cu:311-314 with width = ngrams: the positions that the permutation looks at
+  int64_t const positions = max(static_cast<int64_t>(1), n - ngrams + 1);
+  for (int64_t base = static_cast<int64_t>(wave) * kWave; base < positions; base += kWaves * kWave) {
+    int64_t const idx = base + lane;
+    bool valid        = false;
+    T hv              = 0;
+    if (idx < positions && in.child.valid(first + idx)) {  // 213-216: a null element starts no run
+      // 218-222: the run ends at element idx + ngrams, clamped to the row; a clamped run counts only at idx 0
+      int64_t const next = min(idx + ngrams, n - 1);
+      if (idx == 0 || next - idx >= ngrams) {
+        // 224-229: the bytes from the start of element idx to the end of element next
+        int64_t const bo = in.child.off(first + idx);
+        int64_t const eo = in.child.off(first + next + 1);
+        AlignedSrc const src(in.child.chars + bo, static_cast<uint32_t>(eo - bo));
+        hv    = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+        hv    = hv < 1 ? T{1} : hv;  // 237
+        valid = true;
+      }
+    }
+    uint64_t const vm = ballot64(valid);
+    if (valid) lds[wave].hashes[lanes_below(vm)] = hv;
+    fold_hashes<T, K>(lds[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
+  }
+
+#pragma unroll
+  for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+  __syncthreads();
+  for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
+    T v = red[0][j];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
+    dst[j] = v;
+  }
+}
+
+struct ListValidTimesP {
+  ListView in;
+  int32_t P;
+  __device__ uint64_t operator()(int64_t i) const { return in.valid(i) ? static_cast<uint64_t>(P) : 0; }
+};
+
+template <typename T, int K>
+void launch_ngrams(const ListView& v, int32_t ngrams, T seed, const T* a, const T* b, int32_t P, const int32_t* offsets, T* child,
+                   hipStream_t stream)
+{
+  int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
+  dim3 grid(static_cast<unsigned>(v.size), static_cast<unsigned>(chunks));
+  ProfileScope ps("minhash_ngrams_kernel", stream);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_ngrams_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, ngrams, seed, a, b, P, offsets, child);
+}
+
+template <typename T>
+nvtext_amd_status minhash_ngrams_impl(const nvtext_amd_list_strings_column* input, int32_t ngrams, T seed, const T* a, const T* b,
+                                      int64_t a_count, int64_t b_count, void* stream_, const nvtext_amd_allocator* mr_,
+                                      nvtext_amd_list_column* out, int32_t type_id)
+{
+  if (!input || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  *out = nvtext_amd_list_column{};
+  // cpp/src/text/minhash.cu:524-536, same order and messages
+  if (ngrams < 2) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameter ngrams should be an integer value of 2 or greater");
+  if (a_count <= 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B cannot be empty");
+  if (a_count != b_count) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B should have the same number of elements");
+  if (static_cast<uint64_t>(input->size) * static_cast<uint64_t>(a_count) >= static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
+    return fail(NVTEXT_AMD_OVERFLOW, "The number of parameters times the number of input rows exceeds the column size limit");
+  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
+  if (input->null_count > 0 && !input->null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
+  if (input->size > 0 && !input->offsets) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "a list column with rows needs offsets");
+  if (input->child.null_count > 0 && !input->child.null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
+
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Mr mr{mr_, stream};
+  int32_t const rows = input->size;
+  int32_t const P    = static_cast<int32_t>(a_count);
+  out->child_type    = type_id;
+  out->size          = rows;
+  out->null_count    = input->null_count;
+  out->offsets_size  = rows + 1;
+  out->offsets_bytes = static_cast<size_t>(rows + 1) * sizeof(int32_t);
+  out->offsets       = static_cast<int32_t*>(mr.allocate(out->offsets_bytes));
+  if (!out->offsets) return fail(NVTEXT_AMD_ALLOC_FAILED, "offsets allocation failed");
+  if (rows == 0) {  // minhash.cu:539 then 616
+    launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, 1, stream);
+    NVTEXT_HIP_TRY(hipGetLastError());
+    return NVTEXT_AMD_SUCCESS;
+  }
+  out->child_size  = static_cast<int64_t>(rows - input->null_count) * P;
+  out->child_bytes = static_cast<size_t>(out->child_size) * sizeof(T);
+  if (out->child_bytes) {
+    out->child = mr.allocate(out->child_bytes);
+    if (!out->child) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
+    }
+  }
+  if (input->null_mask) {
+    out->null_mask_bytes = mask_alloc_bytes(rows);
+    out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
+    if (!out->null_mask) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
+    }
+    launch_copy_bitmask(out->null_mask, input->null_mask, input->offset, rows, stream);
+  }
+
+  ListView v;
+  v.offsets  = input->offsets;
+  v.mask     = input->null_mask;
+  v.size     = rows;
+  v.offset   = input->offset;
+  v.use_mask = (input->null_mask != nullptr && input->null_count > 0) ? 1 : 0;
+  v.child    = make_view(input->child);
+  if (v.use_mask) {
+    Temp scan_tmp(mr, scan_temp_bytes(rows));
+    if (!scan_tmp.ok()) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+    }
+    device_exclusive_scan(ListValidTimesP{v, P}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
+  } else {
+    hipLaunchKernelGGL(uniform_offsets_kernel, dim3((rows + 1 + 255) / 256), dim3(256), 0, stream, out->offsets, rows, P);
+  }
+  T* child = static_cast<T*>(out->child);
+  if (out->child_size > 0) {
+    if (P > 2 * kWave)
+      launch_ngrams<T, 4>(v, ngrams, seed, a, b, P, out->offsets, child, stream);
+    else if (P > kWave)
+      launch_ngrams<T, 2>(v, ngrams, seed, a, b, P, out->offsets, child, stream);
+    else
+      launch_ngrams<T, 1>(v, ngrams, seed, a, b, P, out->offsets, child, stream);
+  }
+  NVTEXT_HIP_TRY(hipGetLastError());
+  return NVTEXT_AMD_SUCCESS;
+}
+
 }  // namespace
 }  // namespace nvtext_amd
 
@@ -511,6 +714,20 @@ nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input, u
                                        int64_t b_count, int32_t width, void* stream, const nvtext_amd_allocator* mr, nvtext_amd_list_column* out)
 {
   return nvtext_amd::minhash_impl<uint64_t>(input, seed, a, b, a_count, b_count, width, stream, mr, out, NVTEXT_AMD_TYPE_UINT64);
+}
+
+nvtext_amd_status nvtext_amd_minhash_ngrams(const nvtext_amd_list_strings_column* input, int32_t ngrams, uint32_t seed, const uint32_t* a,
+                                            const uint32_t* b, int64_t a_count, int64_t b_count, void* stream, const nvtext_amd_allocator* mr,
+                                            nvtext_amd_list_column* out)
+{
+  return nvtext_amd::minhash_ngrams_impl<uint32_t>(input, ngrams, seed, a, b, a_count, b_count, stream, mr, out, NVTEXT_AMD_TYPE_UINT32);
+}
+
+nvtext_amd_status nvtext_amd_minhash64_ngrams(const nvtext_amd_list_strings_column* input, int32_t ngrams, uint64_t seed, const uint64_t* a,
+                                              const uint64_t* b, int64_t a_count, int64_t b_count, void* stream, const nvtext_amd_allocator* mr,
+                                              nvtext_amd_list_column* out)
+{
+  return nvtext_amd::minhash_ngrams_impl<uint64_t>(input, ngrams, seed, a, b, a_count, b_count, stream, mr, out, NVTEXT_AMD_TYPE_UINT64);
 }
 
 }  // extern "C"

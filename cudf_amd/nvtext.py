@@ -118,6 +118,39 @@ class DeviceStringsColumn:
 
 
 @dataclass
+class DeviceListStringsColumn:
+    """LIST<STRING> column in HBM: int32 list offsets, optional row validity, a strings child."""
+    offsets: object          # int32 tensor (parent_size + 1 entries) or None for an empty column
+    child: DeviceStringsColumn
+    mask: object
+    size: int
+    offset: int = 0
+    null_count: int = 0
+
+    @staticmethod
+    def from_host(h, device: str = "cuda") -> "DeviceListStringsColumn":
+        torch = _torch()
+        offsets = torch.from_numpy(np.ascontiguousarray(h.offsets, dtype=np.int32)).to(device) if h.offsets.size else None
+        mask = None
+        if h.mask is not None:
+            mask = torch.from_numpy(np.ascontiguousarray(h.mask).view(np.int32)).to(device)
+        return DeviceListStringsColumn(offsets, DeviceStringsColumn.from_host(h.child, device), mask, int(h.size), int(h.offset),
+                                       int(h.null_count))
+
+    def slice(self, lo: int, hi: int, null_count: int) -> "DeviceListStringsColumn":
+        return DeviceListStringsColumn(self.offsets, self.child, self.mask, hi - lo, self.offset + lo, null_count)
+
+    def _c(self) -> _capi.ListStringsColumn:
+        torch = _torch()
+        if self.offsets is not None and self.offsets.dtype != torch.int32:
+            raise TypeError("list offsets must be int32")
+        return _capi.ListStringsColumn(
+            self.offsets.data_ptr() if self.offsets is not None else None,
+            self.mask.data_ptr() if self.mask is not None else None,
+            self.size, self.offset, self.null_count, self.child._c())
+
+
+@dataclass
 class DeviceListColumn:
     """LIST result in HBM.  offsets: int32 tensor; child: raw tensor viewed as child_dtype."""
     offsets: object
@@ -195,6 +228,38 @@ def minhash64(input: DeviceStringsColumn, seed: int, a, b, width: int) -> Device
     st = L.nvtext_amd_minhash64(C.byref(col), int(seed), ta.data_ptr() if ta.numel() else None,
                                 tb.data_ptr() if tb.numel() else None, ta.numel(), tb.numel(), int(width),
                                 _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    return _wrap(out)
+
+
+def minhash_ngrams(input: DeviceListStringsColumn, ngrams: int, seed: int, a, b) -> DeviceListColumn:
+    """nvtext::minhash_ngrams (cpp/include/nvtext/minhash.hpp:156-163); pylibcudf minhash.pyx minhash_ngrams."""
+    L = _capi.load()
+    if not (0 <= int(seed) < 2**32):
+        raise ValueError("seed must fit uint32")
+    ta, tb = _param_tensor(a, np.uint32), _param_tensor(b, np.uint32)
+    out = _capi.ListColumn()
+    col = input._c()
+    st = L.nvtext_amd_minhash_ngrams(C.byref(col), int(ngrams), int(seed), ta.data_ptr() if ta.numel() else None,
+                                     tb.data_ptr() if tb.numel() else None, ta.numel(), tb.numel(),
+                                     _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    return _wrap(out)
+
+
+def minhash64_ngrams(input: DeviceListStringsColumn, ngrams: int, seed: int, a, b) -> DeviceListColumn:
+    """nvtext::minhash64_ngrams (cpp/include/nvtext/minhash.hpp:203-210); pylibcudf minhash.pyx minhash64_ngrams."""
+    L = _capi.load()
+    if not (0 <= int(seed) < 2**64):
+        raise ValueError("seed must fit uint64")
+    ta, tb = _param_tensor(a, np.uint64), _param_tensor(b, np.uint64)
+    out = _capi.ListColumn()
+    col = input._c()
+    st = L.nvtext_amd_minhash64_ngrams(C.byref(col), int(ngrams), int(seed), ta.data_ptr() if ta.numel() else None,
+                                       tb.data_ptr() if tb.numel() else None, ta.numel(), tb.numel(),
+                                       _stream_handle(), C.byref(_mr().struct), C.byref(out))
     if st != _capi.SUCCESS:
         _raise(st)
     return _wrap(out)

@@ -80,6 +80,18 @@ typedef struct nvtext_amd_list_column {
   size_t    null_mask_bytes;
 } nvtext_amd_list_column;
 
+/* LIST<STRING> input column (cpp/include/cudf/lists/lists_column_view.hpp:33-120): int32 list offsets
+ * (size + offset + 1 entries) that index the elements of `child`, optional row validity, and the view's
+ * offset / size for a sliced column.  `child` describes all the elements (its own offset applies on top). */
+typedef struct nvtext_amd_list_strings_column {
+  const int32_t*  offsets;
+  const uint32_t* null_mask;
+  int32_t         size;
+  int32_t         offset;
+  int32_t         null_count;
+  nvtext_amd_strings_column child;
+} nvtext_amd_list_strings_column;
+
 typedef struct nvtext_amd_wordpiece_vocabulary nvtext_amd_wordpiece_vocabulary;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -116,6 +128,36 @@ nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input,
                                        void* stream,
                                        const nvtext_amd_allocator* mr,
                                        nvtext_amd_list_column* out);
+
+/* Replaces nvtext::minhash_ngrams (cpp/include/nvtext/minhash.hpp:156-163; cpp/src/text/minhash.cu:703-714).
+ * The hashed items are runs of consecutive strings of a LIST<STRING> row: for element i the bytes from the
+ * start of element i to the end of element min(i + ngrams, last) (adjacent elements are contiguous in the
+ * child's chars), MurmurHash3_x86_32(seed), for i in [0, max(1, elements - ngrams + 1)); a run that the row
+ * cuts short counts only at i = 0, a null element starts no run.  Permutation, minimum and result layout
+ * as nvtext_amd_minhash: LIST<UINT32>, param_count values per valid row, zeros for an empty row. */
+nvtext_amd_status nvtext_amd_minhash_ngrams(const nvtext_amd_list_strings_column* input,
+                                            int32_t ngrams,
+                                            uint32_t seed,
+                                            const uint32_t* a,
+                                            const uint32_t* b,
+                                            int64_t a_count,
+                                            int64_t b_count,
+                                            void* stream,
+                                            const nvtext_amd_allocator* mr,
+                                            nvtext_amd_list_column* out);
+
+/* Replaces nvtext::minhash64_ngrams (cpp/include/nvtext/minhash.hpp:203-210; cpp/src/text/minhash.cu:728-739).
+ * MurmurHash3_x64_128(seed) word 0; permutation ((hash*a+b) mod 2^64) % (2^61-1).  Result: LIST<UINT64>. */
+nvtext_amd_status nvtext_amd_minhash64_ngrams(const nvtext_amd_list_strings_column* input,
+                                              int32_t ngrams,
+                                              uint64_t seed,
+                                              const uint64_t* a,
+                                              const uint64_t* b,
+                                              int64_t a_count,
+                                              int64_t b_count,
+                                              void* stream,
+                                              const nvtext_amd_allocator* mr,
+                                              nvtext_amd_list_column* out);
 
 /* Replaces nvtext::load_wordpiece_vocabulary / wordpiece_vocabulary::wordpiece_vocabulary
  * (cpp/include/nvtext/wordpiece_tokenize.hpp:26-66; cpp/src/text/wordpiece_tokenize.cu:213-293).

@@ -1,5 +1,6 @@
 // Exercises the C++ mirror of the nvtext API (cudf_amd/include) on the GPU with the cases of the
-// reference's gtests: cpp/tests/text/minhash_tests.cpp (Permuted, PermutedWide, EmptyTest, ErrorsTest)
+// reference's gtests: cpp/tests/text/minhash_tests.cpp (Permuted, PermutedWide, EmptyTest, ErrorsTest, Ngrams, NgramsWide,
+// NgramsSliced)
 // and cpp/tests/text/subword_tests.cpp (all seven).  Own tiny harness: prints one line per case and
 // exits non-zero on the first failure.
 #include <cudf/column/column.hpp>
@@ -203,6 +204,79 @@ void test_minhash_empty_and_errors()
   EXPECT_THROW(nvtext::minhash64(bview, 0, zeros64, zeros64, 4), std::overflow_error);
 }
 
+// lists column of strings as cudf::test::lists_column_wrapper<cudf::string_view> builds it
+cudf::column_view make_list_strings(std::vector<std::vector<Text>> const& rows)
+{
+  using namespace cudf;
+  std::vector<Text> flat;
+  std::vector<int32_t> offsets{0};
+  for (auto const& r : rows) {
+    flat.insert(flat.end(), r.begin(), r.end());
+    offsets.push_back(static_cast<int32_t>(flat.size()));
+  }
+  if (rows.empty()) return column_view{data_type{type_id::LIST}, 0, nullptr, nullptr, 0};
+  column_view off{data_type{type_id::INT32}, static_cast<size_type>(offsets.size()), upload(offsets), nullptr, 0};
+  return column_view{data_type{type_id::LIST}, static_cast<size_type>(rows.size()), nullptr, nullptr, 0, 0, {off, make_strings(flat).view}};
+}
+
+void test_minhash_ngrams()
+{
+  std::printf("minhash_ngrams (Ngrams, NgramsWide, NgramsSliced, errors)\n");
+  std::vector<Text> const row_a{"The", "quick", "brown", "fox", "jump\xc3\xa9" "d", "over", "the", "lazy", "brown", "dog."};
+  std::vector<Text> const row_b{"The", "quick", "brown", "fox", "jump\xc3\xa9" "d", "over", "the", "lazy", "", "dog."};
+  std::vector<Text> const row_c{"short", "row"};
+  std::vector<Text> const ignored{"ignored", "row"};
+  std::vector<uint32_t> const p32{10, 11, 12};
+  std::vector<uint64_t> const p64{10, 11, 12};
+  auto const a32 = make_fixed(p32);
+  auto const a64 = make_fixed(p64);
+  L<uint32_t> const e32{{{230924604u, 55492793u, 963436400u}}, {{230924604u, 367515795u, 963436400u}}, {{2380648568u, 1330223236u, 279797904u}}};
+  L<uint64_t> const e64{{{208926840193078200ul, 576399628675212695ul, 312927673584437419ul}},
+                        {{677038498284219393ul, 326338087730412201ul, 298455901014050223ul}},
+                        {{1493265692486268500ul, 720255058049417768ul, 2253087432826260995ul}}};
+  {
+    auto const input = make_list_strings({row_a, row_b, row_c});
+    cudf::lists_column_view view(input);
+    CHECK(same(download<uint32_t>(*nvtext::minhash_ngrams(view, 4, 0, a32, a32)), e32));
+    CHECK(same(download<uint64_t>(*nvtext::minhash64_ngrams(view, 4, 0, a64, a64)), e64));
+  }
+  {
+    auto const input = make_list_strings({ignored, row_a, row_b, row_c, ignored});
+    cudf::lists_column_view view(slice(input, 1, 4));
+    CHECK(same(download<uint32_t>(*nvtext::minhash_ngrams(view, 4, 0, a32, a32)), e32));
+    CHECK(same(download<uint64_t>(*nvtext::minhash64_ngrams(view, 4, 0, a64, a64)), e64));
+  }
+  {
+    std::vector<Text> const many(512, Text{"hello"});
+    auto const input = make_list_strings({many, many});
+    cudf::lists_column_view view(input);
+    L<uint32_t> const w32{{{571536396u, 2346676954u, 4121817512u}}, {{571536396u, 2346676954u, 4121817512u}}};
+    L<uint64_t> const w64{{{1947142336021414174ul, 1219519365938078011ul, 491896395854741840ul}},
+                          {{1947142336021414174ul, 1219519365938078011ul, 491896395854741840ul}}};
+    CHECK(same(download<uint32_t>(*nvtext::minhash_ngrams(view, 4, 0, a32, a32)), w32));
+    CHECK(same(download<uint64_t>(*nvtext::minhash64_ngrams(view, 4, 0, a64, a64)), w64));
+  }
+  {
+    auto const empty_list = make_list_strings({});
+    cudf::lists_column_view lview(empty_list);
+    auto const e  = make_fixed(std::vector<uint32_t>{});
+    auto const ee = make_fixed(std::vector<uint64_t>{});
+    EXPECT_THROW(nvtext::minhash_ngrams(lview, 0, 0, e, e), std::invalid_argument);
+    EXPECT_THROW(nvtext::minhash64_ngrams(lview, 0, 0, ee, ee), std::invalid_argument);
+    EXPECT_THROW(nvtext::minhash_ngrams(lview, 4, 0, e, e), std::invalid_argument);
+    EXPECT_THROW(nvtext::minhash64_ngrams(lview, 4, 0, ee, ee), std::invalid_argument);
+    CHECK(nvtext::minhash_ngrams(lview, 4, 0, a32, a32)->size() == 0);
+    CHECK(nvtext::minhash64_ngrams(lview, 4, 0, a64, a64)->size() == 0);
+    std::vector<std::vector<Text>> const big(50000, std::vector<Text>{Text{""}});
+    auto const input = make_list_strings(big);
+    cudf::lists_column_view view(input);
+    auto const z32 = make_fixed(std::vector<uint32_t>(50000, 0u));
+    auto const z64 = make_fixed(std::vector<uint64_t>(50000, 0ul));
+    EXPECT_THROW(nvtext::minhash_ngrams(view, 4, 0, z32, z32), std::overflow_error);
+    EXPECT_THROW(nvtext::minhash64_ngrams(view, 4, 0, z64, z64), std::overflow_error);
+  }
+}
+
 void test_wordpiece()
 {
   std::printf("TextSubwordTest.WordPiece / WordPieceSliced\n");
@@ -282,6 +356,7 @@ int main()
   test_minhash_permuted();
   test_minhash_wide();
   test_minhash_empty_and_errors();
+  test_minhash_ngrams();
   test_wordpiece();
   test_wordpiece_subwords();
   test_wordpiece_edges();

@@ -174,6 +174,74 @@ def test_minhash_errors_and_empty(nv):
     assert got.size == 0 and got.child.size == 0
 
 
+# ----------------------------------------------------------------------------- minhash_ngrams
+def ldev(nv, host):
+    return nv.DeviceListStringsColumn.from_host(host)
+
+
+@pytest.mark.parametrize("case", gc.minhash_ngrams_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_minhash_ngrams_golden(nv, case, dtype):
+    host = gc.list_strings(case["rows"], dtype)
+    d = ldev(nv, host)
+    if "slice" in case:
+        lo, hi = case["slice"]
+        d = d.slice(lo, hi, 0)
+    a32, b32 = np.array(case["a"], np.uint32), np.array(case["b"], np.uint32)
+    assert nv.minhash_ngrams(d, case["ngrams"], case["seed"], a32, b32).to_host().to_pylist() == case["expected32"]
+    got = nv.minhash64_ngrams(d, case["ngrams"], case["seed"], a32.astype(np.uint64), b32.astype(np.uint64)).to_host()
+    assert got.to_pylist() == case["expected64"] and got.child.dtype == np.uint64
+
+
+@pytest.mark.parametrize("P,ngrams", [(3, 2), (64, 5), (100, 3), (260, 10)])
+def test_minhash_ngrams_random_vs_oracle(nv, orc, P, ngrams):
+    rng = np.random.default_rng(1000 + P)
+    letters = list("abcdefghijé漢 ")
+    rows = []
+    for _ in range(700):
+        u = rng.random()
+        if u < 0.05:
+            rows.append(None)
+            continue
+        n = 0 if u < 0.1 else int(rng.integers(1, 40)) if u < 0.9 else int(rng.integers(200, 600))
+        row = []
+        for _ in range(n):
+            t = rng.random()
+            row.append(None if t < 0.04 else "" if t < 0.08 else "".join(rng.choice(letters, int(rng.integers(1, 14)))))
+        rows.append(row)
+    for dtype in (np.int32, np.int64):
+        host = gc.list_strings(rows, dtype)
+        d = ldev(nv, host)
+        a = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        b = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        assert_same(nv.minhash_ngrams(d, ngrams, 7, a, b).to_host(), orc.minhash_ngrams(host, ngrams, 7, a, b, nthreads=4), f"ngrams u32 P={P}")
+        a64 = rng.integers(1, 2**64, P, dtype=np.uint64)
+        b64 = rng.integers(0, 2**64, P, dtype=np.uint64)
+        assert_same(nv.minhash64_ngrams(d, ngrams, 99, a64, b64).to_host(), orc.minhash64_ngrams(host, ngrams, 99, a64, b64, nthreads=4),
+                    f"ngrams u64 P={P}")
+        for lo, hi in [(3, 650), (100, 101)]:
+            hs = host.slice(lo, hi)
+            assert_same(nv.minhash_ngrams(d.slice(lo, hi, hs.null_count), ngrams, 7, a, b).to_host(),
+                        orc.minhash_ngrams(hs, ngrams, 7, a, b), f"ngrams slice {lo}:{hi}")
+
+
+def test_minhash_ngrams_wide_row_and_errors(nv, orc):
+    rng = np.random.default_rng(5)
+    words = ["".join(rng.choice(list("abcdef"), int(rng.integers(1, 9)))) for _ in range(300_000)]
+    host = gc.list_strings([words, words[:3], words[:70_000]])
+    a = np.arange(1, 6, dtype=np.uint32)
+    assert_same(nv.minhash_ngrams(ldev(nv, host), 5, 0, a, a).to_host(), orc.minhash_ngrams(host, 5, 0, a, a, nthreads=8), "wide rows")
+    d = ldev(nv, gc.list_strings([["a", "b"]]))
+    with pytest.raises(ValueError):
+        nv.minhash_ngrams(d, 1, 0, a, a)
+    with pytest.raises(ValueError):
+        nv.minhash_ngrams(d, 2, 0, a[:0], a[:0])
+    with pytest.raises(ValueError):
+        nv.minhash64_ngrams(d, 2, 0, np.zeros(3, np.uint64), np.zeros(2, np.uint64))
+    empty = nv.minhash_ngrams(ldev(nv, gc.list_strings([])), 4, 0, a, a).to_host()
+    assert empty.size == 0 and empty.child.size == 0
+
+
 # ----------------------------------------------------------------------------- wordpiece
 @pytest.mark.parametrize("case", gc.wordpiece_cases(), ids=lambda c: c["name"])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
