@@ -26,9 +26,9 @@ VALU_PEAK_TOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 lanes x 2.4 GHz: one 32
 # raw readings are in profiles/hbm_traffic_pmc_C2_C3_C4.md.  Counters cannot be read from inside this
 # process, so the line reports these figures only for the workload they were measured on.
 MEASURED_TRAFFIC_C2 = {
-    "wordpiece_probe_kernel": (1735_700_000, 1955_600_000),
-    "wordpiece_oov_kernel": (1515_000_000, 1390_600_000),
-    "wordpiece_emit_kernel": (2179_700_000, 848_000_000),
+    "wordpiece_probe_kernel": (1702_800_000, 1962_700_000),
+    "wordpiece_oov_kernel": (1061_400_000, 1428_100_000),
+    "wordpiece_emit_kernel": (2179_500_000, 848_000_000),
 }
 
 
@@ -198,6 +198,48 @@ def main():
             log(f"[bench] {name}: {leg}")
             extra["minhash" if name == "C3" else "minhash64"] = leg
             del dc, keep
+
+    # ------------------------------------------------------------------ minhash_ngrams over the words of C3 (a quarter of its rows)
+    if args.minhash_scale > 0:
+        torch.cuda.empty_cache()
+        t0 = time.time()
+        w = datagen.config3(0.25 * args.minhash_scale)
+        p = w.params
+        lists = datagen.words_as_lists(w.rows)
+        a, b = datagen.make_params(p["P"], 32, p["param_seed"])
+        da = torch.from_numpy(a.view(np.int32)).cuda()
+        db = torch.from_numpy(b.view(np.int32)).cuda()
+        log(f"[bench] word lists of C3 x{0.25 * args.minhash_scale}: rows={lists.size} elements={lists.child.size} in {time.time() - t0:.1f}s")
+        dl = nvtext.DeviceListStringsColumn.from_host(lists)
+        keep = {}
+        ngrams = 5
+
+        def nstep():
+            keep["o"] = nvtext.minhash_ngrams(dl, ngrams, p["seed"], da, db)
+
+        nsec = timed_steps(nstep, max(3, args.steps // 2), 1, torch)
+        nk = kernel_times(nstep, 2, _capi, torch)
+        nb = lists.child.chars.size + (lists.child.size + 1) * lists.child.offsets.dtype.itemsize + (lists.size + 1) * 4
+        leg = {"workload": f"words of C3 x{0.25 * args.minhash_scale} as LIST<STRING>, ngrams={ngrams}, P={p['P']}", "rows": lists.size,
+               "elements": lists.child.size, "ms_per_step": round(nsec * 1e3, 3), "input_GBps": round(nb / nsec / 1e9, 2),
+               "mrows_per_s": round(lists.size / nsec / 1e6, 3), "gperm_per_s": round(lists.child.size * p["P"] / nsec / 1e9, 1),
+               "kernels_ms": {k: round(v, 3) for k, v in nk.items()}}
+        if not args.no_cpu:
+            from oracle import pyoracle as orc
+            n = min(lists.size, 20000)
+            smp = lists.slice(0, n)
+            threads = max(1, min(orc.hardware_threads(), 16))
+            t0 = time.perf_counter()
+            exp = orc.minhash_ngrams(smp, ngrams, p["seed"], a, b, nthreads=threads)
+            cs = time.perf_counter() - t0
+            got = nvtext.minhash_ngrams(dl.slice(0, n, smp.null_count), ngrams, p["seed"], da, db).to_host()
+            sample_bytes = int(lists.child.offsets[lists.offsets[n]])
+            leg["cpu_baseline"] = {"value": round(sample_bytes / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
+                                   "sample": f"first {n} rows ({sample_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+            leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
+        log(f"[bench] minhash_ngrams: {leg}")
+        extra["minhash_ngrams"] = leg
+        del dl, keep
 
     # ------------------------------------------------------------------ C5: UTF-8 rows, int64 offsets, 250k vocabulary
     if args.minhash_scale > 0:

@@ -13,7 +13,7 @@ from typing import Optional
 
 import numpy as np
 
-from ..arrow_host import HostStringsColumn
+from ..arrow_host import HostListStringsColumn, HostStringsColumn
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libnvtext_datagen.so")
@@ -149,6 +149,21 @@ def config5(scale: float = 1.0) -> Workload:
     rows = make_rows(vocab, rows=int(8_000_000 * scale), seed=5, mean_bytes=512.0, sigma=0.6, cap_bytes=8192, zipf_s=1.1,
                      p_oov=0.10, multilingual=True, min_bytes=2, offsets_dtype=np.int64)
     return Workload("C5", rows, vocab, dict(max_words_per_row=256, width=8, seed=5, P=64, hash_bits=64, param_seed=55))
+
+
+def words_as_lists(rows: HostStringsColumn) -> HostListStringsColumn:
+    """The rows of a generated strings column (single spaces, none leading or trailing) as LIST<STRING> rows over the
+    same chars: element = a word together with the space that follows it, so that the elements of a row tile its bytes
+    (the layout a tokenizer's output has when it keeps the separators).  Null rows stay null, empty rows are empty lists."""
+    chars = np.ascontiguousarray(rows.chars)
+    roff = np.ascontiguousarray(rows.offsets).astype(np.int64)
+    assert rows.offset == 0
+    after_space = np.flatnonzero(chars == 0x20).astype(np.int64) + 1
+    starts = np.union1d(after_space, roff[:-1][np.diff(roff) > 0])
+    child_offsets = np.concatenate([starts, roff[-1:]]).astype(rows.offsets.dtype)
+    list_offsets = np.searchsorted(starts, roff, side="left").astype(np.int32)
+    child = HostStringsColumn(chars, child_offsets, None, int(starts.size), 0, 0)
+    return HostListStringsColumn(list_offsets, child, rows.mask, rows.size, 0, rows.null_count)
 
 
 CONFIGS = {"C1": config1, "C2": config2, "C3": config3, "C4": config4, "C5": config5}
