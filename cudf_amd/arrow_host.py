@@ -142,6 +142,35 @@ class HostListStringsColumn:
 
 
 @dataclass
+class HostFixedColumn:
+    """Fixed-width column (here FLOAT32 results): values, optional validity mask."""
+    values: np.ndarray
+    mask: Optional[np.ndarray]
+    size: int
+    null_count: int = 0
+
+    def validity(self) -> np.ndarray:
+        if self.mask is None:
+            return np.ones(self.size, dtype=bool)
+        return unpack_validity(self.mask, self.size, 0)
+
+    def to_pylist(self):
+        v = self.validity()
+        return [self.values[i].item() if v[i] else None for i in range(self.size)]
+
+    def equals(self, other: "HostFixedColumn") -> bool:
+        """Size, null count, validity and the bits of every valid value."""
+        if self.size != other.size or self.null_count != other.null_count or self.values.dtype != other.values.dtype:
+            return False
+        v = self.validity()
+        if not np.array_equal(v, other.validity()):
+            return False
+        a = np.ascontiguousarray(self.values[: self.size]).view(np.uint32)
+        b = np.ascontiguousarray(other.values[: other.size]).view(np.uint32)
+        return bool(np.array_equal(a[v], b[v]))
+
+
+@dataclass
 class HostListColumn:
     """LIST<INT32|UINT32|UINT64> result (cpp/src/lists/lists_column_factories.cu:106-129):
     int32 offsets (size+1 entries, or 0 entries for the canonical empty list column),

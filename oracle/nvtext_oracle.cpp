@@ -22,6 +22,7 @@
 // Build: make -C oracle   (g++ -O2 -std=c++17 -shared -fPIC -pthread)
 
 #include <algorithm>
+#include <iterator>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -413,6 +414,66 @@ int minhash_ngrams_impl(ListStringsCol const& col, int32_t ngrams, T seed, T con
 }
 
 // ---------------------------------------------------------------------------
+// jaccard_index -- cpp/src/text/jaccard.cu:196-292 (substring hashes), 66-170 (unique and
+// intersect counts), 405-479 (index, argument checks, nulls)
+// ---------------------------------------------------------------------------
+// The distinct non-zero MurmurHash3_x86_32(seed 0) values of the `width`-character windows of a row, sorted.
+// jaccard.cu:272-277: a window is hashed at every character start that has `width` characters left, and at
+// the first byte whatever is left; 282-286: hash values of 0 are dropped when the hashes are compacted.
+inline std::vector<uint32_t> window_hash_set(uint8_t const* s, int64_t n, int32_t width)
+{
+  std::vector<uint32_t> h;
+  for (int64_t i = 0; i < n; ++i) {
+    if (is_utf8_continuation_char(s[i])) continue;
+    int64_t bytes;
+    int left;
+    bytes_to_character_position(s + i, n - i, width, bytes, left);
+    if (i != 0 && left > 0) continue;
+    bytes             = std::min<int64_t>(bytes, n - i);
+    uint32_t const hv = murmur3_x86_32(s + i, bytes, 0);
+    if (hv != 0) h.push_back(hv);
+  }
+  std::sort(h.begin(), h.end());
+  h.erase(std::unique(h.begin(), h.end()), h.end());
+  return h;
+}
+
+int jaccard_impl(StringsCol const& c1, StringsCol const& c2, int32_t width, int nthreads, float* out, uint32_t* out_mask,
+                 int32_t* out_null_count)
+{
+  // jaccard.cu:441-446, in this order
+  if (c1.size != c2.size) return INVALID_ARGUMENT;
+  if (width < 2) return INVALID_ARGUMENT;
+  *out_null_count = 0;
+  if (c1.size == 0) return OK;
+  parallel_rows(c1.size, nthreads, [&](int, int32_t lo, int32_t hi) {
+    for (int32_t r = lo; r < hi; ++r) {
+      // 211-220: null and empty rows have no hashes
+      std::vector<uint32_t> a, b;
+      if (c1.valid(r)) a = window_hash_set(c1.chars + c1.off(r), c1.off(r + 1) - c1.off(r), width);
+      if (c2.valid(r)) b = window_hash_set(c2.chars + c2.off(r), c2.off(r + 1) - c2.off(r), width);
+      std::vector<uint32_t> both;
+      std::set_intersection(a.begin(), a.end(), b.begin(), b.end(), std::back_inserter(both));
+      // 414-425
+      int32_t const intersects = static_cast<int32_t>(both.size());
+      int32_t const unions     = static_cast<int32_t>(a.size()) + static_cast<int32_t>(b.size()) - intersects;
+      out[r]                   = unions ? static_cast<float>(intersects) / static_cast<float>(unions) : 0.f;
+    }
+  });
+  // 471-476: with nulls in either input the validity is the AND of both
+  if (c1.null_count > 0 || c2.null_count > 0) {
+    int32_t nulls = 0;
+    for (int32_t r = 0; r < c1.size; ++r) {
+      bool const v = c1.valid(r) && c2.valid(r);
+      if (v) out_mask[r >> 5] |= 1u << (r & 31);
+      nulls += !v;
+    }
+    *out_null_count = nulls;
+  }
+  return OK;
+}
+
+// ---------------------------------------------------------------------------
 // wordpiece vocabulary -- cpp/src/text/wordpiece_tokenize.cu:184-209, 213-282
 // ---------------------------------------------------------------------------
 struct Vocab {
@@ -563,6 +624,18 @@ int oracle_minhash64_ngrams(int32_t const* list_offsets, uint32_t const* list_ma
   ListStringsCol c{list_offsets, list_mask, size, offset, null_count,
                    StringsCol{chars, child_offsets, child_offsets_is_int64, child_mask, child_size, child_offset, 0}};
   return minhash_ngrams_impl<uint64_t>(c, ngrams, seed, a, b, P, nthreads, out_offsets, out_child, out_child_len);
+}
+
+// out: size floats; out_mask: ceil(size/32) zeroed words, written only when an input has nulls (then *out_has_mask = 1).
+int oracle_jaccard_index(uint8_t const* chars1, void const* offsets1, int offsets1_is_int64, uint32_t const* mask1, int32_t size1,
+                         int32_t offset1, int32_t null_count1, uint8_t const* chars2, void const* offsets2, int offsets2_is_int64,
+                         uint32_t const* mask2, int32_t size2, int32_t offset2, int32_t null_count2, int32_t width, int nthreads,
+                         float* out, uint32_t* out_mask, int32_t* out_null_count, int32_t* out_has_mask)
+{
+  StringsCol a{chars1, offsets1, offsets1_is_int64, mask1, size1, offset1, null_count1};
+  StringsCol b{chars2, offsets2, offsets2_is_int64, mask2, size2, offset2, null_count2};
+  *out_has_mask = (null_count1 > 0 || null_count2 > 0) ? 1 : 0;
+  return jaccard_impl(a, b, width, nthreads, out, out_mask, out_null_count);
 }
 
 // wordpiece_tokenize.cu:213-282.  Returns INVALID_ARGUMENT for an empty vocabulary

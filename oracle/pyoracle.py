@@ -58,6 +58,9 @@ def lib():
         L.oracle_minhash64_ngrams.restype = C.c_int
         L.oracle_minhash64_ngrams.argtypes = lcol + [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int,
                                                      C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
+        L.oracle_jaccard_index.restype = C.c_int
+        L.oracle_jaccard_index.argtypes = col + col + [C.c_int32, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32),
+                                                       C.POINTER(C.c_int32)]
         L.oracle_vocab_create.restype = C.c_int
         L.oracle_vocab_create.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int32, C.c_int32, C.c_int32,
                                           C.POINTER(C.c_void_p)]
@@ -177,6 +180,22 @@ def minhash_ngrams(col, ngrams, seed, a, b, nthreads: int = 1):
 
 def minhash64_ngrams(col, ngrams, seed, a, b, nthreads: int = 1):
     return _minhash_ngrams(col, ngrams, seed, a, b, np.uint64, lib().oracle_minhash64_ngrams, nthreads)
+
+
+def jaccard_index(col1, col2, width, nthreads: int = 1):
+    from cudf_amd.arrow_host import HostFixedColumn
+    keep1, a1 = _col_args(col1)
+    keep2, a2 = _col_args(col2)
+    rows = int(col1.size)
+    out = np.zeros(rows, dtype=np.float32)
+    mask = np.zeros((rows + 31) // 32, dtype=np.uint32)
+    nulls = C.c_int32(0)
+    has_mask = C.c_int32(0)
+    rc = lib().oracle_jaccard_index(*a1, *a2, width, nthreads, _p(out) if rows else None, _p(mask) if rows else None,
+                                    C.byref(nulls), C.byref(has_mask))
+    if rc != OK:
+        raise OracleError(rc)
+    return HostFixedColumn(out, mask if has_mask.value and rows else None, rows, int(nulls.value))
 
 
 class Vocabulary:

@@ -45,6 +45,10 @@ def list_strings(rows, child_offsets_dtype=np.int32) -> HostListStringsColumn:
     return HostListStringsColumn.from_pylist(rows, child_offsets_dtype)
 
 
+def jaccard_cases():
+    return json.load(open(os.path.join(GOLDEN, "jaccard_vectors.json"), encoding="utf-8"))["cases"]
+
+
 def murmur64_vectors():
     return json.load(open(os.path.join(GOLDEN, "minhash_vectors.json"), encoding="utf-8"))["murmurhash3_x64_128_word0"]
 

@@ -126,6 +126,56 @@ def test_minhash_errors_and_empty():
 
 
 # ----------------------------------------------------------------------------- wordpiece
+def check_jaccard_case(got, case):
+    exp = np.array(case["expected"], np.float32)
+    valid = np.array(case.get("expected_valid", [True] * len(exp)))
+    assert got.size == len(exp) and np.array_equal(got.validity(), valid)
+    assert got.null_count == int((~valid).sum()) and (got.mask is not None) == ("expected_valid" in case)
+    if "tolerance" in case:  # values printed with six digits
+        assert np.allclose(got.values[valid], exp[valid], atol=case["tolerance"], rtol=0)
+    else:  # float32 literals: bit-exact
+        assert np.array_equal(got.values[valid].view(np.uint32), exp[valid].view(np.uint32))
+
+
+@pytest.mark.parametrize("case", gc.jaccard_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_jaccard_golden(case, dtype):
+    got = orc.jaccard_index(strings(case["input1"], dtype), strings(case["input2"], dtype), case["width"])
+    check_jaccard_case(got, case)
+    check_jaccard_case(orc.jaccard_index(strings(case["input2"], dtype), strings(case["input1"], dtype), case["width"]), case)
+
+
+def brute_force_jaccard(s1, s2, width):
+    """The definition on the substrings themselves (no hashing), as the reference's Python test builds it from
+    character_ngrams (test_text_methods.py:971-1010); rows shorter than width contribute the whole row."""
+    def grams(t):
+        if len(t) == 0:
+            return set()
+        return {t} if len(t) < width else {t[i:i + width] for i in range(len(t) - width + 1)}
+    a, b = grams(s1), grams(s2)
+    u = len(a | b)
+    return np.float32(len(a & b)) / np.float32(u) if u else np.float32(0)
+
+
+def test_jaccard_matches_the_set_definition():
+    rng = np.random.default_rng(31)
+    alphabet = list("abcdé漢 ")
+    rows1, rows2 = [], []
+    for _ in range(400):
+        common = "".join(rng.choice(alphabet, int(rng.integers(0, 60))))
+        rows1.append("".join(rng.choice(alphabet, int(rng.integers(0, 12)))) + common)
+        rows2.append("".join(rng.choice(alphabet, int(rng.integers(0, 25)))) + common)
+    for width in (2, 5, 9):
+        got = orc.jaccard_index(strings(rows1), strings(rows2), width, nthreads=2)
+        exp = np.array([brute_force_jaccard(x, y, width) for x, y in zip(rows1, rows2)], np.float32)
+        assert np.array_equal(got.values.view(np.uint32), exp.view(np.uint32)), width
+    with pytest.raises(OracleError):
+        orc.jaccard_index(strings(["1", "2", "3"]), strings(["1", "2", "3"]), 1)
+    with pytest.raises(OracleError):
+        orc.jaccard_index(strings(["1", "2", "3"]), strings(["1", "2"]), 5)
+    assert orc.jaccard_index(strings([]), strings([]), 5).size == 0
+
+
 @pytest.mark.parametrize("case", gc.minhash_ngrams_cases(), ids=lambda c: c["name"])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_minhash_ngrams_golden(case, dtype):
