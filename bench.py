@@ -241,6 +241,41 @@ def main():
         extra["minhash_ngrams"] = leg
         del dl, keep
 
+    # ------------------------------------------------------------------ jaccard_index of neighbouring rows of C3 (a quarter of its rows)
+    if args.minhash_scale > 0:
+        torch.cuda.empty_cache()
+        w = datagen.config3(0.25 * args.minhash_scale)
+        n = w.rows.size - 1
+        dc = nvtext.DeviceStringsColumn.from_host(w.rows)
+        d1, d2 = dc.slice(0, n, 0), dc.slice(1, n + 1, 0)
+        keep = {}
+        jwidth = 5
+
+        def jstep():
+            keep["o"] = nvtext.jaccard_index(d1, d2, jwidth)
+
+        jsec = timed_steps(jstep, max(3, args.steps // 2), 1, torch)
+        jk = kernel_times(jstep, 2, _capi, torch)
+        jb = 2 * input_bytes(w.rows)
+        leg = {"workload": f"rows r and r+1 of C3 x{0.25 * args.minhash_scale}, width={jwidth}", "rows": n,
+               "ms_per_step": round(jsec * 1e3, 3), "input_GBps": round(jb / jsec / 1e9, 2), "mrows_per_s": round(n / jsec / 1e6, 3),
+               "kernels_ms": {k: round(v, 3) for k, v in jk.items()}}
+        if not args.no_cpu:
+            from oracle import pyoracle as orc
+            m = min(n, 20000)
+            s1, s2 = w.rows.slice(0, m), w.rows.slice(1, m + 1)
+            threads = max(1, min(orc.hardware_threads(), 16))
+            t0 = time.perf_counter()
+            exp = orc.jaccard_index(s1, s2, jwidth, nthreads=threads)
+            cs = time.perf_counter() - t0
+            got = nvtext.jaccard_index(dc.slice(0, m, 0), dc.slice(1, m + 1, 0), jwidth).to_host()
+            leg["cpu_baseline"] = {"value": round(2 * input_bytes(s1) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
+                                   "sample": f"first {m} row pairs ({2 * s1.chars_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+            leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
+        log(f"[bench] jaccard_index: {leg}")
+        extra["jaccard_index"] = leg
+        del dc, d1, d2, keep
+
     # ------------------------------------------------------------------ C5: UTF-8 rows, int64 offsets, 250k vocabulary
     if args.minhash_scale > 0:
         torch.cuda.empty_cache()

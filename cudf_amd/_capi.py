@@ -8,7 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnvtext_amd.so")
 
 SUCCESS, INVALID_ARGUMENT, OVERFLOW, LOGIC_ERROR, DEVICE_ERROR, ALLOC_FAILED = range(6)
-TYPE_INT32, TYPE_UINT32, TYPE_UINT64 = 3, 7, 8
+TYPE_INT32, TYPE_UINT32, TYPE_UINT64, TYPE_FLOAT32 = 3, 7, 8, 9
 
 EXPORTS = [
     "nvtext_amd_version",
@@ -17,6 +17,8 @@ EXPORTS = [
     "nvtext_amd_minhash64",
     "nvtext_amd_minhash_ngrams",
     "nvtext_amd_minhash64_ngrams",
+    "nvtext_amd_jaccard_index",
+    "nvtext_amd_fixed_column_free",
     "nvtext_amd_wordpiece_vocabulary_create",
     "nvtext_amd_wordpiece_vocabulary_destroy",
     "nvtext_amd_wordpiece_vocabulary_unk_id",
@@ -74,6 +76,18 @@ class ListColumn(C.Structure):
     ]
 
 
+class FixedColumn(C.Structure):
+    _fields_ = [
+        ("type", C.c_int32),
+        ("size", C.c_int32),
+        ("null_count", C.c_int32),
+        ("data", C.c_void_p),
+        ("null_mask", C.c_void_p),
+        ("data_bytes", C.c_size_t),
+        ("null_mask_bytes", C.c_size_t),
+    ]
+
+
 _lib = None
 
 
@@ -107,6 +121,11 @@ def load():
     L.nvtext_amd_minhash64_ngrams.restype = C.c_int
     L.nvtext_amd_minhash64_ngrams.argtypes = [C.POINTER(ListStringsColumn), C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p,
                                               C.c_int64, C.c_int64] + common_tail[1:]
+    L.nvtext_amd_jaccard_index.restype = C.c_int
+    L.nvtext_amd_jaccard_index.argtypes = [C.POINTER(StringsColumn), C.POINTER(StringsColumn), C.c_int32, C.c_void_p,
+                                           C.POINTER(Allocator), C.POINTER(FixedColumn)]
+    L.nvtext_amd_fixed_column_free.restype = None
+    L.nvtext_amd_fixed_column_free.argtypes = [C.POINTER(FixedColumn), C.c_void_p, C.POINTER(Allocator)]
     L.nvtext_amd_wordpiece_vocabulary_create.restype = C.c_int
     L.nvtext_amd_wordpiece_vocabulary_create.argtypes = [C.POINTER(StringsColumn), C.c_void_p,
                                                          C.POINTER(Allocator), C.POINTER(C.c_void_p)]

@@ -40,4 +40,13 @@ inline std::unique_ptr<cudf::column> make_list_result(nvtext_amd_list_column con
                                   device_buffer{r.null_mask, r.null_mask_bytes, stream, mr}, r.null_count, std::move(kids));
 }
 
+// cudf::make_numeric_column with the null mask set afterwards (cpp/src/text/jaccard.cu:458-476)
+inline std::unique_ptr<cudf::column> make_fixed_result(nvtext_amd_fixed_column const& r, cuda::stream_ref stream,
+                                                       rmm::device_async_resource_ref mr)
+{
+  using namespace cudf;
+  return std::make_unique<column>(data_type{static_cast<type_id>(r.type)}, r.size, device_buffer{r.data, r.data_bytes, stream, mr},
+                                  device_buffer{r.null_mask, r.null_mask_bytes, stream, mr}, r.null_count);
+}
+
 }  // namespace nvtext::detail

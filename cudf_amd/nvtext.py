@@ -18,7 +18,7 @@ from typing import Dict, Optional
 import numpy as np
 
 from . import _capi
-from .arrow_host import HostListColumn, HostStringsColumn
+from .arrow_host import HostFixedColumn, HostListColumn, HostStringsColumn
 
 
 def _torch():
@@ -176,6 +176,26 @@ class DeviceListColumn:
         return HostListColumn(offsets, child, mask, self.size, self.null_count)
 
 
+@dataclass
+class DeviceFixedColumn:
+    """Fixed-width result in HBM (FLOAT32 here): raw data tensor, optional validity words."""
+    data: object
+    mask: object
+    size: int
+    null_count: int
+    dtype: np.dtype
+
+    def to_host(self) -> "HostFixedColumn":
+        torch = _torch()
+        torch.cuda.current_stream().synchronize()
+        values = (self.data.cpu().numpy().view(self.dtype)[: self.size].copy() if self.data is not None
+                  else np.zeros(0, self.dtype))
+        mask = None
+        if self.mask is not None:
+            mask = self.mask.cpu().numpy().view(np.uint32)[: (self.size + 31) // 32].copy()
+        return HostFixedColumn(values, mask, self.size, self.null_count)
+
+
 _DTYPES = {_capi.TYPE_INT32: np.dtype(np.int32), _capi.TYPE_UINT32: np.dtype(np.uint32),
            _capi.TYPE_UINT64: np.dtype(np.uint64)}
 
@@ -263,6 +283,18 @@ def minhash64_ngrams(input: DeviceListStringsColumn, ngrams: int, seed: int, a, 
     if st != _capi.SUCCESS:
         _raise(st)
     return _wrap(out)
+
+
+def jaccard_index(input1: DeviceStringsColumn, input2: DeviceStringsColumn, width: int) -> DeviceFixedColumn:
+    """nvtext::jaccard_index (cpp/include/nvtext/jaccard.hpp:66-71); pylibcudf jaccard.pyx jaccard_index."""
+    L = _capi.load()
+    out = _capi.FixedColumn()
+    c1, c2 = input1._c(), input2._c()
+    st = L.nvtext_amd_jaccard_index(C.byref(c1), C.byref(c2), int(width), _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    mr = _mr()
+    return DeviceFixedColumn(mr.take(out.data), mr.take(out.null_mask), int(out.size), int(out.null_count), np.dtype(np.float32))
 
 
 class WordPieceVocabulary:

@@ -36,7 +36,8 @@ typedef enum nvtext_amd_status {
 enum {
   NVTEXT_AMD_TYPE_INT32  = 3,
   NVTEXT_AMD_TYPE_UINT32 = 7,
-  NVTEXT_AMD_TYPE_UINT64 = 8
+  NVTEXT_AMD_TYPE_UINT64 = 8,
+  NVTEXT_AMD_TYPE_FLOAT32 = 9
 };
 
 /* Non-owning view of an Arrow-layout strings column as libcudf lays it out
@@ -91,6 +92,19 @@ typedef struct nvtext_amd_list_strings_column {
   int32_t         null_count;
   nvtext_amd_strings_column child;
 } nvtext_amd_list_strings_column;
+
+/* Fixed-width result column (cudf::make_numeric_column, cpp/include/cudf/column/column_factories.hpp):
+ * `size` values of `type`, optional validity.  The buffers come from the caller's allocator and are
+ * returned with nvtext_amd_fixed_column_free. */
+typedef struct nvtext_amd_fixed_column {
+  int32_t   type;            /* NVTEXT_AMD_TYPE_* */
+  int32_t   size;
+  int32_t   null_count;
+  void*     data;
+  uint32_t* null_mask;       /* NULL when the column has no nulls */
+  size_t    data_bytes;
+  size_t    null_mask_bytes;
+} nvtext_amd_fixed_column;
 
 typedef struct nvtext_amd_wordpiece_vocabulary nvtext_amd_wordpiece_vocabulary;
 
@@ -158,6 +172,21 @@ nvtext_amd_status nvtext_amd_minhash64_ngrams(const nvtext_amd_list_strings_colu
                                               void* stream,
                                               const nvtext_amd_allocator* mr,
                                               nvtext_amd_list_column* out);
+
+/* Replaces nvtext::jaccard_index (cpp/include/nvtext/jaccard.hpp:66-71; cpp/src/text/jaccard.cu:490-498).
+ * For every row r: A, B = the sets of non-zero MurmurHash3_x86_32(seed 0) values of the `width`-character
+ * windows of input1[r], input2[r] (the window rule of nvtext_amd_minhash); result[r] = |A n B| / |A u B| as
+ * float32 (0 when both sets are empty).  A row that is null in either input is null in the result (its value
+ * is unspecified); the result has a null mask only if an input has nulls.  Synchronises the stream once. */
+nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* input1,
+                                           const nvtext_amd_strings_column* input2,
+                                           int32_t width,
+                                           void* stream,
+                                           const nvtext_amd_allocator* mr,
+                                           nvtext_amd_fixed_column* out);
+
+/* Returns the buffers of a fixed-width result to the allocator they came from. */
+void nvtext_amd_fixed_column_free(nvtext_amd_fixed_column* col, void* stream, const nvtext_amd_allocator* mr);
 
 /* Replaces nvtext::load_wordpiece_vocabulary / wordpiece_vocabulary::wordpiece_vocabulary
  * (cpp/include/nvtext/wordpiece_tokenize.hpp:26-66; cpp/src/text/wordpiece_tokenize.cu:213-293).

@@ -1,12 +1,13 @@
 // Exercises the C++ mirror of the nvtext API (cudf_amd/include) on the GPU with the cases of the
 // reference's gtests: cpp/tests/text/minhash_tests.cpp (Permuted, PermutedWide, EmptyTest, ErrorsTest, Ngrams, NgramsWide,
-// NgramsSliced)
+// NgramsSliced), cpp/tests/text/jaccard_tests.cpp (Basic, WithNulls, Errors)
 // and cpp/tests/text/subword_tests.cpp (all seven).  Own tiny harness: prints one line per case and
 // exits non-zero on the first failure.
 #include <cudf/column/column.hpp>
 #include <cudf/lists/lists_column_view.hpp>
 #include <cudf/strings/strings_column_view.hpp>
 #include <hip/hip_runtime.h>
+#include <nvtext/jaccard.hpp>
 #include <nvtext/minhash.hpp>
 #include <nvtext/wordpiece_tokenize.hpp>
 
@@ -277,6 +278,56 @@ void test_minhash_ngrams()
   }
 }
 
+void test_jaccard()
+{
+  std::printf("JaccardTest.Basic / WithNulls / Errors\n");
+  auto fetch = [](cudf::column const& col, std::vector<float>& values, std::vector<bool>& valid) {
+    HIP_OK(hipDeviceSynchronize());
+    auto const v = col.view();
+    values.assign(v.size(), 0.f);
+    if (v.size()) HIP_OK(hipMemcpy(values.data(), v.head<void>(), v.size() * sizeof(float), hipMemcpyDeviceToHost));
+    std::vector<uint32_t> mask((v.size() + 31) / 32, 0xFFFFFFFFu);
+    if (v.null_mask() && v.size()) HIP_OK(hipMemcpy(mask.data(), v.null_mask(), mask.size() * 4, hipMemcpyDeviceToHost));
+    valid.clear();
+    for (int i = 0; i < v.size(); ++i) valid.push_back((mask[i / 32] >> (i % 32)) & 1u);
+  };
+  std::vector<float> values;
+  std::vector<bool> valid;
+  {
+    auto input1 = make_strings({"the quick brown fox", "jumped over the lazy dog."});
+    auto input2 = make_strings({"the slowest brown cat", "crawled under the jumping fox"});
+    cudf::strings_column_view view1(input1.view), view2(input2.view);
+    auto results = nvtext::jaccard_index(view1, view2, 5);
+    fetch(*results, values, valid);
+    CHECK(results->type().id() == cudf::type_id::FLOAT32 && results->null_count() == 0);
+    CHECK(values == (std::vector<float>{0.103448279f, 0.0697674453f}));
+    fetch(*nvtext::jaccard_index(view1, view1, 5), values, valid);
+    CHECK(values == (std::vector<float>{1.0f, 1.0f}));
+    fetch(*nvtext::jaccard_index(view2, view2, 10), values, valid);
+    CHECK(values == (std::vector<float>{1.0f, 1.0f}));
+  }
+  {
+    auto input1 = make_strings({"brown fox", "jumps over dog", std::nullopt, ""});
+    auto input2 = make_strings({"brown cat", "jumps on fox", "", std::nullopt});
+    cudf::strings_column_view view1(input1.view), view2(input2.view);
+    auto results = nvtext::jaccard_index(view1, view2, 5);
+    fetch(*results, values, valid);
+    CHECK(values[0] == 0.25f && values[1] == 0.200000003f);
+    CHECK(valid == (std::vector<bool>{true, true, false, false}) && results->null_count() == 2);
+    results = nvtext::jaccard_index(view1, view1, 7);
+    fetch(*results, values, valid);
+    CHECK(values[0] == 1.0f && values[1] == 1.0f && values[3] == 0.f);
+    CHECK(valid == (std::vector<bool>{true, true, false, true}) && results->null_count() == 1);
+  }
+  {
+    auto input  = make_strings({"1", "2", "3"});
+    auto input2 = make_strings({"1", "2"});
+    cudf::strings_column_view view(input.view), view2(input2.view);
+    EXPECT_THROW(nvtext::jaccard_index(view, view, 1), std::invalid_argument);
+    EXPECT_THROW(nvtext::jaccard_index(view, view2, 5), std::invalid_argument);
+  }
+}
+
 void test_wordpiece()
 {
   std::printf("TextSubwordTest.WordPiece / WordPieceSliced\n");
@@ -357,6 +408,7 @@ int main()
   test_minhash_wide();
   test_minhash_empty_and_errors();
   test_minhash_ngrams();
+  test_jaccard();
   test_wordpiece();
   test_wordpiece_subwords();
   test_wordpiece_edges();

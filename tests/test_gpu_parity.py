@@ -242,6 +242,71 @@ def test_minhash_ngrams_wide_row_and_errors(nv, orc):
     assert empty.size == 0 and empty.child.size == 0
 
 
+# ----------------------------------------------------------------------------- jaccard_index
+def assert_same_fixed(got, exp, what=""):
+    assert got.size == exp.size and got.null_count == exp.null_count, what
+    assert (got.mask is None) == (exp.mask is None), what
+    v = exp.validity()
+    assert np.array_equal(got.validity(), v), what
+    a, b = got.values.view(np.uint32)[v], exp.values.view(np.uint32)[v]
+    if not np.array_equal(a, b):
+        bad = np.flatnonzero(a != b)
+        raise AssertionError(f"{what}: {bad.size} values differ, first at {bad[:5]}: got {got.values[v][bad[:5]]} expected {exp.values[v][bad[:5]]}")
+
+
+@pytest.mark.parametrize("case", gc.jaccard_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_jaccard_golden(nv, orc, case, dtype):
+    h1, h2 = strings(case["input1"], dtype), strings(case["input2"], dtype)
+    got = nv.jaccard_index(dev(nv, h1), dev(nv, h2), case["width"]).to_host()
+    assert_same_fixed(got, orc.jaccard_index(h1, h2, case["width"]), case["name"])
+    exp = np.array(case["expected"], np.float32)
+    valid = np.array(case.get("expected_valid", [True] * len(exp)))
+    assert np.allclose(got.values[valid], exp[valid], atol=case.get("tolerance", 0), rtol=0)
+
+
+@pytest.mark.parametrize("width", [2, 5, 40])
+def test_jaccard_random_vs_oracle(nv, orc, width):
+    rng = np.random.default_rng(400 + width)
+    alphabet = list("abcdefgé漢 ")
+    r1, r2 = [], []
+    for _ in range(1200):
+        common = "".join(rng.choice(alphabet, int(rng.integers(0, 300))))
+        u = rng.random()
+        r1.append(None if u < 0.04 else "" if u < 0.08 else "".join(rng.choice(alphabet, int(rng.integers(0, 40)))) + common)
+        u = rng.random()
+        r2.append(None if u < 0.04 else "" if u < 0.08 else common + "".join(rng.choice(alphabet, int(rng.integers(0, 80)))))
+    # pairs beyond the 4096 bytes of the LDS set, and one far beyond
+    for n1, n2 in [(3000, 3000), (9000, 100), (100, 20000), (300_000, 250_000)]:
+        base = "".join(rng.choice(alphabet[:6], 64))
+        r1.append((base * (n1 // 64 + 1))[:n1])
+        r2.append("".join(rng.choice(alphabet[:6], n2 // 2)) + (base * (n2 // 128 + 1))[: n2 // 2])
+    for dtype in (np.int32, np.int64):
+        h1, h2 = strings(r1, dtype), strings(r2, dtype)
+        d1, d2 = dev(nv, h1), dev(nv, h2)
+        assert_same_fixed(nv.jaccard_index(d1, d2, width).to_host(), orc.jaccard_index(h1, h2, width, nthreads=8), f"jaccard width={width}")
+        lo, hi = 7, 1150
+        s1, s2 = h1.slice(lo, hi), h2.slice(lo + 3, hi + 3)
+        assert_same_fixed(nv.jaccard_index(d1.slice(lo, hi, s1.null_count), d2.slice(lo + 3, hi + 3, s2.null_count), width).to_host(),
+                          orc.jaccard_index(s1, s2, width, nthreads=4), "jaccard sliced")
+    # no nulls: no mask; same column twice: all ones (or 0 for empty rows)
+    clean = strings([x or "" for x in r1[:300]])
+    same = nv.jaccard_index(dev(nv, clean), dev(nv, clean), width).to_host()
+    assert same.mask is None and same.null_count == 0
+    lens = np.diff(clean.offsets)
+    assert np.array_equal(same.values, np.where(lens > 0, np.float32(1), np.float32(0)))
+
+
+def test_jaccard_errors_and_empty(nv):
+    three, two = dev(nv, strings(["1", "2", "3"])), dev(nv, strings(["1", "2"]))
+    with pytest.raises(ValueError):
+        nv.jaccard_index(three, three, 1)
+    with pytest.raises(ValueError):
+        nv.jaccard_index(three, two, 5)
+    empty = nv.jaccard_index(dev(nv, strings([])), dev(nv, strings([])), 5).to_host()
+    assert empty.size == 0 and empty.values.size == 0
+
+
 # ----------------------------------------------------------------------------- wordpiece
 @pytest.mark.parametrize("case", gc.wordpiece_cases(), ids=lambda c: c["name"])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
