@@ -73,7 +73,11 @@ struct VocabTable {
   // Entries are shared by hashing, so a set bit promises nothing, a clear bit rules the length out.
   const uint32_t* lens;
   uint32_t lens_mask;
+  // Direct tables for keys of one and two bytes: short_ids[kind * 65536 + (byte0 | byte1 << 8)] for two bytes,
+  // short_ids[131072 + kind * 256 + byte0] for one; the token id, or INT32_MIN when there is no such key.
+  const int32_t* short_ids;
 };
+constexpr uint32_t kShortIds = 2 * 65536 + 2 * 256;
 
 __host__ __device__ __forceinline__ uint32_t length_filter_index(uint32_t kind, uint32_t first3)
 {
@@ -99,6 +103,7 @@ struct nvtext_amd_wordpiece_vocabulary {
   void* d_slots     = nullptr;
   void* d_pool      = nullptr;
   void* d_lens      = nullptr;
+  void* d_short     = nullptr;
   size_t slot_bytes = 0;
   size_t pool_bytes = 0;
   int32_t entries   = 0;
@@ -869,6 +874,7 @@ struct ShortWord {
   uint32_t bnd;    // bit i: start + i is a character boundary (bit rem is set)
   uint32_t cand;   // lengths still to try for the piece at start (bit l - 1), longest first
   uint32_t count;  // tokens so far
+  int32_t id1, id2;  // ids of the piece's first byte and first two bytes as keys (kNone: no such key)
   bool done;
 
   __device__ __forceinline__ uint32_t byte(uint32_t k) const
@@ -893,6 +899,8 @@ struct ShortWord {
     uint32_t const lens = rem >= 3 ? t.lens[length_filter_index(kind, r[0] & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
     uint32_t const lim  = min(min(rem, t.max_len[kind]), 16u);
     cand                = (bnd >> 1) & ((1u << lim) - 1u) & ((lens << 2) | 3u);
+    id1                 = t.short_ids[2 * 65536 + kind * 256 + (r[0] & 0xFFu)];
+    id2                 = rem >= 2 ? t.short_ids[kind * 65536 + (r[0] & 0xFFFFu)] : kNone;
   }
 
   __device__ __forceinline__ void begin(VocabTable const& t, const uint32_t (&head)[4], uint32_t len)
@@ -943,46 +951,62 @@ struct ShortWord {
     bnd >>= l;
   }
 
-  // Examines the two longest remaining candidates (their table reads are in flight together).
+  // One trip: probes the two longest remaining candidates of three bytes and more (their table reads are in
+  // flight together); when none of those is left, the candidates of two bytes and of one byte are settled
+  // from the ids fetched when the piece was opened, without hashing or further reads.
   template <typename Emit>
   __device__ __forceinline__ void step(VocabTable const& t, Emit&& emit)
   {
-    uint32_t const kind = count ? 1u : 0u;
-    bool const none     = cand == 0;
-    uint32_t const c1   = none ? 1u : cand;
-    uint32_t const la   = 32u - static_cast<uint32_t>(__builtin_clz(c1));
-    uint32_t const rest = c1 ^ (1u << (la - 1));
-    bool const has_b    = rest != 0;
-    uint32_t const lb   = has_b ? 32u - static_cast<uint32_t>(__builtin_clz(rest)) : 1u;
-    Probe const pa      = probe_of(t, kind, la);
-    Probe const pb      = probe_of(t, kind, lb);
-    uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
-    uint4 const b0 = t.slots[2 * pb.bucket], b1 = t.slots[2 * pb.bucket + 1];
-    int32_t ida, idb;
-    uint32_t va = verdict(pa, a0, a1, la, &ida);
-    uint32_t vb = verdict(pb, b0, b1, lb, &idb);
-    if (va == 2u || (va == 0u && has_b && vb == 2u)) {
-      // the general lookup (keys in the pool, overflowing buckets)
-      if (va == 2u) {
-        ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
-        va  = ida == kNone ? 0u : 1u;
+    uint32_t const kind   = count ? 1u : 0u;
+    uint32_t const longer = cand & ~3u;
+    bool const has_a      = longer != 0;
+    uint32_t const c1     = has_a ? longer : 4u;
+    uint32_t const la     = 32u - static_cast<uint32_t>(__builtin_clz(c1));
+    uint32_t const rest   = c1 ^ (1u << (la - 1));
+    bool const has_b      = has_a && rest != 0;
+    uint32_t const lb     = has_b ? 32u - static_cast<uint32_t>(__builtin_clz(rest)) : 3u;
+    bool hit_a = false, hit_b = false;
+    int32_t ida = kNone, idb = kNone;
+    if (has_a) {
+      Probe const pa = probe_of(t, kind, la);
+      Probe const pb = probe_of(t, kind, lb);
+      uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
+      uint4 const b0 = t.slots[2 * pb.bucket], b1 = t.slots[2 * pb.bucket + 1];
+      uint32_t va = verdict(pa, a0, a1, la, &ida);
+      uint32_t vb = verdict(pb, b0, b1, lb, &idb);
+      if (va == 2u || (va == 0u && has_b && vb == 2u)) {
+        // the general lookup (keys in the pool, overflowing buckets)
+        if (va == 2u) {
+          ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
+          va  = ida == kNone ? 0u : 1u;
+        }
+        if (va == 0u && vb == 2u) {
+          idb = finish_probe(t, pb, b0, b1, *this, 0u, lb);
+          vb  = idb == kNone ? 0u : 1u;
+        }
       }
-      if (va == 0u && vb == 2u) {
-        idb = finish_probe(t, pb, b0, b1, *this, 0u, lb);
-        vb  = idb == kNone ? 0u : 1u;
-      }
+      hit_a = va == 1u;
+      hit_b = !hit_a && has_b && vb == 1u;
     }
-    bool const hit_a   = !none && va == 1u;
-    bool const hit_b   = !none && !hit_a && has_b && vb == 1u;
-    bool const hit     = hit_a || hit_b;
-    uint32_t const len = hit_a ? la : lb;
-    // no candidate left: no prefix of the word matched (375-379), or a later piece has no match and the word
-    // collapses (396-404): either way a single unknown token
-    bool const unknown = none || (!hit && !has_b) || (!hit && (rest ^ (1u << (lb - 1))) == 0);
-    if (hit || unknown) emit(unknown ? 0u : count, unknown ? t.unk_id : (hit_a ? ida : idb));
+    uint32_t const longer_left = has_b ? rest ^ (1u << (lb - 1)) : 0u;  // after two misses
+    bool hit     = hit_a || hit_b;
+    uint32_t len = hit_a ? la : lb;
+    int32_t id   = hit_a ? ida : idb;
+    bool unknown = false;
+    if (!hit && longer_left == 0) {
+      // two bytes, then one byte; else no prefix of the word matched (375-379), or a later piece has no match and
+      // the word collapses (396-404): either way a single unknown token
+      bool const two = (cand & 2u) != 0 && id2 != kNone;
+      bool const one = (cand & 1u) != 0 && id1 != kNone;
+      hit            = two || one;
+      len            = two ? 2u : 1u;
+      id             = two ? id2 : id1;
+      unknown        = !hit;
+    }
+    if (hit || unknown) emit(unknown ? 0u : count, unknown ? t.unk_id : id);
     count = unknown ? 1u : count + (hit ? 1u : 0u);
     done  = unknown || (hit && len == rem);
-    cand  = has_b ? rest ^ (1u << (lb - 1)) : 0u;  // after two misses
+    cand  = longer_left | (cand & 3u);
     if (hit && !done) {
       advance(len);  // next piece: the rest of the word (381-395)
       open_piece(t, 1);
@@ -1408,6 +1432,20 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
     if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') note_length(1, pool.data() + b + 2, static_cast<uint32_t>(len - 2));
   }
 
+  // direct tables for the keys of one and two bytes (the first entry with a key wins, as in the table)
+  std::vector<int32_t> short_ids(kShortIds, kNone);
+  auto note_short = [&](uint32_t kind, const uint8_t* key, uint32_t len, int32_t id) {
+    if (len > 2) return;
+    size_t const at = len == 2 ? kind * 65536u + (key[0] | (uint32_t{key[1]} << 8)) : 2 * 65536u + kind * 256u + key[0];
+    if (short_ids[at] == kNone) short_ids[at] = id;
+  };
+  for (int32_t i = 0; i < V; ++i) {
+    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
+    int64_t const len = e - b;
+    if (len >= 1 && len <= 2) note_short(0, pool.data() + b, static_cast<uint32_t>(len), i);
+    if (len >= 3 && len <= 4 && pool[b] == '#' && pool[b + 1] == '#') note_short(1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), i);
+  }
+
   auto* v = new nvtext_amd_wordpiece_vocabulary;
   v->entries = V;
   // wordpiece_tokenize.cu:199-209, 273-275
@@ -1416,15 +1454,16 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->slot_bytes = capacity * sizeof(HostSlot);
   v->pool_bytes = blocks.size() + 16;
   if (hipMalloc(&v->d_slots, v->slot_bytes) != hipSuccess || hipMalloc(&v->d_pool, v->pool_bytes) != hipSuccess ||
-      hipMalloc(&v->d_lens, lens.size() * sizeof(uint32_t)) != hipSuccess) {
+      hipMalloc(&v->d_lens, lens.size() * sizeof(uint32_t)) != hipSuccess || hipMalloc(&v->d_short, short_ids.size() * sizeof(int32_t)) != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
   hipError_t e1 = hipMemcpyAsync(v->d_slots, slots.data(), v->slot_bytes, hipMemcpyHostToDevice, stream);
   hipError_t e2 = blocks.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, blocks.data(), blocks.size(), hipMemcpyHostToDevice, stream);
   hipError_t e4 = hipMemcpyAsync(v->d_lens, lens.data(), lens.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
+  hipError_t e5 = hipMemcpyAsync(v->d_short, short_ids.data(), short_ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
   hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
-  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess) {
+  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_DEVICE_ERROR, "vocabulary upload failed");
   }
@@ -1436,6 +1475,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.max_len[1]  = max_len[1];
   v->table.lens        = static_cast<const uint32_t*>(v->d_lens);
   v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
+  v->table.short_ids   = static_cast<const int32_t*>(v->d_short);
   *out            = v;
   return NVTEXT_AMD_SUCCESS;
 }
@@ -1446,6 +1486,7 @@ void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
   if (v->d_slots) (void)hipFree(v->d_slots);
   if (v->d_pool) (void)hipFree(v->d_pool);
   if (v->d_lens) (void)hipFree(v->d_lens);
+  if (v->d_short) (void)hipFree(v->d_short);
   delete v;
 }
 
