@@ -459,7 +459,7 @@ __device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return 
 // with lanes <-> words.  The next chunk of every group (the rest of its row, else the start of its next
 // row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
 // For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
-// marker carrying the queue index; nwords[r] = words kept; counts[r] = one per hit.
+// marker carrying the queue index; nwords[r] = counts[r] = words kept.
 __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
                                                                       uint32_t* __restrict__ arena,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
@@ -501,7 +501,6 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
   RowCtx ctx       = make_row_ctx(col, o_cur, e_cur - o_cur);
   uint32_t cbase   = 0;
   uint32_t wdone   = 0;     // words kept so far in this row
-  uint32_t hits    = 0;     // of which found in the vocabulary
   uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
   uint32_t prev_space  = 1; // the byte before the chunk is a space (or the row starts here)
   // the chunk about to be processed: my sixteen bytes and (last lane of the group) the byte after the chunk
@@ -599,7 +598,6 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     // ---- probes (lanes <-> words, all groups pooled)
-    uint32_t my_hits = 0;
     for (uint32_t w0 = 0; w0 < total; w0 += kWave) {
       uint32_t const ws = w0 + lane;  // word slot
       int const gw      = (ws >= gb1) + (ws >= gb2) + (ws >= gb3);
@@ -677,21 +675,11 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView co
         int64_t const s = static_cast<int64_t>((static_cast<uint64_t>(gb.w) << 32) | gb.z) + ga.w + idx;
         store_stream(arena + s, value);
       }
-      uint64_t const hit = ballot64(active && !miss);
-      if (hit) {
-        // credit the hits to the groups that own the words
-        uint64_t const in_g0 = ballot64(gw == 0), in_g1 = ballot64(gw == 1), in_g2 = ballot64(gw == 2);
-        uint64_t const mine_mask = g == 0 ? in_g0 : g == 1 ? in_g1 : g == 2 ? in_g2 : ~(in_g0 | in_g1 | in_g2);
-        my_hits += static_cast<uint32_t>(__builtin_popcountll(hit & mine_mask));
-      }
     }
-    hits += my_hits;
-    if (row_done) {
-      if (gl == 0) {
-        nwords[r_now] = static_cast<int32_t>(wd_after);
-        counts[r_now] = static_cast<int32_t>(hits);
-      }
-      hits = 0;
+    if (row_done && gl == 0) {
+      // one token per word; the out-of-vocabulary pass adds what its words give beyond that
+      nwords[r_now] = static_cast<int32_t>(wd_after);
+      counts[r_now] = static_cast<int32_t>(wd_after);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1020,7 +1008,7 @@ struct ShortWord {
 // bytes (whole in their queue record) run in registers; the few longer ones are set aside for the kernel
 // below: their queue indices go to longer[first entry of the part ...], their number to
 // longer[queue_capacity + wavefront].
-// results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count.
+// results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count - 1.
 __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
                                                                     const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
                                                                     OovResult* __restrict__ results, int32_t* __restrict__ counts,
@@ -1046,7 +1034,7 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col,
     uint4* const dst = reinterpret_cast<uint4*>(results + q);
     store_stream(dst, make_uint4(static_cast<uint32_t>(tok[0]), static_cast<uint32_t>(tok[1]), static_cast<uint32_t>(tok[2]), static_cast<uint32_t>(tok[3])));
     store_stream(dst + 1, make_uint4(static_cast<uint32_t>(tok[4]), static_cast<uint32_t>(tok[5]), static_cast<uint32_t>(tok[6]), count));
-    atomicAdd(&counts[row], static_cast<int32_t>(count));
+    if (count > 1) atomicAdd(&counts[row], static_cast<int32_t>(count - 1));  // the probe pass has counted one token per word
   };
 
   {
@@ -1132,7 +1120,7 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView
       }
       res.count  = st.count;
       results[q] = res;
-      atomicAdd(&counts[e.row], static_cast<int32_t>(st.count));
+      if (st.count > 1) atomicAdd(&counts[e.row], static_cast<int32_t>(st.count - 1));
     }
   }
 }
