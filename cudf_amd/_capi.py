@@ -19,6 +19,10 @@ EXPORTS = [
     "nvtext_amd_minhash64_ngrams",
     "nvtext_amd_jaccard_index",
     "nvtext_amd_fixed_column_free",
+    "nvtext_amd_strings_from_arrow_device",
+    "nvtext_amd_list_strings_from_arrow_device",
+    "nvtext_amd_list_to_arrow_device",
+    "nvtext_amd_fixed_to_arrow_device",
     "nvtext_amd_wordpiece_vocabulary_create",
     "nvtext_amd_wordpiece_vocabulary_destroy",
     "nvtext_amd_wordpiece_vocabulary_unk_id",
@@ -88,6 +92,35 @@ class FixedColumn(C.Structure):
     ]
 
 
+# ---- Arrow C data / device interface (arrow/c/abi.h)
+class ArrowSchema(C.Structure):
+    pass
+
+
+ArrowSchema._fields_ = [
+    ("format", C.c_char_p), ("name", C.c_char_p), ("metadata", C.c_char_p), ("flags", C.c_int64), ("n_children", C.c_int64),
+    ("children", C.POINTER(C.POINTER(ArrowSchema))), ("dictionary", C.POINTER(ArrowSchema)),
+    ("release", C.CFUNCTYPE(None, C.POINTER(ArrowSchema))), ("private_data", C.c_void_p)]
+
+
+class ArrowArray(C.Structure):
+    pass
+
+
+ArrowArray._fields_ = [
+    ("length", C.c_int64), ("null_count", C.c_int64), ("offset", C.c_int64), ("n_buffers", C.c_int64), ("n_children", C.c_int64),
+    ("buffers", C.POINTER(C.c_void_p)), ("children", C.POINTER(C.POINTER(ArrowArray))), ("dictionary", C.POINTER(ArrowArray)),
+    ("release", C.CFUNCTYPE(None, C.POINTER(ArrowArray))), ("private_data", C.c_void_p)]
+
+
+class ArrowDeviceArray(C.Structure):
+    _fields_ = [("array", ArrowArray), ("device_id", C.c_int64), ("device_type", C.c_int32), ("sync_event", C.c_void_p),
+                ("reserved", C.c_int64 * 3)]
+
+
+ARROW_DEVICE_CPU, ARROW_DEVICE_ROCM, ARROW_DEVICE_ROCM_HOST = 1, 10, 11
+ARROW_FLAG_NULLABLE = 2
+
 _lib = None
 
 
@@ -126,6 +159,17 @@ def load():
                                            C.POINTER(Allocator), C.POINTER(FixedColumn)]
     L.nvtext_amd_fixed_column_free.restype = None
     L.nvtext_amd_fixed_column_free.argtypes = [C.POINTER(FixedColumn), C.c_void_p, C.POINTER(Allocator)]
+    L.nvtext_amd_strings_from_arrow_device.restype = C.c_int
+    L.nvtext_amd_strings_from_arrow_device.argtypes = [C.POINTER(ArrowSchema), C.POINTER(ArrowDeviceArray), C.c_void_p, C.POINTER(StringsColumn)]
+    L.nvtext_amd_list_strings_from_arrow_device.restype = C.c_int
+    L.nvtext_amd_list_strings_from_arrow_device.argtypes = [C.POINTER(ArrowSchema), C.POINTER(ArrowDeviceArray), C.c_void_p,
+                                                            C.POINTER(ListStringsColumn)]
+    L.nvtext_amd_list_to_arrow_device.restype = C.c_int
+    L.nvtext_amd_list_to_arrow_device.argtypes = [C.POINTER(ListColumn), C.c_void_p, C.POINTER(Allocator), C.POINTER(ArrowSchema),
+                                                  C.POINTER(ArrowDeviceArray)]
+    L.nvtext_amd_fixed_to_arrow_device.restype = C.c_int
+    L.nvtext_amd_fixed_to_arrow_device.argtypes = [C.POINTER(FixedColumn), C.c_void_p, C.POINTER(Allocator), C.POINTER(ArrowSchema),
+                                                   C.POINTER(ArrowDeviceArray)]
     L.nvtext_amd_wordpiece_vocabulary_create.restype = C.c_int
     L.nvtext_amd_wordpiece_vocabulary_create.argtypes = [C.POINTER(StringsColumn), C.c_void_p,
                                                          C.POINTER(Allocator), C.POINTER(C.c_void_p)]

@@ -1,4 +1,4 @@
-"""The C-ABI library loads and exports every symbol include/nvtext_amd.h declares (no GPU work)."""
+"""The C-ABI library loads and exports every symbol the headers under include/ declare (no GPU work)."""
 import ctypes
 import os
 import re
@@ -9,9 +9,14 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_functions():
-    text = open(os.path.join(ROOT, "include", "nvtext_amd.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(nvtext_amd_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in sorted(os.listdir(os.path.join(ROOT, "include"))):
+        if not header.endswith(".h"):
+            continue
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(nvtext_amd_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_and_binding_agree():
