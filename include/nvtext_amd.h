@@ -1,7 +1,8 @@
 /*
  * nvtext_amd.h -- C ABI of the MI355X (gfx950) implementation of libcudf's nvtext
  * text-dedup hot path: minhash / minhash64 over character windows and
- * wordpiece_tokenize with its wordpiece_vocabulary.
+ * wordpiece_tokenize with its wordpiece_vocabulary, plus the calls either side of them
+ * (minhash_ngrams, jaccard_index, normalize_characters).
  *
  * Plain pointers and sizes only.  Every pointer named "device" is HIP device memory
  * that must stay valid until the work queued on `stream` has completed.  All work is
@@ -106,7 +107,24 @@ typedef struct nvtext_amd_fixed_column {
   size_t    null_mask_bytes;
 } nvtext_amd_fixed_column;
 
+/* Owning result: a STRING column (cudf::make_strings_column, cpp/include/cudf/column/column_factories.hpp).
+ * int32 offsets; the buffers come from the caller's allocator and are returned with
+ * nvtext_amd_strings_result_free. */
+typedef struct nvtext_amd_strings_result {
+  int32_t   size;            /* rows                                                        */
+  int32_t   null_count;
+  int32_t   offsets_size;    /* size+1, or 0 for the canonical empty strings column         */
+  int32_t*  offsets;         /* device, offsets_size entries (NULL if 0)                    */
+  char*     chars;           /* device, chars_size bytes (NULL if 0)                        */
+  int64_t   chars_size;
+  uint32_t* null_mask;       /* device or NULL; bit i = row i                               */
+  size_t    offsets_bytes;   /* allocation sizes, for deallocate()                          */
+  size_t    chars_bytes;
+  size_t    null_mask_bytes;
+} nvtext_amd_strings_result;
+
 typedef struct nvtext_amd_wordpiece_vocabulary nvtext_amd_wordpiece_vocabulary;
+typedef struct nvtext_amd_character_normalizer nvtext_amd_character_normalizer;
 
 /* Library version (major*10000 + minor*100 + patch). */
 int32_t nvtext_amd_version(void);
@@ -214,6 +232,38 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
                                                 void* stream,
                                                 const nvtext_amd_allocator* mr,
                                                 nvtext_amd_list_column* out);
+
+/* Replaces nvtext::create_character_normalizer / character_normalizer::character_normalizer
+ * (cpp/include/nvtext/normalize.hpp:170-213; cpp/src/text/normalize.cu:219-256).  The object owns the device
+ * tables that say, per Unicode code point, whether it is padded with spaces (punctuation, CJK ideographs),
+ * removed (control and format characters; accents when lower-casing), replaced by a space (whitespace) or
+ * replaced by its lower-cased, accent-stripped form of one to three code points.  special_tokens (NULL or
+ * empty for none) are bracketed tokens such as "[PAD]" that keep their case and their brackets unpadded;
+ * nulls among them give INVALID_ARGUMENT.  Belongs to the device that is current at creation; immutable and
+ * shareable between concurrent calls. */
+nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case,
+                                                         const nvtext_amd_strings_column* special_tokens,
+                                                         void* stream,
+                                                         const nvtext_amd_allocator* mr,
+                                                         nvtext_amd_character_normalizer** out);
+
+/* Replaces character_normalizer::~character_normalizer (cpp/src/text/normalize.cu:247). */
+void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* normalizer);
+
+/* Replaces nvtext::normalize_characters (cpp/include/nvtext/normalize.hpp:215-254;
+ * cpp/src/text/normalize.cu:491-573): the BERT basic-tokenizer clean-up that precedes wordpiece_tokenize.
+ * Works on the bytes between the first and the last offset of the view as one flat sequence, so a null row
+ * keeps whatever its offsets span and the result has the input's validity.  Result: STRING column with int32
+ * offsets; OVERFLOW if the normalized bytes exceed INT32_MAX.  Synchronises the stream twice (the byte range
+ * of the view, the size of the result). */
+nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_column* input,
+                                                  const nvtext_amd_character_normalizer* normalizer,
+                                                  void* stream,
+                                                  const nvtext_amd_allocator* mr,
+                                                  nvtext_amd_strings_result* out);
+
+/* Returns the buffers of a strings result to the allocator they came from. */
+void nvtext_amd_strings_result_free(nvtext_amd_strings_result* col, void* stream, const nvtext_amd_allocator* mr);
 
 /* Kernel timing for benchmarks.  The reference marks these entry points with NVTX ranges
  * (CUDF_FUNC_RANGE, cpp/src/text/minhash.cu:699, cpp/src/text/wordpiece_tokenize.cu:897) and is

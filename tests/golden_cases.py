@@ -49,6 +49,15 @@ def jaccard_cases():
     return json.load(open(os.path.join(GOLDEN, "jaccard_vectors.json"), encoding="utf-8"))["cases"]
 
 
+def normalize_cases():
+    """Each case: rows (None = null row), optional slice [offset, size], do_lower_case, special_tokens, expected."""
+    return json.load(open(os.path.join(GOLDEN, "normalize_vectors.json"), encoding="utf-8"))["cases"]
+
+
+def codepoint_behaviour_digests():
+    return json.load(open(os.path.join(GOLDEN, "codepoint_behaviour_digests.json"), encoding="utf-8"))
+
+
 def murmur64_vectors():
     return json.load(open(os.path.join(GOLDEN, "minhash_vectors.json"), encoding="utf-8"))["murmurhash3_x64_128_word0"]
 

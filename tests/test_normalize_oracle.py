@@ -1,0 +1,149 @@
+"""The normalize_characters oracle against the reference's known answers, and the per-code-point rules (the
+oracle's and the library's table generator's) against digests of the reference's tables."""
+import importlib.util
+import os
+
+import numpy as np
+import pytest
+
+from oracle import normalize_py as onorm
+from tests import golden_cases as gc
+from tests.golden.digest_codepoint_metadata import LIMIT, canonical, digests
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def load_generator():
+    spec = importlib.util.spec_from_file_location(
+        "gen_codepoint_tables", os.path.join(ROOT, "cudf_amd", "csrc", "gen_codepoint_tables.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def case_column(case, dtype=np.int32):
+    col = gc.strings(case["rows"], dtype)
+    if "slice" in case:
+        lo, n = case["slice"]
+        col = col.slice(lo, lo + n)
+    return col
+
+
+def expected_bytes(case):
+    return [None if r is None else r.encode("utf-8") for r in case["expected"]]
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("case", gc.normalize_cases(), ids=lambda c: c["name"])
+def test_normalize_golden(case, dtype):
+    tokens = [t.encode("utf-8") for t in case["special_tokens"]]
+    got = onorm.normalize_characters(case_column(case, dtype), case["do_lower_case"], tokens)
+    assert got.to_pylist() == expected_bytes(case)
+    assert got.offsets.dtype == np.int32
+
+
+def mismatched_blocks(entries):
+    want = gc.codepoint_behaviour_digests()
+    got = digests(entries)
+    assert len(got) == len(want["digests"])
+    return [hex(i * want["block"]) for i, (g, w) in enumerate(zip(got, want["digests"])) if g != w]
+
+
+def test_oracle_rules_match_reference_tables():
+    def entries():
+        for cp in range(LIMIT):
+            kind, low = onorm.classify(cp)
+            new = 0x20 if kind == onorm.REPLACE else (0 if low == [cp] or not low else low[0])
+            multi = int(len(low) > 1)
+            aux = ((low[1] << 32) | (low[2] if len(low) > 2 else 0)) if multi else 0
+            yield canonical(kind, multi, new, aux)
+    assert mismatched_blocks(entries()) == []
+
+
+def test_generated_tables_match_reference_tables():
+    gen = load_generator()
+
+    def entries():
+        for cp in range(LIMIT):
+            v, a = gen.entry(cp)
+            yield canonical((v >> 24) & 7, (v >> 23) & 1, v & 0x1FFFFF, a)
+    assert mismatched_blocks(entries()) == []
+
+
+def committed_tables():
+    """The three arrays of cudf_amd/csrc/codepoint_tables.inc, the data the library is compiled from."""
+    import re
+    text = open(os.path.join(ROOT, "cudf_amd", "csrc", "codepoint_tables.inc")).read()
+
+    def rows(name):
+        body = re.search(name + r"\[\]\[\d\] = \{(.*?)\};", text, re.S).group(1)
+        return [tuple(int(x.rstrip("UL"), 0) for x in r.split(",")) for r in re.findall(r"\{([^{}]*)\}", body)]
+    return rows("kCodepointRuns"), rows("kCodepointSecond"), rows("kLowerCase")
+
+
+def test_committed_tables_match_reference_tables():
+    gen = load_generator()
+    runs, second, _ = committed_tables()
+    first = [gen.DEFAULT] * LIMIT
+    for cp, count, value in runs:
+        first[cp: cp + count] = [value] * count
+    aux = dict(second)
+    for cp in range(0xAC00, 0xD7A4):  # the library fills the Hangul syllables the same way
+        first[cp], aux[cp] = gen.hangul(cp)
+    entries = (canonical((v >> 24) & 7, (v >> 23) & 1, v & 0x1FFFFF, aux.get(cp, 0)) for cp, v in enumerate(first))
+    assert mismatched_blocks(entries) == []
+
+
+def test_committed_tables_are_what_the_generator_writes():
+    import unicodedata
+    if unicodedata.unidata_version != "13.0.0":
+        pytest.skip("the tables were generated with the Unicode 13.0.0 database")
+    gen = load_generator()
+    runs, second, lower = committed_tables()
+    want_runs, want_second = gen.tables()
+    assert runs == want_runs and second == want_second and lower == gen.lower_map()
+
+
+def test_lower_case_table_matches_ascii_and_latin1():
+    _, _, lower = committed_tables()
+    table = {row[0]: row[1:] for row in lower}
+    for c in range(ord("A"), ord("Z") + 1):
+        assert table[c] == (c + 32, 0, 0)
+    assert table[0xC9] == (0xE9, 0, 0) and table[0x130] == (0x69, 0x307, 0) and table[0x212A] == (0x6B, 0, 0)
+    assert all(cp <= 0xFFFF for cp in table) and ord("a") not in table
+
+
+def test_special_tokens_sorted_then_lowered():
+    # "[B]" sorts before "[a]" but lower-cases to "[b]": the halving search then misses "[a]" in a list of two
+    # only when it looks at the wrong half; with these two it still finds both
+    assert onorm.sorted_special_tokens([b"[a]", b"[B]"], True) == [b"[b]", b"[a]"]
+    assert onorm._binary_search([b"[b]", b"[a]"], b"[a]") is False
+    assert onorm._binary_search([b"[b]", b"[a]"], b"[b]") is False
+    assert onorm._binary_search([b"[a]", b"[b]"], b"[b]") is True
+
+
+def test_decode_follows_the_lead_byte():
+    # a lead byte decides the length alone: continuation bytes are not checked, bytes past the end read as 0
+    assert onorm._decode("é".encode(), 0) == 0xE9
+    assert onorm._decode("丏".encode(), 0) == 0x4E0F
+    assert onorm._decode("😀".encode(), 0) == 0x1F600
+    assert onorm._decode(b"\xc3", 0) == (0x03 << 6)
+    assert onorm._decode(b"\xe4\xb8", 0) == ((0x4 << 12) | (0x38 << 6))
+
+
+def test_special_token_rules():
+    # a token is recognised only when '[' ... ']' spans at most 6 input characters and matches exactly
+    rows = ["[PAD]", "[PADS]", "[LONGER]", "x[pad]y", "[PAD", "[P-D]"]
+    col = gc.strings(rows)
+    got = onorm.normalize_characters(col, True, [b"[PAD]", b"[LONGER]", b"[XPADS]"]).to_pylist()
+    assert got == [b" [PAD] ", b" [ pads ] ", b" [ longer ] ", b"x [PAD] y", b" [ pad", b" [ p - d ] "]
+    got = onorm.normalize_characters(col, False, [b"[PAD]", b"[PADS]"]).to_pylist()
+    assert got == [b" [PAD] ", b" [PADS] ", b" [ LONGER ] ", b"x [ pad ] y", b" [ PAD", b" [ P - D ] "]
+
+
+def test_special_tokens_lowered_after_sorting_can_be_missed():
+    # "[PADS]" sorts before "[PAD]" ('S' < ']'), "[pads]" after "[pad]" (']' < 's'): the reference sorts, then
+    # lower-cases, then searches by halving, so with both tokens "[pad]" is no longer found
+    col = gc.strings(["[PAD]", "[PADS]"])
+    got = onorm.normalize_characters(col, True, [b"[PAD]", b"[PADS]", b"[LONGER]"]).to_pylist()
+    assert got == [b" [ pad ] ", b" [PADS] "]
