@@ -92,6 +92,7 @@ def main():
     import numpy as np
     import torch
     from cudf_amd import _capi, datagen, nvtext
+    from cudf_amd.arrow_host import HostStringsColumn
     _capi.load()
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
@@ -298,6 +299,33 @@ def main():
                "tokenize": {"ms_per_step": round(tsec * 1e3, 3), "input_GBps": round(ib / tsec / 1e9, 2),
                             "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": keep["o"].child_size,
                             "kernels_ms": {k: round(v, 3) for k, v in tk.items()}}}
+        keep.clear()
+        # normalize_characters, the step that precedes the tokenizer in a BERT pipeline (lower-casing, five special tokens)
+        special = nvtext.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(["[CLS]", "[SEP]", "[PAD]", "[MASK]", "[UNK]"]))
+        normalizer = nvtext.CharacterNormalizer(True, special)
+
+        def zstep():
+            keep["o"] = nvtext.normalize_characters(dc, normalizer)
+
+        zsec = timed_steps(zstep, max(3, args.steps // 2), 1, torch)
+        zk = kernel_times(zstep, 2, _capi, torch)
+        out_bytes = int(keep["o"].chars.numel())
+        leg["normalize_characters"] = {"ms_per_step": round(zsec * 1e3, 3), "input_GBps": round(ib / zsec / 1e9, 2),
+                                       "mrows_per_s": round(w.rows.size / zsec / 1e6, 3), "chars_out": out_bytes,
+                                       "kernels_ms": {k: round(v, 3) for k, v in zk.items()}}
+        if not args.no_cpu:
+            from oracle import normalize_py
+            n = 4000
+            smp = w.rows.slice(0, n)
+            t0 = time.perf_counter()
+            exp = normalize_py.normalize_characters(smp, True, [b"[CLS]", b"[SEP]", b"[PAD]", b"[MASK]", b"[UNK]"])
+            cs = time.perf_counter() - t0
+            got = nvtext.normalize_characters(dc.slice(0, n, smp.null_count), normalizer).to_host()
+            leg["normalize_characters"]["cpu_baseline"] = {
+                "value": round(input_bytes(smp) / cs / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.2f} MB), {cs:.2f} s, pure-Python restatement"}
+            same = np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets)
+            leg["normalize_characters"]["parity"] = "PASS" if same else "FAIL"
         keep.clear()
         a, b = datagen.make_params(p["P"], 64, p["param_seed"])
         da = torch.from_numpy(a.view(np.int64)).cuda()

@@ -23,6 +23,10 @@ EXPORTS = [
     "nvtext_amd_list_strings_from_arrow_device",
     "nvtext_amd_list_to_arrow_device",
     "nvtext_amd_fixed_to_arrow_device",
+    "nvtext_amd_character_normalizer_create",
+    "nvtext_amd_character_normalizer_destroy",
+    "nvtext_amd_normalize_characters",
+    "nvtext_amd_strings_result_free",
     "nvtext_amd_wordpiece_vocabulary_create",
     "nvtext_amd_wordpiece_vocabulary_destroy",
     "nvtext_amd_wordpiece_vocabulary_unk_id",
@@ -88,6 +92,21 @@ class FixedColumn(C.Structure):
         ("data", C.c_void_p),
         ("null_mask", C.c_void_p),
         ("data_bytes", C.c_size_t),
+        ("null_mask_bytes", C.c_size_t),
+    ]
+
+
+class StringsResult(C.Structure):
+    _fields_ = [
+        ("size", C.c_int32),
+        ("null_count", C.c_int32),
+        ("offsets_size", C.c_int32),
+        ("offsets", C.c_void_p),
+        ("chars", C.c_void_p),
+        ("chars_size", C.c_int64),
+        ("null_mask", C.c_void_p),
+        ("offsets_bytes", C.c_size_t),
+        ("chars_bytes", C.c_size_t),
         ("null_mask_bytes", C.c_size_t),
     ]
 
@@ -170,6 +189,16 @@ def load():
     L.nvtext_amd_fixed_to_arrow_device.restype = C.c_int
     L.nvtext_amd_fixed_to_arrow_device.argtypes = [C.POINTER(FixedColumn), C.c_void_p, C.POINTER(Allocator), C.POINTER(ArrowSchema),
                                                    C.POINTER(ArrowDeviceArray)]
+    L.nvtext_amd_character_normalizer_create.restype = C.c_int
+    L.nvtext_amd_character_normalizer_create.argtypes = [C.c_int32, C.POINTER(StringsColumn), C.c_void_p, C.POINTER(Allocator),
+                                                         C.POINTER(C.c_void_p)]
+    L.nvtext_amd_character_normalizer_destroy.restype = None
+    L.nvtext_amd_character_normalizer_destroy.argtypes = [C.c_void_p]
+    L.nvtext_amd_normalize_characters.restype = C.c_int
+    L.nvtext_amd_normalize_characters.argtypes = [C.POINTER(StringsColumn), C.c_void_p, C.c_void_p, C.POINTER(Allocator),
+                                                  C.POINTER(StringsResult)]
+    L.nvtext_amd_strings_result_free.restype = None
+    L.nvtext_amd_strings_result_free.argtypes = [C.POINTER(StringsResult), C.c_void_p, C.POINTER(Allocator)]
     L.nvtext_amd_wordpiece_vocabulary_create.restype = C.c_int
     L.nvtext_amd_wordpiece_vocabulary_create.argtypes = [C.POINTER(StringsColumn), C.c_void_p,
                                                          C.POINTER(Allocator), C.POINTER(C.c_void_p)]

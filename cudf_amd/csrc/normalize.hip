@@ -1,0 +1,591 @@
+// nvtext::normalize_characters for gfx950: the BERT basic-tokenizer clean-up of a strings column
+// (cpp/src/text/normalize.cu:219-573).
+//
+// The reference expands every input byte into three uint32 slots in global memory, fixes the special tokens up
+// in a second kernel, reduces the slots to row sizes and compacts them.  Here a workgroup takes a tile of
+// 1024 input bytes (plus a few either side), keeps the slots in LDS, and the column is walked twice: once to
+// learn how many bytes each tile produces, once to write them, coalesced, at the offsets a scan of those
+// counts gives.  HBM sees the input twice and the output once; the slots never leave the CU.
+#include <algorithm>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "common.cuh"
+
+struct nvtext_amd_character_normalizer {
+  int device            = 0;
+  int32_t do_lower      = 0;
+  uint32_t* entries     = nullptr;  // device, kCodepoints: category << 24 | multi << 23 | replacement
+  uint64_t* second      = nullptr;  // device, kCodepoints: second << 32 | third replacement code point
+  uint8_t* token_chars  = nullptr;  // device: the special tokens, sorted then lower-cased
+  int32_t* token_offset = nullptr;  // device, tokens + 1
+  int32_t tokens        = 0;
+};
+
+namespace nvtext_amd {
+namespace {
+
+#include "codepoint_tables.inc"
+
+constexpr uint32_t kCodepoints   = 0x110000;
+constexpr uint32_t kDefaultEntry = 5u << 24;
+
+// categories of an entry (cpp/src/text/detail/cp_data.h, read through the accessors of normalize.cu:44-98)
+constexpr uint32_t kPad = 0, kPadIfLower = 1, kRemove = 2, kRemoveIfLower = 3, kReplace = 4;
+
+constexpr int kNormThreads = 256;
+constexpr int kNormTile    = 1024;  // input bytes per workgroup
+constexpr int kNormItems   = kNormTile / kNormThreads;
+constexpr int kBefore      = 5;   // a '[' this many bytes before the tile can still change the tile's slots
+constexpr int kAfter       = 6;   // a '[' of the tile reads slots this many bytes past it
+constexpr int kSlots       = kNormTile + kBefore + kAfter;
+constexpr int kRawBefore   = 8;   // bytes staged before the tile (>= kBefore)
+constexpr int kRawAfter    = 12;  // bytes staged after it (>= kAfter + 3 for the longest character)
+constexpr int kRawWords    = (kNormTile + kRawBefore + kRawAfter + 3 + 3) / 4;
+constexpr int kMaxOut      = 12;  // bytes one input byte can produce: three characters of four bytes
+
+struct NormTables {
+  const uint32_t* entries;
+  const uint64_t* second;
+  const uint8_t* token_chars;
+  const int32_t* token_offset;
+  int32_t tokens;
+  int32_t do_lower;
+};
+
+// cudf::strings::detail::codepoint_to_utf8 then from_char_utf8 (cpp/include/cudf/strings/detail/utf8.hpp:170-197,
+// 143-168): the bytes of the character, first byte in the low bits, as the reference leaves them in a slot.
+__device__ __forceinline__ uint32_t utf8_le(uint32_t cp)
+{
+  if (cp < 0x80u) return cp;
+  uint32_t const t0 = 0x80u | (cp & 0x3Fu);
+  uint32_t const t1 = 0x80u | ((cp >> 6) & 0x3Fu);
+  if (cp < 0x800u) return (0xC0u | (cp >> 6)) | (t0 << 8);
+  uint32_t const t2 = 0x80u | ((cp >> 12) & 0x3Fu);
+  if (cp < 0x10000u) return (0xE0u | (cp >> 12)) | (t1 << 8) | (t0 << 16);
+  return (0xF0u | ((cp >> 18) & 0x07u)) | (t2 << 8) | (t1 << 16) | (t0 << 24);
+}
+
+__device__ __forceinline__ uint32_t bytes_of(uint32_t slot) { return (slot != 0) + (slot > 0xFFu) + (slot > 0xFFFFu) + (slot > 0xFFFFFFu); }
+
+// The code point of the character that starts with b0, the next bytes being b1..b3
+// (to_char_utf8 and utf8_to_codepoint, cpp/include/cudf/strings/detail/utf8.hpp:68-97,118-140: the first byte
+// alone says how many bytes belong to the character).
+__device__ __forceinline__ uint32_t decode(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3)
+{
+  if (b0 < 0x80u) return b0;
+  if (b0 < 0xE0u) return ((b0 & 0x1Fu) << 6) | (b1 & 0x3Fu);
+  if (b0 < 0xF0u) return ((b0 & 0x0Fu) << 12) | ((b1 & 0x3Fu) << 6) | (b2 & 0x3Fu);
+  // packed value above 0xF8000000 decodes to 0
+  uint32_t const packed = (b0 << 24) | (b1 << 16) | (b2 << 8) | b3;
+  if (packed > 0xF8000000u) return 0u;
+  return ((b0 & 0x07u) << 18) | ((b1 & 0x3Fu) << 12) | ((b2 & 0x3Fu) << 6) | (b3 & 0x3Fu);
+}
+
+// The slots of one code point (data_normalizer_kernel, cpp/src/text/normalize.cu:331-378).
+__device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
+{
+  s0 = s1 = s2               = 0;
+  uint32_t const e           = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
+  uint32_t const cat         = (e >> 24) & 7u;
+  bool const lower           = t.do_lower != 0;
+  if (cat == kRemove || (lower && cat == kRemoveIfLower)) return;
+  uint32_t const repl = (lower || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
+  uint32_t r0 = repl ? repl : cp, r1 = 0, r2 = 0;
+  bool single = true;
+  if (lower && ((e >> 23) & 1u)) {
+    uint64_t const next = t.second[cp];
+    r1                  = static_cast<uint32_t>(next >> 32);
+    r2                  = static_cast<uint32_t>(next);
+    single              = false;
+  }
+  if ((cat == kPad || (lower && cat == kPadIfLower)) && single) {
+    r1 = r0;
+    r0 = r2 = 0x20u;
+  }
+  s0 = r0 ? utf8_le(r0) : 0u;
+  s1 = r1 ? utf8_le(r1) : 0u;
+  s2 = r2 ? utf8_le(r2) : 0u;
+}
+
+struct NormLds {
+  uint32_t raw[kRawWords];           // the input bytes of the tile and its surroundings, zero outside the column
+  uint32_t slot[3][kSlots];          // slot k of position i - kBefore
+  uint32_t sizes[kNormTile / 4];     // output bytes of each tile position, one byte each
+  uint16_t prefix[kNormTile + 4];    // bytes the tile writes before each position; [tile] = all of them
+  uint32_t scan[kNormThreads / kWave + 1];
+};
+
+// Slot `at` of the flat slot sequence (three per position).
+__device__ __forceinline__ uint32_t& flat_slot(NormLds& lds, int at) { return lds.slot[at % 3][at / 3]; }
+
+// Compares the candidate in flat slots [from, to] (spaces and empty slots skipped, one byte per character) with
+// special token `i`: < 0, 0, > 0 as the candidate sorts before, equal to or after it.
+__device__ int compare_candidate(NormLds& lds, int from, int to, NormTables const& t, int32_t i)
+{
+  const uint8_t* tok = t.token_chars + t.token_offset[i];
+  int32_t const tl   = t.token_offset[i + 1] - t.token_offset[i];
+  int32_t j          = 0;
+  for (int at = from; at <= to; ++at) {
+    uint32_t const c = flat_slot(lds, at) & 0xFFu;
+    if (c == 0u || c == 0x20u) continue;
+    if (j >= tl) return 1;
+    uint32_t const b = tok[j++];
+    if (c != b) return c < b ? -1 : 1;
+  }
+  return j < tl ? -1 : 0;
+}
+
+// One tile: fills lds.slot for the tile and its surroundings, applies the special tokens, leaves the output size
+// of every tile position in lds.sizes.
+__device__ __forceinline__ void tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t)
+{
+  int const tid = threadIdx.x;
+  // stage [t0 - kRawBefore, t0 + kNormTile + kRawAfter) with aligned dword loads; bytes outside [0, n) read as 0
+  const uint8_t* const wb = chars + t0 - kRawBefore;
+  uint32_t const mis      = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 3u);
+  const uint32_t* const ap = reinterpret_cast<const uint32_t*>(wb - mis);
+  for (int w = tid; w < kRawWords; w += kNormThreads) {
+    int64_t const p = t0 - kRawBefore - mis + 4 * static_cast<int64_t>(w);  // column position of the word's first byte
+    uint32_t v      = 0;
+    if (p + 3 >= 0 && p < n) {
+      v = ap[w];
+      if (p < 0) v &= 0xFFFFFFFFu << (8 * static_cast<uint32_t>(-p));
+      if (p + 4 > n) v &= 0xFFFFFFFFu >> (8 * static_cast<uint32_t>(p + 4 - n));
+    }
+    lds.raw[w] = v;
+  }
+  __syncthreads();
+  const uint8_t* const rawb = reinterpret_cast<const uint8_t*>(lds.raw) + mis + kRawBefore - kBefore;  // byte of slot index 0
+  for (int i = tid; i < kSlots; i += kNormThreads) {
+    uint32_t const b0 = rawb[i];
+    uint32_t s0 = 0, s1 = 0, s2 = 0;
+    if (b0 != 0u && (b0 & 0xC0u) != 0x80u) {  // byte 0 is U+0000, which is removed
+      uint32_t cp = b0;
+      if (b0 >= 0xC0u) cp = decode(b0, rawb[i + 1], rawb[i + 2], rawb[i + 3]);
+      slots_of(cp, t, s0, s1, s2);
+    }
+    lds.slot[0][i] = s0;
+    lds.slot[1][i] = s1;
+    lds.slot[2][i] = s2;
+  }
+  __syncthreads();
+  if (t.tokens > 0) {
+    // special_tokens_kernel (normalize.cu:270-316), in two steps so that every decision reads unchanged slots
+    int found_from[(kSlots + kNormThreads - 1) / kNormThreads];
+    int found_to[(kSlots + kNormThreads - 1) / kNormThreads];
+#pragma unroll
+    for (int k = 0; k < (kSlots + kNormThreads - 1) / kNormThreads; ++k) {
+      int const i   = tid + k * kNormThreads;
+      found_from[k] = -1;
+      found_to[k]   = -1;
+      // a '[' in the last kAfter positions belongs to the next tile
+      if (i < kNormTile + kBefore && lds.slot[1][i] == '[') {
+        int const from = 3 * i + 1;
+        int to         = -1;
+        for (int at = from + 1; at < from + 18; ++at) {
+          if (flat_slot(lds, at) == ']') {
+            to = at;
+            break;
+          }
+        }
+        if (to > 0) {
+          int32_t first = 0, count = t.tokens;  // thrust::binary_search: lower_bound by halving, then !(value < *it)
+          while (count > 0) {
+            int32_t const half = count >> 1;
+            if (compare_candidate(lds, from, to, t, first + half) > 0) {
+              first += half + 1;
+              count -= half + 1;
+            } else {
+              count = half;
+            }
+          }
+          if (first < t.tokens && compare_candidate(lds, from, to, t, first) >= 0) {
+            found_from[k] = from;
+            found_to[k]   = to;
+          }
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < (kSlots + kNormThreads - 1) / kNormThreads; ++k) {
+      if (found_from[k] < 0) continue;
+      flat_slot(lds, found_from[k] + 1) = 0u;  // the space after '['
+      flat_slot(lds, found_to[k] - 1)   = 0u;  // the space before ']'
+      if (t.do_lower) {
+        for (int at = found_from[k] + 2; at < found_to[k] - 2; ++at) {
+          uint32_t const c = flat_slot(lds, at);
+          if (c >= 'a' && c <= 'z') flat_slot(lds, at) = c - 'a' + 'A';
+        }
+      }
+    }
+    __syncthreads();
+  }
+  uint8_t* const sizes = reinterpret_cast<uint8_t*>(lds.sizes);
+  for (int i = tid; i < kNormTile; i += kNormThreads) {
+    int const s = i + kBefore;
+    sizes[i]    = static_cast<uint8_t>(bytes_of(lds.slot[0][s]) + bytes_of(lds.slot[1][s]) + bytes_of(lds.slot[2][s]));
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ uint32_t sum_bytes(uint32_t v) { return (v & 0xFFu) + ((v >> 8) & 0xFFu) + ((v >> 16) & 0xFFu) + (v >> 24); }
+
+// tile_bytes[tile] = bytes the tile's input positions produce
+__global__ void __launch_bounds__(kNormThreads) normalize_count_kernel(const uint8_t* __restrict__ chars, int64_t n, NormTables t,
+                                                                       uint32_t* __restrict__ tile_bytes)
+{
+  __shared__ NormLds lds;
+  int64_t const t0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
+  tile_slots(lds, chars, t0, n, t);
+  uint32_t total;
+  block_exclusive_scan<kNormThreads>(sum_bytes(lds.sizes[threadIdx.x]), lds.scan, &total);
+  if (threadIdx.x == 0) tile_bytes[blockIdx.x] = total;
+}
+
+// Writes the tile's bytes at tile_offset[tile] and the output offset of every row that starts in the tile.
+__global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView col, int64_t first, int64_t n, NormTables t,
+                                                                       const uint64_t* __restrict__ tile_offset, uint8_t* __restrict__ out_chars,
+                                                                       int32_t* __restrict__ out_offsets)
+{
+  __shared__ NormLds lds;
+  __shared__ uint32_t staged[(kNormTile * kMaxOut + 4) / 4];
+  int const tid        = threadIdx.x;
+  int64_t const t0     = static_cast<int64_t>(blockIdx.x) * kNormTile;
+  int64_t const t1     = min(t0 + kNormTile, n);
+  uint64_t const base  = tile_offset[blockIdx.x];
+  tile_slots(lds, col.chars + first, t0, n, t);
+
+  uint32_t const four = lds.sizes[tid];
+  uint32_t total;
+  uint32_t run = block_exclusive_scan<kNormThreads>(sum_bytes(four), lds.scan, &total);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    lds.prefix[4 * tid + k] = static_cast<uint16_t>(run);
+    run += (four >> (8 * k)) & 0xFFu;
+  }
+  if (tid == kNormThreads - 1) lds.prefix[kNormTile] = static_cast<uint16_t>(run);
+  __syncthreads();
+
+  // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword
+  uint8_t* const dst  = out_chars + base;
+  uint32_t const lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 3u);
+  uint8_t* const sb   = reinterpret_cast<uint8_t*>(staged);
+#pragma unroll
+  for (int k = 0; k < kNormItems; ++k) {
+    int const i = tid + k * kNormThreads;
+    uint32_t o  = lead + lds.prefix[i];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      uint32_t v = lds.slot[s][i + kBefore];
+      while (v) {
+        sb[o++] = static_cast<uint8_t>(v);
+        v >>= 8;
+      }
+    }
+  }
+  __syncthreads();
+  uint32_t const end      = lead + total;
+  uint32_t const w_lo     = (lead + 3u) >> 2;
+  uint32_t const w_hi     = end >> 2;
+  uint32_t* const dw      = reinterpret_cast<uint32_t*>(dst - lead);
+  for (uint32_t w = w_lo + tid; w < w_hi; w += kNormThreads) dw[w] = staged[w];
+  uint32_t const head_end   = min(4u * w_lo, end);
+  uint32_t const tail_begin = max(4u * w_hi, head_end);
+  if (tid < 4) {
+    uint32_t const at = lead + tid;
+    if (at < head_end) (dst - lead)[at] = sb[at];
+  } else if (tid < 8) {
+    uint32_t const at = tail_begin + (tid - 4);
+    if (at < end) (dst - lead)[at] = sb[at];
+  }
+
+  // rows whose first byte lies in [t0, t1) -- in [t0, n] for the last tile -- start at base + prefix
+  int64_t const rows = col.size;
+  int64_t lo = 0, hi = rows + 1;
+  while (lo < hi) {
+    int64_t const mid = (lo + hi) >> 1;
+    if (col.off(mid) - first < t0) lo = mid + 1;
+    else hi = mid;
+  }
+  bool const last_tile = blockIdx.x == gridDim.x - 1;
+  for (int64_t r = lo + tid; r <= rows; r += kNormThreads) {
+    int64_t const p = col.off(r) - first;
+    if (p > t1 || (p == t1 && !last_tile)) break;
+    out_offsets[r] = static_cast<int32_t>(base + lds.prefix[p - t0]);
+  }
+}
+
+struct TileBytes {
+  const uint32_t* counts;
+  __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
+};
+
+// ------------------------------------------------------------------ host: tables and tokens
+void append_utf8(std::string& s, uint32_t cp)
+{
+  if (cp < 0x80u) {
+    s.push_back(static_cast<char>(cp));
+  } else if (cp < 0x800u) {
+    s.push_back(static_cast<char>(0xC0u | (cp >> 6)));
+    s.push_back(static_cast<char>(0x80u | (cp & 0x3Fu)));
+  } else if (cp < 0x10000u) {
+    s.push_back(static_cast<char>(0xE0u | (cp >> 12)));
+    s.push_back(static_cast<char>(0x80u | ((cp >> 6) & 0x3Fu)));
+    s.push_back(static_cast<char>(0x80u | (cp & 0x3Fu)));
+  } else {
+    s.push_back(static_cast<char>(0xF0u | ((cp >> 18) & 0x07u)));
+    s.push_back(static_cast<char>(0x80u | ((cp >> 12) & 0x3Fu)));
+    s.push_back(static_cast<char>(0x80u | ((cp >> 6) & 0x3Fu)));
+    s.push_back(static_cast<char>(0x80u | (cp & 0x3Fu)));
+  }
+}
+
+// cudf::strings::to_lower of one string (cpp/src/strings/case.cu:142-148: code points above U+FFFF stay).
+// Bytes that are not well-formed UTF-8 are copied as they are.
+std::string to_lower_bmp(std::string const& in)
+{
+  std::string out;
+  size_t i = 0;
+  auto cont = [&](size_t k) { return k < in.size() && (static_cast<uint8_t>(in[k]) & 0xC0u) == 0x80u; };
+  while (i < in.size()) {
+    uint32_t const b0 = static_cast<uint8_t>(in[i]);
+    uint32_t cp       = b0;
+    size_t len        = 1;
+    if (b0 >= 0xC2u && b0 < 0xE0u && cont(i + 1)) {
+      cp  = ((b0 & 0x1Fu) << 6) | (static_cast<uint8_t>(in[i + 1]) & 0x3Fu);
+      len = 2;
+    } else if (b0 >= 0xE0u && b0 < 0xF0u && cont(i + 1) && cont(i + 2)) {
+      cp  = ((b0 & 0x0Fu) << 12) | ((static_cast<uint8_t>(in[i + 1]) & 0x3Fu) << 6) | (static_cast<uint8_t>(in[i + 2]) & 0x3Fu);
+      len = 3;
+    } else if (b0 >= 0x80u) {
+      len = 1;
+      cp  = 0xFFFFFFFFu;  // not a BMP character: copied
+      if (b0 >= 0xF0u && cont(i + 1) && cont(i + 2) && cont(i + 3)) len = 4;
+    }
+    const uint32_t(*row)[4] = nullptr;
+    if (cp <= 0xFFFFu) {
+      auto const* end = kLowerCase + sizeof(kLowerCase) / sizeof(kLowerCase[0]);
+      auto const* it  = std::lower_bound(kLowerCase, end, cp, [](const uint32_t(&r)[4], uint32_t v) { return r[0] < v; });
+      if (it != end && (*it)[0] == cp) row = it;
+    }
+    if (row) {
+      for (int k = 1; k < 4; ++k)
+        if ((*row)[k]) append_utf8(out, (*row)[k]);
+    } else {
+      out.append(in, i, len);
+    }
+    i += len;
+  }
+  return out;
+}
+
+}  // namespace
+}  // namespace nvtext_amd
+
+extern "C" {
+
+nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, const nvtext_amd_strings_column* special_tokens, void* stream_,
+                                                         const nvtext_amd_allocator* mr, nvtext_amd_character_normalizer** out)
+{
+  using namespace nvtext_amd;
+  (void)mr;  // the tables live as long as the object: plain hipMalloc / hipFree
+  if (!out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  *out               = nullptr;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  std::vector<std::string> tokens;
+  if (special_tokens && special_tokens->size > 0) {
+    // cpp/src/text/normalize.cu:227-228
+    if (special_tokens->null_count > 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "special tokens should not have nulls");
+    int32_t const count = special_tokens->size;
+    size_t const ow     = special_tokens->offsets_is_int64 ? 8 : 4;
+    std::vector<uint8_t> h_off((static_cast<size_t>(count) + 1) * ow);
+    const uint8_t* d_off = static_cast<const uint8_t*>(special_tokens->offsets) + static_cast<size_t>(special_tokens->offset) * ow;
+    NVTEXT_HIP_TRY(hipMemcpyAsync(h_off.data(), d_off, h_off.size(), hipMemcpyDeviceToHost, stream));
+    NVTEXT_HIP_TRY(hipStreamSynchronize(stream));
+    auto off_at = [&](int32_t i) -> int64_t {
+      if (ow == 8) {
+        int64_t v;
+        std::memcpy(&v, h_off.data() + static_cast<size_t>(i) * 8, 8);
+        return v;
+      }
+      int32_t v;
+      std::memcpy(&v, h_off.data() + static_cast<size_t>(i) * 4, 4);
+      return v;
+    };
+    int64_t const first = off_at(0), last = off_at(count);
+    if (last < first) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "special token offsets are not monotone");
+    std::string pool(static_cast<size_t>(last - first), '\0');
+    if (!pool.empty()) {
+      NVTEXT_HIP_TRY(hipMemcpyAsync(&pool[0], special_tokens->chars + first, pool.size(), hipMemcpyDeviceToHost, stream));
+      NVTEXT_HIP_TRY(hipStreamSynchronize(stream));
+    }
+    for (int32_t i = 0; i < count; ++i) tokens.emplace_back(pool, static_cast<size_t>(off_at(i) - first), static_cast<size_t>(off_at(i + 1) - off_at(i)));
+    // cpp/src/text/normalize.cu:230-235: sorted by bytes first, lower-cased afterwards
+    std::sort(tokens.begin(), tokens.end(), [](std::string const& a, std::string const& b) {
+      int const c = std::memcmp(a.data(), b.data(), std::min(a.size(), b.size()));
+      return c != 0 ? c < 0 : a.size() < b.size();
+    });
+    if (do_lower_case)
+      for (auto& tk : tokens) tk = to_lower_bmp(tk);
+  }
+
+  // dense tables from the generated runs; the Hangul syllables decompose by arithmetic (The Unicode Standard, 3.12)
+  std::vector<uint32_t> entries(kCodepoints, kDefaultEntry);
+  std::vector<uint64_t> second(kCodepoints, 0);
+  for (auto const& run : kCodepointRuns) std::fill(entries.begin() + run[0], entries.begin() + run[0] + run[1], run[2]);
+  for (auto const& pair : kCodepointSecond) second[static_cast<size_t>(pair[0])] = pair[1];
+  for (uint32_t s = 0; s < 11172u; ++s) {
+    uint32_t const lead = 0x1100u + s / 588u, vowel = 0x1161u + (s % 588u) / 28u, trail = s % 28u;
+    entries[0xAC00u + s] = (5u << 24) | (1u << 23) | lead;
+    second[0xAC00u + s]  = (static_cast<uint64_t>(vowel) << 32) | (trail ? 0x11A7u + trail : 0u);
+  }
+
+  auto* obj      = new nvtext_amd_character_normalizer();
+  obj->do_lower  = do_lower_case ? 1 : 0;
+  obj->tokens    = static_cast<int32_t>(tokens.size());
+  auto fail_with = [&](hipError_t e) {
+    nvtext_amd_character_normalizer_destroy(obj);
+    return fail(e == hipErrorOutOfMemory ? NVTEXT_AMD_ALLOC_FAILED : NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+  };
+  hipError_t e = hipGetDevice(&obj->device);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->entries), entries.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->second), second.size() * sizeof(uint64_t));
+  if (e == hipSuccess) e = hipMemcpy(obj->entries, entries.data(), entries.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(obj->second, second.data(), second.size() * sizeof(uint64_t), hipMemcpyHostToDevice);
+  if (e != hipSuccess) return fail_with(e);
+  if (!tokens.empty()) {
+    std::vector<int32_t> offsets(tokens.size() + 1, 0);
+    std::string chars;
+    for (size_t i = 0; i < tokens.size(); ++i) {
+      chars += tokens[i];
+      if (chars.size() > 0x7FFFFFFFull) {
+        nvtext_amd_character_normalizer_destroy(obj);
+        return fail(NVTEXT_AMD_OVERFLOW, "special tokens too large");
+      }
+      offsets[i + 1] = static_cast<int32_t>(chars.size());
+    }
+    e = hipMalloc(reinterpret_cast<void**>(&obj->token_offset), offsets.size() * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->token_chars), std::max<size_t>(chars.size(), 1));
+    if (e == hipSuccess) e = hipMemcpy(obj->token_offset, offsets.data(), offsets.size() * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e == hipSuccess && !chars.empty()) e = hipMemcpy(obj->token_chars, chars.data(), chars.size(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return fail_with(e);
+  }
+  *out = obj;
+  return NVTEXT_AMD_SUCCESS;
+}
+
+void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* normalizer)
+{
+  if (!normalizer) return;
+  (void)hipFree(normalizer->entries);
+  (void)hipFree(normalizer->second);
+  (void)hipFree(normalizer->token_chars);
+  (void)hipFree(normalizer->token_offset);
+  delete normalizer;
+}
+
+nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_column* input, const nvtext_amd_character_normalizer* normalizer,
+                                                  void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_strings_result* out)
+{
+  using namespace nvtext_amd;
+  if (!input || !normalizer || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  *out = nvtext_amd_strings_result{};
+  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
+  if (input->null_count > 0 && !input->null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
+  int device = 0;
+  NVTEXT_HIP_TRY(hipGetDevice(&device));
+  if (device != normalizer->device) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "the normalizer belongs to another device");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Mr mr{mr_, stream};
+  int32_t const rows = input->size;
+  if (rows == 0) return NVTEXT_AMD_SUCCESS;  // normalize.cu:497: the empty strings column
+  if (!input->offsets) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "offsets missing");
+
+  // normalize.cu:499-501: the byte range of the view
+  size_t const ow      = input->offsets_is_int64 ? 8 : 4;
+  const uint8_t* d_off = static_cast<const uint8_t*>(input->offsets) + static_cast<size_t>(input->offset) * ow;
+  int64_t ends[2]      = {0, 0};
+  int32_t ends32[2]    = {0, 0};
+  for (int k = 0; k < 2; ++k) {
+    void* host = ow == 8 ? static_cast<void*>(&ends[k]) : static_cast<void*>(&ends32[k]);
+    NVTEXT_HIP_TRY(hipMemcpyAsync(host, d_off + (k ? static_cast<size_t>(rows) * ow : 0), ow, hipMemcpyDeviceToHost, stream));
+  }
+  NVTEXT_HIP_TRY(hipStreamSynchronize(stream));
+  int64_t const first = ow == 8 ? ends[0] : ends32[0];
+  int64_t const last  = ow == 8 ? ends[1] : ends32[1];
+  if (last < first) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "offsets are not monotone");
+  int64_t const n = last - first;
+  if (n > 0 && !input->chars) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "chars missing");
+
+  auto release = [&](nvtext_amd_status st, const char* msg) {
+    nvtext_amd_strings_result_free(out, stream_, mr_);
+    return fail(st, msg);
+  };
+  out->size          = rows;
+  out->null_count    = input->null_count;
+  out->offsets_size  = rows + 1;
+  out->offsets_bytes = (static_cast<size_t>(rows) + 1) * sizeof(int32_t);
+  out->offsets       = static_cast<int32_t*>(mr.allocate(out->offsets_bytes));
+  if (!out->offsets) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
+  if (input->null_mask) {  // copy_bitmask(input): cpp/src/bitmask/null_mask.cu:381-391
+    out->null_mask_bytes = mask_alloc_bytes(rows);
+    out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
+    if (!out->null_mask) return release(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
+    launch_copy_bitmask(out->null_mask, input->null_mask, input->offset, rows, stream);
+  }
+  if (n == 0) {  // normalize.cu:504: nothing to normalize, every row is empty
+    launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, static_cast<int64_t>(rows) + 1, stream);
+    NVTEXT_HIP_TRY(hipGetLastError());
+    return NVTEXT_AMD_SUCCESS;
+  }
+
+  int64_t const tiles = (n + kNormTile - 1) / kNormTile;
+  if (tiles > 0x7FFFFFFFll) return release(NVTEXT_AMD_OVERFLOW, "input too large");
+  Temp tile_bytes(mr, static_cast<size_t>(tiles) * sizeof(uint32_t));
+  Temp tile_offset(mr, (static_cast<size_t>(tiles) + 1) * sizeof(uint64_t));
+  Temp scan_temp(mr, scan_temp_bytes(tiles));
+  if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+  NormTables const tables{normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
+                          normalizer->do_lower};
+  ColView const view = make_view(*input);
+  {
+    ProfileScope ps("normalize_count_kernel", stream);
+    hipLaunchKernelGGL(normalize_count_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view.chars + first, n, tables,
+                       tile_bytes.as<uint32_t>());
+  }
+  device_exclusive_scan(TileBytes{tile_bytes.as<uint32_t>()}, tiles, tile_offset.as<uint64_t>(), scan_temp.as<uint64_t>(), stream);
+  uint64_t total = 0;
+  hipError_t e   = hipMemcpyAsync(&total, tile_offset.as<uint64_t>() + tiles, sizeof(total), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) return release(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+  if (total > 0x7FFFFFFFull) return release(NVTEXT_AMD_OVERFLOW, "normalized strings exceed the int32 offset range");
+  out->chars_size = static_cast<int64_t>(total);
+  if (total > 0) {
+    out->chars_bytes = static_cast<size_t>(total);
+    out->chars       = static_cast<char*>(mr.allocate(out->chars_bytes));
+    if (!out->chars) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
+  }
+  {
+    ProfileScope ps("normalize_write_kernel", stream);
+    hipLaunchKernelGGL(normalize_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view, first, n, tables,
+                       tile_offset.as<uint64_t>(), reinterpret_cast<uint8_t*>(out->chars), out->offsets);
+  }
+  e = hipGetLastError();
+  if (e != hipSuccess) return release(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+  return NVTEXT_AMD_SUCCESS;
+}
+
+void nvtext_amd_strings_result_free(nvtext_amd_strings_result* col, void* stream, const nvtext_amd_allocator* mr)
+{
+  if (!col) return;
+  nvtext_amd::Mr m{mr, static_cast<hipStream_t>(stream)};
+  m.deallocate(col->offsets, col->offsets_bytes);
+  m.deallocate(col->chars, col->chars_bytes);
+  m.deallocate(col->null_mask, col->null_mask_bytes);
+  *col = nvtext_amd_strings_result{};
+}
+
+}  // extern "C"

@@ -101,6 +101,13 @@ class DeviceStringsColumn:
     def slice(self, lo: int, hi: int, null_count: int) -> "DeviceStringsColumn":
         return DeviceStringsColumn(self.chars, self.offsets, self.mask, hi - lo, self.offset + lo, null_count)
 
+    def to_host(self) -> HostStringsColumn:
+        torch = _torch()
+        torch.cuda.current_stream().synchronize()
+        offsets = self.offsets.cpu().numpy().copy() if self.offsets is not None else np.zeros(0, np.int32)
+        mask = self.mask.cpu().numpy().view(np.uint32).copy() if self.mask is not None else None
+        return HostStringsColumn(self.chars.cpu().numpy().copy(), offsets, mask, self.size, self.offset, self.null_count)
+
     def _c(self) -> _capi.StringsColumn:
         torch = _torch()
         is64 = 0
@@ -295,6 +302,54 @@ def jaccard_index(input1: DeviceStringsColumn, input2: DeviceStringsColumn, widt
         _raise(st)
     mr = _mr()
     return DeviceFixedColumn(mr.take(out.data), mr.take(out.null_mask), int(out.size), int(out.null_count), np.dtype(np.float32))
+
+
+class CharacterNormalizer:
+    """nvtext::character_normalizer (cpp/include/nvtext/normalize.hpp:81-124); pylibcudf normalize.pyx CharacterNormalizer."""
+
+    def __init__(self, do_lower_case: bool, special_tokens: Optional[DeviceStringsColumn] = None):
+        L = _capi.load()
+        h = C.c_void_p()
+        col = special_tokens._c() if special_tokens is not None else None
+        st = L.nvtext_amd_character_normalizer_create(int(bool(do_lower_case)), C.byref(col) if col is not None else None,
+                                                      _stream_handle(), C.byref(_mr().struct), C.byref(h))
+        if st != _capi.SUCCESS:
+            _raise(st)
+        self._h = h
+        self.do_lower_case = bool(do_lower_case)
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            try:
+                _capi.load().nvtext_amd_character_normalizer_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+
+def normalize_characters(input: DeviceStringsColumn, normalizer: CharacterNormalizer) -> DeviceStringsColumn:
+    """nvtext::normalize_characters (cpp/include/nvtext/normalize.hpp:126-160); pylibcudf normalize.pyx normalize_characters."""
+    L = _capi.load()
+    out = _capi.StringsResult()
+    col = input._c()
+    st = L.nvtext_amd_normalize_characters(C.byref(col), normalizer._h, _stream_handle(), C.byref(_mr().struct), C.byref(out))
+    if st != _capi.SUCCESS:
+        _raise(st)
+    mr = _mr()
+    torch = _torch()
+    chars = mr.take(out.chars)
+    offsets = mr.take(out.offsets)
+    mask = mr.take(out.null_mask)
+    if chars is None:
+        chars = torch.empty(0, dtype=torch.uint8, device="cuda")
+    else:
+        chars = chars[: int(out.chars_size)]
+    if offsets is not None:
+        offsets = offsets.view(torch.int32)[: int(out.offsets_size)]
+    if mask is not None:
+        mask = mask[: (int(out.size) + 31) // 32 * 4].view(torch.int32)
+    return DeviceStringsColumn(chars, offsets, mask, int(out.size), 0, int(out.null_count))
 
 
 class WordPieceVocabulary:

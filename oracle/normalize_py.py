@@ -186,3 +186,24 @@ def normalize_characters(col, do_lower_case: bool, special_tokens: Sequence[byte
     out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(np.int32)
     chars = np.frombuffer(b"".join(pieces), dtype=np.uint8).copy()
     return HostStringsColumn(chars, out_off, copy_bitmask(col), col.size, 0, col.null_count)
+
+
+def normalize_ascii(col, do_lower_case: bool):
+    """normalize_characters for a column whose bytes are all below 0x80, no special tokens: the same rules through a
+    256-entry table and numpy, for inputs too large for the loops above.  Tests check it against
+    normalize_characters on small inputs before relying on it."""
+    from cudf_amd.arrow_host import HostStringsColumn
+    from oracle.pyoracle import copy_bitmask
+    table = np.zeros((128, 3), np.uint8)
+    for cp in range(128):
+        slots = normalize_flat(bytes([cp]), do_lower_case)[0]
+        table[cp] = [s[0] if s else 0 for s in slots]
+    off = np.asarray(col.offsets).astype(np.int64)
+    first, last = int(off[col.offset]), int(off[col.offset + col.size])
+    data = np.ascontiguousarray(col.chars[first:last])
+    assert data.size == 0 or int(data.max()) < 0x80
+    slots = table[data]                                   # (n, 3)
+    keep = slots != 0
+    prefix = np.concatenate([[0], np.cumsum(keep.sum(axis=1, dtype=np.int64))])
+    out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(np.int32)
+    return HostStringsColumn(slots[keep], out_off, copy_bitmask(col), col.size, 0, col.null_count)

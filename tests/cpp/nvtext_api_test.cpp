@@ -1,7 +1,8 @@
 // Exercises the C++ mirror of the nvtext API (cudf_amd/include) on the GPU with the cases of the
 // reference's gtests: cpp/tests/text/minhash_tests.cpp (Permuted, PermutedWide, EmptyTest, ErrorsTest, Ngrams, NgramsWide,
 // NgramsSliced), cpp/tests/text/jaccard_tests.cpp (Basic, WithNulls, Errors)
-// and cpp/tests/text/subword_tests.cpp (all seven).  Own tiny harness: prints one line per case and
+// cpp/tests/text/normalize_tests.cpp (NormalizeEmptyTest, AllNullStrings, SomeNullStrings, WithNormalizer, SpecialTokens,
+// NormalizeSlicedColumn) and cpp/tests/text/subword_tests.cpp (all seven).  Own tiny harness: prints one line per case and
 // exits non-zero on the first failure.
 #include <cudf/column/column.hpp>
 #include <cudf/lists/lists_column_view.hpp>
@@ -9,6 +10,7 @@
 #include <hip/hip_runtime.h>
 #include <nvtext/jaccard.hpp>
 #include <nvtext/minhash.hpp>
+#include <nvtext/normalize.hpp>
 #include <nvtext/wordpiece_tokenize.hpp>
 
 #include <cstdio>
@@ -328,6 +330,89 @@ void test_jaccard()
   }
 }
 
+// rows of a STRING column, nullopt for nulls
+std::vector<Text> download_strings(cudf::column const& col)
+{
+  HIP_OK(hipDeviceSynchronize());
+  auto const v = col.view();
+  int const n  = v.size();
+  std::vector<Text> rows;
+  if (n == 0) return rows;
+  std::vector<int32_t> off(n + 1);
+  HIP_OK(hipMemcpy(off.data(), v.child(0).head<void>(), off.size() * 4, hipMemcpyDeviceToHost));
+  std::vector<char> chars(off[n]);
+  if (!chars.empty()) HIP_OK(hipMemcpy(chars.data(), v.head<void>(), chars.size(), hipMemcpyDeviceToHost));
+  std::vector<uint32_t> mask((n + 31) / 32, 0xFFFFFFFFu);
+  if (v.null_mask()) HIP_OK(hipMemcpy(mask.data(), v.null_mask(), mask.size() * 4, hipMemcpyDeviceToHost));
+  for (int i = 0; i < n; ++i) {
+    if ((mask[i / 32] >> (i % 32)) & 1u) rows.emplace_back(std::string(chars.begin() + off[i], chars.begin() + off[i + 1]));
+    else rows.emplace_back(std::nullopt);
+  }
+  return rows;
+}
+
+void test_normalize()
+{
+  std::printf("TextNormalizeTest.NormalizeEmptyTest / AllNullStrings / SomeNullStrings / WithNormalizer / SpecialTokens / NormalizeSlicedColumn\n");
+  std::string const long_row = "this entry is intended to pad out past 256 bytes which is currently the block size";
+  {
+    auto empty      = make_strings({});
+    auto normalizer = nvtext::create_character_normalizer(true);
+    CHECK(nvtext::normalize_characters(cudf::strings_column_view(empty.view), *normalizer)->size() == 0);
+    auto nulls   = make_strings({std::nullopt, std::nullopt, std::nullopt});
+    auto results = nvtext::normalize_characters(cudf::strings_column_view(nulls.view), *normalizer);
+    CHECK(download_strings(*results) == (std::vector<Text>{std::nullopt, std::nullopt, std::nullopt}) && results->null_count() == 3);
+    auto some = make_strings({std::nullopt, ".", "a"});
+    results   = nvtext::normalize_characters(cudf::strings_column_view(some.view), *normalizer);
+    CHECK(download_strings(*results) == (std::vector<Text>{std::nullopt, " . ", "a"}));
+  }
+  {
+    auto input = make_strings({"abc\xC2\xA3" "def", std::nullopt, "\xC3\xA9\xC3\xA8 \xC3\xA2 \xC3\xAE\xC3\xB4\taeio",
+                               "\t\xC4\x82\xC4\x86\xC4\x96\xC3\x91  \xC3\x9C", "ACEN U", "P^NP", "$41.07", "[a,b]",
+                               "\xE4\xB8\x8F\xE4\xB8\x9F", "", long_row, long_row, long_row});
+    cudf::strings_column_view sv(input.view);
+    auto normalizer = nvtext::create_character_normalizer(true);
+    std::vector<Text> const lower{"abc\xC2\xA3" "def", std::nullopt, "ee a io aeio", " acen  u", "acen u", "p ^ np", " $ 41 . 07", " [ a , b ] ",
+                                  " \xE4\xB8\x8F  \xE4\xB8\x9F ", "", long_row, long_row, long_row};
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == lower);
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == lower);  // normalizer re-use
+    normalizer = nvtext::create_character_normalizer(false);
+    std::vector<Text> const keep{"abc\xC2\xA3" "def", std::nullopt, "\xC3\xA9\xC3\xA8 \xC3\xA2 \xC3\xAE\xC3\xB4 aeio",
+                                 " \xC4\x82\xC4\x86\xC4\x96\xC3\x91  \xC3\x9C", "ACEN U", "P ^ NP", " $ 41 . 07", " [ a , b ] ",
+                                 " \xE4\xB8\x8F  \xE4\xB8\x9F ", "", long_row, long_row, long_row};
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == keep);
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == keep);
+  }
+  {
+    auto input  = make_strings({"[BOS]Some strings with [PAD] special[SEP]tokens[EOS]", "[bos]these should[sep]work for lowercase[eos]",
+                                "some[non]tokens[eol]too", long_row, long_row, long_row});
+    auto tokens = make_strings({"[BOS]", "[EOS]", "[SEP]", "[PAD]"});
+    cudf::strings_column_view sv(input.view), stv(tokens.view);
+    auto normalizer = nvtext::create_character_normalizer(true, stv);
+    std::vector<Text> const lower{" [BOS] some strings with  [PAD]  special [SEP] tokens [EOS] ", " [BOS] these should [SEP] work for lowercase [EOS] ",
+                                  "some [ non ] tokens [ eol ] too", long_row, long_row, long_row};
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == lower);
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == lower);
+    normalizer = nvtext::create_character_normalizer(false, stv);
+    std::vector<Text> const keep{" [BOS] Some strings with  [PAD]  special [SEP] tokens [EOS] ",
+                                 " [ bos ] these should [ sep ] work for lowercase [ eos ] ", "some [ non ] tokens [ eol ] too", long_row, long_row,
+                                 long_row};
+    CHECK(download_strings(*nvtext::normalize_characters(sv, *normalizer)) == keep);
+    auto with_null = make_strings({"[PAD]", std::nullopt});
+    EXPECT_THROW(nvtext::create_character_normalizer(true, cudf::strings_column_view(with_null.view)), std::invalid_argument);
+  }
+  {
+    auto input = make_strings({"abc\xC2\xA3" "def", "\xC3\xA9\xC3\xA8 \xC3\xA2 \xC3\xAE\xC3\xB4\taeio", "ACEN U", "P^NP", "$41.07", "[a,b]",
+                               "\xE4\xB8\x8F\xE4\xB8\x9F"});
+    auto normalizer = nvtext::create_character_normalizer(true);
+    auto results    = nvtext::normalize_characters(cudf::strings_column_view(slice(input.view, 0, 4)), *normalizer);
+    CHECK(download_strings(*results) == (std::vector<Text>{"abc\xC2\xA3" "def", "ee a io aeio", "acen u", "p ^ np"}));
+    normalizer = nvtext::create_character_normalizer(false);
+    results    = nvtext::normalize_characters(cudf::strings_column_view(slice(input.view, 4, 7)), *normalizer);
+    CHECK(download_strings(*results) == (std::vector<Text>{" $ 41 . 07", " [ a , b ] ", " \xE4\xB8\x8F  \xE4\xB8\x9F "}));
+  }
+}
+
 void test_wordpiece()
 {
   std::printf("TextSubwordTest.WordPiece / WordPieceSliced\n");
@@ -409,6 +494,7 @@ int main()
   test_minhash_empty_and_errors();
   test_minhash_ngrams();
   test_jaccard();
+  test_normalize();
   test_wordpiece();
   test_wordpiece_subwords();
   test_wordpiece_edges();
