@@ -101,6 +101,7 @@ class StringsResult(C.Structure):
         ("size", C.c_int32),
         ("null_count", C.c_int32),
         ("offsets_size", C.c_int32),
+        ("offsets_is_int64", C.c_int32),
         ("offsets", C.c_void_p),
         ("chars", C.c_void_p),
         ("chars_size", C.c_int64),

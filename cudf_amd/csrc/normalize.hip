@@ -245,10 +245,27 @@ __global__ void __launch_bounds__(kNormThreads) normalize_count_kernel(const uin
   if (threadIdx.x == 0) tile_bytes[blockIdx.x] = total;
 }
 
+// tile_row[tile] = the first row (of rows + 1: the end counts as one) whose first byte lies at or after the tile's
+// first byte.  One thread per tile: the searches of a launch hide each other's latency.
+__global__ void __launch_bounds__(256) normalize_tile_rows_kernel(ColView col, int64_t first, int64_t tiles, int32_t* __restrict__ tile_row)
+{
+  int64_t const tile = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tile >= tiles) return;
+  int64_t const t0 = tile * kNormTile;
+  int64_t lo = 0, hi = static_cast<int64_t>(col.size) + 1;
+  while (lo < hi) {
+    int64_t const mid = (lo + hi) >> 1;
+    if (col.off(mid) - first < t0) lo = mid + 1;
+    else hi = mid;
+  }
+  tile_row[tile] = static_cast<int32_t>(lo);
+}
+
 // Writes the tile's bytes at tile_offset[tile] and the output offset of every row that starts in the tile.
 __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView col, int64_t first, int64_t n, NormTables t,
-                                                                       const uint64_t* __restrict__ tile_offset, uint8_t* __restrict__ out_chars,
-                                                                       int32_t* __restrict__ out_offsets)
+                                                                       const uint64_t* __restrict__ tile_offset,
+                                                                       const int32_t* __restrict__ tile_row, uint8_t* __restrict__ out_chars,
+                                                                       void* __restrict__ out_offsets, int offsets_are_int64)
 {
   __shared__ NormLds lds;
   __shared__ uint32_t staged[(kNormTile * kMaxOut + 4) / 4];
@@ -303,18 +320,14 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   }
 
   // rows whose first byte lies in [t0, t1) -- in [t0, n] for the last tile -- start at base + prefix
-  int64_t const rows = col.size;
-  int64_t lo = 0, hi = rows + 1;
-  while (lo < hi) {
-    int64_t const mid = (lo + hi) >> 1;
-    if (col.off(mid) - first < t0) lo = mid + 1;
-    else hi = mid;
-  }
+  int64_t const rows   = col.size;
   bool const last_tile = blockIdx.x == gridDim.x - 1;
-  for (int64_t r = lo + tid; r <= rows; r += kNormThreads) {
+  for (int64_t r = static_cast<int64_t>(tile_row[blockIdx.x]) + tid; r <= rows; r += kNormThreads) {
     int64_t const p = col.off(r) - first;
     if (p > t1 || (p == t1 && !last_tile)) break;
-    out_offsets[r] = static_cast<int32_t>(base + lds.prefix[p - t0]);
+    uint64_t const at = base + lds.prefix[p - t0];
+    if (offsets_are_int64) static_cast<int64_t*>(out_offsets)[r] = static_cast<int64_t>(at);
+    else static_cast<int32_t*>(out_offsets)[r] = static_cast<int32_t>(at);
   }
 }
 
@@ -524,12 +537,15 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
     nvtext_amd_strings_result_free(out, stream_, mr_);
     return fail(st, msg);
   };
-  out->size          = rows;
-  out->null_count    = input->null_count;
-  out->offsets_size  = rows + 1;
-  out->offsets_bytes = (static_cast<size_t>(rows) + 1) * sizeof(int32_t);
-  out->offsets       = static_cast<int32_t*>(mr.allocate(out->offsets_bytes));
-  if (!out->offsets) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
+  out->size         = rows;
+  out->null_count   = input->null_count;
+  out->offsets_size = rows + 1;
+  auto allocate_offsets = [&](bool wide) {
+    out->offsets_is_int64 = wide ? 1 : 0;
+    out->offsets_bytes    = (static_cast<size_t>(rows) + 1) * (wide ? sizeof(int64_t) : sizeof(int32_t));
+    out->offsets          = mr.allocate(out->offsets_bytes);
+    return out->offsets != nullptr;
+  };
   if (input->null_mask) {  // copy_bitmask(input): cpp/src/bitmask/null_mask.cu:381-391
     out->null_mask_bytes = mask_alloc_bytes(rows);
     out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
@@ -537,7 +553,8 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
     launch_copy_bitmask(out->null_mask, input->null_mask, input->offset, rows, stream);
   }
   if (n == 0) {  // normalize.cu:504: nothing to normalize, every row is empty
-    launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, static_cast<int64_t>(rows) + 1, stream);
+    if (!allocate_offsets(false)) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
+    launch_fill_u32(static_cast<uint32_t*>(out->offsets), 0u, static_cast<int64_t>(rows) + 1, stream);
     NVTEXT_HIP_TRY(hipGetLastError());
     return NVTEXT_AMD_SUCCESS;
   }
@@ -547,7 +564,8 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   Temp tile_bytes(mr, static_cast<size_t>(tiles) * sizeof(uint32_t));
   Temp tile_offset(mr, (static_cast<size_t>(tiles) + 1) * sizeof(uint64_t));
   Temp scan_temp(mr, scan_temp_bytes(tiles));
-  if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+  Temp tile_row(mr, static_cast<size_t>(tiles) * sizeof(int32_t));
+  if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok() || !tile_row.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   NormTables const tables{normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
                           normalizer->do_lower};
   ColView const view = make_view(*input);
@@ -556,12 +574,15 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
     hipLaunchKernelGGL(normalize_count_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view.chars + first, n, tables,
                        tile_bytes.as<uint32_t>());
   }
+  hipLaunchKernelGGL(normalize_tile_rows_kernel, dim3(static_cast<unsigned>((tiles + 255) / 256)), dim3(256), 0, stream, view, first, tiles,
+                     tile_row.as<int32_t>());
   device_exclusive_scan(TileBytes{tile_bytes.as<uint32_t>()}, tiles, tile_offset.as<uint64_t>(), scan_temp.as<uint64_t>(), stream);
   uint64_t total = 0;
   hipError_t e   = hipMemcpyAsync(&total, tile_offset.as<uint64_t>() + tiles, sizeof(total), hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e != hipSuccess) return release(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
-  if (total > 0x7FFFFFFFull) return release(NVTEXT_AMD_OVERFLOW, "normalized strings exceed the int32 offset range");
+  // int64 offsets from the large-strings threshold on (cpp/include/cudf/strings/detail/strings_children.cuh:164-175)
+  if (!allocate_offsets(total >= 0x7FFFFFFFull)) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
   out->chars_size = static_cast<int64_t>(total);
   if (total > 0) {
     out->chars_bytes = static_cast<size_t>(total);
@@ -571,7 +592,8 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   {
     ProfileScope ps("normalize_write_kernel", stream);
     hipLaunchKernelGGL(normalize_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view, first, n, tables,
-                       tile_offset.as<uint64_t>(), reinterpret_cast<uint8_t*>(out->chars), out->offsets);
+                       tile_offset.as<uint64_t>(), tile_row.as<int32_t>(), reinterpret_cast<uint8_t*>(out->chars), out->offsets,
+                       out->offsets_is_int64);
   }
   e = hipGetLastError();
   if (e != hipSuccess) return release(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));

@@ -30,14 +30,14 @@ inline cudf::strings_column_view no_special_tokens()
   return cudf::strings_column_view(cudf::column_view{cudf::data_type{cudf::type_id::STRING}, 0, nullptr, nullptr, 0});
 }
 
-// cudf::make_strings_column: STRING parent owning the chars, child[0] = INT32 offsets
+// cudf::make_strings_column: STRING parent owning the chars, child[0] = INT32 (INT64 for large strings) offsets
 inline std::unique_ptr<cudf::column> make_strings_result(nvtext_amd_strings_result const& r, cuda::stream_ref stream,
                                                          rmm::device_async_resource_ref mr)
 {
   using namespace cudf;
   std::vector<std::unique_ptr<column>> kids;
   if (r.offsets_size > 0) {
-    kids.push_back(std::make_unique<column>(data_type{type_id::INT32}, r.offsets_size, device_buffer{r.offsets, r.offsets_bytes, stream, mr},
+    kids.push_back(std::make_unique<column>(data_type{r.offsets_is_int64 ? type_id::INT64 : type_id::INT32}, r.offsets_size, device_buffer{r.offsets, r.offsets_bytes, stream, mr},
                                             device_buffer{}, 0));
   }
   return std::make_unique<column>(data_type{type_id::STRING}, r.size, device_buffer{r.chars, r.chars_bytes, stream, mr},
@@ -56,7 +56,6 @@ inline std::unique_ptr<character_normalizer> create_character_normalizer(
  * Normalizes the characters of every row for tokenizing: punctuation and CJK ideographs padded with spaces,
  * whitespace replaced by a space, control characters removed and, when the normalizer lower-cases, characters
  * lower-cased with their accents stripped.  The normalizer's special tokens keep their brackets and case.
- * Throws std::overflow_error if the result exceeds the int32 offset range.
  */
 inline std::unique_ptr<cudf::column> normalize_characters(cudf::strings_column_view const& input, character_normalizer const& normalizer,
                                                           cuda::stream_ref stream           = cudf::get_default_stream(),

@@ -346,7 +346,7 @@ def normalize_characters(input: DeviceStringsColumn, normalizer: CharacterNormal
     else:
         chars = chars[: int(out.chars_size)]
     if offsets is not None:
-        offsets = offsets.view(torch.int32)[: int(out.offsets_size)]
+        offsets = offsets.view(torch.int64 if out.offsets_is_int64 else torch.int32)[: int(out.offsets_size)]
     if mask is not None:
         mask = mask[: (int(out.size) + 31) // 32 * 4].view(torch.int32)
     return DeviceStringsColumn(chars, offsets, mask, int(out.size), 0, int(out.null_count))

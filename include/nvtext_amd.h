@@ -108,13 +108,15 @@ typedef struct nvtext_amd_fixed_column {
 } nvtext_amd_fixed_column;
 
 /* Owning result: a STRING column (cudf::make_strings_column, cpp/include/cudf/column/column_factories.hpp).
- * int32 offsets; the buffers come from the caller's allocator and are returned with
- * nvtext_amd_strings_result_free. */
+ * The offsets are int32 unless the chars reach INT32_MAX bytes, then int64 (large strings:
+ * cpp/include/cudf/strings/detail/strings_children.cuh:164-175, cpp/src/strings/utilities.cu:150-157).
+ * The buffers come from the caller's allocator and are returned with nvtext_amd_strings_result_free. */
 typedef struct nvtext_amd_strings_result {
   int32_t   size;            /* rows                                                        */
   int32_t   null_count;
   int32_t   offsets_size;    /* size+1, or 0 for the canonical empty strings column         */
-  int32_t*  offsets;         /* device, offsets_size entries (NULL if 0)                    */
+  int32_t   offsets_is_int64;
+  void*     offsets;         /* device, offsets_size entries (NULL if 0)                    */
   char*     chars;           /* device, chars_size bytes (NULL if 0)                        */
   int64_t   chars_size;
   uint32_t* null_mask;       /* device or NULL; bit i = row i                               */
@@ -253,9 +255,9 @@ void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* no
 /* Replaces nvtext::normalize_characters (cpp/include/nvtext/normalize.hpp:215-254;
  * cpp/src/text/normalize.cu:491-573): the BERT basic-tokenizer clean-up that precedes wordpiece_tokenize.
  * Works on the bytes between the first and the last offset of the view as one flat sequence, so a null row
- * keeps whatever its offsets span and the result has the input's validity.  Result: STRING column with int32
- * offsets; OVERFLOW if the normalized bytes exceed INT32_MAX.  Synchronises the stream twice (the byte range
- * of the view, the size of the result). */
+ * keeps whatever its offsets span and the result has the input's validity.  Result: STRING column (int64
+ * offsets when it holds INT32_MAX bytes or more).  Synchronises the stream twice (the byte range of the view,
+ * the size of the result). */
 nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_column* input,
                                                   const nvtext_amd_character_normalizer* normalizer,
                                                   void* stream,

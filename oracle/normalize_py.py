@@ -170,8 +170,14 @@ def normalize_flat(data: bytes, do_lower_case: bool, special_tokens: Sequence[by
     return slots
 
 
+def _offsets_dtype(total: int):
+    """int64 offsets from the large-strings threshold on (cpp/include/cudf/strings/detail/strings_children.cuh:164-175,
+    cpp/src/strings/utilities.cu:150-157: INT32_MAX unless the environment lowers it)."""
+    return np.int64 if int(total) >= 0x7FFFFFFF else np.int32
+
+
 def normalize_characters(col, do_lower_case: bool, special_tokens: Sequence[bytes] = ()):
-    """col: cudf_amd.arrow_host.HostStringsColumn.  Returns a HostStringsColumn (int32 offsets)."""
+    """col: cudf_amd.arrow_host.HostStringsColumn.  Returns a HostStringsColumn."""
     from cudf_amd.arrow_host import HostStringsColumn
     from oracle.pyoracle import copy_bitmask
     if col.size == 0:
@@ -183,7 +189,7 @@ def normalize_characters(col, do_lower_case: bool, special_tokens: Sequence[byte
     pieces = [b"".join(s) for s in slots]
     sizes = np.array([len(p) for p in pieces], dtype=np.int64)
     prefix = np.concatenate([[0], np.cumsum(sizes)])
-    out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(np.int32)
+    out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(_offsets_dtype(prefix[-1]))
     chars = np.frombuffer(b"".join(pieces), dtype=np.uint8).copy()
     return HostStringsColumn(chars, out_off, copy_bitmask(col), col.size, 0, col.null_count)
 
@@ -205,5 +211,5 @@ def normalize_ascii(col, do_lower_case: bool):
     slots = table[data]                                   # (n, 3)
     keep = slots != 0
     prefix = np.concatenate([[0], np.cumsum(keep.sum(axis=1, dtype=np.int64))])
-    out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(np.int32)
+    out_off = prefix[off[col.offset: col.offset + col.size + 1] - first].astype(_offsets_dtype(prefix[-1]))
     return HostStringsColumn(slots[keep], out_off, copy_bitmask(col), col.size, 0, col.null_count)

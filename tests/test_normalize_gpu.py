@@ -178,3 +178,22 @@ def test_normalize_ascii_at_scale(nv, onorm, do_lower):
     small = host.slice(5, 400)
     assert_same(onorm.normalize_ascii(small, do_lower), onorm.normalize_characters(small, do_lower), "numpy restatement")
     assert_same(run(nv, host, do_lower), onorm.normalize_ascii(host, do_lower), "64 MiB")
+
+
+@pytest.mark.parametrize("total", [0x7FFFFFFF - 1, 0x7FFFFFFF, (1 << 31) + 4097])
+def test_normalize_large_strings_offsets(nv, total):
+    # lower-case letters and single spaces come back unchanged, so the result must equal the input; its offsets are
+    # int32 below INT32_MAX bytes of chars and int64 from there on.  Built and compared on the device.
+    import torch
+    phrase = torch.tensor(list(b"the quick brown fox jumps over the lazy dog "), dtype=torch.uint8, device="cuda")
+    chars = phrase.repeat(total // phrase.numel() + 1)[:total].contiguous()
+    row = 65521
+    offsets = torch.arange(0, total, row, dtype=torch.int64, device="cuda")
+    offsets = torch.cat([offsets, torch.tensor([total], dtype=torch.int64, device="cuda")])
+    col = nv.DeviceStringsColumn(chars, offsets, None, offsets.numel() - 1, 0, 0)
+    out = nv.normalize_characters(col, nv.CharacterNormalizer(True))
+    torch.cuda.synchronize()
+    assert out.size == col.size and out.null_count == 0
+    assert out.offsets.dtype == (torch.int64 if total >= 0x7FFFFFFF else torch.int32)
+    assert out.chars.numel() == total and torch.equal(out.chars, chars)
+    assert torch.equal(out.offsets.to(torch.int64), offsets)
