@@ -16,6 +16,7 @@
 struct nvtext_amd_character_normalizer {
   int device            = 0;
   int32_t do_lower      = 0;
+  uint32_t* ascii       = nullptr;  // device, 128: slot 0 | slot 1 << 8 | slot 2 << 16 of the code points below 0x80
   uint32_t* entries     = nullptr;  // device, kCodepoints: category << 24 | multi << 23 | replacement
   uint64_t* second      = nullptr;  // device, kCodepoints: second << 32 | third replacement code point
   uint8_t* token_chars  = nullptr;  // device: the special tokens, sorted then lower-cased
@@ -46,6 +47,7 @@ constexpr int kRawWords    = (kNormTile + kRawBefore + kRawAfter + 3 + 3) / 4;
 constexpr int kMaxOut      = 12;  // bytes one input byte can produce: three characters of four bytes
 
 struct NormTables {
+  const uint32_t* ascii;  // 128 entries: the slots of the code points below 0x80
   const uint32_t* entries;
   const uint64_t* second;
   const uint8_t* token_chars;
@@ -67,7 +69,7 @@ __device__ __forceinline__ uint32_t utf8_le(uint32_t cp)
   return (0xF0u | ((cp >> 18) & 0x07u)) | (t2 << 8) | (t1 << 16) | (t0 << 24);
 }
 
-__device__ __forceinline__ uint32_t bytes_of(uint32_t slot) { return (slot != 0) + (slot > 0xFFu) + (slot > 0xFFFFu) + (slot > 0xFFFFFFu); }
+__device__ __forceinline__ uint32_t bytes_of(uint32_t slot) { return (39u - static_cast<uint32_t>(__clz(slot))) >> 3; }
 
 // The code point of the character that starts with b0, the next bytes being b1..b3
 // (to_char_utf8 and utf8_to_codepoint, cpp/include/cudf/strings/detail/utf8.hpp:68-97,118-140: the first byte
@@ -86,35 +88,45 @@ __device__ __forceinline__ uint32_t decode(uint32_t b0, uint32_t b1, uint32_t b2
 // The slots of one code point (data_normalizer_kernel, cpp/src/text/normalize.cu:331-378).
 __device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
 {
-  s0 = s1 = s2               = 0;
-  uint32_t const e           = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
-  uint32_t const cat         = (e >> 24) & 7u;
-  bool const lower           = t.do_lower != 0;
+  s0 = s1 = s2       = 0;
+  uint32_t const e   = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
+  uint32_t const cat = (e >> 24) & 7u;
+  bool const lower   = t.do_lower != 0;
   if (cat == kRemove || (lower && cat == kRemoveIfLower)) return;
   uint32_t const repl = (lower || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
-  uint32_t r0 = repl ? repl : cp, r1 = 0, r2 = 0;
-  bool single = true;
-  if (lower && ((e >> 23) & 1u)) {
+  uint32_t const r0   = repl ? repl : cp;
+  if (lower && ((e >> 23) & 1u)) {  // two or three code points, never padded
     uint64_t const next = t.second[cp];
-    r1                  = static_cast<uint32_t>(next >> 32);
-    r2                  = static_cast<uint32_t>(next);
-    single              = false;
+    uint32_t const r1 = static_cast<uint32_t>(next >> 32), r2 = static_cast<uint32_t>(next);
+    s0 = utf8_le(r0);
+    s1 = r1 ? utf8_le(r1) : 0u;
+    s2 = r2 ? utf8_le(r2) : 0u;
+    return;
   }
-  if ((cat == kPad || (lower && cat == kPadIfLower)) && single) {
-    r1 = r0;
-    r0 = r2 = 0x20u;
+  uint32_t const one = utf8_le(r0);
+  if (cat == kPad || (lower && cat == kPadIfLower)) {
+    s0 = s2 = 0x20u;
+    s1      = one;
+  } else {
+    s0 = one;
   }
-  s0 = r0 ? utf8_le(r0) : 0u;
-  s1 = r1 ? utf8_le(r1) : 0u;
-  s2 = r2 ? utf8_le(r2) : 0u;
 }
 
 struct NormLds {
   uint32_t raw[kRawWords];           // the input bytes of the tile and its surroundings, zero outside the column
-  uint32_t slot[3][kSlots];          // slot k of position i - kBefore
-  uint32_t sizes[kNormTile / 4];     // output bytes of each tile position, one byte each
-  uint16_t prefix[kNormTile + 4];    // bytes the tile writes before each position; [tile] = all of them
+  uint32_t ascii[128];               // slots of the code points below 0x80: slot 0 | slot 1 << 8 | slot 2 << 16
+  union {
+    uint32_t slot[3][kSlots];        // slot k of position i - kBefore; only filled where special tokens can be
+    uint32_t staged[(kNormTile * kMaxOut + 4) / 4];  // afterwards: the tile's output bytes
+  };
+  alignas(8) uint16_t prefix[kNormTile + 4];  // bytes the tile writes before each position; [tile] = all of them
   uint32_t scan[kNormThreads / kWave + 1];
+};
+
+// The slots of the four tile positions a thread owns (4 * thread .. 4 * thread + 3): consecutive bytes in, consecutive
+// bytes out.
+struct Owned {
+  uint32_t s[kNormItems][3];
 };
 
 // Slot `at` of the flat slot sequence (three per position).
@@ -137,101 +149,197 @@ __device__ int compare_candidate(NormLds& lds, int from, int to, NormTables cons
   return j < tl ? -1 : 0;
 }
 
-// One tile: fills lds.slot for the tile and its surroundings, applies the special tokens, leaves the output size
-// of every tile position in lds.sizes.
-__device__ __forceinline__ void tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t)
+// Slots of the character whose bytes start `window` (first byte in the low bits; at least four bytes of it valid).
+__device__ __forceinline__ void window_slots(NormLds const& lds, uint64_t window, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
+{
+  uint32_t const b0 = static_cast<uint32_t>(window) & 0xFFu;
+  if (b0 < 0x80u) {
+    uint32_t const d = lds.ascii[b0];
+    s0               = d & 0xFFu;
+    s1               = (d >> 8) & 0xFFu;
+    s2               = d >> 16;
+    return;
+  }
+  s0 = s1 = s2 = 0;
+  if ((b0 & 0xC0u) == 0x80u) return;
+  uint32_t const w = static_cast<uint32_t>(window);
+  slots_of(decode(b0, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
+}
+
+__device__ __forceinline__ bool has_byte(uint32_t v, uint32_t byte)
+{
+  uint32_t const x = v ^ (byte * 0x01010101u);
+  return ((x - 0x01010101u) & ~x & 0x80808080u) != 0u;
+}
+
+// special_tokens_kernel (normalize.cu:270-316) over lds.slot, in two steps so that every decision reads unchanged slots
+__device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
+{
+  int const tid       = threadIdx.x;
+  constexpr int kEach = (kSlots + kNormThreads - 1) / kNormThreads;
+  int found_from[kEach];
+  int found_to[kEach];
+#pragma unroll
+  for (int k = 0; k < kEach; ++k) {
+    int const i   = tid + k * kNormThreads;
+    found_from[k] = -1;
+    found_to[k]   = -1;
+    // a '[' in the last kAfter positions belongs to the next tile
+    if (i < kNormTile + kBefore && lds.slot[1][i] == '[') {
+      int const from = 3 * i + 1;
+      int to         = -1;
+      for (int at = from + 1; at < from + 18; ++at) {
+        if (flat_slot(lds, at) == ']') {
+          to = at;
+          break;
+        }
+      }
+      if (to > 0) {
+        int32_t first = 0, count = t.tokens;  // thrust::binary_search: lower_bound by halving, then !(value < *it)
+        while (count > 0) {
+          int32_t const half = count >> 1;
+          if (compare_candidate(lds, from, to, t, first + half) > 0) {
+            first += half + 1;
+            count -= half + 1;
+          } else {
+            count = half;
+          }
+        }
+        if (first < t.tokens && compare_candidate(lds, from, to, t, first) >= 0) {
+          found_from[k] = from;
+          found_to[k]   = to;
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kEach; ++k) {
+    if (found_from[k] < 0) continue;
+    flat_slot(lds, found_from[k] + 1) = 0u;  // the space after '['
+    flat_slot(lds, found_to[k] - 1)   = 0u;  // the space before ']'
+    if (t.do_lower) {
+      for (int at = found_from[k] + 2; at < found_to[k] - 2; ++at) {
+        uint32_t const c = flat_slot(lds, at);
+        if (c >= 'a' && c <= 'z') flat_slot(lds, at) = c - 'a' + 'A';
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// One tile: the slots of the thread's four positions, special tokens applied.  Returns the bytes they produce.
+__device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t, Owned& mine,
+                                               uint32_t (&size)[kNormItems])
 {
   int const tid = threadIdx.x;
   // stage [t0 - kRawBefore, t0 + kNormTile + kRawAfter) with aligned dword loads; bytes outside [0, n) read as 0
-  const uint8_t* const wb = chars + t0 - kRawBefore;
-  uint32_t const mis      = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 3u);
+  const uint8_t* const wb  = chars + t0 - kRawBefore;
+  uint32_t const mis       = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 3u);
   const uint32_t* const ap = reinterpret_cast<const uint32_t*>(wb - mis);
   for (int w = tid; w < kRawWords; w += kNormThreads) {
     int64_t const p = t0 - kRawBefore - mis + 4 * static_cast<int64_t>(w);  // column position of the word's first byte
     uint32_t v      = 0;
     if (p + 3 >= 0 && p < n) {
-      v = ap[w];
+      v = load_stream(ap + w);
       if (p < 0) v &= 0xFFFFFFFFu << (8 * static_cast<uint32_t>(-p));
       if (p + 4 > n) v &= 0xFFFFFFFFu >> (8 * static_cast<uint32_t>(p + 4 - n));
     }
     lds.raw[w] = v;
   }
+  if (tid < 128) lds.ascii[tid] = t.ascii[tid];
   __syncthreads();
-  const uint8_t* const rawb = reinterpret_cast<const uint8_t*>(lds.raw) + mis + kRawBefore - kBefore;  // byte of slot index 0
-  for (int i = tid; i < kSlots; i += kNormThreads) {
-    uint32_t const b0 = rawb[i];
-    uint32_t s0 = 0, s1 = 0, s2 = 0;
-    if (b0 != 0u && (b0 & 0xC0u) != 0x80u) {  // byte 0 is U+0000, which is removed
-      uint32_t cp = b0;
-      if (b0 >= 0xC0u) cp = decode(b0, rawb[i + 1], rawb[i + 2], rawb[i + 3]);
-      slots_of(cp, t, s0, s1, s2);
-    }
-    lds.slot[0][i] = s0;
-    lds.slot[1][i] = s1;
-    lds.slot[2][i] = s2;
-  }
-  __syncthreads();
-  if (t.tokens > 0) {
-    // special_tokens_kernel (normalize.cu:270-316), in two steps so that every decision reads unchanged slots
-    int found_from[(kSlots + kNormThreads - 1) / kNormThreads];
-    int found_to[(kSlots + kNormThreads - 1) / kNormThreads];
-#pragma unroll
-    for (int k = 0; k < (kSlots + kNormThreads - 1) / kNormThreads; ++k) {
-      int const i   = tid + k * kNormThreads;
-      found_from[k] = -1;
-      found_to[k]   = -1;
-      // a '[' in the last kAfter positions belongs to the next tile
-      if (i < kNormTile + kBefore && lds.slot[1][i] == '[') {
-        int const from = 3 * i + 1;
-        int to         = -1;
-        for (int at = from + 1; at < from + 18; ++at) {
-          if (flat_slot(lds, at) == ']') {
-            to = at;
-            break;
-          }
-        }
-        if (to > 0) {
-          int32_t first = 0, count = t.tokens;  // thrust::binary_search: lower_bound by halving, then !(value < *it)
-          while (count > 0) {
-            int32_t const half = count >> 1;
-            if (compare_candidate(lds, from, to, t, first + half) > 0) {
-              first += half + 1;
-              count -= half + 1;
-            } else {
-              count = half;
-            }
-          }
-          if (first < t.tokens && compare_candidate(lds, from, to, t, first) >= 0) {
-            found_from[k] = from;
-            found_to[k]   = to;
-          }
-        }
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < (kSlots + kNormThreads - 1) / kNormThreads; ++k) {
-      if (found_from[k] < 0) continue;
-      flat_slot(lds, found_from[k] + 1) = 0u;  // the space after '['
-      flat_slot(lds, found_to[k] - 1)   = 0u;  // the space before ']'
-      if (t.do_lower) {
-        for (int at = found_from[k] + 2; at < found_to[k] - 2; ++at) {
-          uint32_t const c = flat_slot(lds, at);
-          if (c >= 'a' && c <= 'z') flat_slot(lds, at) = c - 'a' + 'A';
-        }
-      }
-    }
-    __syncthreads();
-  }
-  uint8_t* const sizes = reinterpret_cast<uint8_t*>(lds.sizes);
-  for (int i = tid; i < kNormTile; i += kNormThreads) {
-    int const s = i + kBefore;
-    sizes[i]    = static_cast<uint8_t>(bytes_of(lds.slot[0][s]) + bytes_of(lds.slot[1][s]) + bytes_of(lds.slot[2][s]));
-  }
-  __syncthreads();
-}
 
-__device__ __forceinline__ uint32_t sum_bytes(uint32_t v) { return (v & 0xFFu) + ((v >> 8) & 0xFFu) + ((v >> 16) & 0xFFu) + (v >> 24); }
+  // the thread's four bytes and the four after them, whatever the alignment of the tile in memory
+  uint32_t const shift = 8u * mis;
+  int const word       = kRawBefore / 4 + tid;
+  uint32_t const r0 = lds.raw[word], r1 = lds.raw[word + 1], r2 = lds.raw[word + 2];
+  uint32_t const own  = __builtin_amdgcn_alignbit(r1, r0, shift);
+  uint32_t const next = __builtin_amdgcn_alignbit(r2, r1, shift);
+  if ((own & 0x80808080u) == 0u) {
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+      uint32_t const d = lds.ascii[(own >> (8 * j)) & 0xFFu];
+      mine.s[j][0]     = d & 0xFFu;
+      mine.s[j][1]     = (d >> 8) & 0xFFu;
+      mine.s[j][2]     = d >> 16;
+    }
+  } else {
+    // one-byte characters through the table, continuation bytes give nothing, and each first byte of a longer
+    // character (seldom more than two in four bytes) goes through the code point tables
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+      uint32_t const b = (own >> (8 * j)) & 0xFFu;
+      uint32_t const d = b < 0x80u ? lds.ascii[b] : 0u;
+      mine.s[j][0]     = d & 0xFFu;
+      mine.s[j][1]     = (d >> 8) & 0xFFu;
+      mine.s[j][2]     = d >> 16;
+    }
+    uint64_t const both = (static_cast<uint64_t>(next) << 32) | own;
+    uint32_t leads      = own & (own << 1) & 0x80808080u;  // bit 7 of the bytes >= 0xC0
+    while (leads) {
+      int const at = (__ffs(static_cast<int>(leads)) - 1) >> 3;
+      leads &= leads - 1u;
+      uint32_t const w = static_cast<uint32_t>(both >> (8 * at));
+      uint32_t s0, s1, s2;
+      slots_of(decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
+#pragma unroll
+      for (int j = 0; j < kNormItems; ++j) {
+        if (j == at) {
+          mine.s[j][0] = s0;
+          mine.s[j][1] = s1;
+          mine.s[j][2] = s2;
+        }
+      }
+    }
+  }
+
+  if (t.tokens > 0) {
+    // A special token starts at a position whose slot 1 is '['.  Tiles without one skip the exchange through LDS.
+    // For the positions before the tile (eight looked at, five needed) the bytes decide: a '[', or one of the
+    // first bytes 0xC1, 0xE0, 0xF0 with which an over-long encoding of '[' would start (no other code point's
+    // replacement is a '[').
+    bool bracket = false;
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
+    if (tid < 2) {
+      uint32_t const v = __builtin_amdgcn_alignbit(lds.raw[tid + 1], lds.raw[tid], shift);
+      bracket = bracket || has_byte(v, '[') || has_byte(v, 0xC1u) || has_byte(v, 0xE0u) || has_byte(v, 0xF0u);
+    }
+    if (__syncthreads_or(bracket)) {
+#pragma unroll
+      for (int j = 0; j < kNormItems; ++j) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) lds.slot[k][kBefore + kNormItems * tid + j] = mine.s[j][k];
+      }
+      if (tid < kBefore + kAfter) {  // the positions either side of the tile
+        int const i               = tid < kBefore ? tid : kNormTile + tid;
+        const uint8_t* const rawb = reinterpret_cast<const uint8_t*>(lds.raw) + mis + kRawBefore - kBefore + i;
+        uint64_t window           = 0;
+        for (int k = 3; k >= 0; --k) window = (window << 8) | rawb[k];
+        uint32_t s0, s1, s2;
+        window_slots(lds, window, t, s0, s1, s2);
+        lds.slot[0][i] = s0;
+        lds.slot[1][i] = s1;
+        lds.slot[2][i] = s2;
+      }
+      __syncthreads();
+      apply_special_tokens(lds, t);
+#pragma unroll
+      for (int j = 0; j < kNormItems; ++j) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) mine.s[j][k] = lds.slot[k][kBefore + kNormItems * tid + j];
+      }
+    }
+  }
+  uint32_t sum = 0;
+#pragma unroll
+  for (int j = 0; j < kNormItems; ++j) {
+    size[j] = bytes_of(mine.s[j][0]) + bytes_of(mine.s[j][1]) + bytes_of(mine.s[j][2]);
+    sum += size[j];
+  }
+  return sum;
+}
 
 // tile_bytes[tile] = bytes the tile's input positions produce
 __global__ void __launch_bounds__(kNormThreads) normalize_count_kernel(const uint8_t* __restrict__ chars, int64_t n, NormTables t,
@@ -239,9 +347,11 @@ __global__ void __launch_bounds__(kNormThreads) normalize_count_kernel(const uin
 {
   __shared__ NormLds lds;
   int64_t const t0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
-  tile_slots(lds, chars, t0, n, t);
+  Owned mine;
+  uint32_t size[kNormItems];
+  uint32_t const sum = tile_slots(lds, chars, t0, n, t, mine, size);
   uint32_t total;
-  block_exclusive_scan<kNormThreads>(sum_bytes(lds.sizes[threadIdx.x]), lds.scan, &total);
+  block_exclusive_scan<kNormThreads>(sum, lds.scan, &total);
   if (threadIdx.x == 0) tile_bytes[blockIdx.x] = total;
 }
 
@@ -268,38 +378,43 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
                                                                        void* __restrict__ out_offsets, int offsets_are_int64)
 {
   __shared__ NormLds lds;
-  __shared__ uint32_t staged[(kNormTile * kMaxOut + 4) / 4];
   int const tid        = threadIdx.x;
   int64_t const t0     = static_cast<int64_t>(blockIdx.x) * kNormTile;
   int64_t const t1     = min(t0 + kNormTile, n);
   uint64_t const base  = tile_offset[blockIdx.x];
-  tile_slots(lds, col.chars + first, t0, n, t);
-
-  uint32_t const four = lds.sizes[tid];
+  Owned mine;
+  uint32_t size[kNormItems];
+  uint32_t const sum = tile_slots(lds, col.chars + first, t0, n, t, mine, size);
   uint32_t total;
-  uint32_t run = block_exclusive_scan<kNormThreads>(sum_bytes(four), lds.scan, &total);
+  uint32_t const before = block_exclusive_scan<kNormThreads>(sum, lds.scan, &total);
+  {
+    uint32_t run = before;
+    uint32_t packed[2];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    lds.prefix[4 * tid + k] = static_cast<uint16_t>(run);
-    run += (four >> (8 * k)) & 0xFFu;
+    for (int j = 0; j < kNormItems; ++j) {
+      if (j & 1) packed[j >> 1] |= run << 16;
+      else packed[j >> 1] = run;
+      run += size[j];
+    }
+    *reinterpret_cast<uint2*>(&lds.prefix[kNormItems * tid]) = make_uint2(packed[0], packed[1]);
+    if (tid == kNormThreads - 1) lds.prefix[kNormTile] = static_cast<uint16_t>(run);
   }
-  if (tid == kNormThreads - 1) lds.prefix[kNormTile] = static_cast<uint16_t>(run);
-  __syncthreads();
 
   // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword
   uint8_t* const dst  = out_chars + base;
   uint32_t const lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 3u);
-  uint8_t* const sb   = reinterpret_cast<uint8_t*>(staged);
+  uint8_t* const sb   = reinterpret_cast<uint8_t*>(lds.staged);
+  {
+    uint32_t o = lead + before;
 #pragma unroll
-  for (int k = 0; k < kNormItems; ++k) {
-    int const i = tid + k * kNormThreads;
-    uint32_t o  = lead + lds.prefix[i];
+    for (int j = 0; j < kNormItems; ++j) {
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      uint32_t v = lds.slot[s][i + kBefore];
-      while (v) {
-        sb[o++] = static_cast<uint8_t>(v);
-        v >>= 8;
+      for (int k = 0; k < 3; ++k) {
+        uint32_t v = mine.s[j][k];
+        while (v) {
+          sb[o++] = static_cast<uint8_t>(v);
+          v >>= 8;
+        }
       }
     }
   }
@@ -308,7 +423,7 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   uint32_t const w_lo     = (lead + 3u) >> 2;
   uint32_t const w_hi     = end >> 2;
   uint32_t* const dw      = reinterpret_cast<uint32_t*>(dst - lead);
-  for (uint32_t w = w_lo + tid; w < w_hi; w += kNormThreads) dw[w] = staged[w];
+  for (uint32_t w = w_lo + tid; w < w_hi; w += kNormThreads) dw[w] = lds.staged[w];
   uint32_t const head_end   = min(4u * w_lo, end);
   uint32_t const tail_begin = max(4u * w_hi, head_end);
   if (tid < 4) {
@@ -456,6 +571,19 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
     second[0xAC00u + s]  = (static_cast<uint64_t>(vowel) << 32) | (trail ? 0x11A7u + trail : 0u);
   }
 
+  // the slots of the one-byte code points, decided here once (the rules of slots_of)
+  uint32_t ascii[128];
+  for (uint32_t cp = 0; cp < 128u; ++cp) {
+    uint32_t const e = entries[cp], cat = (e >> 24) & 7u;
+    uint32_t d       = 0;
+    if (!(cat == kRemove || (do_lower_case && cat == kRemoveIfLower))) {
+      uint32_t const repl = (do_lower_case || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
+      uint32_t const r0   = repl ? repl : cp;
+      d                   = (cat == kPad || (do_lower_case && cat == kPadIfLower)) ? (0x20u | (r0 << 8) | (0x20u << 16)) : r0;
+    }
+    ascii[cp] = d;
+  }
+
   auto* obj      = new nvtext_amd_character_normalizer();
   obj->do_lower  = do_lower_case ? 1 : 0;
   obj->tokens    = static_cast<int32_t>(tokens.size());
@@ -464,6 +592,8 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
     return fail(e == hipErrorOutOfMemory ? NVTEXT_AMD_ALLOC_FAILED : NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
   };
   hipError_t e = hipGetDevice(&obj->device);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->ascii), sizeof(ascii));
+  if (e == hipSuccess) e = hipMemcpy(obj->ascii, ascii, sizeof(ascii), hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->entries), entries.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->second), second.size() * sizeof(uint64_t));
   if (e == hipSuccess) e = hipMemcpy(obj->entries, entries.data(), entries.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
@@ -493,6 +623,7 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
 void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* normalizer)
 {
   if (!normalizer) return;
+  (void)hipFree(normalizer->ascii);
   (void)hipFree(normalizer->entries);
   (void)hipFree(normalizer->second);
   (void)hipFree(normalizer->token_chars);
@@ -566,7 +697,7 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   Temp scan_temp(mr, scan_temp_bytes(tiles));
   Temp tile_row(mr, static_cast<size_t>(tiles) * sizeof(int32_t));
   if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok() || !tile_row.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-  NormTables const tables{normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
+  NormTables const tables{normalizer->ascii, normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
                           normalizer->do_lower};
   ColView const view = make_view(*input);
   {

@@ -129,6 +129,11 @@ def test_normalize_malformed_utf8(nv, onorm, do_lower):
     rows = [bytes(rng.integers(0, 256, rng.integers(0, 40), dtype=np.uint8)) for _ in range(200)]
     rows += [b"abc\xe4", b"\xf0\x9f", b"\xc3", b"\xf8\x80\x80\x80z", b"\xf4\x90\x80\x80", b"\xed\xa0\x80", b"\x80\x80a"]
     check(nv, onorm, strings(rows), do_lower, ["[PAD]"], "random bytes")
+    # over-long encodings of '[' decode to it and open a special token like the plain byte does
+    for opener in (b"\xc1\x9b", b"\xe0\x81\x9b", b"\xf0\x80\x81\x9b", b"\xc1\x1b"):
+        for shift in range(0, 9):
+            rows = [b"a" * (TILE - 6 + shift) + opener + b"PAD]" + b"b" * 40, opener + b"PAD]"]
+            check(nv, onorm, strings(rows), do_lower, ["[PAD]"], f"over-long bracket {opener!r} shift {shift}")
 
 
 def test_normalize_nulls_keep_their_bytes_and_empty_shapes(nv, onorm):
