@@ -3,9 +3,10 @@
 //
 // The reference expands every input byte into three uint32 slots in global memory, fixes the special tokens up
 // in a second kernel, reduces the slots to row sizes and compacts them.  Here a workgroup takes a tile of
-// 1024 input bytes (plus a few either side), keeps the slots in LDS, and the column is walked twice: once to
-// learn how many bytes each tile produces, once to write them, coalesced, at the offsets a scan of those
-// counts gives.  HBM sees the input twice and the output once; the slots never leave the CU.
+// 2048 input bytes (plus a few either side), each lane keeps the slots of eight consecutive bytes in registers,
+// and the column is walked twice: once to learn how many bytes each tile produces, once to write them,
+// coalesced, at the offsets a scan of those counts gives.  HBM sees the input twice and the output once; the
+// slots never leave the CU.
 #include <algorithm>
 #include <cstring>
 #include <string>
@@ -16,7 +17,7 @@
 struct nvtext_amd_character_normalizer {
   int device            = 0;
   int32_t do_lower      = 0;
-  uint32_t* ascii       = nullptr;  // device, 128: slot 0 | slot 1 << 8 | slot 2 << 16 of the code points below 0x80
+  uint32_t* ascii       = nullptr;  // device, 128: slot 0 | slot 1 << 8 | slot 2 << 16 | bytes << 24 of the code points below 0x80
   uint32_t* entries     = nullptr;  // device, kCodepoints: category << 24 | multi << 23 | replacement
   uint64_t* second      = nullptr;  // device, kCodepoints: second << 32 | third replacement code point
   uint8_t* token_chars  = nullptr;  // device: the special tokens, sorted then lower-cased
@@ -36,15 +37,16 @@ constexpr uint32_t kDefaultEntry = 5u << 24;
 constexpr uint32_t kPad = 0, kPadIfLower = 1, kRemove = 2, kRemoveIfLower = 3, kReplace = 4;
 
 constexpr int kNormThreads = 256;
-constexpr int kNormTile    = 1024;  // input bytes per workgroup
-constexpr int kNormItems   = kNormTile / kNormThreads;
+constexpr int kNormItems   = 8;     // consecutive input bytes per lane
+constexpr int kNormTile    = kNormThreads * kNormItems;  // input bytes per workgroup
 constexpr int kBefore      = 5;   // a '[' this many bytes before the tile can still change the tile's slots
 constexpr int kAfter       = 6;   // a '[' of the tile reads slots this many bytes past it
-constexpr int kSlots       = kNormTile + kBefore + kAfter;
+constexpr int kSlotBase    = 8;   // index of the tile's first position in the slot arrays (>= kBefore; 8 keeps a lane's bytes aligned)
+constexpr int kSlots       = kSlotBase + kNormTile + 8;
 constexpr int kRawBefore   = 8;   // bytes staged before the tile (>= kBefore)
 constexpr int kRawAfter    = 12;  // bytes staged after it (>= kAfter + 3 for the longest character)
 constexpr int kRawWords    = (kNormTile + kRawBefore + kRawAfter + 3 + 3) / 4;
-constexpr int kMaxOut      = 12;  // bytes one input byte can produce: three characters of four bytes
+constexpr int kStageBytes  = 4 * kNormTile;  // output bytes of a tile that are assembled in LDS; a tile with more writes them one by one
 
 struct NormTables {
   const uint32_t* ascii;  // 128 entries: the slots of the code points below 0x80
@@ -113,24 +115,25 @@ __device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint3
 }
 
 struct NormLds {
-  uint32_t raw[kRawWords];           // the input bytes of the tile and its surroundings, zero outside the column
-  uint32_t ascii[128];               // slots of the code points below 0x80: slot 0 | slot 1 << 8 | slot 2 << 16
+  alignas(8) uint32_t raw[kRawWords];  // the input bytes of the tile and its surroundings, zero outside the column
+  uint32_t ascii[128];                 // code points below 0x80: slot 0 | slot 1 << 8 | slot 2 << 16 | bytes << 24
   union {
-    uint32_t slot[3][kSlots];        // slot k of position i - kBefore; only filled where special tokens can be
-    uint32_t staged[(kNormTile * kMaxOut + 4) / 4];  // afterwards: the tile's output bytes
+    // first byte of slot k of tile position i - kSlotBase; only filled where special tokens can be.  A first byte
+    // tells '[', ']', a space and a-z from everything else, which is all the special tokens look at or change.
+    alignas(8) uint8_t slot[3][kSlots];
+    uint32_t staged[(kStageBytes + 8) / 4];  // afterwards: the tile's output bytes
   };
-  alignas(8) uint16_t prefix[kNormTile + 4];  // bytes the tile writes before each position; [tile] = all of them
+  alignas(16) uint16_t prefix[kNormTile + 8];  // bytes the tile writes before each position; [tile] = all of them
   uint32_t scan[kNormThreads / kWave + 1];
 };
 
-// The slots of the four tile positions a thread owns (4 * thread .. 4 * thread + 3): consecutive bytes in, consecutive
-// bytes out.
+// The slots of the tile positions a lane owns (kNormItems * lane ..): consecutive bytes in, consecutive bytes out.
 struct Owned {
   uint32_t s[kNormItems][3];
 };
 
 // Slot `at` of the flat slot sequence (three per position).
-__device__ __forceinline__ uint32_t& flat_slot(NormLds& lds, int at) { return lds.slot[at % 3][at / 3]; }
+__device__ __forceinline__ uint8_t& flat_slot(NormLds& lds, int at) { return lds.slot[at % 3][at / 3]; }
 
 // Compares the candidate in flat slots [from, to] (spaces and empty slots skipped, one byte per character) with
 // special token `i`: < 0, 0, > 0 as the candidate sorts before, equal to or after it.
@@ -140,7 +143,7 @@ __device__ int compare_candidate(NormLds& lds, int from, int to, NormTables cons
   int32_t const tl   = t.token_offset[i + 1] - t.token_offset[i];
   int32_t j          = 0;
   for (int at = from; at <= to; ++at) {
-    uint32_t const c = flat_slot(lds, at) & 0xFFu;
+    uint32_t const c = flat_slot(lds, at);
     if (c == 0u || c == 0x20u) continue;
     if (j >= tl) return 1;
     uint32_t const b = tok[j++];
@@ -149,86 +152,77 @@ __device__ int compare_candidate(NormLds& lds, int from, int to, NormTables cons
   return j < tl ? -1 : 0;
 }
 
-// Slots of the character whose bytes start `window` (first byte in the low bits; at least four bytes of it valid).
-__device__ __forceinline__ void window_slots(NormLds const& lds, uint64_t window, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
-{
-  uint32_t const b0 = static_cast<uint32_t>(window) & 0xFFu;
-  if (b0 < 0x80u) {
-    uint32_t const d = lds.ascii[b0];
-    s0               = d & 0xFFu;
-    s1               = (d >> 8) & 0xFFu;
-    s2               = d >> 16;
-    return;
-  }
-  s0 = s1 = s2 = 0;
-  if ((b0 & 0xC0u) == 0x80u) return;
-  uint32_t const w = static_cast<uint32_t>(window);
-  slots_of(decode(b0, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
-}
-
 __device__ __forceinline__ bool has_byte(uint32_t v, uint32_t byte)
 {
   uint32_t const x = v ^ (byte * 0x01010101u);
   return ((x - 0x01010101u) & ~x & 0x80808080u) != 0u;
 }
 
-// special_tokens_kernel (normalize.cu:270-316) over lds.slot, in two steps so that every decision reads unchanged slots
+// Whether a special token opens at slot index i (its slot 1 holds '['): the flat slot of its ']' if so, else -1.
+// special_tokens_kernel, cpp/src/text/normalize.cu:283-301.
+__device__ int token_opens_at(NormLds& lds, NormTables const& t, int i)
+{
+  if (lds.slot[1][i] != '[') return -1;
+  int const from = 3 * i + 1;
+  int to         = -1;
+  for (int at = from + 1; at < from + 18; ++at) {
+    if (flat_slot(lds, at) == ']') {
+      to = at;
+      break;
+    }
+  }
+  if (to < 0) return -1;
+  int32_t first = 0, count = t.tokens;  // thrust::binary_search: lower_bound by halving, then !(value < *it)
+  while (count > 0) {
+    int32_t const half = count >> 1;
+    if (compare_candidate(lds, from, to, t, first + half) > 0) {
+      first += half + 1;
+      count -= half + 1;
+    } else {
+      count = half;
+    }
+  }
+  if (first >= t.tokens || compare_candidate(lds, from, to, t, first) < 0) return -1;
+  return to;
+}
+
+// special_tokens_kernel (normalize.cu:270-316) over lds.slot, in two steps so that every decision reads unchanged
+// slots.  A lane looks at its own positions; the first kBefore lanes also at the positions before the tile (a '['
+// in the positions after the tile belongs to the next tile).
 __device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
 {
-  int const tid       = threadIdx.x;
-  constexpr int kEach = (kSlots + kNormThreads - 1) / kNormThreads;
-  int found_from[kEach];
-  int found_to[kEach];
+  int const tid = threadIdx.x;
+  int found_to[kNormItems + 1];
 #pragma unroll
-  for (int k = 0; k < kEach; ++k) {
-    int const i   = tid + k * kNormThreads;
-    found_from[k] = -1;
-    found_to[k]   = -1;
-    // a '[' in the last kAfter positions belongs to the next tile
-    if (i < kNormTile + kBefore && lds.slot[1][i] == '[') {
-      int const from = 3 * i + 1;
-      int to         = -1;
-      for (int at = from + 1; at < from + 18; ++at) {
-        if (flat_slot(lds, at) == ']') {
-          to = at;
-          break;
-        }
-      }
-      if (to > 0) {
-        int32_t first = 0, count = t.tokens;  // thrust::binary_search: lower_bound by halving, then !(value < *it)
-        while (count > 0) {
-          int32_t const half = count >> 1;
-          if (compare_candidate(lds, from, to, t, first + half) > 0) {
-            first += half + 1;
-            count -= half + 1;
-          } else {
-            count = half;
-          }
-        }
-        if (first < t.tokens && compare_candidate(lds, from, to, t, first) >= 0) {
-          found_from[k] = from;
-          found_to[k]   = to;
-        }
-      }
-    }
+  for (int k = 0; k <= kNormItems; ++k) {
+    int const i = k < kNormItems ? kSlotBase + kNormItems * tid + k : kSlotBase - kBefore + tid;
+    found_to[k] = (k < kNormItems || tid < kBefore) ? token_opens_at(lds, t, i) : -1;
   }
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < kEach; ++k) {
-    if (found_from[k] < 0) continue;
-    flat_slot(lds, found_from[k] + 1) = 0u;  // the space after '['
-    flat_slot(lds, found_to[k] - 1)   = 0u;  // the space before ']'
+  for (int k = 0; k <= kNormItems; ++k) {
+    if (found_to[k] < 0) continue;
+    int const i    = k < kNormItems ? kSlotBase + kNormItems * tid + k : kSlotBase - kBefore + tid;
+    int const from = 3 * i + 1;
+    flat_slot(lds, from + 1)        = 0u;  // the space after '['
+    flat_slot(lds, found_to[k] - 1) = 0u;  // the space before ']'
     if (t.do_lower) {
-      for (int at = found_from[k] + 2; at < found_to[k] - 2; ++at) {
+      for (int at = from + 2; at < found_to[k] - 2; ++at) {
         uint32_t const c = flat_slot(lds, at);
-        if (c >= 'a' && c <= 'z') flat_slot(lds, at) = c - 'a' + 'A';
+        if (c >= 'a' && c <= 'z') flat_slot(lds, at) = static_cast<uint8_t>(c - 'a' + 'A');
       }
     }
   }
   __syncthreads();
 }
 
-// One tile: the slots of the thread's four positions, special tokens applied.  Returns the bytes they produce.
+// Slots of the character whose bytes start `w` (first byte in the low bits), through the code point tables.
+__device__ __forceinline__ void wide_slots(uint32_t w, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
+{
+  slots_of(decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
+}
+
+// One tile: the slots of the lane's positions, special tokens applied.  Returns the bytes they produce.
 __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t, Owned& mine,
                                                uint32_t (&size)[kNormItems])
 {
@@ -237,8 +231,9 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
   const uint8_t* const wb  = chars + t0 - kRawBefore;
   uint32_t const mis       = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 3u);
   const uint32_t* const ap = reinterpret_cast<const uint32_t*>(wb - mis);
+  int64_t const p0         = t0 - kRawBefore - mis;  // column position of the first staged byte
   for (int w = tid; w < kRawWords; w += kNormThreads) {
-    int64_t const p = t0 - kRawBefore - mis + 4 * static_cast<int64_t>(w);  // column position of the word's first byte
+    int64_t const p = p0 + 4 * w;
     uint32_t v      = 0;
     if (p + 3 >= 0 && p < n) {
       v = load_stream(ap + w);
@@ -250,48 +245,48 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
   if (tid < 128) lds.ascii[tid] = t.ascii[tid];
   __syncthreads();
 
-  // the thread's four bytes and the four after them, whatever the alignment of the tile in memory
+  // the lane's eight bytes and the four after them, whatever the alignment of the tile in memory
   uint32_t const shift = 8u * mis;
-  int const word       = kRawBefore / 4 + tid;
-  uint32_t const r0 = lds.raw[word], r1 = lds.raw[word + 1], r2 = lds.raw[word + 2];
-  uint32_t const own  = __builtin_amdgcn_alignbit(r1, r0, shift);
-  uint32_t const next = __builtin_amdgcn_alignbit(r2, r1, shift);
-  if ((own & 0x80808080u) == 0u) {
+  int const word       = kRawBefore / 4 + 2 * tid;
+  uint2 const ra = *reinterpret_cast<const uint2*>(&lds.raw[word]), rb = *reinterpret_cast<const uint2*>(&lds.raw[word + 2]);
+  uint32_t const own0 = __builtin_amdgcn_alignbit(ra.y, ra.x, shift);
+  uint32_t const own1 = __builtin_amdgcn_alignbit(rb.x, ra.y, shift);
+  uint32_t const next = __builtin_amdgcn_alignbit(rb.y, rb.x, shift);
+  uint64_t const lo64 = (static_cast<uint64_t>(own1) << 32) | own0;
+  uint32_t sum        = 0;
+  // one-byte characters through the table; continuation bytes give nothing
 #pragma unroll
-    for (int j = 0; j < kNormItems; ++j) {
-      uint32_t const d = lds.ascii[(own >> (8 * j)) & 0xFFu];
-      mine.s[j][0]     = d & 0xFFu;
-      mine.s[j][1]     = (d >> 8) & 0xFFu;
-      mine.s[j][2]     = d >> 16;
-    }
-  } else {
-    // one-byte characters through the table, continuation bytes give nothing, and each first byte of a longer
-    // character (seldom more than two in four bytes) goes through the code point tables
-#pragma unroll
-    for (int j = 0; j < kNormItems; ++j) {
-      uint32_t const b = (own >> (8 * j)) & 0xFFu;
-      uint32_t const d = b < 0x80u ? lds.ascii[b] : 0u;
-      mine.s[j][0]     = d & 0xFFu;
-      mine.s[j][1]     = (d >> 8) & 0xFFu;
-      mine.s[j][2]     = d >> 16;
-    }
-    uint64_t const both = (static_cast<uint64_t>(next) << 32) | own;
-    uint32_t leads      = own & (own << 1) & 0x80808080u;  // bit 7 of the bytes >= 0xC0
-    while (leads) {
-      int const at = (__ffs(static_cast<int>(leads)) - 1) >> 3;
-      leads &= leads - 1u;
-      uint32_t const w = static_cast<uint32_t>(both >> (8 * at));
+  for (int j = 0; j < kNormItems; ++j) {
+    uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
+    uint32_t const d = b < 0x80u ? lds.ascii[b] : 0u;
+    mine.s[j][0]     = d & 0xFFu;
+    mine.s[j][1]     = (d >> 8) & 0xFFu;
+    mine.s[j][2]     = (d >> 16) & 0xFFu;
+    size[j]          = d >> 24;
+    sum += size[j];
+  }
+  // each first byte of a longer character (seldom more than four in eight bytes) goes through the code point tables
+  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;  // bit 7 of the bytes >= 0xC0
+  if (leads) {
+    uint64_t const hi64 = (static_cast<uint64_t>(next) << 32) | own1;
+    do {
+      int const at = (__ffsll(static_cast<long long>(leads)) - 1) >> 3;
+      leads &= leads - 1ull;
+      uint32_t const w = static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3)));
       uint32_t s0, s1, s2;
-      slots_of(decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
+      wide_slots(w, t, s0, s1, s2);
+      uint32_t const bytes = bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+      sum += bytes;
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
         if (j == at) {
           mine.s[j][0] = s0;
           mine.s[j][1] = s1;
           mine.s[j][2] = s2;
+          size[j]      = bytes;
         }
       }
-    }
+    } while (leads);
   }
 
   if (t.tokens > 0) {
@@ -304,45 +299,58 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
     for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
     if (tid < 2) {
       uint32_t const v = __builtin_amdgcn_alignbit(lds.raw[tid + 1], lds.raw[tid], shift);
-      bracket = bracket || has_byte(v, '[') || has_byte(v, 0xC1u) || has_byte(v, 0xE0u) || has_byte(v, 0xF0u);
+      bracket          = bracket || has_byte(v, '[') || has_byte(v, 0xC1u) || has_byte(v, 0xE0u) || has_byte(v, 0xF0u);
     }
     if (__syncthreads_or(bracket)) {
 #pragma unroll
-      for (int j = 0; j < kNormItems; ++j) {
+      for (int k = 0; k < 3; ++k) {
+        uint32_t a = 0, b = 0;
 #pragma unroll
-        for (int k = 0; k < 3; ++k) lds.slot[k][kBefore + kNormItems * tid + j] = mine.s[j][k];
+        for (int j = 0; j < 4; ++j) {
+          a |= (mine.s[j][k] & 0xFFu) << (8 * j);
+          b |= (mine.s[j + 4][k] & 0xFFu) << (8 * j);
+        }
+        *reinterpret_cast<uint2*>(&lds.slot[k][kSlotBase + kNormItems * tid]) = make_uint2(a, b);
       }
       if (tid < kBefore + kAfter) {  // the positions either side of the tile
-        int const i               = tid < kBefore ? tid : kNormTile + tid;
-        const uint8_t* const rawb = reinterpret_cast<const uint8_t*>(lds.raw) + mis + kRawBefore - kBefore + i;
-        uint64_t window           = 0;
-        for (int k = 3; k >= 0; --k) window = (window << 8) | rawb[k];
-        uint32_t s0, s1, s2;
-        window_slots(lds, window, t, s0, s1, s2);
-        lds.slot[0][i] = s0;
-        lds.slot[1][i] = s1;
-        lds.slot[2][i] = s2;
+        int const pos             = tid < kBefore ? tid - kBefore : kNormTile + tid - kBefore;
+        const uint8_t* const rawb = reinterpret_cast<const uint8_t*>(lds.raw) + mis + kRawBefore + pos;
+        uint32_t const b0         = rawb[0];
+        uint32_t s0 = 0, s1 = 0, s2 = 0;
+        if (b0 < 0x80u) {
+          uint32_t const d = lds.ascii[b0];
+          s0               = d & 0xFFu;
+          s1               = (d >> 8) & 0xFFu;
+          s2               = (d >> 16) & 0xFFu;
+        } else if (b0 >= 0xC0u) {
+          wide_slots(b0 | (static_cast<uint32_t>(rawb[1]) << 8) | (static_cast<uint32_t>(rawb[2]) << 16) | (static_cast<uint32_t>(rawb[3]) << 24),
+                     t, s0, s1, s2);
+        }
+        lds.slot[0][kSlotBase + pos] = static_cast<uint8_t>(s0);
+        lds.slot[1][kSlotBase + pos] = static_cast<uint8_t>(s1);
+        lds.slot[2][kSlotBase + pos] = static_cast<uint8_t>(s2);
       }
       __syncthreads();
       apply_special_tokens(lds, t);
+      // the tokens only ever empty a slot or turn its letter into upper case: take over the first bytes that changed
+      sum = 0;
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
 #pragma unroll
-        for (int k = 0; k < 3; ++k) mine.s[j][k] = lds.slot[k][kBefore + kNormItems * tid + j];
+        for (int k = 0; k < 3; ++k) {
+          uint32_t const now = lds.slot[k][kSlotBase + kNormItems * tid + j];
+          if (now != (mine.s[j][k] & 0xFFu)) mine.s[j][k] = now;
+        }
+        size[j] = bytes_of(mine.s[j][0]) + bytes_of(mine.s[j][1]) + bytes_of(mine.s[j][2]);
+        sum += size[j];
       }
     }
-  }
-  uint32_t sum = 0;
-#pragma unroll
-  for (int j = 0; j < kNormItems; ++j) {
-    size[j] = bytes_of(mine.s[j][0]) + bytes_of(mine.s[j][1]) + bytes_of(mine.s[j][2]);
-    sum += size[j];
   }
   return sum;
 }
 
 // tile_bytes[tile] = bytes the tile's input positions produce
-__global__ void __launch_bounds__(kNormThreads) normalize_count_kernel(const uint8_t* __restrict__ chars, int64_t n, NormTables t,
+__global__ void __launch_bounds__(kNormThreads, 8) normalize_count_kernel(const uint8_t* __restrict__ chars, int64_t n, NormTables t,
                                                                        uint32_t* __restrict__ tile_bytes)
 {
   __shared__ NormLds lds;
@@ -382,6 +390,10 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   int64_t const t0     = static_cast<int64_t>(blockIdx.x) * kNormTile;
   int64_t const t1     = min(t0 + kNormTile, n);
   uint64_t const base  = tile_offset[blockIdx.x];
+  // the rows that start in this tile are looked up now, so that the loads are back when the tile is done
+  int64_t const rows     = col.size;
+  int64_t const my_row   = static_cast<int64_t>(tile_row[blockIdx.x]) + tid;
+  int64_t const my_start = my_row <= rows ? col.off(my_row) - first : n + 1;
   Owned mine;
   uint32_t size[kNormItems];
   uint32_t const sum = tile_slots(lds, col.chars + first, t0, n, t, mine, size);
@@ -389,23 +401,23 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   uint32_t const before = block_exclusive_scan<kNormThreads>(sum, lds.scan, &total);
   {
     uint32_t run = before;
-    uint32_t packed[2];
+    uint32_t packed[kNormItems / 2];
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) {
       if (j & 1) packed[j >> 1] |= run << 16;
       else packed[j >> 1] = run;
       run += size[j];
     }
-    *reinterpret_cast<uint2*>(&lds.prefix[kNormItems * tid]) = make_uint2(packed[0], packed[1]);
+    *reinterpret_cast<uint4*>(&lds.prefix[kNormItems * tid]) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     if (tid == kNormThreads - 1) lds.prefix[kNormTile] = static_cast<uint16_t>(run);
   }
 
-  // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword
-  uint8_t* const dst  = out_chars + base;
-  uint32_t const lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 3u);
-  uint8_t* const sb   = reinterpret_cast<uint8_t*>(lds.staged);
-  {
-    uint32_t o = lead + before;
+  uint8_t* const dst = out_chars + base;
+  if (total <= static_cast<uint32_t>(kStageBytes)) {
+    // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword
+    uint32_t const lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 3u);
+    uint8_t* const sb   = reinterpret_cast<uint8_t*>(lds.staged);
+    uint32_t o          = lead + before;
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) {
 #pragma unroll
@@ -417,28 +429,42 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
         }
       }
     }
-  }
-  __syncthreads();
-  uint32_t const end      = lead + total;
-  uint32_t const w_lo     = (lead + 3u) >> 2;
-  uint32_t const w_hi     = end >> 2;
-  uint32_t* const dw      = reinterpret_cast<uint32_t*>(dst - lead);
-  for (uint32_t w = w_lo + tid; w < w_hi; w += kNormThreads) dw[w] = lds.staged[w];
-  uint32_t const head_end   = min(4u * w_lo, end);
-  uint32_t const tail_begin = max(4u * w_hi, head_end);
-  if (tid < 4) {
-    uint32_t const at = lead + tid;
-    if (at < head_end) (dst - lead)[at] = sb[at];
-  } else if (tid < 8) {
-    uint32_t const at = tail_begin + (tid - 4);
-    if (at < end) (dst - lead)[at] = sb[at];
+    __syncthreads();
+    uint32_t const end  = lead + total;
+    uint32_t const w_lo = (lead + 3u) >> 2;
+    uint32_t const w_hi = end >> 2;
+    uint32_t* const dw  = reinterpret_cast<uint32_t*>(dst - lead);
+    for (uint32_t w = w_lo + tid; w < w_hi; w += kNormThreads) store_stream(dw + w, lds.staged[w]);
+    uint32_t const head_end   = min(4u * w_lo, end);
+    uint32_t const tail_begin = max(4u * w_hi, head_end);
+    if (tid < 4) {
+      uint32_t const at = lead + tid;
+      if (at < head_end) (dst - lead)[at] = sb[at];
+    } else if (tid < 8) {
+      uint32_t const at = tail_begin + (tid - 4);
+      if (at < end) (dst - lead)[at] = sb[at];
+    }
+  } else {
+    // more than four output bytes per input byte (only input that is not UTF-8 gets there): byte by byte
+    uint8_t* o = dst + before;
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        uint32_t v = mine.s[j][k];
+        while (v) {
+          *o++ = static_cast<uint8_t>(v);
+          v >>= 8;
+        }
+      }
+    }
+    __syncthreads();  // lds.prefix is complete for the rows below
   }
 
   // rows whose first byte lies in [t0, t1) -- in [t0, n] for the last tile -- start at base + prefix
-  int64_t const rows   = col.size;
   bool const last_tile = blockIdx.x == gridDim.x - 1;
-  for (int64_t r = static_cast<int64_t>(tile_row[blockIdx.x]) + tid; r <= rows; r += kNormThreads) {
-    int64_t const p = col.off(r) - first;
+  for (int64_t r = my_row; r <= rows; r += kNormThreads) {
+    int64_t const p = r == my_row ? my_start : col.off(r) - first;
     if (p > t1 || (p == t1 && !last_tile)) break;
     uint64_t const at = base + lds.prefix[p - t0];
     if (offsets_are_int64) static_cast<int64_t*>(out_offsets)[r] = static_cast<int64_t>(at);
@@ -579,7 +605,7 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
     if (!(cat == kRemove || (do_lower_case && cat == kRemoveIfLower))) {
       uint32_t const repl = (do_lower_case || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
       uint32_t const r0   = repl ? repl : cp;
-      d                   = (cat == kPad || (do_lower_case && cat == kPadIfLower)) ? (0x20u | (r0 << 8) | (0x20u << 16)) : r0;
+      d                   = (cat == kPad || (do_lower_case && cat == kPadIfLower)) ? (0x20u | (r0 << 8) | (0x20u << 16) | (3u << 24)) : (r0 | (1u << 24));
     }
     ascii[cp] = d;
   }
