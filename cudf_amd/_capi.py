@@ -23,6 +23,7 @@ EXPORTS = [
     "nvtext_amd_list_strings_from_arrow_device",
     "nvtext_amd_list_to_arrow_device",
     "nvtext_amd_fixed_to_arrow_device",
+    "nvtext_amd_strings_to_arrow_device",
     "nvtext_amd_character_normalizer_create",
     "nvtext_amd_character_normalizer_destroy",
     "nvtext_amd_normalize_characters",
@@ -190,6 +191,9 @@ def load():
     L.nvtext_amd_fixed_to_arrow_device.restype = C.c_int
     L.nvtext_amd_fixed_to_arrow_device.argtypes = [C.POINTER(FixedColumn), C.c_void_p, C.POINTER(Allocator), C.POINTER(ArrowSchema),
                                                    C.POINTER(ArrowDeviceArray)]
+    L.nvtext_amd_strings_to_arrow_device.restype = C.c_int
+    L.nvtext_amd_strings_to_arrow_device.argtypes = [C.POINTER(StringsResult), C.c_void_p, C.POINTER(Allocator), C.POINTER(ArrowSchema),
+                                                     C.POINTER(ArrowDeviceArray)]
     L.nvtext_amd_character_normalizer_create.restype = C.c_int
     L.nvtext_amd_character_normalizer_create.argtypes = [C.c_int32, C.POINTER(StringsColumn), C.c_void_p, C.POINTER(Allocator),
                                                          C.POINTER(C.c_void_p)]

@@ -89,7 +89,7 @@ struct Exported {
   bool has_event;
   void* buffers_to_free[3];
   size_t bytes_to_free[3];
-  const void* parent_buffers[2];
+  const void* parent_buffers[3];
   const void* child_buffers[2];
   ArrowArray child;
   ArrowArray* children[1];
@@ -262,6 +262,45 @@ nvtext_amd_status nvtext_amd_fixed_to_arrow_device(nvtext_amd_fixed_column* col,
   auto* s               = new ExportedSchema{};
   *out_schema = ArrowSchema{format, "", nullptr, col->null_mask ? ARROW_FLAG_NULLABLE : 0, 0, nullptr, nullptr, release_exported_schema, s};
   *col        = nvtext_amd_fixed_column{};
+  return NVTEXT_AMD_SUCCESS;
+}
+
+nvtext_amd_status nvtext_amd_strings_to_arrow_device(nvtext_amd_strings_result* col, void* stream, const nvtext_amd_allocator* mr,
+                                                     ArrowSchema* out_schema, ArrowDeviceArray* out_array)
+{
+  using namespace nvtext_amd;
+  if (!col || !out_schema || !out_array) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  Exported* x = new_exported(stream, mr);
+  auto give_up = [&](nvtext_amd_status st) {
+    if (x->has_event) (void)hipEventDestroy(x->event);
+    delete x;
+    return st;
+  };
+  if (col->size == 0 && !col->offsets) {
+    // the canonical empty column has no offsets child; an Arrow string array holds length + 1 of them
+    Mr m{mr, x->stream};
+    col->offsets_bytes    = sizeof(int32_t);
+    col->offsets          = m.allocate(col->offsets_bytes);
+    col->offsets_is_int64 = 0;
+    if (!col->offsets) return give_up(fail(NVTEXT_AMD_ALLOC_FAILED, "offsets allocation failed"));
+    launch_fill_u32(static_cast<uint32_t*>(col->offsets), 0u, 1, x->stream);
+  }
+  nvtext_amd_status st = finish_device_array(x, x->stream, out_array);
+  if (st != NVTEXT_AMD_SUCCESS) return give_up(st);
+  x->buffers_to_free[0] = col->offsets;
+  x->bytes_to_free[0]   = col->offsets_bytes;
+  x->buffers_to_free[1] = col->chars;
+  x->bytes_to_free[1]   = col->chars_bytes;
+  x->buffers_to_free[2] = col->null_mask;
+  x->bytes_to_free[2]   = col->null_mask_bytes;
+  x->parent_buffers[0]  = col->null_mask;
+  x->parent_buffers[1]  = col->offsets;
+  x->parent_buffers[2]  = col->chars;
+  out_array->array      = ArrowArray{col->size, col->null_count, 0, 3, 0, x->parent_buffers, nullptr, nullptr, release_exported_array, x};
+  auto* s               = new ExportedSchema{};
+  *out_schema = ArrowSchema{col->offsets_is_int64 ? "U" : "u", "", nullptr, col->null_mask ? ARROW_FLAG_NULLABLE : 0, 0, nullptr, nullptr,
+                            release_exported_schema, s};
+  *col        = nvtext_amd_strings_result{};
   return NVTEXT_AMD_SUCCESS;
 }
 

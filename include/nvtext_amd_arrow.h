@@ -105,6 +105,14 @@ nvtext_amd_status nvtext_amd_fixed_to_arrow_device(nvtext_amd_fixed_column* col,
                                                    struct ArrowSchema* out_schema,
                                                    struct ArrowDeviceArray* out_array);
 
+/* As above for a strings result: "u" (utf8, int32 offsets) or "U" (large_utf8, int64 offsets), buffers
+ * [validity, offsets, data].  An empty result gets the single offset an Arrow string array of length 0 holds. */
+nvtext_amd_status nvtext_amd_strings_to_arrow_device(nvtext_amd_strings_result* col,
+                                                     void* stream,
+                                                     const nvtext_amd_allocator* mr,
+                                                     struct ArrowSchema* out_schema,
+                                                     struct ArrowDeviceArray* out_array);
+
 #ifdef __cplusplus
 }
 #endif

@@ -212,6 +212,43 @@ def test_ngrams_and_jaccard_through_arrow(env):
     fa.array.release(C.byref(fa.array))
 
 
+def test_normalize_characters_through_arrow(env):
+    capi, lib = env["capi"], env["lib"]
+    from oracle import normalize_py
+    rows = ["Stock^ $1", None, "éâîô\teaio", "[PAD] ĂĆĖÑÜ", "", "丏丟"]
+    normalizer = C.c_void_p()
+    tokens = env["nv"].DeviceStringsColumn.from_host(host_strings(pa.array(["[PAD]"], type=pa.string())))._c()
+    assert lib.nvtext_amd_character_normalizer_create(1, C.byref(tokens), stream_of(env), C.byref(env["mr"].struct), C.byref(normalizer)) == capi.SUCCESS
+    for typ, want in ((pa.string(), pa.string()), (pa.large_string(), pa.string())):
+        arr = pa.array(rows, type=typ)
+        schema = export_schema(env, typ)
+        darr = device_array_of(env, arr)
+        col = capi.StringsColumn()
+        assert lib.nvtext_amd_strings_from_arrow_device(C.byref(schema), C.byref(darr), stream_of(env), C.byref(col)) == capi.SUCCESS
+        out = capi.StringsResult()
+        assert lib.nvtext_amd_normalize_characters(C.byref(col), normalizer, stream_of(env), C.byref(env["mr"].struct), C.byref(out)) == capi.SUCCESS
+        out_schema, out_arr = capi.ArrowSchema(), capi.ArrowDeviceArray()
+        assert lib.nvtext_amd_strings_to_arrow_device(C.byref(out), stream_of(env), C.byref(env["mr"].struct), C.byref(out_schema),
+                                                      C.byref(out_arr)) == capi.SUCCESS
+        assert not out.offsets and not out.chars  # moved out
+        got, keep = import_result(env, out_schema, out_arr)
+        exp = normalize_py.normalize_characters(host_strings(arr), True, [b"[PAD]"])
+        assert got.type == want and got.null_count == 1
+        assert [None if v is None else v.encode("utf-8") for v in got.to_pylist()] == exp.to_pylist()
+        out_arr.array.release(C.byref(out_arr.array))
+    # an empty result still is a well-formed Arrow string array
+    empty = capi.StringsResult()
+    col = env["nv"].DeviceStringsColumn.from_host(host_strings(pa.array([], type=pa.string())))._c()
+    assert lib.nvtext_amd_normalize_characters(C.byref(col), normalizer, stream_of(env), C.byref(env["mr"].struct), C.byref(empty)) == capi.SUCCESS
+    out_schema, out_arr = capi.ArrowSchema(), capi.ArrowDeviceArray()
+    assert lib.nvtext_amd_strings_to_arrow_device(C.byref(empty), stream_of(env), C.byref(env["mr"].struct), C.byref(out_schema),
+                                                  C.byref(out_arr)) == capi.SUCCESS
+    got, keep = import_result(env, out_schema, out_arr)
+    assert got.type == pa.string() and len(got) == 0
+    out_arr.array.release(C.byref(out_arr.array))
+    lib.nvtext_amd_character_normalizer_destroy(normalizer)
+
+
 def test_arrow_argument_checks(env):
     capi, lib = env["capi"], env["lib"]
     arr = pa.array(["a", "b"], type=pa.string())
