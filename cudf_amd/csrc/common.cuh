@@ -226,6 +226,37 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* l
   return base + i - v;
 }
 
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight (a __syncthreads()
+// waits for them).  For kernels whose lanes exchange data through LDS alone.
+__device__ __forceinline__ void lds_barrier()
+{
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// block_exclusive_scan with lds_barrier() in place of __syncthreads().
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_exclusive_scan_lds(uint32_t v, uint32_t* lds, uint32_t* total)
+{
+  constexpr int W  = THREADS / kWave;
+  int const lane   = lane_id();
+  int const wave   = threadIdx.x / kWave;
+  uint32_t const i = wave_inclusive_scan(v);
+  lds_barrier();  // protect lds reuse between calls
+  if (lane == kWave - 1) lds[wave] = i;
+  lds_barrier();
+  uint32_t base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    uint32_t const t = lds[w];
+    if (w < wave) base += t;
+    sum += t;
+  }
+  *total = sum;
+  return base + i - v;
+}
+
 template <int THREADS>
 __device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t v, uint64_t* lds, uint64_t* total)
 {

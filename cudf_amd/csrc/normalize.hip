@@ -45,7 +45,7 @@ constexpr int kSlotBase    = 8;   // index of the tile's first position in the s
 constexpr int kSlots       = kSlotBase + kNormTile + 8;
 constexpr int kRawBefore   = 8;   // bytes staged before the tile (>= kBefore)
 constexpr int kRawAfter    = 12;  // bytes staged after it (>= kAfter + 3 for the longest character)
-constexpr int kRawWords    = (kNormTile + kRawBefore + kRawAfter + 3 + 3) / 4;
+constexpr int kRawWords    = (kNormTile + kRawBefore + kRawAfter + 15 + 15) / 16 * 4;  // whole 16-byte blocks, any alignment
 constexpr int kStageBytes  = 4 * kNormTile;  // output bytes of a tile that are assembled in LDS; a tile with more writes them one by one
 
 struct NormTables {
@@ -115,7 +115,7 @@ __device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint3
 }
 
 struct NormLds {
-  alignas(8) uint32_t raw[kRawWords];  // the input bytes of the tile and its surroundings, zero outside the column
+  alignas(16) uint32_t raw[kRawWords];  // the input bytes of the tile and its surroundings, zero outside the column
   uint32_t ascii[128];                 // code points below 0x80: slot 0 | slot 1 << 8 | slot 2 << 16 | bytes << 24
   union {
     // first byte of slot k of tile position i - kSlotBase; only filled where special tokens can be.  A first byte
@@ -125,6 +125,7 @@ struct NormLds {
   };
   alignas(16) uint16_t prefix[kNormTile + 8];  // bytes the tile writes before each position; [tile] = all of them
   uint32_t scan[kNormThreads / kWave + 1];
+  uint32_t bracket;  // some lane of the tile saw what can open a special token
 };
 
 // The slots of the tile positions a lane owns (kNormItems * lane ..): consecutive bytes in, consecutive bytes out.
@@ -198,7 +199,7 @@ __device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
     int const i = k < kNormItems ? kSlotBase + kNormItems * tid + k : kSlotBase - kBefore + tid;
     found_to[k] = (k < kNormItems || tid < kBefore) ? token_opens_at(lds, t, i) : -1;
   }
-  __syncthreads();
+  lds_barrier();
 #pragma unroll
   for (int k = 0; k <= kNormItems; ++k) {
     if (found_to[k] < 0) continue;
@@ -213,7 +214,7 @@ __device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
 }
 
 // Slots of the character whose bytes start `w` (first byte in the low bits), through the code point tables.
@@ -227,38 +228,49 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
                                                uint32_t (&size)[kNormItems])
 {
   int const tid = threadIdx.x;
-  // stage [t0 - kRawBefore, t0 + kNormTile + kRawAfter) with aligned dword loads; bytes outside [0, n) read as 0
-  const uint8_t* const wb  = chars + t0 - kRawBefore;
-  uint32_t const mis       = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 3u);
-  const uint32_t* const ap = reinterpret_cast<const uint32_t*>(wb - mis);
-  int64_t const p0         = t0 - kRawBefore - mis;  // column position of the first staged byte
-  for (int w = tid; w < kRawWords; w += kNormThreads) {
-    int64_t const p = p0 + 4 * w;
-    uint32_t v      = 0;
-    if (p + 3 >= 0 && p < n) {
-      v = load_stream(ap + w);
-      if (p < 0) v &= 0xFFFFFFFFu << (8 * static_cast<uint32_t>(-p));
-      if (p + 4 > n) v &= 0xFFFFFFFFu >> (8 * static_cast<uint32_t>(p + 4 - n));
+  // stage [t0 - kRawBefore, t0 + kNormTile + kRawAfter) with one aligned 16-byte load per lane (the first 131 lanes);
+  // bytes outside [0, n) read as 0.  Everything is requested before anything is waited for.
+  uint32_t const table_entry = tid < 128 ? t.ascii[tid] : 0u;
+  const uint8_t* const wb    = chars + t0 - kRawBefore;
+  uint32_t const mis         = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wb) & 15u);
+  if (tid < kRawWords / 4) {
+    int64_t const p = t0 - kRawBefore - mis + 16 * static_cast<int64_t>(tid);  // column position of the block's first byte
+    uint4 v         = make_uint4(0u, 0u, 0u, 0u);
+    if (p + 15 >= 0 && p < n) {
+      v = load_stream(reinterpret_cast<const uint4*>(wb - mis) + tid);
+      if (p < 0 || p + 16 > n) {  // the first or the last block of the column: clear what lies outside
+        uint32_t* const part = &v.x;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          int64_t const q = p + 4 * k;
+          uint32_t keep   = 0xFFFFFFFFu;
+          if (q < 0) keep = q <= -4 ? 0u : keep << (8 * static_cast<uint32_t>(-q));
+          if (q + 4 > n) keep = q >= n ? 0u : keep & (0xFFFFFFFFu >> (8 * static_cast<uint32_t>(q + 4 - n)));
+          part[k] &= keep;
+        }
+      }
     }
-    lds.raw[w] = v;
+    *reinterpret_cast<uint4*>(&lds.raw[4 * tid]) = v;
   }
-  if (tid < 128) lds.ascii[tid] = t.ascii[tid];
-  __syncthreads();
+  if (tid < 128) lds.ascii[tid] = table_entry;
+  if (tid == 0) lds.bracket = 0u;
+  lds_barrier();
 
   // the lane's eight bytes and the four after them, whatever the alignment of the tile in memory
-  uint32_t const shift = 8u * mis;
-  int const word       = kRawBefore / 4 + 2 * tid;
-  uint2 const ra = *reinterpret_cast<const uint2*>(&lds.raw[word]), rb = *reinterpret_cast<const uint2*>(&lds.raw[word + 2]);
-  uint32_t const own0 = __builtin_amdgcn_alignbit(ra.y, ra.x, shift);
-  uint32_t const own1 = __builtin_amdgcn_alignbit(rb.x, ra.y, shift);
-  uint32_t const next = __builtin_amdgcn_alignbit(rb.y, rb.x, shift);
+  uint32_t const shift = 8u * (mis & 3u);
+  int const word       = static_cast<int>((mis + kRawBefore) >> 2) + 2 * tid;
+  uint32_t const r0 = lds.raw[word], r1 = lds.raw[word + 1], r2 = lds.raw[word + 2], r3 = lds.raw[word + 3];
+  uint32_t const own0 = __builtin_amdgcn_alignbit(r1, r0, shift);
+  uint32_t const own1 = __builtin_amdgcn_alignbit(r2, r1, shift);
+  uint32_t const next = __builtin_amdgcn_alignbit(r3, r2, shift);
   uint64_t const lo64 = (static_cast<uint64_t>(own1) << 32) | own0;
   uint32_t sum        = 0;
   // one-byte characters through the table; continuation bytes give nothing
 #pragma unroll
   for (int j = 0; j < kNormItems; ++j) {
     uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
-    uint32_t const d = b < 0x80u ? lds.ascii[b] : 0u;
+    uint32_t const e = lds.ascii[b & 0x7Fu];  // read in any case: no branch
+    uint32_t const d = b < 0x80u ? e : 0u;
     mine.s[j][0]     = d & 0xFFu;
     mine.s[j][1]     = (d >> 8) & 0xFFu;
     mine.s[j][2]     = (d >> 16) & 0xFFu;
@@ -298,10 +310,13 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
     if (tid < 2) {
-      uint32_t const v = __builtin_amdgcn_alignbit(lds.raw[tid + 1], lds.raw[tid], shift);
+      int const at     = static_cast<int>(mis >> 2) + tid;
+      uint32_t const v = __builtin_amdgcn_alignbit(lds.raw[at + 1], lds.raw[at], shift);
       bracket          = bracket || has_byte(v, '[') || has_byte(v, 0xC1u) || has_byte(v, 0xE0u) || has_byte(v, 0xF0u);
     }
-    if (__syncthreads_or(bracket)) {
+    if (ballot64(bracket) != 0 && lane_id() == 0) lds.bracket = 1u;
+    lds_barrier();
+    if (lds.bracket != 0u) {
 #pragma unroll
       for (int k = 0; k < 3; ++k) {
         uint32_t a = 0, b = 0;
@@ -330,7 +345,7 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
         lds.slot[1][kSlotBase + pos] = static_cast<uint8_t>(s1);
         lds.slot[2][kSlotBase + pos] = static_cast<uint8_t>(s2);
       }
-      __syncthreads();
+      lds_barrier();
       apply_special_tokens(lds, t);
       // the tokens only ever empty a slot or turn its letter into upper case: take over the first bytes that changed
       sum = 0;
@@ -340,6 +355,19 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
         for (int k = 0; k < 3; ++k) {
           uint32_t const now = lds.slot[k][kSlotBase + kNormItems * tid + j];
           if (now != (mine.s[j][k] & 0xFFu)) mine.s[j][k] = now;
+        }
+        // keep the filled slots of a position in front (the output is the same): the writer relies on it
+#pragma unroll
+        for (int again = 0; again < 2; ++again) {
+          if (mine.s[j][0] == 0u) {
+            mine.s[j][0] = mine.s[j][1];
+            mine.s[j][1] = mine.s[j][2];
+            mine.s[j][2] = 0u;
+          }
+        }
+        if (mine.s[j][1] == 0u) {
+          mine.s[j][1] = mine.s[j][2];
+          mine.s[j][2] = 0u;
         }
         size[j] = bytes_of(mine.s[j][0]) + bytes_of(mine.s[j][1]) + bytes_of(mine.s[j][2]);
         sum += size[j];
@@ -359,7 +387,7 @@ __global__ void __launch_bounds__(kNormThreads, 8) normalize_count_kernel(const 
   uint32_t size[kNormItems];
   uint32_t const sum = tile_slots(lds, chars, t0, n, t, mine, size);
   uint32_t total;
-  block_exclusive_scan<kNormThreads>(sum, lds.scan, &total);
+  block_exclusive_scan_lds<kNormThreads>(sum, lds.scan, &total);
   if (threadIdx.x == 0) tile_bytes[blockIdx.x] = total;
 }
 
@@ -390,15 +418,25 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   int64_t const t0     = static_cast<int64_t>(blockIdx.x) * kNormTile;
   int64_t const t1     = min(t0 + kNormTile, n);
   uint64_t const base  = tile_offset[blockIdx.x];
-  // the rows that start in this tile are looked up now, so that the loads are back when the tile is done
+  // the rows that start in this tile are looked up now; the barriers below do not wait for global loads, so this
+  // one is back when the tile is done
   int64_t const rows     = col.size;
   int64_t const my_row   = static_cast<int64_t>(tile_row[blockIdx.x]) + tid;
-  int64_t const my_start = my_row <= rows ? col.off(my_row) - first : n + 1;
+  uint32_t start_lo = 0, start_hi = 0;  // the raw offset entry; not touched before the end
+  if (my_row <= rows) {
+    if (col.is64) {
+      uint2 const v = static_cast<const uint2*>(col.offsets)[my_row + col.offset];
+      start_lo      = v.x;
+      start_hi      = v.y;
+    } else {
+      start_lo = static_cast<const uint32_t*>(col.offsets)[my_row + col.offset];
+    }
+  }
   Owned mine;
   uint32_t size[kNormItems];
   uint32_t const sum = tile_slots(lds, col.chars + first, t0, n, t, mine, size);
   uint32_t total;
-  uint32_t const before = block_exclusive_scan<kNormThreads>(sum, lds.scan, &total);
+  uint32_t const before = block_exclusive_scan_lds<kNormThreads>(sum, lds.scan, &total);
   {
     uint32_t run = before;
     uint32_t packed[kNormItems / 2];
@@ -414,22 +452,53 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
 
   uint8_t* const dst = out_chars + base;
   if (total <= static_cast<uint32_t>(kStageBytes)) {
-    // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword
+    // the output bytes, laid out in LDS as they will lie in memory relative to an aligned dword.  A slot is stored
+    // as one (unaligned) dword wherever the three bytes that may follow it still belong to this lane: later slots
+    // overwrite them.  The last slots of the lane go byte by byte.
     uint32_t const lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst) & 3u);
     uint8_t* const sb   = reinterpret_cast<uint8_t*>(lds.staged);
     uint32_t o          = lead + before;
+    uint32_t const mine_end = o + sum;
+    uint32_t all = 0;
 #pragma unroll
-    for (int j = 0; j < kNormItems; ++j) {
+    for (int j = 0; j < kNormItems; ++j) all |= mine.s[j][0] | mine.s[j][1] | mine.s[j][2];
+    if (ballot64(all > 0xFFu) == 0) {
+      // every character of the wavefront's output is one byte: a position's (up to three) bytes travel together
 #pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        uint32_t v = mine.s[j][k];
-        while (v) {
-          sb[o++] = static_cast<uint8_t>(v);
-          v >>= 8;
+      for (int j = 0; j < kNormItems; ++j) {
+        uint32_t const three = mine.s[j][0] | (mine.s[j][1] << 8) | (mine.s[j][2] << 16);
+        if (size[j]) {
+          if (o + 4u <= mine_end) {
+            __builtin_memcpy(sb + o, &three, 4);
+          } else {
+            sb[o] = static_cast<uint8_t>(three);
+            if (size[j] > 1u) sb[o + 1] = static_cast<uint8_t>(three >> 8);
+            if (size[j] > 2u) sb[o + 2] = static_cast<uint8_t>(three >> 16);
+          }
+          o += size[j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kNormItems; ++j) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+          uint32_t v = mine.s[j][k];
+          if (v) {
+            if (o + 4u <= mine_end) {
+              __builtin_memcpy(sb + o, &v, 4);
+              o += bytes_of(v);
+            } else {
+              do {
+                sb[o++] = static_cast<uint8_t>(v);
+                v >>= 8;
+              } while (v);
+            }
+          }
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
     uint32_t const end  = lead + total;
     uint32_t const w_lo = (lead + 3u) >> 2;
     uint32_t const w_hi = end >> 2;
@@ -458,11 +527,13 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
         }
       }
     }
-    __syncthreads();  // lds.prefix is complete for the rows below
+    lds_barrier();  // lds.prefix is complete for the rows below
   }
 
   // rows whose first byte lies in [t0, t1) -- in [t0, n] for the last tile -- start at base + prefix
-  bool const last_tile = blockIdx.x == gridDim.x - 1;
+  bool const last_tile   = blockIdx.x == gridDim.x - 1;
+  int64_t const my_start = (col.is64 ? static_cast<int64_t>((static_cast<uint64_t>(start_hi) << 32) | start_lo)
+                                     : static_cast<int64_t>(static_cast<int32_t>(start_lo))) - first;
   for (int64_t r = my_row; r <= rows; r += kNormThreads) {
     int64_t const p = r == my_row ? my_start : col.off(r) - first;
     if (p > t1 || (p == t1 && !last_tile)) break;
