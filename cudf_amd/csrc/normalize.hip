@@ -463,21 +463,20 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) all |= mine.s[j][0] | mine.s[j][1] | mine.s[j][2];
     if (ballot64(all > 0xFFu) == 0) {
-      // every character of the wavefront's output is one byte: a position's (up to three) bytes travel together
+      // every character of the wavefront's output is one byte: a position's (up to three) bytes travel together.
+      // A position that starts in the lane's last three bytes is skipped; those bytes are kept in `last` (the
+      // four bytes written last, newest on top) and stored one by one at the end.
+      uint32_t last = 0;
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
         uint32_t const three = mine.s[j][0] | (mine.s[j][1] << 8) | (mine.s[j][2] << 16);
-        if (size[j]) {
-          if (o + 4u <= mine_end) {
-            __builtin_memcpy(sb + o, &three, 4);
-          } else {
-            sb[o] = static_cast<uint8_t>(three);
-            if (size[j] > 1u) sb[o + 1] = static_cast<uint8_t>(three >> 8);
-            if (size[j] > 2u) sb[o + 2] = static_cast<uint8_t>(three >> 16);
-          }
-          o += size[j];
-        }
+        if (size[j] != 0u && o + 4u <= mine_end) __builtin_memcpy(sb + o, &three, 4);
+        last = __builtin_amdgcn_alignbit(three, last, 8u * size[j]);
+        o += size[j];
       }
+      if (sum >= 1u) sb[mine_end - 1u] = static_cast<uint8_t>(last >> 24);
+      if (sum >= 2u) sb[mine_end - 2u] = static_cast<uint8_t>(last >> 16);
+      if (sum >= 3u) sb[mine_end - 3u] = static_cast<uint8_t>(last >> 8);
     } else {
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
