@@ -23,12 +23,12 @@ VALU_PEAK_TOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 lanes x 2.4 GHz: one 32
 
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload, from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; the commands and
-# raw readings are in profiles/hbm_traffic_pmc_C2_C3_C4.md.  Counters cannot be read from inside this
+# raw readings are in profiles/hbm_traffic_pmc_all_workloads.md.  Counters cannot be read from inside this
 # process, so the line reports these figures only for the workload they were measured on.
 MEASURED_TRAFFIC_C2 = {
-    "wordpiece_probe_kernel": (1702_800_000, 1962_700_000),
-    "wordpiece_oov_kernel": (1061_400_000, 1428_100_000),
-    "wordpiece_emit_kernel": (2179_500_000, 848_000_000),
+    "wordpiece_probe_kernel": (1699400000, 1963300000),
+    "wordpiece_oov_kernel": (1037400000, 1435100000),
+    "wordpiece_emit_kernel": (2179500000, 848000000),
 }
 
 
