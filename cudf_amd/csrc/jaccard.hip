@@ -103,7 +103,8 @@ __device__ __forceinline__ void jaccard_pair(ColView const& c1, ColView const& c
   constexpr uint32_t kPairThreads = WAVES * kWave;
   int const lane = lane_id();
   int const wave = threadIdx.x / kWave;
-  for (uint32_t i = threadIdx.x; i < nslots; i += kPairThreads) slots[i] = 0u;
+  // (nslots is a power of two of at least 64 and the arrays are 16-byte aligned: whole uint4 stores)
+  for (uint32_t i = threadIdx.x; i < nslots / 4; i += kPairThreads) reinterpret_cast<uint4*>(slots)[i] = make_uint4(0u, 0u, 0u, 0u);
   for (uint32_t i = threadIdx.x; i < nslots / 32; i += kPairThreads) {
     in1[i] = 0u;
     in2[i] = 0u;
@@ -180,7 +181,7 @@ __device__ __forceinline__ void list_pair(uint32_t* lists, int which, int64_t ro
 __global__ void __launch_bounds__(kThreads) jaccard_small_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
                                                                  uint32_t* __restrict__ lists)
 {
-  __shared__ uint32_t slots[kSmallSlots];
+  __shared__ alignas(16) uint32_t slots[kSmallSlots];
   __shared__ uint32_t in1[kSmallSlots / 32], in2[kSmallSlots / 32];
   __shared__ PairScratch<kWaves> scratch;
   int64_t const rows = c1.size;
@@ -199,7 +200,7 @@ __global__ void __launch_bounds__(kThreads) jaccard_small_kernel(ColView c1, Col
 __global__ void __launch_bounds__(kMediumWaves * kWave) jaccard_medium_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
                                                                               uint32_t* __restrict__ lists)
 {
-  __shared__ uint32_t slots[kMediumSlots];
+  __shared__ alignas(16) uint32_t slots[kMediumSlots];
   __shared__ uint32_t in1[kMediumSlots / 32], in2[kMediumSlots / 32];
   __shared__ PairScratch<kMediumWaves> scratch;
   int64_t const rows   = c1.size;
