@@ -310,9 +310,17 @@ def main():
         zsec = timed_steps(zstep, max(3, args.steps // 2), 1, torch)
         zk = kernel_times(zstep, 2, _capi, torch)
         out_bytes = int(keep["o"].chars.numel())
+        # algorithmic bytes of a call: chars + offsets in, chars + offsets (int64 from INT32_MAX bytes on) out; priced against the longest kernel
+        zalg = ib + out_bytes + (8 if out_bytes >= 0x7FFFFFFF else 4) * (w.rows.size + 1)
+        zdom = max(zk, key=zk.get)
         leg["normalize_characters"] = {"ms_per_step": round(zsec * 1e3, 3), "input_GBps": round(ib / zsec / 1e9, 2),
                                        "mrows_per_s": round(w.rows.size / zsec / 1e6, 3), "chars_out": out_bytes,
-                                       "kernels_ms": {k: round(v, 3) for k, v in zk.items()}}
+                                       "kernels_ms": {k: round(v, 3) for k, v in zk.items()},
+                                       "roofline": {"bound": "hbm", "kernel": zdom, "achieved": round(zalg / (zk[zdom] * 1e-3) / 1e9, 1),
+                                                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                                    "frac": round(zalg / (zk[zdom] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                                    "algorithmic_bytes": zalg, "frac_whole_op": round(zalg / zsec / 1e9 / HBM_PEAK_GBS, 4),
+                                                    "traffic": None}}
         if not args.no_cpu:
             from oracle import normalize_py
             n = 4000
