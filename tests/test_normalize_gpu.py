@@ -202,3 +202,24 @@ def test_normalize_large_strings_offsets(nv, total):
     assert out.offsets.dtype == (torch.int64 if total >= 0x7FFFFFFF else torch.int32)
     assert out.chars.numel() == total and torch.equal(out.chars, chars)
     assert torch.equal(out.offsets.to(torch.int64), offsets)
+
+
+def test_normalize_feeds_the_tokenizer(nv, onorm):
+    # the BERT pipeline on the device: the STRING result of normalize_characters goes straight into wordpiece_tokenize
+    from oracle import pyoracle as orc
+    d = gc.bert_case()
+    vocab = strings(d["vocab"])
+    words = [v.decode("utf-8") for v in d["vocab"] if v.isalpha() and len(v) > 2][:500]
+    rng = np.random.default_rng(21)
+    styles = [str.upper, str.title, lambda s: s, lambda s: s + ",", lambda s: "(" + s + ")", lambda s: s.replace("e", "é"),
+              lambda s: s + "\t", lambda s: "[CLS]" + s, lambda s: s + "丏", lambda s: s + "!?"]
+    rows = [None if rng.random() < 0.05 else
+            " ".join(styles[int(rng.integers(0, len(styles)))](words[int(rng.integers(0, len(words)))]) for _ in range(int(rng.integers(0, 40))))
+            for _ in range(3000)]
+    host = strings(rows)
+    normalizer = nv.CharacterNormalizer(True, nv.DeviceStringsColumn.from_host(strings(["[CLS]"])))
+    normalized = nv.normalize_characters(nv.DeviceStringsColumn.from_host(host), normalizer)
+    got = nv.wordpiece_tokenize(normalized, nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(vocab)), 0).to_host()
+    exp = orc.wordpiece_tokenize(onorm.normalize_characters(host, True, [b"[CLS]"]), orc.Vocabulary(vocab), 0)
+    assert got.equals(exp)
+    assert got.child.size > 3 * 3000

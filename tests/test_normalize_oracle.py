@@ -147,3 +147,61 @@ def test_special_tokens_lowered_after_sorting_can_be_missed():
     col = gc.strings(["[PAD]", "[PADS]"])
     got = onorm.normalize_characters(col, True, [b"[PAD]", b"[PADS]", b"[LONGER]"]).to_pylist()
     assert got == [b" [ pad ] ", b" [PADS] "]
+
+
+# Unicode blocks whose characters and properties have not changed for many Unicode versions: an implementation with
+# older or newer character tables than the reference's (Unicode 11) must still agree there
+STABLE_BLOCKS = [(1, 0x0780), (0x1E00, 0x1F00), (0x2000, 0x2070), (0x3000, 0x3100), (0x4E00, 0x9FA6), (0xAC00, 0xD7A4),
+                 (0xFB00, 0xFB50), (0xFF00, 0xFFF0)]
+
+
+def test_rules_match_hf_bert_normalizer_and_pre_tokenizer():
+    """An independent implementation of the same BERT clean-up (tokenizers' BertNormalizer + BertPreTokenizer, written in
+    Rust with its own character tables): the words it finds in "x<c>y" must be the words of the oracle's output, for every
+    assigned character c of the stable blocks, lower-casing and not."""
+    import unicodedata
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers import normalizers, pre_tokenizers
+    pre = pre_tokenizers.BertPreTokenizer()
+    checked = 0
+    for lower in (True, False):
+        norm = normalizers.BertNormalizer(clean_text=True, handle_chinese_chars=True, strip_accents=None if lower else False, lowercase=lower)
+        for lo, hi in STABLE_BLOCKS:
+            cps = [cp for cp in range(lo, hi) if unicodedata.category(chr(cp)) not in ("Cn", "Co")]
+            rows = ["x" + chr(cp) + "y" for cp in cps]
+            got = onorm.normalize_characters(gc.strings(rows), lower).to_pylist()
+            for cp, text, g in zip(cps, rows, got):
+                want = [w for w, _ in pre.pre_tokenize_str(norm.normalize_str(text))]
+                assert [w for w in g.decode("utf-8").split(" ") if w] == want, (hex(cp), lower)
+                checked += 1
+    assert checked > 60000
+
+
+def test_normalize_then_tokenize_matches_hf_bert_pipeline():
+    """normalize_characters followed by wordpiece_tokenize is BERT's tokenizer: ids equal tokenizers' Bert pipeline."""
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers import Tokenizer, normalizers, pre_tokenizers
+    from tokenizers.models import WordPiece
+    from oracle import pyoracle as orc
+    d = gc.bert_case()
+    vocab = [v.decode("utf-8") for v in d["vocab"]]
+    ids = {}
+    for i, t in enumerate(vocab):
+        ids.setdefault(t, i)
+    tok = Tokenizer(WordPiece(ids, unk_token="[UNK]", max_input_chars_per_word=100))
+    tok.normalizer = normalizers.BertNormalizer(clean_text=True, handle_chinese_chars=True, strip_accents=None, lowercase=True)
+    tok.pre_tokenizer = pre_tokenizers.BertPreTokenizer()
+    rng = np.random.default_rng(5)
+    stems = [t for t in vocab if t.isalpha() and t.isascii() and len(t) > 2][:600]
+    decorate = [str.upper, str.title, lambda s: s, lambda s: s + ",", lambda s: "(" + s + ")", lambda s: s.replace("e", "é").replace("a", "Â"),
+                lambda s: s + "\t", lambda s: s + "ing", lambda s: "un" + s, lambda s: s + "丏", lambda s: s + "­", lambda s: s + "!?"]
+    rows = [" ".join(decorate[int(rng.integers(0, len(decorate)))](stems[int(rng.integers(0, len(stems)))]) for _ in range(int(rng.integers(1, 25))))
+            for _ in range(400)]
+    normalized = onorm.normalize_characters(gc.strings(rows), True)
+    got = orc.wordpiece_tokenize(normalized, orc.Vocabulary(gc.strings(d["vocab"])), 0).to_pylist()
+    split = 0
+    for row, g in zip(rows, got):
+        want = tok.encode(row, add_special_tokens=False).ids
+        assert g == want, row
+        split += len(want) > len(row.split(" "))
+    assert split > 200  # punctuation and sub-word splits were exercised
