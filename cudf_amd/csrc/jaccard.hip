@@ -7,9 +7,11 @@
 // Here a workgroup takes a row pair and needs no sort and no temporary: the window hashes of both rows go
 // into ONE open-addressing set in LDS (load <= 2/3) with two membership bits per slot, "seen in row 1" and
 // "seen in row 2".  |A|, |B| and |A n B| are then population counts of the two bit arrays and of their
-// AND.  Two launches cover the pairs by size: a 32 KiB set (four workgroups per CU) for pairs of up to
-// 5461 bytes together, a 128 KiB set (one workgroup of eight wavefronts per CU) up to 21845 bytes; the
-// few longer pairs are listed and done by a third kernel with the same code over a set in global memory.
+// AND.  The launches cover the pairs by size: an 8 KiB set per WAVEFRONT (each wavefront its own pair, nothing
+// shared, so that many short pairs are in flight per CU) for pairs of up to 1365 bytes together, a 32 KiB set
+// (four workgroups per CU) up to 5461 bytes, a 128 KiB set (one workgroup of eight wavefronts per CU) up to
+// 21845 bytes; the few longer pairs are done by a last kernel with the same code over a set in global memory.
+// Each kernel lists the pairs that are too large for it for the next one.
 #include "common.cuh"
 #include "murmur.cuh"
 #include "windows.cuh"
@@ -19,6 +21,7 @@
 namespace nvtext_amd {
 namespace {
 
+constexpr uint32_t kTinySlots   = 2048;   // slots of a wavefront's own LDS set
 constexpr uint32_t kSmallSlots  = 8192;   // slots of the small LDS set
 constexpr uint32_t kMediumSlots = 32768;  // slots of the large LDS set
 constexpr int kMediumWaves      = 8;
@@ -45,7 +48,7 @@ struct PairSet {
 
 // Hashes the windows of one row (jaccard.cu:249-292) and inserts the non-zero hashes into the set.
 // The wavefronts of the workgroup take the tiles of the row in turn.
-__device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_t width, PairSet const& set, int which, WaveLds<uint32_t>& lds,
+__device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_t width, PairSet const& set, int which, uint32_t* stage,
                                            int wave, int nwaves, int lane)
 {
   if (static_cast<int64_t>(width) * 4 <= kHalo) {
@@ -54,7 +57,7 @@ __device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_
       uint32_t const cnt = static_cast<uint32_t>(min(static_cast<int64_t>(kTile), n - base));
       uint32_t const len = static_cast<uint32_t>(min(n - base, static_cast<int64_t>(cnt + halo)));
       bool all_ascii;
-      uint32_t const mis = stage_bytes(row, base, len, lds.bytes, lane, &all_ascii);
+      uint32_t const mis = stage_bytes(row, base, len, stage, lane, &all_ascii);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -62,7 +65,7 @@ __device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_
         uint32_t const p = q + lane;
         if (p < cnt) {
           int64_t const gpos = base + p;
-          WordSrc const src{lds.bytes, mis + p};
+          WordSrc const src{stage, mis + p};
           uint32_t hlen;
           if (window_at(src, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen)) {
             uint32_t const hv = murmur3_x86_32(src, hlen, 0u);  // jaccard.cu:258: seed 0
@@ -114,11 +117,11 @@ __device__ __forceinline__ void jaccard_pair(ColView const& c1, ColView const& c
   // 211-220: null rows and empty rows have no hashes
   if (c1.valid(r)) {
     int64_t const o = c1.off(r);
-    insert_row(c1.chars + o, c1.off(r + 1) - o, width, set, 0, scratch.wave[wave], wave, WAVES, lane);
+    insert_row(c1.chars + o, c1.off(r + 1) - o, width, set, 0, scratch.wave[wave].bytes, wave, WAVES, lane);
   }
   if (c2.valid(r)) {
     int64_t const o = c2.off(r);
-    insert_row(c2.chars + o, c2.off(r + 1) - o, width, set, 1, scratch.wave[wave], wave, WAVES, lane);
+    insert_row(c2.chars + o, c2.off(r + 1) - o, width, set, 1, scratch.wave[wave].bytes, wave, WAVES, lane);
   }
   __syncthreads();
   uint32_t u1 = 0, u2 = 0, both = 0;
@@ -167,25 +170,106 @@ __device__ __host__ __forceinline__ uint64_t slots_for(int64_t bytes)
   return s;
 }
 
-// Work lists in `lists`: [0] = pairs listed for the global-memory kernel, [1] = pairs listed for the medium
-// kernel, [2..3] = the most bytes a pair of the first list has (64 bits), then `rows` entries of the first
-// list and `rows` entries of the second.
+// Work lists in `lists`: a header of 8 words -- [0] = pairs listed for the global-memory kernel, [1] = for the
+// medium kernel, [2..3] = the most bytes a pair of the first list has (64 bits), [4] = pairs listed for the small
+// kernel -- then `rows` entries each for the global, the medium and the small list.
+constexpr int kListHeader = 8;
+__device__ __forceinline__ uint32_t* list_count(uint32_t* lists, int which) { return &lists[which == 2 ? 4 : which]; }
+__device__ __forceinline__ uint32_t* list_entries(uint32_t* lists, int which, int64_t rows) { return lists + kListHeader + which * rows; }
 __device__ __forceinline__ void list_pair(uint32_t* lists, int which, int64_t rows, int64_t r, int64_t bytes)
 {
-  uint32_t const at = atomicAdd(&lists[which], 1u);
-  lists[4 + (which ? rows : 0) + at] = static_cast<uint32_t>(r);
+  uint32_t const at                  = atomicAdd(list_count(lists, which), 1u);
+  list_entries(lists, which, rows)[at] = static_cast<uint32_t>(r);
   if (which == 0) atomicMax(reinterpret_cast<unsigned long long*>(&lists[2]), static_cast<unsigned long long>(bytes));
 }
 
-// All pairs whose set fits kSmallSlots; the others are listed for the medium kernel.
+struct TinyLds {
+  alignas(16) uint32_t slots[kTinySlots];
+  uint32_t in1[kTinySlots / 32], in2[kTinySlots / 32];
+  uint32_t stage[kTileWords];  // the bytes of the tile being hashed
+};
+
+// Every wavefront on its own: it sizes 64 consecutive pairs at once (lanes <-> pairs, coalesced offset loads), lists
+// those that need more than kTinySlots for the small kernel with one atomic, and does the others one after the
+// other with its own set.  No workgroup barrier anywhere.
+__global__ void __launch_bounds__(kThreads) jaccard_tiny_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
+                                                                uint32_t* __restrict__ lists)
+{
+  __shared__ TinyLds lds_all[kWaves];
+  int const lane       = lane_id();
+  TinyLds& lds         = lds_all[threadIdx.x / kWave];
+  int64_t const rows   = c1.size;
+  int64_t const nwaves = static_cast<int64_t>(gridDim.x) * kWaves;
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  for (int64_t base = (static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave) * kWave; base < rows; base += nwaves * kWave) {
+    int64_t const r = base + lane;
+    int64_t o1 = 0, n1 = 0, o2 = 0, n2 = 0;  // 211-220: null rows and empty rows have no hashes
+    if (r < rows) {
+      if (c1.valid(r)) {
+        o1 = c1.off(r);
+        n1 = c1.off(r + 1) - o1;
+      }
+      if (c2.valid(r)) {
+        o2 = c2.off(r);
+        n2 = c2.off(r + 1) - o2;
+      }
+    }
+    uint64_t const need = slots_for(n1 + n2);
+    bool const mine     = r < rows && need <= kTinySlots;
+    uint64_t const later = ballot64(r < rows && !mine);
+    if (later != 0) {
+      uint32_t at = 0;
+      if (lane == 0) at = atomicAdd(list_count(lists, 2), static_cast<uint32_t>(__builtin_popcountll(later)));
+      at = wave_bcast(at, 0);
+      if (r < rows && !mine) list_entries(lists, 2, rows)[at + lanes_below(later)] = static_cast<uint32_t>(r);
+    }
+    for (uint64_t todo = ballot64(mine); todo != 0; todo &= todo - 1) {
+      int const b           = __builtin_ctzll(todo);
+      uint32_t const nslots = static_cast<uint32_t>(wave_bcast64(need, b));
+      int64_t const ro1 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(o1), b)), rn1 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(n1), b));
+      int64_t const ro2 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(o2), b)), rn2 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(n2), b));
+      for (uint32_t i = lane; i < nslots / 4; i += kWave) reinterpret_cast<uint4*>(lds.slots)[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (static_cast<uint32_t>(lane) < nslots / 32) {
+        lds.in1[lane] = 0u;
+        lds.in2[lane] = 0u;
+      }
+      wave_sync();
+      PairSet const set{lds.slots, lds.in1, lds.in2, nslots - 1u, static_cast<uint32_t>(__builtin_clz(nslots)) + 1u};
+      if (rn1 > 0) insert_row(c1.chars + ro1, rn1, width, set, 0, lds.stage, 0, 1, lane);
+      if (rn2 > 0) insert_row(c2.chars + ro2, rn2, width, set, 1, lds.stage, 0, 1, lane);
+      wave_sync();
+      uint32_t u1 = 0, u2 = 0, both = 0;
+      if (static_cast<uint32_t>(lane) < nslots / 32) {  // at most 64 words of bits
+        uint32_t const a = lds.in1[lane], bb = lds.in2[lane];
+        u1   = __builtin_popcount(a);
+        u2   = __builtin_popcount(bb);
+        both = __builtin_popcount(a & bb);
+      }
+      int32_t const count1     = static_cast<int32_t>(wave_bcast(wave_inclusive_scan(u1), kWave - 1));
+      int32_t const count2     = static_cast<int32_t>(wave_bcast(wave_inclusive_scan(u2), kWave - 1));
+      int32_t const intersects = static_cast<int32_t>(wave_bcast(wave_inclusive_scan(both), kWave - 1));
+      int32_t const unions     = count1 + count2 - intersects;  // jaccard.cu:414-425
+      if (lane == 0) out[base + b] = unions ? static_cast<float>(intersects) / static_cast<float>(unions) : 0.f;
+      wave_sync();
+    }
+  }
+}
+
+// The pairs listed by the tiny kernel whose set fits kSmallSlots; the others are listed for the medium kernel.
 __global__ void __launch_bounds__(kThreads) jaccard_small_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
                                                                  uint32_t* __restrict__ lists)
 {
   __shared__ alignas(16) uint32_t slots[kSmallSlots];
   __shared__ uint32_t in1[kSmallSlots / 32], in2[kSmallSlots / 32];
   __shared__ PairScratch<kWaves> scratch;
-  int64_t const rows = c1.size;
-  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+  int64_t const rows   = c1.size;
+  uint32_t const count = *list_count(lists, 2);
+  for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
+    int64_t const r     = list_entries(lists, 2, rows)[i];
     int64_t const bytes = pair_bytes(c1, c2, r);
     uint64_t const need = slots_for(bytes);
     if (need > kSmallSlots) {
@@ -206,7 +290,7 @@ __global__ void __launch_bounds__(kMediumWaves * kWave) jaccard_medium_kernel(Co
   int64_t const rows   = c1.size;
   uint32_t const count = lists[1];
   for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
-    int64_t const r     = lists[4 + rows + i];
+    int64_t const r     = list_entries(lists, 1, rows)[i];
     int64_t const bytes = pair_bytes(c1, c2, r);
     uint64_t const need = slots_for(bytes);
     if (need > kMediumSlots) {
@@ -226,7 +310,7 @@ __global__ void __launch_bounds__(kThreads) jaccard_global_kernel(ColView c1, Co
   uint32_t const count = big[0];
   uint32_t* const mine = tables + static_cast<uint64_t>(blockIdx.x) * (table_slots + 2 * (table_slots / 32));
   for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
-    int64_t const r     = big[4 + i];
+    int64_t const r     = big[kListHeader + i];
     uint32_t const need = static_cast<uint32_t>(slots_for(pair_bytes(c1, c2, r)));
     jaccard_pair<kWaves>(c1, c2, r, width, mine, mine + table_slots, mine + table_slots + table_slots / 32, need, scratch, out);
   }
@@ -294,14 +378,14 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
       return fail(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
     }
   }
-  // the two work lists (see list_pair) and the null counter behind them
-  Temp big(mr, (2 * static_cast<size_t>(rows) + 8) * sizeof(uint32_t));
+  // the three work lists (see list_pair) and the null counter behind them
+  Temp big(mr, (3 * static_cast<size_t>(rows) + kListHeader + 4) * sizeof(uint32_t));
   if (!big.ok()) {
     nvtext_amd_fixed_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
-  launch_fill_u32(big.as<uint32_t>(), 0u, 4, stream);
-  uint32_t* const null_counter = big.as<uint32_t>() + 4 + 2 * static_cast<size_t>(rows);
+  launch_fill_u32(big.as<uint32_t>(), 0u, kListHeader, stream);
+  uint32_t* const null_counter = big.as<uint32_t>() + kListHeader + 3 * static_cast<size_t>(rows);
   launch_fill_u32(null_counter, 0u, 1, stream);
 
   ColView const v1 = make_view(*input1);
@@ -310,6 +394,12 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
   int device = 0, cus = 256;
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+  {
+    ProfileScope ps("jaccard_tiny_kernel", stream);
+    int64_t const batches = (static_cast<int64_t>(rows) + kWave * kWaves - 1) / (kWave * kWaves);
+    unsigned const grid   = static_cast<unsigned>(std::min<int64_t>(batches, static_cast<int64_t>(cus) * 8));
+    hipLaunchKernelGGL(jaccard_tiny_kernel, dim3(grid), dim3(kThreads), 0, stream, v1, v2, width, values, big.as<uint32_t>());
+  }
   {
     ProfileScope ps("jaccard_small_kernel", stream);
     unsigned const grid = static_cast<unsigned>(std::min<int64_t>(rows, static_cast<int64_t>(cus) * 16));
