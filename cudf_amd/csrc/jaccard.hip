@@ -162,7 +162,8 @@ __device__ __forceinline__ int64_t pair_bytes(ColView const& c1, ColView const& 
   return n;
 }
 
-// Slots for a pair: a power of two that keeps the load at or below 2/3 (window starts <= bytes).
+// Slots a pair needs: a power of two that keeps the load at or below 2/3 (window starts <= bytes).  This decides
+// the kernel that takes the pair; where that kernel's set has room it uses twice as many (shorter probe runs).
 __device__ __host__ __forceinline__ uint64_t slots_for(int64_t bytes)
 {
   uint64_t s = 64;
@@ -229,7 +230,7 @@ __global__ void __launch_bounds__(kThreads) jaccard_tiny_kernel(ColView c1, ColV
     }
     for (uint64_t todo = ballot64(mine); todo != 0; todo &= todo - 1) {
       int const b           = __builtin_ctzll(todo);
-      uint32_t const nslots = static_cast<uint32_t>(wave_bcast64(need, b));
+      uint32_t const nslots = min(kTinySlots, 2u * static_cast<uint32_t>(wave_bcast64(need, b)));
       int64_t const ro1 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(o1), b)), rn1 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(n1), b));
       int64_t const ro2 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(o2), b)), rn2 = static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(n2), b));
       for (uint32_t i = lane; i < nslots / 4; i += kWave) reinterpret_cast<uint4*>(lds.slots)[i] = make_uint4(0u, 0u, 0u, 0u);
@@ -276,7 +277,7 @@ __global__ void __launch_bounds__(kThreads) jaccard_small_kernel(ColView c1, Col
       if (threadIdx.x == 0) list_pair(lists, 1, rows, r, bytes);
       continue;
     }
-    jaccard_pair<kWaves>(c1, c2, r, width, slots, in1, in2, static_cast<uint32_t>(need), scratch, out);
+    jaccard_pair<kWaves>(c1, c2, r, width, slots, in1, in2, min(kSmallSlots, 2u * static_cast<uint32_t>(need)), scratch, out);
   }
 }
 
@@ -297,7 +298,7 @@ __global__ void __launch_bounds__(kMediumWaves * kWave) jaccard_medium_kernel(Co
       if (threadIdx.x == 0) list_pair(lists, 0, rows, r, bytes);
       continue;
     }
-    jaccard_pair<kMediumWaves>(c1, c2, r, width, slots, in1, in2, static_cast<uint32_t>(need), scratch, out);
+    jaccard_pair<kMediumWaves>(c1, c2, r, width, slots, in1, in2, min(kMediumSlots, 2u * static_cast<uint32_t>(need)), scratch, out);
   }
 }
 
