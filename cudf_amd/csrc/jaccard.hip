@@ -9,8 +9,9 @@
 // "seen in row 2".  |A|, |B| and |A n B| are then population counts of the two bit arrays and of their
 // AND.  The launches cover the pairs by size: an 8 KiB set per WAVEFRONT (each wavefront its own pair, nothing
 // shared, so that many short pairs are in flight per CU) for pairs of up to 1365 bytes together, a 32 KiB set
-// (four workgroups per CU) up to 5461 bytes, a 128 KiB set (one workgroup of eight wavefronts per CU) up to
-// 21845 bytes; the few longer pairs are done by a last kernel with the same code over a set in global memory.
+// (four workgroups per CU) up to 5461 bytes, a 64 KiB set (two workgroups of eight wavefronts per CU) up to 10922
+// bytes, a 128 KiB set (one workgroup per CU) up to 21845 bytes; the few longer pairs are done by a last kernel
+// with the same code over a set in global memory.
 // Each kernel lists the pairs that are too large for it for the next one.
 #include "common.cuh"
 #include "murmur.cuh"
@@ -23,6 +24,7 @@ namespace {
 
 constexpr uint32_t kTinySlots   = 2048;   // slots of a wavefront's own LDS set
 constexpr uint32_t kSmallSlots  = 8192;   // slots of the small LDS set
+constexpr uint32_t kMidSlots    = 16384;  // slots of the 64 KiB LDS set
 constexpr uint32_t kMediumSlots = 32768;  // slots of the large LDS set
 constexpr int kMediumWaves      = 8;
 
@@ -93,7 +95,7 @@ __device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_
 
 template <int WAVES>
 struct PairScratch {
-  WaveLds<uint32_t> wave[WAVES];
+  uint32_t stage[WAVES][kTileWords];  // per wavefront: the bytes of the tile being hashed
   uint32_t sums[3][WAVES];
 };
 
@@ -117,11 +119,11 @@ __device__ __forceinline__ void jaccard_pair(ColView const& c1, ColView const& c
   // 211-220: null rows and empty rows have no hashes
   if (c1.valid(r)) {
     int64_t const o = c1.off(r);
-    insert_row(c1.chars + o, c1.off(r + 1) - o, width, set, 0, scratch.wave[wave].bytes, wave, WAVES, lane);
+    insert_row(c1.chars + o, c1.off(r + 1) - o, width, set, 0, scratch.stage[wave], wave, WAVES, lane);
   }
   if (c2.valid(r)) {
     int64_t const o = c2.off(r);
-    insert_row(c2.chars + o, c2.off(r + 1) - o, width, set, 1, scratch.wave[wave].bytes, wave, WAVES, lane);
+    insert_row(c2.chars + o, c2.off(r + 1) - o, width, set, 1, scratch.stage[wave], wave, WAVES, lane);
   }
   __syncthreads();
   uint32_t u1 = 0, u2 = 0, both = 0;
@@ -172,10 +174,10 @@ __device__ __host__ __forceinline__ uint64_t slots_for(int64_t bytes)
 }
 
 // Work lists in `lists`: a header of 8 words -- [0] = pairs listed for the global-memory kernel, [1] = for the
-// medium kernel, [2..3] = the most bytes a pair of the first list has (64 bits), [4] = pairs listed for the small
-// kernel -- then `rows` entries each for the global, the medium and the small list.
+// 128 KiB kernel, [2..3] = the most bytes a pair of the first list has (64 bits), [4] = pairs listed for the 32 KiB
+// kernel, [5] = for the 64 KiB kernel -- then `rows` entries for each of these four lists, in the order 0, 1, [4], [5].
 constexpr int kListHeader = 8;
-__device__ __forceinline__ uint32_t* list_count(uint32_t* lists, int which) { return &lists[which == 2 ? 4 : which]; }
+__device__ __forceinline__ uint32_t* list_count(uint32_t* lists, int which) { return &lists[which >= 2 ? which + 2 : which]; }
 __device__ __forceinline__ uint32_t* list_entries(uint32_t* lists, int which, int64_t rows) { return lists + kListHeader + which * rows; }
 __device__ __forceinline__ void list_pair(uint32_t* lists, int which, int64_t rows, int64_t r, int64_t bytes)
 {
@@ -260,45 +262,26 @@ __global__ void __launch_bounds__(kThreads) jaccard_tiny_kernel(ColView c1, ColV
   }
 }
 
-// The pairs listed by the tiny kernel whose set fits kSmallSlots; the others are listed for the medium kernel.
-__global__ void __launch_bounds__(kThreads) jaccard_small_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
-                                                                 uint32_t* __restrict__ lists)
+// The pairs of list FROM whose set fits SLOTS slots, one workgroup of WAVES wavefronts per pair; the others are put on
+// list TO.  Three instances: 8192 slots (32 KiB, four workgroups per CU), 16384 (64 KiB, two per CU), 32768 (128 KiB, one).
+template <uint32_t SLOTS, int WAVES, int FROM, int TO>
+__global__ void __launch_bounds__(WAVES* kWave) jaccard_listed_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
+                                                                       uint32_t* __restrict__ lists)
 {
-  __shared__ alignas(16) uint32_t slots[kSmallSlots];
-  __shared__ uint32_t in1[kSmallSlots / 32], in2[kSmallSlots / 32];
-  __shared__ PairScratch<kWaves> scratch;
+  __shared__ alignas(16) uint32_t slots[SLOTS];
+  __shared__ uint32_t in1[SLOTS / 32], in2[SLOTS / 32];
+  __shared__ PairScratch<WAVES> scratch;
   int64_t const rows   = c1.size;
-  uint32_t const count = *list_count(lists, 2);
+  uint32_t const count = *list_count(lists, FROM);
   for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
-    int64_t const r     = list_entries(lists, 2, rows)[i];
+    int64_t const r     = list_entries(lists, FROM, rows)[i];
     int64_t const bytes = pair_bytes(c1, c2, r);
     uint64_t const need = slots_for(bytes);
-    if (need > kSmallSlots) {
-      if (threadIdx.x == 0) list_pair(lists, 1, rows, r, bytes);
+    if (need > SLOTS) {
+      if (threadIdx.x == 0) list_pair(lists, TO, rows, r, bytes);
       continue;
     }
-    jaccard_pair<kWaves>(c1, c2, r, width, slots, in1, in2, min(kSmallSlots, 2u * static_cast<uint32_t>(need)), scratch, out);
-  }
-}
-
-// The pairs listed by the small kernel whose set fits kMediumSlots; the others are listed for the global-memory kernel.
-__global__ void __launch_bounds__(kMediumWaves * kWave) jaccard_medium_kernel(ColView c1, ColView c2, int32_t width, float* __restrict__ out,
-                                                                              uint32_t* __restrict__ lists)
-{
-  __shared__ alignas(16) uint32_t slots[kMediumSlots];
-  __shared__ uint32_t in1[kMediumSlots / 32], in2[kMediumSlots / 32];
-  __shared__ PairScratch<kMediumWaves> scratch;
-  int64_t const rows   = c1.size;
-  uint32_t const count = lists[1];
-  for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
-    int64_t const r     = list_entries(lists, 1, rows)[i];
-    int64_t const bytes = pair_bytes(c1, c2, r);
-    uint64_t const need = slots_for(bytes);
-    if (need > kMediumSlots) {
-      if (threadIdx.x == 0) list_pair(lists, 0, rows, r, bytes);
-      continue;
-    }
-    jaccard_pair<kMediumWaves>(c1, c2, r, width, slots, in1, in2, min(kMediumSlots, 2u * static_cast<uint32_t>(need)), scratch, out);
+    jaccard_pair<WAVES>(c1, c2, r, width, slots, in1, in2, min(SLOTS, 2u * static_cast<uint32_t>(need)), scratch, out);
   }
 }
 
@@ -379,14 +362,14 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
       return fail(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
     }
   }
-  // the three work lists (see list_pair) and the null counter behind them
-  Temp big(mr, (3 * static_cast<size_t>(rows) + kListHeader + 4) * sizeof(uint32_t));
+  // the four work lists (see list_pair) and the null counter behind them
+  Temp big(mr, (4 * static_cast<size_t>(rows) + kListHeader + 4) * sizeof(uint32_t));
   if (!big.ok()) {
     nvtext_amd_fixed_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
   launch_fill_u32(big.as<uint32_t>(), 0u, kListHeader, stream);
-  uint32_t* const null_counter = big.as<uint32_t>() + kListHeader + 3 * static_cast<size_t>(rows);
+  uint32_t* const null_counter = big.as<uint32_t>() + kListHeader + 4 * static_cast<size_t>(rows);
   launch_fill_u32(null_counter, 0u, 1, stream);
 
   ColView const v1 = make_view(*input1);
@@ -404,12 +387,20 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
   {
     ProfileScope ps("jaccard_small_kernel", stream);
     unsigned const grid = static_cast<unsigned>(std::min<int64_t>(rows, static_cast<int64_t>(cus) * 16));
-    hipLaunchKernelGGL(jaccard_small_kernel, dim3(grid), dim3(kThreads), 0, stream, v1, v2, width, values, big.as<uint32_t>());
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(jaccard_listed_kernel<kSmallSlots, kWaves, 2, 3>), dim3(grid), dim3(kThreads), 0, stream, v1, v2, width, values,
+                       big.as<uint32_t>());
+  }
+  {
+    ProfileScope ps("jaccard_mid_kernel", stream);
+    unsigned const grid = static_cast<unsigned>(std::min<int64_t>(rows, static_cast<int64_t>(cus) * 4));
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(jaccard_listed_kernel<kMidSlots, kMediumWaves, 3, 1>), dim3(grid), dim3(kMediumWaves * kWave), 0, stream, v1, v2,
+                       width, values, big.as<uint32_t>());
   }
   {
     ProfileScope ps("jaccard_medium_kernel", stream);
     unsigned const grid = static_cast<unsigned>(std::min<int64_t>(rows, static_cast<int64_t>(cus) * 2));
-    hipLaunchKernelGGL(jaccard_medium_kernel, dim3(grid), dim3(kMediumWaves * kWave), 0, stream, v1, v2, width, values, big.as<uint32_t>());
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(jaccard_listed_kernel<kMediumSlots, kMediumWaves, 1, 0>), dim3(grid), dim3(kMediumWaves * kWave), 0, stream, v1, v2,
+                       width, values, big.as<uint32_t>());
   }
   if (with_mask) {
     int32_t const words = (rows + 31) / 32;
