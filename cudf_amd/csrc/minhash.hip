@@ -475,6 +475,9 @@ struct AlignedSrc {
   }
 };
 
+constexpr uint32_t kNgramStageBytes = 4096;                             // longest stretch of chars hashed out of LDS
+constexpr uint32_t kNgramStageWords = (kNgramStageBytes + 4 + 28) / 4;  // + misalignment, + over-read of the hash tail
+
 // One workgroup per (row, parameter chunk); its wavefronts take the positions of the row 64 at a time.
 template <typename T, int K>
 __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, int32_t ngrams, T seed, const T* __restrict__ pa,
@@ -484,6 +487,7 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
   using H = HashTraits<T>;
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][K * kWave];
+  __shared__ uint32_t run_bytes[kWaves][kNgramStageWords];  // the chars of the elements a wavefront is hashing
 
   int64_t const r = blockIdx.x;
   if (!in.valid(r)) return;
@@ -507,19 +511,39 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
     int64_t const idx = base + lane;
     bool valid        = false;
     T hv              = 0;
+    int64_t bo = 0, eo = 0;
     if (idx < positions && in.child.valid(first + idx)) {  // 213-216: a null element starts no run
       // 218-222: the run ends at element idx + ngrams, clamped to the row; a clamped run counts only at idx 0
       int64_t const next = min(idx + ngrams, n - 1);
       if (idx == 0 || next - idx >= ngrams) {
         // 224-229: the bytes from the start of element idx to the end of element next
-        int64_t const bo = in.child.off(first + idx);
-        int64_t const eo = in.child.off(first + next + 1);
-        AlignedSrc const src(in.child.chars + bo, static_cast<uint32_t>(eo - bo));
-        hv    = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
-        hv    = hv < 1 ? T{1} : hv;  // 237
+        bo    = in.child.off(first + idx);
+        eo    = in.child.off(first + next + 1);
         valid = true;
       }
     }
+    // The runs of these 64 elements overlap and lie side by side in the chars: fetch that stretch once, with
+    // coalesced loads, and hash out of LDS (the hash walks a run dword by dword, each step a dependent read).
+    // A stretch too long for the buffer is hashed straight from memory.
+    int64_t const span_begin = in.child.off(first + base);
+    int64_t const span_end   = in.child.off(first + min(base + kWave + ngrams, n));
+    if (span_end - span_begin <= static_cast<int64_t>(kNgramStageBytes)) {
+      bool ascii;
+      uint32_t const mis = stage_bytes(in.child.chars, span_begin, static_cast<uint32_t>(span_end - span_begin), run_bytes[wave], lane, &ascii);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (valid) {
+        WordSrc const src{run_bytes[wave], mis + static_cast<uint32_t>(bo - span_begin)};
+        hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    } else if (valid) {
+      AlignedSrc const src(in.child.chars + bo, static_cast<uint32_t>(eo - bo));
+      hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+    }
+    if (valid) hv = hv < 1 ? T{1} : hv;  // 237
     uint64_t const vm = ballot64(valid);
     if (valid) lds[wave].hashes[lanes_below(vm)] = hv;
     fold_hashes<T, K>(lds[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
