@@ -129,6 +129,13 @@ def test_normalize_malformed_utf8(nv, onorm, do_lower):
     rows = [bytes(rng.integers(0, 256, rng.integers(0, 40), dtype=np.uint8)) for _ in range(200)]
     rows += [b"abc\xe4", b"\xf0\x9f", b"\xc3", b"\xf8\x80\x80\x80z", b"\xf4\x90\x80\x80", b"\xed\xa0\x80", b"\x80\x80a"]
     check(nv, onorm, strings(rows), do_lower, ["[PAD]"], "random bytes")
+    # more than four output bytes per input byte (a first byte that swallows ASCII into a Hangul syllable, which then
+    # decomposes, and the swallowed bytes count once more on their own): the tile's output no longer fits the LDS
+    # staging and is written byte by byte
+    rows = [b"\xea\x30\x21" * 2000, b"ab" + b"\xea\x30\x21" * 700 + b"cd", b"plain"]
+    got = check(nv, onorm, strings(rows), do_lower, (), "expansion beyond the staging buffer")
+    if do_lower:
+        assert got.chars.size > 4 * sum(len(r) for r in rows[:2])
     # over-long encodings of '[' decode to it and open a special token like the plain byte does
     for opener in (b"\xc1\x9b", b"\xe0\x81\x9b", b"\xf0\x80\x81\x9b", b"\xc1\x1b"):
         for shift in range(0, 9):
