@@ -156,6 +156,10 @@ def test_normalize_nulls_keep_their_bytes_and_empty_shapes(nv, onorm):
     # empty column
     got = run(nv, strings([]), False)
     assert got.size == 0 and got.offsets.size == 0 and got.chars.size == 0
+    # thousands of empty rows that all start at one byte position, before, between and after the text
+    rows = [""] * 3000 + ["Ab, c"] + [""] * 2500 + ["D!"] + [""] * 1000
+    got = check(nv, onorm, strings(rows), True)
+    assert got.offsets[3000] == 0 and got.offsets[3001] == 7 and got.offsets[-1] == 7 + 4
     # sliced view whose first offset is not 0, int64 offsets
     host = strings(["skip me", "Keep, THIS", "and\tthis"], np.int64).slice(1, 3)
     assert check(nv, onorm, host, True).to_pylist() == [b"keep ,  this", b"and this"]
