@@ -223,7 +223,88 @@ __device__ __forceinline__ void wide_slots(uint32_t w, NormTables const& t, uint
   slots_of(decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
 }
 
-// One tile: the slots of the lane's positions, special tokens applied.  Returns the bytes they produce.
+__device__ __forceinline__ uint32_t utf8_length(uint32_t cp) { return 1u + (cp > 0x7Fu) + (cp > 0x7FFu) + (cp > 0xFFFFu); }
+
+// Bytes that the character whose bytes start `w` produces: slots_of without building the slots.
+__device__ __forceinline__ uint32_t wide_size(uint32_t w, NormTables const& t)
+{
+  uint32_t const cp  = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
+  uint32_t const e   = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
+  uint32_t const cat = (e >> 24) & 7u;
+  bool const lower   = t.do_lower != 0;
+  if (cat == kRemove || (lower && cat == kRemoveIfLower)) return 0u;
+  uint32_t const repl = (lower || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
+  uint32_t const r0   = repl ? repl : cp;
+  if (lower && ((e >> 23) & 1u)) {
+    uint64_t const next = t.second[cp];
+    uint32_t const r1 = static_cast<uint32_t>(next >> 32), r2 = static_cast<uint32_t>(next);
+    return utf8_length(r0) + (r1 ? utf8_length(r1) : 0u) + (r2 ? utf8_length(r2) : 0u);
+  }
+  return utf8_length(r0) + ((cat == kPad || (lower && cat == kPadIfLower)) ? 2u : 0u);
+}
+
+// The slots (and sizes) of the eight positions whose bytes are lo64; hi64 = bytes 4..11.  Returns the bytes they produce.
+__device__ __forceinline__ uint32_t owned_slots(NormLds const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t, Owned& mine,
+                                                uint32_t (&size)[kNormItems])
+{
+  uint32_t sum = 0;
+  // one-byte characters through the table; continuation bytes give nothing
+#pragma unroll
+  for (int j = 0; j < kNormItems; ++j) {
+    uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
+    uint32_t const e = lds.ascii[b & 0x7Fu];  // read in any case: no branch
+    uint32_t const d = b < 0x80u ? e : 0u;
+    mine.s[j][0]     = d & 0xFFu;
+    mine.s[j][1]     = (d >> 8) & 0xFFu;
+    mine.s[j][2]     = (d >> 16) & 0xFFu;
+    size[j]          = d >> 24;
+    sum += size[j];
+  }
+  // each first byte of a longer character (seldom more than four in eight bytes) goes through the code point tables
+  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;  // bit 7 of the bytes >= 0xC0
+  while (leads) {
+    int const at = (__ffsll(static_cast<long long>(leads)) - 1) >> 3;
+    leads &= leads - 1ull;
+    uint32_t const w = static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3)));
+    uint32_t s0, s1, s2;
+    wide_slots(w, t, s0, s1, s2);
+    uint32_t const bytes = bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+    sum += bytes;
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+      if (j == at) {
+        mine.s[j][0] = s0;
+        mine.s[j][1] = s1;
+        mine.s[j][2] = s2;
+        size[j]      = bytes;
+      }
+    }
+  }
+  return sum;
+}
+
+// The same count without the slots, for the pass that only sizes the output.
+__device__ __forceinline__ uint32_t owned_size(NormLds const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t)
+{
+  uint32_t sum = 0;
+#pragma unroll
+  for (int j = 0; j < kNormItems; ++j) {
+    uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
+    uint32_t const e = lds.ascii[b & 0x7Fu];
+    sum += b < 0x80u ? e >> 24 : 0u;
+  }
+  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;
+  while (leads) {
+    int const at = (__ffsll(static_cast<long long>(leads)) - 1) >> 3;
+    leads &= leads - 1ull;
+    sum += wide_size(static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3))), t);
+  }
+  return sum;
+}
+
+// One tile: the slots of the lane's positions, special tokens applied.  Returns the bytes they produce.  Without
+// SLOTS only that number is wanted: the slots are then built only in tiles that may hold a special token.
+template <bool SLOTS>
 __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t, Owned& mine,
                                                uint32_t (&size)[kNormItems])
 {
@@ -264,51 +345,24 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
   uint32_t const own1 = __builtin_amdgcn_alignbit(r2, r1, shift);
   uint32_t const next = __builtin_amdgcn_alignbit(r3, r2, shift);
   uint64_t const lo64 = (static_cast<uint64_t>(own1) << 32) | own0;
-  uint32_t sum        = 0;
-  // one-byte characters through the table; continuation bytes give nothing
-#pragma unroll
-  for (int j = 0; j < kNormItems; ++j) {
-    uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
-    uint32_t const e = lds.ascii[b & 0x7Fu];  // read in any case: no branch
-    uint32_t const d = b < 0x80u ? e : 0u;
-    mine.s[j][0]     = d & 0xFFu;
-    mine.s[j][1]     = (d >> 8) & 0xFFu;
-    mine.s[j][2]     = (d >> 16) & 0xFFu;
-    size[j]          = d >> 24;
-    sum += size[j];
-  }
-  // each first byte of a longer character (seldom more than four in eight bytes) goes through the code point tables
-  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;  // bit 7 of the bytes >= 0xC0
-  if (leads) {
-    uint64_t const hi64 = (static_cast<uint64_t>(next) << 32) | own1;
-    do {
-      int const at = (__ffsll(static_cast<long long>(leads)) - 1) >> 3;
-      leads &= leads - 1ull;
-      uint32_t const w = static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3)));
-      uint32_t s0, s1, s2;
-      wide_slots(w, t, s0, s1, s2);
-      uint32_t const bytes = bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
-      sum += bytes;
-#pragma unroll
-      for (int j = 0; j < kNormItems; ++j) {
-        if (j == at) {
-          mine.s[j][0] = s0;
-          mine.s[j][1] = s1;
-          mine.s[j][2] = s2;
-          size[j]      = bytes;
-        }
-      }
-    } while (leads);
-  }
+  uint64_t const hi64 = (static_cast<uint64_t>(next) << 32) | own1;
+  uint32_t sum        = SLOTS ? owned_slots(lds, lo64, hi64, t, mine, size) : owned_size(lds, lo64, hi64, t);
 
   if (t.tokens > 0) {
     // A special token starts at a position whose slot 1 is '['.  Tiles without one skip the exchange through LDS.
-    // For the positions before the tile (eight looked at, five needed) the bytes decide: a '[', or one of the
-    // first bytes 0xC1, 0xE0, 0xF0 with which an over-long encoding of '[' would start (no other code point's
-    // replacement is a '[').
+    // No code point's replacement is a '[', so it takes a '[' byte or an over-long encoding of it, which starts
+    // with 0xC1, 0xE0 or 0xF0: that is what decides for the positions before the tile (eight looked at, five
+    // needed) and, when the slots have not been built, for the lane's own bytes (a superset, which is harmless).
     bool bracket = false;
+    if (SLOTS) {
 #pragma unroll
-    for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
+      for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
+    } else {
+      bracket = has_byte(own0, '[') || has_byte(own1, '[');
+      if ((lo64 & (lo64 << 1) & 0x8080808080808080ull) != 0)
+        bracket = bracket || has_byte(own0, 0xC1u) || has_byte(own0, 0xE0u) || has_byte(own0, 0xF0u) || has_byte(own1, 0xC1u) ||
+                  has_byte(own1, 0xE0u) || has_byte(own1, 0xF0u);
+    }
     if (tid < 2) {
       int const at     = static_cast<int>(mis >> 2) + tid;
       uint32_t const v = __builtin_amdgcn_alignbit(lds.raw[at + 1], lds.raw[at], shift);
@@ -317,6 +371,7 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
     if (ballot64(bracket) != 0 && lane_id() == 0) lds.bracket = 1u;
     lds_barrier();
     if (lds.bracket != 0u) {
+      if (!SLOTS) owned_slots(lds, lo64, hi64, t, mine, size);
 #pragma unroll
       for (int k = 0; k < 3; ++k) {
         uint32_t a = 0, b = 0;
@@ -385,7 +440,7 @@ __global__ void __launch_bounds__(kNormThreads, 8) normalize_count_kernel(const 
   int64_t const t0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
   Owned mine;
   uint32_t size[kNormItems];
-  uint32_t const sum = tile_slots(lds, chars, t0, n, t, mine, size);
+  uint32_t const sum = tile_slots<false>(lds, chars, t0, n, t, mine, size);
   uint32_t total;
   block_exclusive_scan_lds<kNormThreads>(sum, lds.scan, &total);
   if (threadIdx.x == 0) tile_bytes[blockIdx.x] = total;
@@ -434,7 +489,7 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   }
   Owned mine;
   uint32_t size[kNormItems];
-  uint32_t const sum = tile_slots(lds, col.chars + first, t0, n, t, mine, size);
+  uint32_t const sum = tile_slots<true>(lds, col.chars + first, t0, n, t, mine, size);
   uint32_t total;
   uint32_t const before = block_exclusive_scan_lds<kNormThreads>(sum, lds.scan, &total);
   {
