@@ -18,6 +18,7 @@ struct nvtext_amd_character_normalizer {
   int device            = 0;
   int32_t do_lower      = 0;
   uint32_t* ascii       = nullptr;  // device, 128: slot 0 | slot 1 << 8 | slot 2 << 16 | bytes << 24 of the code points below 0x80
+  uint4* bmp            = nullptr;  // device, 65536: {slot 0, slot 1, slot 2, bytes} of the code points below 0x10000
   uint32_t* entries     = nullptr;  // device, kCodepoints: category << 24 | multi << 23 | replacement
   uint64_t* second      = nullptr;  // device, kCodepoints: second << 32 | third replacement code point
   uint8_t* token_chars  = nullptr;  // device: the special tokens, sorted then lower-cased
@@ -50,6 +51,7 @@ constexpr int kStageBytes  = 4 * kNormTile;  // output bytes of a tile that are 
 
 struct NormTables {
   const uint32_t* ascii;  // 128 entries: the slots of the code points below 0x80
+  const uint4* bmp;       // 65536 entries: the three slots and their bytes together, of the code points below 0x10000
   const uint32_t* entries;
   const uint64_t* second;
   const uint8_t* token_chars;
@@ -60,7 +62,7 @@ struct NormTables {
 
 // cudf::strings::detail::codepoint_to_utf8 then from_char_utf8 (cpp/include/cudf/strings/detail/utf8.hpp:170-197,
 // 143-168): the bytes of the character, first byte in the low bits, as the reference leaves them in a slot.
-__device__ __forceinline__ uint32_t utf8_le(uint32_t cp)
+__host__ __device__ __forceinline__ uint32_t utf8_le(uint32_t cp)
 {
   if (cp < 0x80u) return cp;
   uint32_t const t0 = 0x80u | (cp & 0x3Fu);
@@ -71,7 +73,14 @@ __device__ __forceinline__ uint32_t utf8_le(uint32_t cp)
   return (0xF0u | ((cp >> 18) & 0x07u)) | (t2 << 8) | (t1 << 16) | (t0 << 24);
 }
 
-__device__ __forceinline__ uint32_t bytes_of(uint32_t slot) { return (39u - static_cast<uint32_t>(__clz(slot))) >> 3; }
+__host__ __device__ __forceinline__ uint32_t bytes_of(uint32_t slot)
+{
+#ifdef __HIP_DEVICE_COMPILE__
+  return (39u - static_cast<uint32_t>(__clz(slot))) >> 3;
+#else
+  return (slot != 0) + (slot > 0xFFu) + (slot > 0xFFFFu) + (slot > 0xFFFFFFu);
+#endif
+}
 
 // The code point of the character that starts with b0, the next bytes being b1..b3
 // (to_char_utf8 and utf8_to_codepoint, cpp/include/cudf/strings/detail/utf8.hpp:68-97,118-140: the first byte
@@ -88,7 +97,7 @@ __device__ __forceinline__ uint32_t decode(uint32_t b0, uint32_t b1, uint32_t b2
 }
 
 // The slots of one code point (data_normalizer_kernel, cpp/src/text/normalize.cu:331-378).
-__device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
+__host__ __device__ __forceinline__ void slots_of(uint32_t cp, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
 {
   s0 = s1 = s2       = 0;
   uint32_t const e   = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
@@ -217,30 +226,30 @@ __device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
   lds_barrier();
 }
 
-// Slots of the character whose bytes start `w` (first byte in the low bits), through the code point tables.
-__device__ __forceinline__ void wide_slots(uint32_t w, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
+// Slots of the character whose bytes start `w` (first byte in the low bits) and the bytes they hold together.  The
+// Basic Multilingual Plane has them ready in one 16-byte table entry; the rest goes through the code point tables.
+__device__ __forceinline__ uint32_t wide_slots(uint32_t w, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
 {
-  slots_of(decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24), t, s0, s1, s2);
+  uint32_t const cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
+  if (cp < 0x10000u) {
+    uint4 const e = t.bmp[cp];
+    s0            = e.x;
+    s1            = e.y;
+    s2            = e.z;
+    return e.w;
+  }
+  slots_of(cp, t, s0, s1, s2);
+  return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
 }
 
-__device__ __forceinline__ uint32_t utf8_length(uint32_t cp) { return 1u + (cp > 0x7Fu) + (cp > 0x7FFu) + (cp > 0xFFFFu); }
-
-// Bytes that the character whose bytes start `w` produces: slots_of without building the slots.
+// Bytes that the character whose bytes start `w` produces, without its slots.
 __device__ __forceinline__ uint32_t wide_size(uint32_t w, NormTables const& t)
 {
-  uint32_t const cp  = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
-  uint32_t const e   = cp < kCodepoints ? t.entries[cp] : kDefaultEntry;
-  uint32_t const cat = (e >> 24) & 7u;
-  bool const lower   = t.do_lower != 0;
-  if (cat == kRemove || (lower && cat == kRemoveIfLower)) return 0u;
-  uint32_t const repl = (lower || cat == kReplace) ? (e & 0x1FFFFFu) : cp;
-  uint32_t const r0   = repl ? repl : cp;
-  if (lower && ((e >> 23) & 1u)) {
-    uint64_t const next = t.second[cp];
-    uint32_t const r1 = static_cast<uint32_t>(next >> 32), r2 = static_cast<uint32_t>(next);
-    return utf8_length(r0) + (r1 ? utf8_length(r1) : 0u) + (r2 ? utf8_length(r2) : 0u);
-  }
-  return utf8_length(r0) + ((cat == kPad || (lower && cat == kPadIfLower)) ? 2u : 0u);
+  uint32_t const cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
+  if (cp < 0x10000u) return t.bmp[cp].w;
+  uint32_t s0, s1, s2;
+  slots_of(cp, t, s0, s1, s2);
+  return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
 }
 
 // The slots (and sizes) of the eight positions whose bytes are lo64; hi64 = bytes 4..11.  Returns the bytes they produce.
@@ -267,8 +276,7 @@ __device__ __forceinline__ uint32_t owned_slots(NormLds const& lds, uint64_t lo6
     leads &= leads - 1ull;
     uint32_t const w = static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3)));
     uint32_t s0, s1, s2;
-    wide_slots(w, t, s0, s1, s2);
-    uint32_t const bytes = bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+    uint32_t const bytes = wide_slots(w, t, s0, s1, s2);
     sum += bytes;
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) {
@@ -735,6 +743,17 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
     ascii[cp] = d;
   }
 
+  // the finished slots of the Basic Multilingual Plane (the rules of slots_of, run here once per code point)
+  std::vector<uint4> bmp(0x10000);
+  {
+    NormTables const host_tables{nullptr, nullptr, entries.data(), second.data(), nullptr, nullptr, 0, do_lower_case ? 1 : 0};
+    for (uint32_t cp = 0; cp < 0x10000u; ++cp) {
+      uint32_t s0, s1, s2;
+      slots_of(cp, host_tables, s0, s1, s2);
+      bmp[cp] = make_uint4(s0, s1, s2, bytes_of(s0) + bytes_of(s1) + bytes_of(s2));
+    }
+  }
+
   auto* obj      = new nvtext_amd_character_normalizer();
   obj->do_lower  = do_lower_case ? 1 : 0;
   obj->tokens    = static_cast<int32_t>(tokens.size());
@@ -745,6 +764,8 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
   hipError_t e = hipGetDevice(&obj->device);
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->ascii), sizeof(ascii));
   if (e == hipSuccess) e = hipMemcpy(obj->ascii, ascii, sizeof(ascii), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->bmp), bmp.size() * sizeof(uint4));
+  if (e == hipSuccess) e = hipMemcpy(obj->bmp, bmp.data(), bmp.size() * sizeof(uint4), hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->entries), entries.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->second), second.size() * sizeof(uint64_t));
   if (e == hipSuccess) e = hipMemcpy(obj->entries, entries.data(), entries.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
@@ -775,6 +796,7 @@ void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* no
 {
   if (!normalizer) return;
   (void)hipFree(normalizer->ascii);
+  (void)hipFree(normalizer->bmp);
   (void)hipFree(normalizer->entries);
   (void)hipFree(normalizer->second);
   (void)hipFree(normalizer->token_chars);
@@ -848,7 +870,7 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   Temp scan_temp(mr, scan_temp_bytes(tiles));
   Temp tile_row(mr, static_cast<size_t>(tiles) * sizeof(int32_t));
   if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok() || !tile_row.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-  NormTables const tables{normalizer->ascii, normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
+  NormTables const tables{normalizer->ascii, normalizer->bmp, normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
                           normalizer->do_lower};
   ColView const view = make_view(*input);
   {
