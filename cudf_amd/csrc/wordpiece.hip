@@ -939,47 +939,33 @@ struct ShortWord {
     bnd >>= l;
   }
 
-  // One trip: probes the two longest remaining candidates of three bytes and more (their table reads are in
-  // flight together); when none of those is left, the candidates of two bytes and of one byte are settled
-  // from the ids fetched when the piece was opened, without hashing or further reads.
+  // One trip: probes the longest remaining candidate of three bytes and more; when none of those is left, the
+  // candidates of two bytes and of one byte are settled from the ids fetched when the piece was opened, without
+  // hashing or further reads.  (The length filter leaves few candidates: a piece that has any has 1.4 on average,
+  // so a second probe in the same trip would mostly be wasted work.)
   template <typename Emit>
   __device__ __forceinline__ void step(VocabTable const& t, Emit&& emit)
   {
     uint32_t const kind   = count ? 1u : 0u;
     uint32_t const longer = cand & ~3u;
     bool const has_a      = longer != 0;
-    uint32_t const c1     = has_a ? longer : 4u;
-    uint32_t const la     = 32u - static_cast<uint32_t>(__builtin_clz(c1));
-    uint32_t const rest   = c1 ^ (1u << (la - 1));
-    bool const has_b      = has_a && rest != 0;
-    uint32_t const lb     = has_b ? 32u - static_cast<uint32_t>(__builtin_clz(rest)) : 3u;
-    bool hit_a = false, hit_b = false;
-    int32_t ida = kNone, idb = kNone;
+    uint32_t const la     = 32u - static_cast<uint32_t>(__builtin_clz(has_a ? longer : 4u));
+    bool hit_a            = false;
+    int32_t ida           = kNone;
     if (has_a) {
       Probe const pa = probe_of(t, kind, la);
-      Probe const pb = probe_of(t, kind, lb);
       uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
-      uint4 const b0 = t.slots[2 * pb.bucket], b1 = t.slots[2 * pb.bucket + 1];
-      uint32_t va = verdict(pa, a0, a1, la, &ida);
-      uint32_t vb = verdict(pb, b0, b1, lb, &idb);
-      if (va == 2u || (va == 0u && has_b && vb == 2u)) {
-        // the general lookup (keys in the pool, overflowing buckets)
-        if (va == 2u) {
-          ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
-          va  = ida == kNone ? 0u : 1u;
-        }
-        if (va == 0u && vb == 2u) {
-          idb = finish_probe(t, pb, b0, b1, *this, 0u, lb);
-          vb  = idb == kNone ? 0u : 1u;
-        }
+      uint32_t va    = verdict(pa, a0, a1, la, &ida);
+      if (va == 2u) {  // the general lookup (keys in the pool, overflowing buckets)
+        ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
+        va  = ida == kNone ? 0u : 1u;
       }
       hit_a = va == 1u;
-      hit_b = !hit_a && has_b && vb == 1u;
     }
-    uint32_t const longer_left = has_b ? rest ^ (1u << (lb - 1)) : 0u;  // after two misses
-    bool hit     = hit_a || hit_b;
-    uint32_t len = hit_a ? la : lb;
-    int32_t id   = hit_a ? ida : idb;
+    uint32_t const longer_left = has_a ? longer ^ (1u << (la - 1)) : 0u;  // after a miss
+    bool hit     = hit_a;
+    uint32_t len = la;
+    int32_t id   = ida;
     bool unknown = false;
     if (!hit && longer_left == 0) {
       // two bytes, then one byte; else no prefix of the word matched (375-379), or a later piece has no match and
