@@ -323,15 +323,18 @@ def main():
                                                     "traffic": None}}
         if not args.no_cpu:
             from oracle import normalize_py
-            n = 4000
+            from oracle import pyoracle as orc
+            threads = max(1, min(orc.hardware_threads(), 16))
+            normalize_py.rule_tables()  # built once, outside the timed part (the library's tables are built at create time)
+            n = min(w.rows.size, 400000)
             smp = w.rows.slice(0, n)
             t0 = time.perf_counter()
-            exp = normalize_py.normalize_characters(smp, True, [b"[CLS]", b"[SEP]", b"[PAD]", b"[MASK]", b"[UNK]"])
+            exp = normalize_py.normalize_characters_native(smp, True, [b"[CLS]", b"[SEP]", b"[PAD]", b"[MASK]", b"[UNK]"], nthreads=threads)
             cs = time.perf_counter() - t0
             got = nvtext.normalize_characters(dc.slice(0, n, smp.null_count), normalizer).to_host()
             leg["normalize_characters"]["cpu_baseline"] = {
-                "value": round(input_bytes(smp) / cs / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.2f} MB), {cs:.2f} s, pure-Python restatement"}
+                "value": round(input_bytes(smp) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB), {cs:.2f} s"}
             same = np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets)
             leg["normalize_characters"]["parity"] = "PASS" if same else "FAIL"
         keep.clear()

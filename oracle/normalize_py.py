@@ -194,6 +194,57 @@ def normalize_characters(col, do_lower_case: bool, special_tokens: Sequence[byte
     return HostStringsColumn(chars, out_off, copy_bitmask(col), col.size, 0, col.null_count)
 
 
+_RULES = None
+
+
+def rule_tables():
+    """classify() of every code point as two arrays for oracle/nvtext_oracle.cpp: kind[cp] and lower[3 * cp + k]
+    (the characters cp becomes when lower-casing, 0 = none).  Unassigned code points are all alike, so only the
+    assigned ones go through classify()."""
+    global _RULES
+    if _RULES is None:
+        kind = np.full(0x110000, PLAIN, np.uint8)
+        lower = np.zeros((0x110000, 3), np.uint32)
+        lower[:, 0] = np.arange(0x110000, dtype=np.uint32)
+        plain_unassigned = classify(0x0378) == (PLAIN, [0x0378])  # an unassigned code point
+        assert plain_unassigned
+        for cp in range(0x110000):
+            if unicodedata.category(chr(cp)) == "Cn" and not _cjk(cp):
+                continue
+            k, low = classify(cp)
+            kind[cp] = k
+            lower[cp, :] = 0
+            lower[cp, :len(low)] = low
+        _RULES = (kind, np.ascontiguousarray(lower.reshape(-1)))
+    return _RULES
+
+
+def normalize_characters_native(col, do_lower_case: bool, special_tokens: Sequence[bytes] = (), nthreads: int = 1):
+    """normalize_characters through the C++ restatement in oracle/nvtext_oracle.cpp (same rules, from rule_tables()):
+    for inputs too large for the loops above.  Tests hold the two against each other."""
+    import ctypes as C
+    from cudf_amd.arrow_host import HostStringsColumn
+    from oracle import pyoracle
+    if col.size == 0:
+        return HostStringsColumn(np.zeros(0, np.uint8), np.zeros(0, np.int32), None, 0, 0, 0)
+    kind, lower = rule_tables()
+    tokens = sorted_special_tokens(special_tokens, do_lower_case)
+    tok_chars = np.frombuffer(b"".join(tokens) or b"\0", dtype=np.uint8).copy()
+    tok_off = np.concatenate([[0], np.cumsum([len(t) for t in tokens])]).astype(np.int32)
+    keep, cargs = pyoracle._col_args(col)
+    out_off = np.zeros(col.size + 1, np.int64)
+    out_chars, out_bytes = C.c_void_p(), C.c_int64(0)
+    rc = pyoracle.lib().oracle_normalize_characters(*cargs, pyoracle._p(kind), pyoracle._p(lower), int(bool(do_lower_case)),
+                                                     pyoracle._p(tok_chars), pyoracle._p(tok_off), len(tokens), int(nthreads),
+                                                     pyoracle._p(out_off), C.byref(out_chars), C.byref(out_bytes))
+    if rc != pyoracle.OK:
+        raise pyoracle.OracleError(rc)
+    n = out_bytes.value
+    chars = np.ctypeslib.as_array(C.cast(out_chars, C.POINTER(C.c_uint8)), shape=(max(n, 1),))[:n].copy()
+    pyoracle.lib().oracle_free(out_chars)
+    return HostStringsColumn(chars, out_off.astype(_offsets_dtype(n)), pyoracle.copy_bitmask(col), col.size, 0, col.null_count)
+
+
 def normalize_ascii(col, do_lower_case: bool):
     """normalize_characters for a column whose bytes are all below 0x80, no special tokens: the same rules through a
     256-entry table and numpy, for inputs too large for the loops above.  Tests check it against

@@ -1,7 +1,7 @@
 // nvtext_oracle.cpp -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
 //
-// Scalar host restatement of libcudf's nvtext::minhash / minhash64 /
-// wordpiece_tokenize (+ wordpiece_vocabulary) semantics.  It exists only to
+// Scalar host restatement of libcudf's nvtext::minhash / minhash64 (+ _ngrams) /
+// jaccard_index / wordpiece_tokenize (+ wordpiece_vocabulary) / normalize_characters semantics.  It exists only to
 // check the HIP implementation (tests, the smoke check and the bench's
 // cpu_baseline leg); the product library never links or loads it.
 //
@@ -13,7 +13,7 @@
 // published algorithm.
 //
 // Parity status: every function below is pinned by the reference's own test
-// vectors (tests/test_oracle_golden.py); two behaviours are pinned by code
+// vectors (tests/test_oracle_golden.py, tests/test_normalize_oracle.py); two behaviours are pinned by code
 // reading only -- the size_bytes/2 word cap and validity being ignored when
 // max_words_per_row == 0 -- and one reference behaviour is racy and therefore
 // unpinnable: rows ending in >= 2 spaces with max_words_per_row > 0.  For that
@@ -568,6 +568,180 @@ inline void tokenize_row(Vocab const& v, uint8_t const* s, int64_t n, bool valid
   }
 }
 
+// ---------------------------------------------------------------------------
+// normalize_characters -- cpp/src/text/normalize.cu:331-388 (per-character replacement into three
+// slots per input byte), 270-316 (special tokens), 491-561 (flat pass over the column's chars).
+// The per-code-point rules are data here: oracle/normalize_py.py works them out (classify) and
+// hands them over as two tables, so this file and that one state the algorithm twice (tests hold
+// them against each other and against the reference's vectors) over ONE statement of the rules.
+// ---------------------------------------------------------------------------
+enum : uint8_t { N_PAD = 0, N_PAD_IF_LOWER = 1, N_REMOVE = 2, N_REMOVE_IF_LOWER = 3, N_REPLACE = 4, N_PLAIN = 5 };
+constexpr uint32_t n_codepoints = 0x110000;
+
+struct NormRules {
+  uint8_t const* kind;    // n_codepoints entries
+  uint32_t const* lower;  // 3 per code point: what it becomes when lower-casing (0 = no further character)
+  bool do_lower;
+  std::vector<std::string> tokens;  // sorted by bytes, then lower-cased (normalize.cu:230-235): maybe not in order
+};
+
+// cpp/include/cudf/strings/detail/utf8.hpp:68-97,118-140: the first byte alone says how many bytes are read,
+// the magnitude of the packed value picks the decoding.  Bytes past the end read as 0.
+inline uint32_t norm_decode(uint8_t const* d, int64_t n, int64_t i)
+{
+  uint8_t const b0 = d[i];
+  int const len    = 1 + (b0 >= 0xC0) + (b0 >= 0xE0) + (b0 >= 0xF0);
+  uint32_t packed  = 0;
+  for (int k = 0; k < len; ++k) packed = (packed << 8) | (i + k < n ? d[i + k] : 0u);
+  if (packed < 0x80u) return packed;
+  if (packed < 0xE000u) return ((packed & 0x1F00u) >> 2) | (packed & 0x3Fu);
+  if (packed < 0xF00000u) return ((packed & 0x0F0000u) >> 4) | ((packed & 0x3F00u) >> 2) | (packed & 0x3Fu);
+  if (packed <= 0xF8000000u)
+    return ((packed & 0x07000000u) >> 6) | ((packed & 0x3F0000u) >> 4) | ((packed & 0x3F00u) >> 2) | (packed & 0x3Fu);
+  return 0;
+}
+
+// cudf::strings::detail::codepoint_to_utf8 (utf8.hpp:170-197); returns the number of bytes put at out
+inline int norm_encode(uint32_t cp, uint8_t* out)
+{
+  if (cp < 0x80u) {
+    out[0] = uint8_t(cp);
+    return 1;
+  }
+  if (cp < 0x800u) {
+    out[0] = uint8_t(0xC0u | (cp >> 6));
+    out[1] = uint8_t(0x80u | (cp & 0x3Fu));
+    return 2;
+  }
+  if (cp < 0x10000u) {
+    out[0] = uint8_t(0xE0u | (cp >> 12));
+    out[1] = uint8_t(0x80u | ((cp >> 6) & 0x3Fu));
+    out[2] = uint8_t(0x80u | (cp & 0x3Fu));
+    return 3;
+  }
+  out[0] = uint8_t(0xF0u | ((cp >> 18) & 0x07u));
+  out[1] = uint8_t(0x80u | ((cp >> 12) & 0x3Fu));
+  out[2] = uint8_t(0x80u | ((cp >> 6) & 0x3Fu));
+  out[3] = uint8_t(0x80u | (cp & 0x3Fu));
+  return 4;
+}
+
+// normalize.cu:331-378: the three slots (code points, 0 = empty) of the character that starts at byte i
+inline void norm_slots(NormRules const& r, uint8_t const* d, int64_t n, int64_t i, uint32_t* s)
+{
+  s[0] = s[1] = s[2] = 0;
+  if ((d[i] & 0xC0u) == 0x80u) return;
+  uint32_t const cp = norm_decode(d, n, i);
+  uint8_t const k   = cp < n_codepoints ? r.kind[cp] : uint8_t(N_PLAIN);
+  if (k == N_REMOVE || (r.do_lower && k == N_REMOVE_IF_LOWER)) return;
+  uint32_t out[3] = {cp, 0, 0};
+  if (k == N_REPLACE) {
+    out[0] = 0x20;
+  } else if (r.do_lower && cp < n_codepoints) {
+    for (int j = 0; j < 3; ++j) out[j] = r.lower[3 * size_t(cp) + j];
+  }
+  if ((k == N_PAD || (r.do_lower && k == N_PAD_IF_LOWER)) && out[1] == 0) {
+    s[0] = 0x20;
+    s[1] = out[0];
+    s[2] = 0x20;
+  } else {
+    s[0] = out[0];
+    s[1] = out[1];
+    s[2] = out[2];
+  }
+}
+
+inline uint8_t norm_first_byte(uint32_t cp)
+{
+  uint8_t b[4];
+  norm_encode(cp, b);
+  return b[0];
+}
+
+// thrust::binary_search over tokens that need not be in order (normalize.cu:299): lower_bound by halving,
+// then "not value < *it"
+inline bool norm_is_token(NormRules const& r, std::string const& v)
+{
+  size_t first = 0, count = r.tokens.size();
+  while (count > 0) {
+    size_t const half = count >> 1;
+    if (r.tokens[first + half] < v) {
+      first += half + 1;
+      count -= half + 1;
+    } else {
+      count = half;
+    }
+  }
+  return first < r.tokens.size() && !(v < r.tokens[first]);
+}
+
+// special_tokens_kernel (normalize.cu:270-316) for the '[' in slot 1 of position i; the slots of the positions
+// from lo on are at base (3 each), n = bytes in the column
+inline void norm_special_token(NormRules const& r, uint32_t* base, int64_t lo, int64_t i, int64_t n)
+{
+  auto slot = [&](int64_t j, int k) -> uint32_t* { return base + 3 * (j - lo) + k; };
+  int64_t const span = std::min<int64_t>(6, n - i);
+  // the slots after the one holding '[': `span` positions' worth (normalize.cu:286), ending with slot 0 of
+  // position i + span when there is one
+  uint32_t* seq[20];
+  int m    = 0;
+  seq[m++] = slot(i, 1);
+  seq[m++] = slot(i, 2);
+  for (int64_t j = i + 1; j < i + span; ++j)
+    for (int k = 0; k < 3; ++k) seq[m++] = slot(j, k);
+  if (i + span < n) seq[m++] = slot(i + span, 0);
+  int close = -1;
+  for (int p = 0; p < m; ++p) {
+    if (*seq[p] == ']') {
+      close = p;
+      break;
+    }
+  }
+  if (close < 0) return;
+  std::string cand;  // one byte per character, its first (normalize.cu:289-294 narrows each slot to a char)
+  for (int p = 0; p <= close; ++p)
+    if (*seq[p] != 0 && *seq[p] != 0x20) cand.push_back(char(norm_first_byte(*seq[p])));
+  if (!norm_is_token(r, cand)) return;
+  *seq[1]         = 0;  // the space after '['
+  *seq[close - 1] = 0;  // the space before ']'
+  if (r.do_lower)
+    for (int p = 2; p < close - 2; ++p)
+      if (*seq[p] >= 'a' && *seq[p] <= 'z') *seq[p] -= 32;
+}
+
+// Bytes [b, e) of the flat chars: appends their output to `out` and sets prefix_at[r - row_lo] = bytes of output
+// before the first byte of row r, for the rows r in [row_lo, row_hi) (those that start in [b, e)).
+// Done in blocks; the '[' of up to `reach` positions before a block are looked at as well, because what they change
+// reaches into it; what a '[' still further back changed in THEIR windows is not seen (only nested brackets could tell).
+void norm_range(NormRules const& r, uint8_t const* d, int64_t n, int64_t b, int64_t e, StringsCol const& c, int64_t first,
+                int32_t row_lo, int32_t row_hi, std::vector<uint8_t>& out, int64_t* prefix_at)
+{
+  constexpr int64_t reach = 8, block = 1 << 15;  // in blocks, so that the slots stay in the cache
+  std::vector<uint32_t> slots(size_t(3 * (block + 2 * reach)));
+  out.reserve(size_t((e - b) + (e - b) / 8 + 64));
+  int32_t row = row_lo;
+  for (int64_t bb = b; bb < e; bb += block) {
+    int64_t const be = std::min(e, bb + block);
+    int64_t const lo = std::max<int64_t>(0, bb - reach), hi = std::min(n, be + reach);
+    for (int64_t i = lo; i < hi; ++i) norm_slots(r, d, n, i, &slots[size_t(3 * (i - lo))]);
+    if (!r.tokens.empty())
+      for (int64_t i = lo; i < be; ++i)
+        if (slots[size_t(3 * (i - lo) + 1)] == '[') norm_special_token(r, slots.data(), lo, i, n);
+    for (int64_t i = bb; i < be; ++i) {
+      while (row < row_hi && c.off(row) - first == i) prefix_at[row++ - row_lo] = int64_t(out.size());
+      for (int k = 0; k < 3; ++k) {
+        uint32_t const cp = slots[size_t(3 * (i - lo) + k)];
+        if (cp == 0) continue;
+        uint8_t buf[4];
+        int const nb = norm_encode(cp, buf);
+        out.insert(out.end(), buf, buf + nb);
+      }
+    }
+  }
+  while (row < row_hi) prefix_at[row++ - row_lo] = int64_t(out.size());
+}
+
+
 }  // namespace
 
 // ===========================================================================
@@ -721,6 +895,62 @@ int oracle_wordpiece_tokenize(void const* handle, uint8_t const* chars, void con
   }
   *out_tokens  = toks;
   *out_ntokens = total;
+  return OK;
+}
+
+// normalize.cu:491-561.  `kind` and `lower` are the rule tables (see NormRules); the special tokens come
+// sorted and, when lower-casing, lower-cased by the caller.  out_offsets: size + 1 entries of int64;
+// *out_chars is malloc'ed here and released with oracle_free.
+int oracle_normalize_characters(uint8_t const* chars, void const* offsets, int offsets_is_int64, uint32_t const* mask, int32_t size,
+                                int32_t offset, int32_t null_count, uint8_t const* kind, uint32_t const* lower, int do_lower,
+                                uint8_t const* token_chars, int32_t const* token_offsets, int32_t tokens, int nthreads,
+                                int64_t* out_offsets, uint8_t** out_chars, int64_t* out_bytes)
+{
+  *out_chars = nullptr;
+  *out_bytes = 0;
+  StringsCol c{chars, offsets, offsets_is_int64, mask, size, offset, null_count};
+  NormRules r{kind, lower, do_lower != 0, {}};
+  for (int32_t t = 0; t < tokens; ++t)
+    r.tokens.emplace_back(reinterpret_cast<char const*>(token_chars) + token_offsets[t], size_t(token_offsets[t + 1] - token_offsets[t]));
+  int64_t const first = c.off(0), n = c.off(size) - first;
+  uint8_t const* d    = chars + first;
+  int const nt        = int(std::max<int64_t>(1, std::min<int64_t>(nthreads, n / 4096)));
+  std::vector<std::vector<uint8_t>> parts(static_cast<size_t>(nt));
+  // rows by the part their first byte lies in; rows that start at the very end (and the end itself) go with the last part
+  std::vector<int32_t> row_lo(size_t(nt) + 1);
+  for (int t = 1; t < nt; ++t) {
+    int64_t const b = n * t / nt;
+    int32_t lo = 0, hi = size + 1;
+    while (lo < hi) {
+      int32_t const mid = lo + (hi - lo) / 2;
+      if (c.off(mid) - first < b) lo = mid + 1;
+      else hi = mid;
+    }
+    row_lo[size_t(t)] = lo;
+  }
+  row_lo[0]          = 0;
+  row_lo[size_t(nt)] = size + 1;
+  std::vector<std::thread> ts;
+  for (int t = 0; t < nt; ++t) {
+    ts.emplace_back([&, t] {
+      norm_range(r, d, n, n * t / nt, n * (t + 1) / nt, c, first, row_lo[size_t(t)], row_lo[size_t(t) + 1], parts[size_t(t)],
+                 out_offsets + row_lo[size_t(t)]);
+    });
+  }
+  for (auto& t : ts) t.join();
+  int64_t total = 0;
+  for (int t = 0; t < nt; ++t) {
+    for (int32_t row = row_lo[size_t(t)]; row < row_lo[size_t(t) + 1]; ++row) out_offsets[row] += total;
+    total += int64_t(parts[size_t(t)].size());
+  }
+  auto* bytes = static_cast<uint8_t*>(std::malloc(std::max<size_t>(size_t(total), 1)));
+  int64_t w   = 0;
+  for (auto const& p : parts) {
+    if (!p.empty()) std::memcpy(bytes + w, p.data(), p.size());
+    w += int64_t(p.size());
+  }
+  *out_chars = bytes;
+  *out_bytes = total;
   return OK;
 }
 

@@ -71,6 +71,9 @@ def lib():
         L.oracle_wordpiece_tokenize.restype = C.c_int
         L.oracle_wordpiece_tokenize.argtypes = [C.c_void_p] + col + [
             C.c_int32, C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int64), C.POINTER(C.c_int32)]
+        L.oracle_normalize_characters.restype = C.c_int
+        L.oracle_normalize_characters.argtypes = col + [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int32,
+                                                        C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int64)]
         L.oracle_free.restype = None
         L.oracle_free.argtypes = [C.c_void_p]
         L.oracle_copy_bitmask.restype = None

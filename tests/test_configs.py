@@ -14,6 +14,7 @@ import numpy as np
 import pytest
 
 from cudf_amd import datagen
+from cudf_amd.arrow_host import HostStringsColumn
 
 
 def _crc(col):
@@ -196,6 +197,25 @@ def test_config5_utf8_pipeline_full_size(nv, orc):
         assert torch.equal(_child(got), child[int(offs[lo]): int(offs[hi])]), f"C5 tokenize: slice {lo}:{hi} of the whole"
         assert np.array_equal(exp.offsets.astype(np.int64) + int(offs[lo]), offs[lo: hi + 1].astype(np.int64))
     del full, child
+    torch.cuda.empty_cache()
+    # normalize_characters of the whole column (the output passes 2 GiB: int64 offsets), exact against the oracle on
+    # row ranges, each also as a slice of the whole
+    from oracle import normalize_py
+    tokens = ["[CLS]", "[SEP]", "[PAD]", "[MASK]", "[UNK]"]
+    normalizer = nv.CharacterNormalizer(True, nv.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(tokens)))
+    whole = nv.normalize_characters(d, normalizer)
+    assert whole.offsets.dtype == torch.int64 and whole.size == w.rows.size
+    woff = whole.offsets.cpu().numpy()
+    assert woff[0] == 0 and np.all(np.diff(woff) >= 0) and int(woff[-1]) == whole.chars.numel() > 0x7FFFFFFF
+    for lo, hi in [(0, 400_000), (3_999_999, 4_300_001), (7_700_000, 8_000_000)]:
+        hs = w.rows.slice(lo, hi)
+        exp = normalize_py.normalize_characters_native(hs, True, [t.encode() for t in tokens], nthreads=16)
+        got = nv.normalize_characters(d.slice(lo, hi, hs.null_count), normalizer)
+        gh = got.to_host()
+        assert np.array_equal(gh.offsets, exp.offsets) and np.array_equal(gh.chars, exp.chars), f"C5 normalize rows {lo}:{hi}"
+        assert torch.equal(got.chars, whole.chars[int(woff[lo]): int(woff[hi])]), f"C5 normalize: slice {lo}:{hi} of the whole"
+        assert np.array_equal(exp.offsets.astype(np.int64) + int(woff[lo]), woff[lo: hi + 1])
+    del whole
     torch.cuda.empty_cache()
     a, b, da, db = _params(nv, p)
     _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, [(0, 20_000), (6_000_000, 6_010_000)], "C5 minhash64")

@@ -205,3 +205,78 @@ def test_normalize_then_tokenize_matches_hf_bert_pipeline():
         assert g == want, row
         split += len(want) > len(row.split(" "))
     assert split > 200  # punctuation and sub-word splits were exercised
+
+
+# ---- the C++ restatement (oracle/nvtext_oracle.cpp), which checks the large inputs
+
+def test_rule_tables_hold_classify_of_every_code_point():
+    kind, lower = onorm.rule_tables()
+    lower = lower.reshape(-1, 3)
+    for cp in range(0x110000):
+        k, low = onorm.classify(cp)
+        assert kind[cp] == k and [int(x) for x in lower[cp] if x] == [x for x in low if x], hex(cp)
+
+
+@pytest.mark.parametrize("nthreads", [1, 4])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("case", gc.normalize_cases(), ids=lambda c: c["name"])
+def test_native_normalize_golden(case, dtype, nthreads):
+    tokens = [t.encode("utf-8") for t in case["special_tokens"]]
+    got = onorm.normalize_characters_native(case_column(case, dtype), case["do_lower_case"], tokens, nthreads)
+    assert got.to_pylist() == expected_bytes(case)
+
+
+def random_text_rows(rng, n, max_items):
+    palette = (list("abcdefghijklmnopqrstuvwxyzABCDEFGHIJKLMNOPQRSTUVWXYZ0123456789") * 3 + list("  \t\n\r.,;:!?^$[](){}`~-_'\"") * 2
+               + list("éèâîôÉÈÂĂĆĖÑÜüñßçøåİıŉǅΐΣς") + ["é", "́", "̧", " ", " ", "​", "­", "�", "\x00", "\x7f"]
+               + list("漢字仮名丏丟乾乿中文한글각힣ﬃﬁǰẖ£€„“”«»") + ["😀", "𝄞", "\U00020000", "\U000e0001", "\U0010ffff"]
+               + ["[PAD]", "[CLS]", "[SEP]", "[pad]", "[MASK]", "[UNK]", "[", "]", "[a]", "[é]"])
+    rows = []
+    for _ in range(n):
+        u = rng.random()
+        rows.append(None if u < 0.05 else "" if u < 0.1 else
+                    "".join(palette[i] for i in rng.integers(0, len(palette), rng.integers(1, max_items + 1))))
+    return rows
+
+
+@pytest.mark.parametrize("do_lower", [True, False])
+@pytest.mark.parametrize("seed,dtype", [(11, np.int32), (12, np.int64)])
+def test_native_normalize_matches_the_python_loops(seed, dtype, do_lower):
+    rng = np.random.default_rng(seed)
+    col = gc.strings(random_text_rows(rng, 600, 60), dtype)
+    tokens = [b"[PAD]", b"[CLS]", b"[SEP]", b"[MASK]", b"[UNK]"]
+    for toks in (tokens, []):
+        for view in (col, col.slice(23, 411)):
+            exp = onorm.normalize_characters(view, do_lower, toks)
+            for nthreads in (1, 3, 8):  # parts of 4096 bytes and more: the column has about 40 KB
+                got = onorm.normalize_characters_native(view, do_lower, toks, nthreads)
+                assert np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets), (len(toks), nthreads)
+                assert got.offsets.dtype == exp.offsets.dtype and got.null_count == exp.null_count
+
+
+def test_native_normalize_malformed_bytes():
+    rng = np.random.default_rng(5)
+    data = rng.integers(0, 256, 30000, dtype=np.uint8)
+    data[rng.random(data.size) < 0.3] = 0x5B  # plenty of '['
+    data[rng.random(data.size) < 0.1] = 0x5D
+    cuts = np.sort(rng.integers(0, data.size + 1, 299))
+    offsets = np.concatenate([[0], cuts, [data.size]]).astype(np.int32)
+    from cudf_amd.arrow_host import HostStringsColumn
+    col = HostStringsColumn(data, offsets, None, 300, 0, 0)
+    for do_lower in (True, False):
+        exp = onorm.normalize_characters(col, do_lower, [b"[]", b"[a]"])
+        for nthreads in (1, 5):
+            got = onorm.normalize_characters_native(col, do_lower, [b"[]", b"[a]"], nthreads)
+            assert np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets)
+
+
+def test_native_normalize_special_token_across_its_blocks():
+    # the C++ restatement works through the chars 32 KiB at a time: a token that lies across such a boundary
+    from cudf_amd.arrow_host import HostStringsColumn
+    for shift in range(0, 7):
+        text = b"a" * (32768 - shift) + b"[pad]" + b"b" * 100 + "É".encode() + b"[SEP]"
+        col = HostStringsColumn(np.frombuffer(text, np.uint8).copy(), np.array([0, 5, len(text)], np.int32), None, 2, 0, 0)
+        exp = onorm.normalize_characters(col, True, [b"[PAD]", b"[SEP]"])
+        got = onorm.normalize_characters_native(col, True, [b"[PAD]", b"[SEP]"], 1)
+        assert np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets), shift
+        assert bytes(got.chars).count(b"[PAD]") == 1 and bytes(got.chars).count(b"[SEP]") == 1
