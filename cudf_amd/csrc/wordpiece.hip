@@ -1126,9 +1126,9 @@ struct EmitLds {
 
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
                                                                      const uint32_t* __restrict__ arena,
-                                                                     const int32_t* __restrict__ nwords, const OovEntry* __restrict__ queue,
-                                                                     const OovResult* __restrict__ results, const int32_t* __restrict__ offsets,
-                                                                     int32_t* __restrict__ out, int block_rows)
+                                                                     const int32_t* __restrict__ nwords, OovResult* __restrict__ results,
+                                                                     const int32_t* __restrict__ offsets, int32_t* __restrict__ out, int block_rows,
+                                                                     uint32_t* __restrict__ again, uint32_t* __restrict__ again_count)
 {
   // block_rows (1..64) rows per wavefront at a time: fewer when rows are long, so that the walks stay
   // short and there are enough of them to fill the device
@@ -1215,11 +1215,11 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
           } else if (c <= kOovKeep) {
             dst[done + t] = results[v & ~kOovMark].tok[k];
           } else if (k == 0) {
-            // more pieces than a queue entry keeps: tokenize the word again, straight into place
-            OovEntry const e = queue[v & ~kOovMark];
-            const uint8_t* p = col.chars + col.off(e.row) + e.delta;
-            int32_t* d       = dst + done + t;
-            tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t jj, int32_t id) { d[jj] = id; });
+            // more pieces than a result record keeps (seldom): noted for wordpiece_retokenize_kernel, with the
+            // place of the word's first token in the child left where its tokens would have been
+            uint32_t const q = v & ~kOovMark;
+            again[atomicAdd(again_count, 1u)] = q;
+            results[q].tok[0]                 = base + static_cast<int32_t>(done + t);
           }
         }
         lds_sync();
@@ -1227,6 +1227,25 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
       done += tokens;
     }
     lds_sync();
+  }
+}
+
+// The words that have more pieces than a result record keeps (the emit pass has listed them in again[0 .. *again_count)
+// and left the index of each one's first token in the child in its result record): tokenized again, straight into
+// place.  One lane per word; kept apart from the emit pass so that it is compiled for its common case (a third of
+// the registers, all the wavefronts a unit can hold).
+__global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
+                                                                           const OovResult* __restrict__ results,
+                                                                           const uint32_t* __restrict__ again,
+                                                                           const uint32_t* __restrict__ again_count, int32_t* __restrict__ out)
+{
+  uint32_t const n = *again_count;
+  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
+    uint32_t const q = again[i];
+    OovEntry const e = queue[q];
+    const uint8_t* p = col.chars + col.off(e.row) + e.delta;
+    int32_t* const d = out + results[q].tok[0];
+    tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t j, int32_t id) { d[j] = id; });
   }
 }
 
@@ -1592,7 +1611,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       nvtext_amd_list_column_free(out, stream_, mr_);
       return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
     }
-    launch_fill_u32(qsize.as<uint32_t>(), 0u, 1, stream);
+    launch_fill_u32(qsize.as<uint32_t>(), 0u, 2, stream);  // queue size; words the emit pass hands on
     {
       ProfileScope ps("wordpiece_probe_kernel", stream);
       hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
@@ -1647,9 +1666,13 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
-                         arena.as<uint32_t>(), nwords.as<int32_t>(), queue.as<OovEntry>(), results.as<OovResult>(),
-                         out->offsets,
-                         static_cast<int32_t*>(out->child), block_rows);
+                         arena.as<uint32_t>(), nwords.as<int32_t>(), results.as<OovResult>(), out->offsets,
+                         static_cast<int32_t*>(out->child), block_rows, longer.as<uint32_t>(), qsize.as<uint32_t>() + 1);
+      // (the list of longer words has served its purpose by now: its memory takes the list of words to do again,
+      // at most one entry per queued word)
+      hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
+                         queue.as<OovEntry>(), results.as<OovResult>(), longer.as<uint32_t>(), qsize.as<uint32_t>() + 1,
+                         static_cast<int32_t*>(out->child));
     }
     break;
   }
