@@ -460,7 +460,7 @@ __device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return 
 // row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
 // For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
 // marker carrying the queue index; nwords[r] = counts[r] = words kept.
-__global__ void __launch_bounds__(kTokThreads) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
+__global__ void __launch_bounds__(kTokThreads, 6) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
                                                                       uint32_t* __restrict__ arena,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
                                                                       OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
