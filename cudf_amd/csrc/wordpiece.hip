@@ -460,7 +460,7 @@ __device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return 
 // row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
 // For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
 // marker carrying the queue index; nwords[r] = counts[r] = words kept.
-__global__ void __launch_bounds__(kTokThreads, 6) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
+__global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
                                                                       uint32_t* __restrict__ arena,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
                                                                       OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
@@ -485,20 +485,26 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_probe_kernel(ColView
     return col.valid(row) ? static_cast<uint32_t>(min(static_cast<int64_t>(max_words), bytes / 2)) : 0u;
   };
 
-  // ---- per-group state (the same value in all 16 lanes of a group)
-  int64_t r = (static_cast<int64_t>(blockIdx.x) * kTokWaves + wave) * kGroups + g;
-  int64_t o_cur = 0, e_cur = 0, o_nxt = 0, e_nxt = 0;
-  uint32_t cap = 0;
-  if (r < rows) {
-    o_cur = col.off(r);
-    e_cur = col.off(r + 1);
-    cap   = word_cap(r, e_cur - o_cur);
+  // ---- per-group state (the same value in all 16 lanes of a group).  Kept small: the row being walked is known by its
+  // RowCtx alone (its first byte's address gives back its offset), the row after it by its offset and length.
+  uint32_t r = (blockIdx.x * kTokWaves + wave) * kGroups + g;  // rows fit 31 bits and so does the stride: no wrap
+  int64_t o_nxt  = 0;
+  uint32_t n_nxt = 0;
+  uint32_t cap   = 0;
+  RowCtx ctx;
+  {
+    int64_t o = 0, n = 0;
+    if (r < rows) {
+      o   = col.off(r);
+      n   = col.off(r + 1) - o;
+      cap = word_cap(r, n);
+    }
+    ctx = make_row_ctx(col, o, n);
   }
   if (r + stride < rows) {
     o_nxt = col.off(r + stride);
-    e_nxt = col.off(r + stride + 1);
+    n_nxt = static_cast<uint32_t>(col.off(r + stride + 1) - o_nxt);
   }
-  RowCtx ctx       = make_row_ctx(col, o_cur, e_cur - o_cur);
   uint32_t cbase   = 0;
   uint32_t wdone   = 0;     // words kept so far in this row
   uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
@@ -559,8 +565,9 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_probe_kernel(ColView
     // words of this chunk that count (the row's word limit may cut them short)
     uint32_t const allowed = chunk_ok ? min(my_gtotal, cap - wdone) : 0u;
     uint32_t const wd_after = wdone + allowed;
-    int64_t const r_now     = r;
+    uint32_t const r_now    = r;
     if (gl == 0) {
+      int64_t const o_cur    = reinterpret_cast<const uint8_t*>(ctx.base) + ctx.mis - col.chars;
       int64_t const row_slot = ((o_cur - first_offset) >> 1) + r;
       *reinterpret_cast<uint4*>(&lds.group[g][0]) = make_uint4(my_gbase, allowed, cbase, wdone);
       *reinterpret_cast<uint4*>(&lds.group[g][4]) =
@@ -574,18 +581,16 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_probe_kernel(ColView
         cbase += kChunk;
         wdone = wd_after;
       } else {
-        r += stride;
-        o_cur = o_nxt;
-        e_cur = e_nxt;
-        ctx   = make_row_ctx(col, o_cur, e_cur - o_cur);
+        r += static_cast<uint32_t>(stride);
+        ctx   = make_row_ctx(col, o_nxt, n_nxt);
         cbase = 0;
         wdone = 0;
         carry_start = 0;
         prev_space  = 1;
-        if (r < rows) cap = word_cap(r, e_cur - o_cur);
+        if (r < rows) cap = word_cap(r, n_nxt);
         if (r + stride < rows) {
           o_nxt = col.off(r + stride);
-          e_nxt = col.off(r + stride + 1);
+          n_nxt = static_cast<uint32_t>(col.off(r + stride + 1) - o_nxt);
         }
       }
       if (r < rows) {
