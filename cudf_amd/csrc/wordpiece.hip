@@ -477,6 +477,8 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
   int64_t const rows   = col.size;
   int64_t const stride = static_cast<int64_t>(gridDim.x) * kTokWaves * kGroups;  // rows between two rows of a group
   uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
+  uint32_t my_block       = min(queue_block, 128u);  // entries reserved at a time: doubled up to queue_block when ranges fill fast
+  uint32_t steps_in_range = 0;                       // steps of the loop below since the range was reserved
 
   // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
   // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
@@ -518,6 +520,7 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
   }
 
   while (ballot64(r < rows) != 0) {
+    ++steps_in_range;
     bool const has_row  = r < rows;
     bool const chunk_ok = has_row && cbase < ctx.aend && wdone < cap;
 
@@ -655,18 +658,20 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
       }
       uint64_t const mm = ballot64(miss);
       if (mm) {
-        uint32_t const nm = static_cast<uint32_t>(__builtin_popcountll(mm));
-        if (q_pos + nm > q_lim) {  // queue_block >= 64 >= nm
-          // retire what is left of the old range (entries nobody owns are marked with row -1), take a new one
-          for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-            if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
-          uint32_t base = 0;
-          if (lane == 0) base = atomicAdd(queue_size, queue_block);
-          q_pos = wave_bcast(base, 0);
-          q_lim = q_pos + queue_block;
+        uint32_t const nm   = static_cast<uint32_t>(__builtin_popcountll(mm));
+        uint32_t const room = q_lim - q_pos;  // left of the reserved range: filled up before the next one is begun,
+        uint32_t fresh      = 0;              // so that unused entries only ever follow a wavefront's last word
+        if (nm > room) {                      // my_block >= 64 >= nm
+          // a range that lasted only a few steps is followed by one twice as long: atomics on the one counter
+          // run at about 150 M/s for the whole device, and unused entries cost the next pass time
+          if (steps_in_range < 8u && my_block < queue_block) my_block <<= 1;
+          steps_in_range = 0;
+          if (lane == 0) fresh = atomicAdd(queue_size, my_block);
+          fresh = wave_bcast(fresh, 0);
         }
         if (miss) {
-          uint32_t const q = q_pos + lanes_below(mm);
+          uint32_t const rank = lanes_below(mm);
+          uint32_t const q    = rank < room ? q_pos + rank : fresh + (rank - room);
           if (q < queue_capacity) {
             uint4* const dst = reinterpret_cast<uint4*>(queue + q);
             store_stream(dst, make_uint4(gb.y, wstart - gb.x, ga.w + idx, wl));
@@ -674,7 +679,12 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
           }
           value = kOovMark | q;
         }
-        q_pos += nm;
+        if (nm > room) {
+          q_pos = fresh + (nm - room);
+          q_lim = fresh + my_block;
+        } else {
+          q_pos += nm;
+        }
       }
       if (active) {
         int64_t const s = static_cast<int64_t>((static_cast<uint64_t>(gb.w) << 32) | gb.z) + ga.w + idx;
@@ -1000,7 +1010,7 @@ struct ShortWord {
 // below: their queue indices go to longer[first entry of the part ...], their number to
 // longer[queue_capacity + wavefront].
 // results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count - 1.
-__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
+__global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
                                                                     const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
                                                                     OovResult* __restrict__ results, int32_t* __restrict__ counts,
                                                                     uint32_t* __restrict__ longer)
@@ -1587,11 +1597,12 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   };
   unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves * kGroups - 1) / (kTokWaves * kGroups),
                                                                       resident(reinterpret_cast<const void*>(wordpiece_probe_kernel), kTokThreads)));
-  // Each wavefront reserves queue entries `queue_block` at a time (one atomic per block).
+  // Each wavefront reserves queue entries a range at a time (one atomic per range), at most `queue_block` of them:
+  // it starts with short ranges and doubles them while they fill within a few steps, because atomics on one
+  // address are slow (about 150 M/s) and the unused tail of each wavefront's last range, half a range on
+  // average, is time lost in the pass that reads the queue.
   uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
   uint32_t queue_block = 64;
-  // (atomics on one address are slow: about 150 M/s, so blocks are kept large even though the unused tail of
-  // each wavefront's last block, half a block on average, then makes up a tenth or more of the queue)
   while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
   uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
   Temp arena(mr, arena_slots * sizeof(uint32_t));
