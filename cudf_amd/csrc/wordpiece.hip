@@ -1004,7 +1004,7 @@ struct ShortWord {
 };
 
 // One lane per queued word, and a lane that finishes its word takes the next one: every wavefront owns a
-// contiguous part of the queue and, every fourth trip, lets its idle lanes store their result and pick up
+// contiguous part of the queue and, every eighth trip, lets its idle lanes store their result and pick up
 // new entries, so lanes with short words do not wait for the longest word of a batch.  Words of up to 16
 // bytes (whole in their queue record) run in registers; the few longer ones are set aside for the kernel
 // below: their queue indices go to longer[first entry of the part ...], their number to
@@ -1045,7 +1045,7 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(ColView c
     uint32_t q = 0;
     int32_t row = -1;
     for (uint32_t trip = 0;; ++trip) {
-      if ((trip & 3u) == 0) {
+      if ((trip & 7u) == 0) {
         if (busy && sw.done) {
           deliver(q, row, sw.count);
           busy = false;
