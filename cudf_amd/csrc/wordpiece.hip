@@ -58,10 +58,12 @@ __host__ __device__ __forceinline__ uint32_t key_hash_block(uint32_t h, uint32_t
 }
 
 // slot.x = (tag23 << 9) | (kind << 8) | len   (0 = empty; len in 1..199)
-// slot.y = token id
+// slot.y = token id; in slot 0 of a bucket, bit 31 says that some key has been carried past this bucket
+//          (kSearchOn: a key that is not in a bucket without the bit is not in the table)
 // slot.z, slot.w = the key itself when len <= 8 (zero padded), else (byte offset of the key in the pool, 0);
 // the pool holds the keys of more than 8 bytes, each zero padded to a multiple of 8 at an 8-byte aligned offset
 // Bucket b = slots[2b], slots[2b+1]; a bucket fills slot 0 first, overflow goes to the next bucket.
+constexpr uint32_t kSearchOn = 0x80000000u;
 struct VocabTable {
   const uint4* slots;
   const uint8_t* pool;
@@ -290,7 +292,7 @@ __device__ __forceinline__ int check_slot(VocabTable const& t, uint4 const& s, P
   if (s.x == pr.want) {
     bool const same = len <= 8 ? (s.z == pr.k0 && s.w == pr.k1) : pool_key_equal(t, s.z, w, p, len);
     if (same) {
-      *id = static_cast<int32_t>(s.y);
+      *id = static_cast<int32_t>(s.y & ~kSearchOn);
       return 1;
     }
   }
@@ -325,7 +327,7 @@ __device__ __forceinline__ int32_t finish_probe(VocabTable const& t, Probe const
   if (r == 0) return kNone;
   r = check_slot(t, s1, pr, w, p, len, &id);
   if (r > 0) return id;
-  if (r == 0) return kNone;
+  if (r == 0 || (s0.y & kSearchOn) == 0) return kNone;
   return lookup_further(t, pr, w, p, len);
 }
 
@@ -340,8 +342,8 @@ __device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W 
 }
 
 // What the two home slots say about a key of l bytes without any further memory access:
-// 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or the
-// bucket is full and the search goes on in the next one: both rare).  Straight-line code.
+// 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or keys have been
+// carried past this bucket and the search goes on in the next one).  Straight-line code.
 __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
 {
   bool const tag0  = s0.x == pr.want, tag1 = s1.x == pr.want;
@@ -349,9 +351,28 @@ __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, ui
   bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
   bool const small = l <= 8;
   bool const found = small && (is0 || is1);
-  bool const more  = (!small && (tag0 || tag1)) || (!found && s0.x != 0 && s1.x != 0);
-  *id              = static_cast<int32_t>(is0 ? s0.y : s1.y);
+  bool const more  = (!small && (tag0 || tag1)) || (!found && (s0.y & kSearchOn) != 0);
+  *id              = static_cast<int32_t>((is0 ? s0.y : s1.y) & ~kSearchOn);
   return found ? 1u : more ? 2u : 0u;
+}
+
+// The same for a key of 9 to 16 bytes whose bytes are k[0..3] (zero padded): a home slot with the right tag
+// names the key's place in the pool, and one 16-byte read there decides.  Still undecided (2) only when both home
+// slots carry the tag or the search goes on in the next bucket.
+__device__ __forceinline__ uint32_t verdict_16(VocabTable const& t, Probe const& pr, uint4 const& s0, uint4 const& s1, const uint32_t (&k)[4],
+                                               int32_t* id)
+{
+  bool const tag0 = s0.x == pr.want, tag1 = s1.x == pr.want;
+  bool const on   = (s0.y & kSearchOn) != 0;
+  if (tag0 && tag1) return 2u;
+  if (!tag0 && !tag1) return on ? 2u : 0u;
+  const uint2* const e = reinterpret_cast<const uint2*>(t.pool + (tag0 ? s0.z : s1.z));
+  uint2 const a = e[0], b = e[1];
+  if (a.x == k[0] && a.y == k[1] && b.x == k[2] && b.y == k[3]) {
+    *id = static_cast<int32_t>((tag0 ? s0.y : s1.y) & ~kSearchOn);
+    return 1u;
+  }
+  return on ? 2u : 0u;
 }
 
 // ------------------------------------------------------------------ wavefront helpers of the probe pass
@@ -648,7 +669,8 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
             pr.bucket = b & table.bucket_mask;
             uint4 const s0 = table.slots[2 * pr.bucket];
             uint4 const s1 = table.slots[2 * pr.bucket + 1];
-            uint32_t const v = verdict(pr, s0, s1, wl, &id);
+            uint32_t v = verdict(pr, s0, s1, wl, &id);
+            if (v == 2u && wl > 8 && wl <= 16) v = verdict_16(table, pr, s0, s1, head, &id);
             if (v == 2u) id = finish_probe(table, pr, s0, s1, rw_, 0u, wl);
             else if (v == 0u) id = kNone;
           }
@@ -1320,6 +1342,7 @@ void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::
       // the same key again: the first entry wins (duplicates are undefined in the reference)
       if (host_same(s, w0, pool, key, len, k0, k1)) return;
     }
+    slots[2 * static_cast<size_t>(b)].y |= kSearchOn;  // the key is carried past this bucket
     ++b;
   }
 }
@@ -1337,7 +1360,7 @@ int32_t host_find(const std::vector<HostSlot>& slots, uint32_t bucket_mask, cons
     for (int j = 0; j < 2; ++j) {
       HostSlot const& s = slots[2 * static_cast<size_t>(b) + j];
       if (s.x == 0) return -1;
-      if (host_same(s, w0, pool, key, len, k0, k1)) return static_cast<int32_t>(s.y);
+      if (host_same(s, w0, pool, key, len, k0, k1)) return static_cast<int32_t>(s.y & ~kSearchOn);
     }
     ++b;
   }
