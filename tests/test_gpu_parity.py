@@ -5,6 +5,7 @@ import pytest
 
 from tests import golden_cases as gc
 from tests.golden_cases import strings
+from cudf_amd.arrow_host import HostStringsColumn
 
 pytestmark = pytest.mark.gpu
 
@@ -498,6 +499,34 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
         exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4)
         assert_same(got, exp, f"long keys mw={mw}")
     assert exp.child.size > 5000
+
+
+@pytest.mark.parametrize("which", ["bert 30k", "multilingual 250k"])
+def test_wordpiece_every_vocabulary_entry_is_its_own_token(nv, orc, which):
+    """Each entry of a generated vocabulary, as a word in the middle of a row and as the only word of a row: its
+    token is its own index (the first one, if the entry occurs twice).  This reaches every key wherever the table
+    put it -- in its home bucket, carried past one full bucket or past several -- and every key length."""
+    from cudf_amd import datagen
+    vocab = (datagen.make_vocab(datagen.VOCAB_BERT, 30522, seed=1001) if which == "bert 30k"
+             else datagen.make_vocab(datagen.VOCAB_MULTILINGUAL, 250000, seed=1005))
+    entries = vocab.to_pylist()
+    first = {}
+    for i, e in enumerate(entries):
+        first.setdefault(e, i)
+    words = [(e, first[e]) for e in entries if e and not e.startswith(b"##") and b" " not in e and len(e) < 199]
+    assert len(words) > 0.5 * len(entries)
+    dv = nv.WordPieceVocabulary(dev(nv, vocab))
+    # alone in their rows
+    alone = HostStringsColumn.from_pylist([w for w, _ in words])
+    got = nv.wordpiece_tokenize(dev(nv, alone), dv, 0).to_host()
+    assert np.array_equal(got.offsets, np.arange(len(words) + 1, dtype=np.int32))
+    assert np.array_equal(got.child, np.array([i for _, i in words], np.int32))
+    # sixteen to a row, and against the oracle
+    rows = [b" ".join(w for w, _ in words[k: k + 16]) for k in range(0, len(words), 16)]
+    packed = HostStringsColumn.from_pylist(rows)
+    got = nv.wordpiece_tokenize(dev(nv, packed), dv, 0).to_host()
+    assert np.array_equal(got.child, np.array([i for _, i in words], np.int32))
+    assert_same(got, orc.wordpiece_tokenize(packed, orc.Vocabulary(vocab), 0, nthreads=8), which)
 
 
 def test_cpp_api_program():
