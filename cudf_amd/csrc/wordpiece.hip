@@ -482,7 +482,7 @@ __device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return 
 // For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
 // marker carrying the queue index; nwords[r] = counts[r] = words kept.
 __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                      uint32_t* __restrict__ arena,
+                                                                      int64_t last_offset, uint32_t* __restrict__ arena,
                                                                       int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
                                                                       OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
                                                                       uint32_t* __restrict__ queue_size)
@@ -496,7 +496,6 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
   int const g_last     = g_first + kGroupLanes - 1;
   ProbeLds& lds        = lds_all[wave];
   int64_t const rows   = col.size;
-  int64_t const stride = static_cast<int64_t>(gridDim.x) * kTokWaves * kGroups;  // rows between two rows of a group
   uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
   uint32_t my_block       = min(queue_block, 128u);  // entries reserved at a time: doubled up to queue_block when ranges fill fast
   uint32_t steps_in_range = 0;                       // steps of the loop below since the range was reserved
@@ -508,26 +507,49 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
     return col.valid(row) ? static_cast<uint32_t>(min(static_cast<int64_t>(max_words), bytes / 2)) : 0u;
   };
 
+  // ---- the rows of a group: consecutive ones, [r, r_end), that hold its share of the column's BYTES (group k of G
+  // begins with the first row at or after byte k/G of the chars).  With a share of the rows instead (every G-th row)
+  // the groups with the longest rows walked a seventh more chunks than the average group, and the pass waited for them.
+  // r_end is found together with r: two searches over the offsets in step, 22 dependent reads for 4M rows.
+  uint32_t r = 0, r_end = 0;
+  {
+    uint32_t const groups = gridDim.x * kTokWaves * kGroups;
+    uint32_t const k      = (blockIdx.x * kTokWaves + wave) * kGroups + g;
+    // (bytes < 2^47 and groups < 2^16: the products fit)
+    int64_t const bytes = last_offset - first_offset;
+    int64_t const t0    = first_offset + bytes / groups * k + bytes % groups * k / groups;
+    int64_t const t1    = first_offset + bytes / groups * (k + 1) + bytes % groups * (k + 1) / groups;
+    // number of entries off(0..rows) below t, which is the first row at or after byte t
+    uint32_t below0 = 0, below1 = 0;
+    uint32_t step   = 1;
+    while (step <= static_cast<uint32_t>(rows)) step <<= 1;  // rows + 1 entries; rows < 2^31
+    for (; step > 0; step >>= 1) {
+      uint32_t const p0 = below0 + step, p1 = below1 + step;
+      int64_t const v0  = p0 <= static_cast<uint32_t>(rows) + 1u ? col.off(static_cast<int64_t>(p0) - 1) : std::numeric_limits<int64_t>::max();
+      int64_t const v1  = p1 <= static_cast<uint32_t>(rows) + 1u ? col.off(static_cast<int64_t>(p1) - 1) : std::numeric_limits<int64_t>::max();
+      if (v0 < t0) below0 = p0;
+      if (v1 < t1) below1 = p1;
+    }
+    r     = min(below0, static_cast<uint32_t>(rows));
+    r_end = k + 1 == groups ? static_cast<uint32_t>(rows) : min(below1, static_cast<uint32_t>(rows));
+    if (k == 0) r = 0;
+  }
   // ---- per-group state (the same value in all 16 lanes of a group).  Kept small: the row being walked is known by its
-  // RowCtx alone (its first byte's address gives back its offset), the row after it by its offset and length.
-  uint32_t r = (blockIdx.x * kTokWaves + wave) * kGroups + g;  // rows fit 31 bits and so does the stride: no wrap
-  int64_t o_nxt  = 0;
-  uint32_t n_nxt = 0;
-  uint32_t cap   = 0;
+  // RowCtx alone (its first byte's address gives back its offset; the next row begins where it ends), the row after
+  // it by its end.
+  int64_t e_nxt = 0;
+  uint32_t cap  = 0;
   RowCtx ctx;
   {
     int64_t o = 0, n = 0;
-    if (r < rows) {
+    if (r < r_end) {
       o   = col.off(r);
       n   = col.off(r + 1) - o;
       cap = word_cap(r, n);
     }
     ctx = make_row_ctx(col, o, n);
   }
-  if (r + stride < rows) {
-    o_nxt = col.off(r + stride);
-    n_nxt = static_cast<uint32_t>(col.off(r + stride + 1) - o_nxt);
-  }
+  if (r + 1 < r_end) e_nxt = col.off(static_cast<int64_t>(r) + 2);
   uint32_t cbase   = 0;
   uint32_t wdone   = 0;     // words kept so far in this row
   uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
@@ -535,14 +557,14 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
   // the chunk about to be processed: my sixteen bytes and (last lane of the group) the byte after the chunk
   uint4 mine_cur    = make_uint4(0u, 0u, 0u, 0u);
   uint32_t tail_cur = 0x20u;
-  if (r < rows) {
+  if (r < r_end) {
     mine_cur = ctx.load_raw(16 * gl);
     if (gl == kGroupLanes - 1) tail_cur = ctx.byte_at(kChunk);
   }
 
-  while (ballot64(r < rows) != 0) {
+  while (ballot64(r < r_end) != 0) {
     ++steps_in_range;
-    bool const has_row  = r < rows;
+    bool const has_row  = r < r_end;
     bool const chunk_ok = has_row && cbase < ctx.aend && wdone < cap;
 
     // ---- bytes -> word ends (lanes <-> bytes, per group)
@@ -605,19 +627,19 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
         cbase += kChunk;
         wdone = wd_after;
       } else {
-        r += static_cast<uint32_t>(stride);
-        ctx   = make_row_ctx(col, o_nxt, n_nxt);
+        // the next row begins where this one ends
+        int64_t const o_new = reinterpret_cast<const uint8_t*>(ctx.base) + ctx.aend - col.chars;
+        int64_t const n_new = r + 1 < r_end ? e_nxt - o_new : 0;
+        ++r;
+        ctx   = make_row_ctx(col, o_new, n_new);
         cbase = 0;
         wdone = 0;
         carry_start = 0;
         prev_space  = 1;
-        if (r < rows) cap = word_cap(r, n_nxt);
-        if (r + stride < rows) {
-          o_nxt = col.off(r + stride);
-          n_nxt = static_cast<uint32_t>(col.off(r + stride + 1) - o_nxt);
-        }
+        if (r < r_end) cap = word_cap(r, n_new);
+        if (r + 1 < r_end) e_nxt = col.off(static_cast<int64_t>(r) + 2);
       }
-      if (r < rows) {
+      if (r < r_end) {
         mine_cur = ctx.load_raw(cbase + 16 * gl);
         tail_cur = gl == kGroupLanes - 1 ? ctx.byte_at(cbase + kChunk) : 0x20u;
       }
@@ -1654,7 +1676,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     {
       ProfileScope ps("wordpiece_probe_kernel", stream);
       hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
-                         first_offset, arena.as<uint32_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
+                         first_offset, last_offset, arena.as<uint32_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
                          queue_block, qsize.as<uint32_t>());
     }
     {
