@@ -278,14 +278,15 @@ __device__ __forceinline__ uint32_t owned_slots(NormLds const& lds, uint64_t lo6
     uint32_t s0, s1, s2;
     uint32_t const bytes = wide_slots(w, t, s0, s1, s2);
     sum += bytes;
+    // (as bit masks: written as "if (j == at)", the eight cases become a tree of branches, which lanes with
+    // different `at` walk one leaf after the other)
 #pragma unroll
     for (int j = 0; j < kNormItems; ++j) {
-      if (j == at) {
-        mine.s[j][0] = s0;
-        mine.s[j][1] = s1;
-        mine.s[j][2] = s2;
-        size[j]      = bytes;
-      }
+      uint32_t const here = static_cast<uint32_t>((static_cast<int32_t>(j ^ at) - 1) >> 31);  // all ones where j == at
+      mine.s[j][0] = (mine.s[j][0] & ~here) | (s0 & here);
+      mine.s[j][1] = (mine.s[j][1] & ~here) | (s1 & here);
+      mine.s[j][2] = (mine.s[j][2] & ~here) | (s2 & here);
+      size[j]      = (size[j] & ~here) | (bytes & here);
     }
   }
   return sum;
