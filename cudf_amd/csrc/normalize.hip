@@ -226,30 +226,48 @@ __device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
   lds_barrier();
 }
 
+// Code point of a character of two or three bytes whose bytes start `w` (first byte below 0xF0): decode() without
+// its branches.
+__device__ __forceinline__ uint32_t decode_short(uint32_t w)
+{
+  uint32_t const b1    = (w >> 8) & 0x3Fu;
+  uint32_t const two   = ((w & 0x1Fu) << 6) | b1;
+  uint32_t const three = ((w & 0x0Fu) << 12) | (b1 << 6) | ((w >> 16) & 0x3Fu);
+  return (w & 0xFFu) < 0xE0u ? two : three;
+}
+
 // Slots of the character whose bytes start `w` (first byte in the low bits) and the bytes they hold together.  The
 // Basic Multilingual Plane has them ready in one 16-byte table entry; the rest goes through the code point tables.
 __device__ __forceinline__ uint32_t wide_slots(uint32_t w, NormTables const& t, uint32_t& s0, uint32_t& s1, uint32_t& s2)
 {
-  uint32_t const cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
-  if (cp < 0x10000u) {
-    uint4 const e = t.bmp[cp];
-    s0            = e.x;
-    s1            = e.y;
-    s2            = e.z;
-    return e.w;
+  uint32_t cp = decode_short(w);
+  if ((w & 0xFFu) >= 0xF0u) {  // four bytes (seldom)
+    cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
+    if (cp >= 0x10000u) {
+      slots_of(cp, t, s0, s1, s2);
+      return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+    }
   }
-  slots_of(cp, t, s0, s1, s2);
-  return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+  uint4 const e = t.bmp[cp];
+  s0            = e.x;
+  s1            = e.y;
+  s2            = e.z;
+  return e.w;
 }
 
 // Bytes that the character whose bytes start `w` produces, without its slots.
 __device__ __forceinline__ uint32_t wide_size(uint32_t w, NormTables const& t)
 {
-  uint32_t const cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
-  if (cp < 0x10000u) return t.bmp[cp].w;
-  uint32_t s0, s1, s2;
-  slots_of(cp, t, s0, s1, s2);
-  return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+  uint32_t cp = decode_short(w);
+  if ((w & 0xFFu) >= 0xF0u) {
+    cp = decode(w & 0xFFu, (w >> 8) & 0xFFu, (w >> 16) & 0xFFu, w >> 24);
+    if (cp >= 0x10000u) {
+      uint32_t s0, s1, s2;
+      slots_of(cp, t, s0, s1, s2);
+      return bytes_of(s0) + bytes_of(s1) + bytes_of(s2);
+    }
+  }
+  return t.bmp[cp].w;
 }
 
 // The slots (and sizes) of the eight positions whose bytes are lo64; hi64 = bytes 4..11.  Returns the bytes they produce.
