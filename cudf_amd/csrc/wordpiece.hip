@@ -507,26 +507,29 @@ __global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView
     return col.valid(row) ? static_cast<uint32_t>(min(static_cast<int64_t>(max_words), bytes / 2)) : 0u;
   };
 
-  // ---- the rows of a group: consecutive ones, [r, r_end), that hold its share of the column's BYTES (group k of G
-  // begins with the first row at or after byte k/G of the chars).  With a share of the rows instead (every G-th row)
-  // the groups with the longest rows walked a seventh more chunks than the average group, and the pass waited for them.
-  // r_end is found together with r: two searches over the offsets in step, 22 dependent reads for 4M rows.
+  // ---- the rows of a group: consecutive ones, [r, r_end), that hold its share of the column's WORK, a row counting
+  // as its bytes plus one chunk (which is about what walking it costs; rows without bytes must count, or a long run
+  // of them would fall to one group).  Group k of G begins with the first row at or after k/G of the total.  With a
+  // share of the rows instead (every G-th row) the groups with the longest rows walked a seventh more chunks than the
+  // average group, and the pass waited for them.  r_end is found together with r: two searches over the offsets in
+  // step, 22 dependent reads for 4M rows.
   uint32_t r = 0, r_end = 0;
   {
     uint32_t const groups = gridDim.x * kTokWaves * kGroups;
     uint32_t const k      = (blockIdx.x * kTokWaves + wave) * kGroups + g;
-    // (bytes < 2^47 and groups < 2^16: the products fit)
-    int64_t const bytes = last_offset - first_offset;
-    int64_t const t0    = first_offset + bytes / groups * k + bytes % groups * k / groups;
-    int64_t const t1    = first_offset + bytes / groups * (k + 1) + bytes % groups * (k + 1) / groups;
-    // number of entries off(0..rows) below t, which is the first row at or after byte t
+    auto work_before = [&](int64_t row) -> int64_t { return col.off(row) - first_offset + row * static_cast<int64_t>(kChunk); };
+    // (work < 2^48 and groups < 2^16: the products fit)
+    int64_t const work = last_offset - first_offset + rows * static_cast<int64_t>(kChunk);
+    int64_t const t0   = work / groups * k + work % groups * k / groups;
+    int64_t const t1   = work / groups * (k + 1) + work % groups * (k + 1) / groups;
+    // number of rows 0..rows with less work before them than t, which is the first row at or after t
     uint32_t below0 = 0, below1 = 0;
     uint32_t step   = 1;
     while (step <= static_cast<uint32_t>(rows)) step <<= 1;  // rows + 1 entries; rows < 2^31
     for (; step > 0; step >>= 1) {
       uint32_t const p0 = below0 + step, p1 = below1 + step;
-      int64_t const v0  = p0 <= static_cast<uint32_t>(rows) + 1u ? col.off(static_cast<int64_t>(p0) - 1) : std::numeric_limits<int64_t>::max();
-      int64_t const v1  = p1 <= static_cast<uint32_t>(rows) + 1u ? col.off(static_cast<int64_t>(p1) - 1) : std::numeric_limits<int64_t>::max();
+      int64_t const v0  = p0 <= static_cast<uint32_t>(rows) + 1u ? work_before(static_cast<int64_t>(p0) - 1) : std::numeric_limits<int64_t>::max();
+      int64_t const v1  = p1 <= static_cast<uint32_t>(rows) + 1u ? work_before(static_cast<int64_t>(p1) - 1) : std::numeric_limits<int64_t>::max();
       if (v0 < t0) below0 = p0;
       if (v1 < t1) below1 = p1;
     }

@@ -501,6 +501,18 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
     assert exp.child.size > 5000
 
 
+@pytest.mark.parametrize("max_words", [0, 4])
+def test_wordpiece_long_runs_of_rows_without_bytes(nv, orc, max_words):
+    """Hundreds of thousands of empty and null rows in a row, before, between and after rows with text: the rows are
+    shared out by work, and rows without bytes must neither be lost nor all fall to one group of lanes."""
+    vocab = strings(["[UNK]", "hello", "world", "##s", "a", "b"])
+    rows = [""] * 300_000 + ["hello worlds a b zzz"] * 500 + [None] * 200_000 + ["a"] + [""] * 100_000 + ["b hello"] * 3 + [None] * 7
+    host = strings(rows, np.int32)
+    got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, vocab)), max_words).to_host()
+    assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(vocab), max_words, nthreads=4), f"max_words={max_words}")
+    assert got.offsets[300_000] == 0 and got.offsets[-1] == got.child.size > 0
+
+
 @pytest.mark.parametrize("which", ["bert 30k", "multilingual 250k"])
 def test_wordpiece_every_vocabulary_entry_is_its_own_token(nv, orc, which):
     """Each entry of a generated vocabulary, as a word in the middle of a row and as the only word of a row: its
