@@ -78,6 +78,31 @@ struct Temp {
   }
 };
 
+// Several temporaries in ONE allocation (a call to the caller's allocator can cost tens of microseconds: from Python
+// it is a callback into the interpreter), each part 256-byte aligned.
+template <int N>
+struct TempParts {
+  size_t at[N + 1];
+  Temp whole;
+  static size_t total(const size_t (&bytes)[N])
+  {
+    size_t sum = 0;
+    for (int i = 0; i < N; ++i) sum += (bytes[i] + 255) & ~static_cast<size_t>(255);
+    return sum;
+  }
+  TempParts(Mr m, const size_t (&bytes)[N]) : whole(m, total(bytes))
+  {
+    at[0] = 0;
+    for (int i = 0; i < N; ++i) at[i + 1] = at[i] + ((bytes[i] + 255) & ~static_cast<size_t>(255));
+  }
+  bool ok() const { return whole.ok(); }
+  template <typename T>
+  T* part(int i) const
+  {
+    return reinterpret_cast<T*>(static_cast<char*>(whole.ptr) + at[i]);
+  }
+};
+
 inline size_t mask_alloc_bytes(int64_t bits)
 {
   // libcudf pads bitmask allocations to 64 bytes (cpp/include/cudf/null_mask.hpp:56-57)

@@ -884,24 +884,27 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
 
   int64_t const tiles = (n + kNormTile - 1) / kNormTile;
   if (tiles > 0x7FFFFFFFll) return release(NVTEXT_AMD_OVERFLOW, "input too large");
-  Temp tile_bytes(mr, static_cast<size_t>(tiles) * sizeof(uint32_t));
-  Temp tile_offset(mr, (static_cast<size_t>(tiles) + 1) * sizeof(uint64_t));
-  Temp scan_temp(mr, scan_temp_bytes(tiles));
-  Temp tile_row(mr, static_cast<size_t>(tiles) * sizeof(int32_t));
-  if (!tile_bytes.ok() || !tile_offset.ok() || !scan_temp.ok() || !tile_row.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+  size_t const temp_bytes[4] = {static_cast<size_t>(tiles) * sizeof(uint32_t), (static_cast<size_t>(tiles) + 1) * sizeof(uint64_t),
+                                scan_temp_bytes(tiles), static_cast<size_t>(tiles) * sizeof(int32_t)};
+  TempParts<4> const temps(mr, temp_bytes);
+  uint32_t* const tile_bytes  = temps.part<uint32_t>(0);
+  uint64_t* const tile_offset = temps.part<uint64_t>(1);
+  uint64_t* const scan_temp   = temps.part<uint64_t>(2);
+  int32_t* const tile_row     = temps.part<int32_t>(3);
+  if (!temps.ok()) return release(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   NormTables const tables{normalizer->ascii, normalizer->bmp, normalizer->entries, normalizer->second, normalizer->token_chars, normalizer->token_offset, normalizer->tokens,
                           normalizer->do_lower};
   ColView const view = make_view(*input);
   {
     ProfileScope ps("normalize_count_kernel", stream);
     hipLaunchKernelGGL(normalize_count_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view.chars + first, n, tables,
-                       tile_bytes.as<uint32_t>());
+                       tile_bytes);
   }
   hipLaunchKernelGGL(normalize_tile_rows_kernel, dim3(static_cast<unsigned>((tiles + 255) / 256)), dim3(256), 0, stream, view, first, tiles,
-                     tile_row.as<int32_t>());
-  device_exclusive_scan(TileBytes{tile_bytes.as<uint32_t>()}, tiles, tile_offset.as<uint64_t>(), scan_temp.as<uint64_t>(), stream);
+                     tile_row);
+  device_exclusive_scan(TileBytes{tile_bytes}, tiles, tile_offset, scan_temp, stream);
   uint64_t total = 0;
-  hipError_t e   = hipMemcpyAsync(&total, tile_offset.as<uint64_t>() + tiles, sizeof(total), hipMemcpyDeviceToHost, stream);
+  hipError_t e   = hipMemcpyAsync(&total, tile_offset + tiles, sizeof(total), hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);
   if (e != hipSuccess) return release(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
   // int64 offsets from the large-strings threshold on (cpp/include/cudf/strings/detail/strings_children.cuh:164-175)
@@ -915,7 +918,7 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   {
     ProfileScope ps("normalize_write_kernel", stream);
     hipLaunchKernelGGL(normalize_write_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kNormThreads), 0, stream, view, first, n, tables,
-                       tile_offset.as<uint64_t>(), tile_row.as<int32_t>(), reinterpret_cast<uint8_t*>(out->chars), out->offsets,
+                       tile_offset, tile_row, reinterpret_cast<uint8_t*>(out->chars), out->offsets,
                        out->offsets_is_int64);
   }
   e = hipGetLastError();

@@ -1653,12 +1653,15 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   uint32_t queue_block = 64;
   while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
   uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
-  Temp arena(mr, arena_slots * sizeof(uint32_t));
-  Temp nwords(mr, static_cast<size_t>(rows) * sizeof(int32_t));
-  Temp counts(mr, static_cast<size_t>(rows) * sizeof(int32_t));
-  Temp scan_tmp(mr, scan_temp_bytes(rows));
-  Temp qsize(mr, 256);
-  if (!arena.ok() || !nwords.ok() || !counts.ok() || !scan_tmp.ok() || !qsize.ok()) {
+  size_t const temp_bytes[5] = {arena_slots * sizeof(uint32_t), static_cast<size_t>(rows) * sizeof(int32_t),
+                                static_cast<size_t>(rows) * sizeof(int32_t), scan_temp_bytes(rows), 256};
+  TempParts<5> const temps(mr, temp_bytes);
+  uint32_t* const arena    = temps.part<uint32_t>(0);
+  int32_t* const nwords    = temps.part<int32_t>(1);
+  int32_t* const counts    = temps.part<int32_t>(2);
+  uint64_t* const scan_tmp = temps.part<uint64_t>(3);
+  uint32_t* const qsize    = temps.part<uint32_t>(4);
+  if (!temps.ok()) {
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
@@ -1666,37 +1669,40 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   for (int attempt = 0;; ++attempt) {
     if (queue_capacity > 0x7FFFFFFEull) queue_capacity = 0x7FFFFFFEull;
     uint32_t const qcap = static_cast<uint32_t>(queue_capacity);
-    Temp queue(mr, static_cast<size_t>(qcap) * sizeof(OovEntry));
-    Temp results(mr, static_cast<size_t>(qcap) * sizeof(OovResult));
-    // queue indices of the words of more than 16 bytes, then one count per wavefront of the out-of-vocabulary pass
-    int64_t const oov_blocks = resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads);
-    Temp longer(mr, (static_cast<size_t>(qcap) + static_cast<size_t>(oov_blocks) * (kOovThreads / kWave)) * sizeof(uint32_t));
-    if (!queue.ok() || !results.ok() || !longer.ok()) {
+    // (third part: queue indices of the words of more than 16 bytes, then one count per wavefront of the out-of-vocabulary pass)
+    int64_t const oov_blocks    = resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads);
+    size_t const queue_bytes[3] = {static_cast<size_t>(qcap) * sizeof(OovEntry), static_cast<size_t>(qcap) * sizeof(OovResult),
+                                   (static_cast<size_t>(qcap) + static_cast<size_t>(oov_blocks) * (kOovThreads / kWave)) * sizeof(uint32_t)};
+    TempParts<3> const queue_temps(mr, queue_bytes);
+    OovEntry* const queue    = queue_temps.part<OovEntry>(0);
+    OovResult* const results = queue_temps.part<OovResult>(1);
+    uint32_t* const longer   = queue_temps.part<uint32_t>(2);
+    if (!queue_temps.ok()) {
       nvtext_amd_list_column_free(out, stream_, mr_);
       return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
     }
-    launch_fill_u32(qsize.as<uint32_t>(), 0u, 2, stream);  // queue size; words the emit pass hands on
+    launch_fill_u32(qsize, 0u, 2, stream);  // queue size; words the emit pass hands on
     {
       ProfileScope ps("wordpiece_probe_kernel", stream);
       hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
-                         first_offset, last_offset, arena.as<uint32_t>(), nwords.as<int32_t>(), counts.as<int32_t>(), queue.as<OovEntry>(), qcap,
-                         queue_block, qsize.as<uint32_t>());
+                         first_offset, last_offset, arena, nwords, counts, queue, qcap,
+                         queue_block, qsize);
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
       hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>(), longer.as<uint32_t>());
+                         queue, qsize, qcap, results, counts, longer);
     }
     {
       ProfileScope ps("wordpiece_oov_long_kernel", stream);
       hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue.as<OovEntry>(), qsize.as<uint32_t>(), qcap, results.as<OovResult>(), counts.as<int32_t>(), longer.as<uint32_t>());
+                         queue, qsize, qcap, results, counts, longer);
     }
     // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
-    device_exclusive_scan(CountOf{counts.as<int32_t>()}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
+    device_exclusive_scan(CountOf{counts}, static_cast<int64_t>(rows), out->offsets, scan_tmp, stream);
     uint32_t queued = 0;
-    hipError_t e    = hipMemcpyAsync(&total, scan_tmp.as<uint64_t>() + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(&queued, qsize.as<uint32_t>(), sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+    hipError_t e    = hipMemcpyAsync(&total, scan_tmp + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(&queued, qsize, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
     if (e != hipSuccess) {
       nvtext_amd_list_column_free(out, stream_, mr_);
@@ -1730,12 +1736,12 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
-                         arena.as<uint32_t>(), nwords.as<int32_t>(), results.as<OovResult>(), out->offsets,
-                         static_cast<int32_t*>(out->child), block_rows, longer.as<uint32_t>(), qsize.as<uint32_t>() + 1);
+                         arena, nwords, results, out->offsets,
+                         static_cast<int32_t*>(out->child), block_rows, longer, qsize + 1);
       // (the list of longer words has served its purpose by now: its memory takes the list of words to do again,
       // at most one entry per queued word)
       hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue.as<OovEntry>(), results.as<OovResult>(), longer.as<uint32_t>(), qsize.as<uint32_t>() + 1,
+                         queue, results, longer, qsize + 1,
                          static_cast<int32_t*>(out->child));
     }
     break;
