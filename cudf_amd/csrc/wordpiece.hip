@@ -1311,6 +1311,66 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(ColVi
   }
 }
 
+// ------------------------------------------------------------------ very long rows
+// A row is walked by one group of lanes in the probe pass and by one wavefront in the emit pass, so a row of
+// megabytes would take milliseconds while the rest of the device is idle.  Without a word limit the tokens of a row
+// are simply those of its words in order, so such a row can be cut at spaces into pieces that are tokenized as
+// rows of their own; the list offsets of the original rows are then those of their first pieces.
+constexpr int64_t kLongRow  = 64 * 1024;  // rows beyond this many bytes are cut
+constexpr int64_t kRowPiece = 32 * 1024;  // into pieces of about this many
+
+// pieces[r] = pieces row r is cut into (1 for rows that stay whole); *any_long = 1 when some row is cut
+__global__ void long_rows_kernel(ColView col, uint32_t* __restrict__ pieces, uint32_t* __restrict__ any_long)
+{
+  int64_t const r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (r >= col.size) return;
+  int64_t const bytes = col.off(r + 1) - col.off(r);
+  bool const is_long  = bytes > kLongRow;
+  pieces[r]           = is_long ? static_cast<uint32_t>((bytes + kRowPiece - 1) / kRowPiece) : 1u;
+  if (is_long) *any_long = 1u;
+}
+
+struct PiecesOf {
+  const uint32_t* pieces;
+  __device__ uint64_t operator()(int64_t i) const { return pieces[i]; }
+};
+
+// piece_offset[v] = where piece v begins: piece j > 0 of a row begins at the first space at or after byte
+// j * kRowPiece of the row (the row's end if there is none), so no word is cut.  first_piece[r] = index of row r's
+// first piece, first_piece[rows] = number of pieces.
+__global__ void piece_offsets_kernel(ColView col, const uint32_t* __restrict__ first_piece, int64_t pieces, int64_t* __restrict__ piece_offset)
+{
+  int64_t const v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (v > pieces) return;
+  int64_t const rows = col.size;
+  if (v == pieces) {
+    piece_offset[v] = col.off(rows);
+    return;
+  }
+  int64_t lo = 0, hi = rows - 1;  // the last row whose first piece is at or before v
+  while (lo < hi) {
+    int64_t const mid = (lo + hi + 1) >> 1;
+    if (static_cast<int64_t>(first_piece[mid]) <= v) lo = mid;
+    else hi = mid - 1;
+  }
+  int64_t const j = v - first_piece[lo];
+  int64_t p       = col.off(lo);
+  if (j > 0) {
+    int64_t const end = col.off(lo + 1);
+    p += j * kRowPiece;
+    while (p < end && col.chars[p] != ' ') ++p;
+  }
+  piece_offset[v] = p;
+}
+
+// offsets[r] = piece_token_offsets[first_piece[r]] for r in 0..rows
+__global__ void row_offsets_of_pieces_kernel(const int32_t* __restrict__ piece_token_offsets, const uint32_t* __restrict__ first_piece,
+                                             int64_t rows, int32_t* __restrict__ offsets)
+{
+  int64_t const r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (r <= rows) offsets[r] = piece_token_offsets[first_piece[r]];
+}
+
 struct CountOf {
   const int32_t* counts;
   __device__ uint64_t operator()(int64_t i) const { return static_cast<uint64_t>(counts[i]); }
@@ -1548,9 +1608,21 @@ void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
 
 int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* v) { return v ? v->table.unk_id : -1; }
 
+// may_cut_rows: very long rows may be cut into pieces that are tokenized as rows (false in the call that does the pieces)
+static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
+                                       int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out,
+                                       bool may_cut_rows);
+
 nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
                                                 int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_,
                                                 nvtext_amd_list_column* out)
+{
+  return tokenize_rows(input, vocabulary, max_words_per_row, stream_, mr_, out, true);
+}
+
+static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
+                                       int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out,
+                                       bool may_cut_rows)
 {
   using namespace nvtext_amd;
   if (!input || !vocabulary || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
@@ -1601,6 +1673,24 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   }
 
   ColView const v = make_view(*input);
+  // Without a word limit very long rows are cut into pieces (see long_rows_kernel): are there any?  The answer
+  // comes back with the two offsets read below.
+  bool const look_for_long_rows = may_cut_rows && max_words_per_row == 0;
+  size_t const cut_bytes[3]     = {look_for_long_rows ? static_cast<size_t>(rows) * sizeof(uint32_t) : 0,
+                                   look_for_long_rows ? (static_cast<size_t>(rows) + 1) * sizeof(uint32_t) : 0, look_for_long_rows ? 256u : 0u};
+  TempParts<3> const cut_temps(mr, cut_bytes);
+  uint32_t* const pieces      = cut_temps.part<uint32_t>(0);
+  uint32_t* const first_piece = cut_temps.part<uint32_t>(1);
+  uint32_t* const any_long    = cut_temps.part<uint32_t>(2);
+  uint32_t has_long           = 0;
+  if (look_for_long_rows) {
+    if (!cut_temps.ok()) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+    }
+    launch_fill_u32(any_long, 0u, 1, stream);
+    hipLaunchKernelGGL(long_rows_kernel, dim3(static_cast<unsigned>((rows + 255) / 256)), dim3(256), 0, stream, v, pieces, any_long);
+  }
   // first and last offset of the view (the reference reads the same two scalars,
   // cpp/src/strings/utilities.cu:180-190); they size the token arena
   size_t const ow = input->offsets_is_int64 ? 8 : 4;
@@ -1610,6 +1700,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     const uint8_t* d_off  = static_cast<const uint8_t*>(input->offsets) + static_cast<size_t>(input->offset) * ow;
     hipError_t e          = hipMemcpyAsync(buf, d_off, ow, hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipMemcpyAsync(buf + 8, d_off + static_cast<size_t>(rows) * ow, ow, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess && look_for_long_rows) e = hipMemcpyAsync(&has_long, any_long, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
     if (e != hipSuccess) {
       nvtext_amd_list_column_free(out, stream_, mr_);
@@ -1629,6 +1720,47 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   if (last_offset < first_offset) {
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_INVALID_ARGUMENT, "offsets are not monotone");
+  }
+  if (has_long != 0) {
+    // the pieces as a strings column of their own over the same chars (int64 offsets, no mask: validity is not
+    // consulted without a word limit), tokenized by this same function; then the rows' offsets from their first pieces
+    auto give_up = [&](nvtext_amd_status st, const char* what) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return fail(st, what);
+    };
+    Temp scan_tmp(mr, scan_temp_bytes(rows));
+    if (!scan_tmp.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+    device_exclusive_scan(PiecesOf{pieces}, static_cast<int64_t>(rows), first_piece, scan_tmp.as<uint64_t>(), stream);
+    uint64_t n_pieces = 0;
+    hipError_t e      = hipMemcpyAsync(&n_pieces, scan_tmp.as<uint64_t>() + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+    if (n_pieces > static_cast<uint64_t>(std::numeric_limits<int32_t>::max()) - 1) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+    Temp piece_offset(mr, (static_cast<size_t>(n_pieces) + 1) * sizeof(int64_t));
+    if (!piece_offset.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+    hipLaunchKernelGGL(piece_offsets_kernel, dim3(static_cast<unsigned>((n_pieces + 1 + 255) / 256)), dim3(256), 0, stream, v, first_piece,
+                       static_cast<int64_t>(n_pieces), piece_offset.as<int64_t>());
+    nvtext_amd_strings_column cut{};
+    cut.chars            = input->chars;
+    cut.offsets          = piece_offset.ptr;
+    cut.offsets_is_int64 = 1;
+    cut.size             = static_cast<int32_t>(n_pieces);
+    nvtext_amd_list_column of_pieces{};
+    nvtext_amd_status const st = tokenize_rows(&cut, vocabulary, 0, stream_, mr_, &of_pieces, false);
+    if (st != NVTEXT_AMD_SUCCESS) {
+      nvtext_amd_list_column_free(out, stream_, mr_);
+      return st;
+    }
+    hipLaunchKernelGGL(row_offsets_of_pieces_kernel, dim3(static_cast<unsigned>((rows + 1 + 255) / 256)), dim3(256), 0, stream, of_pieces.offsets,
+                       first_piece, static_cast<int64_t>(rows), out->offsets);
+    out->child       = of_pieces.child;  // the tokens are the pieces' tokens, in the same order
+    out->child_size  = of_pieces.child_size;
+    out->child_bytes = of_pieces.child_bytes;
+    of_pieces.child  = nullptr;
+    of_pieces.child_bytes = 0;
+    nvtext_amd_list_column_free(&of_pieces, stream_, mr_);
+    NVTEXT_HIP_TRY(hipGetLastError());
+    return NVTEXT_AMD_SUCCESS;
   }
   // word arena: one slot per possible word; row r gets floor(bytes/2) + 1 slots
   size_t const arena_slots = static_cast<size_t>((last_offset - first_offset) >> 1) + static_cast<size_t>(rows) + 1;
@@ -1729,9 +1861,10 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
         return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
       }
       ProfileScope ps("wordpiece_emit_kernel", stream);
-      // about 4096 words (at 5.6 bytes each) per walk
+      // about 4096 words (at 5.6 bytes each) per walk, judged by the mean row; where the rows are the pieces of very
+      // long rows (among ordinary rows, so the mean says little) a walk takes one row at a time
       int64_t const mean_bytes = (last_offset - first_offset) / rows + 1;
-      int block_rows           = kWave;
+      int block_rows           = may_cut_rows ? kWave : 1;
       while (block_rows > 1 && block_rows * mean_bytes > 4096 * 56 / 10) block_rows >>= 1;
       int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));

@@ -501,6 +501,34 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
     assert exp.child.size > 5000
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype):
+    """Rows of hundreds of kilobytes (which the library tokenizes in pieces cut at spaces when there is no word limit)
+    among short ones: with words of every length at the places where the cuts fall, a row that is one long word, a
+    row that is mostly spaces, null rows, and the same column sliced."""
+    rng = np.random.default_rng(77)
+    letters = list("abcdefghij")
+    vocab = ["[UNK]"] + letters + ["##" + c for c in letters] + ["ab", "abc", "##cd", "hello", "##llo"]
+    def text(nbytes, max_word):
+        words, total = [], 0
+        while total < nbytes:
+            w = "".join(rng.choice(letters, int(rng.integers(1, max_word + 1))))
+            words.append(w)
+            total += len(w) + 1
+        return " ".join(words)
+    rows = ["hello ab", text(70_000, 6), None, "", text(300_000, 40), "abc", "z" * 150_000, " " * 90_000 + "ab" + " " * 90_000,
+            text(1_100_000, 12), text(65_536, 3)[:65_536], text(65_537, 3)[:65_537], None, "ab cd"]
+    host = strings(rows, dtype)
+    dv = nv.WordPieceVocabulary(dev(nv, strings(vocab)))
+    ov = orc.Vocabulary(strings(vocab))
+    for view in (host, host.slice(1, 10)):
+        got = nv.wordpiece_tokenize(dev(nv, view), dv, 0).to_host()
+        assert_same(got, orc.wordpiece_tokenize(view, ov, 0, nthreads=8), "very long rows")
+    # with a word limit the rows are not cut (and end after the limit)
+    got = nv.wordpiece_tokenize(dev(nv, host), dv, 50).to_host()
+    assert_same(got, orc.wordpiece_tokenize(host, ov, 50, nthreads=8), "very long rows, word limit")
+
+
 @pytest.mark.parametrize("max_words", [0, 4])
 def test_wordpiece_long_runs_of_rows_without_bytes(nv, orc, max_words):
     """Hundreds of thousands of empty and null rows in a row, before, between and after rows with text: the rows are
