@@ -1358,7 +1358,20 @@ __global__ void piece_offsets_kernel(ColView col, const uint32_t* __restrict__ f
   if (j > 0) {
     int64_t const end = col.off(lo + 1);
     p += j * kRowPiece;
-    while (p < end && col.chars[p] != ' ') ++p;
+    // eight bytes at a time from an aligned address (ordinary text has a space within a few bytes; a stretch
+    // without one is read to its end)
+    const uint8_t* const chars = col.chars;
+    while (p < end && (reinterpret_cast<uintptr_t>(chars + p) & 7u) != 0 && chars[p] != ' ') ++p;
+    while (p + 8 <= end && chars[p] != ' ') {
+      uint2 const w      = *reinterpret_cast<const uint2*>(chars + p);
+      uint32_t const lo  = space_bytes(w.x), hi = space_bytes(w.y);
+      if ((lo | hi) != 0) {
+        p += lo ? (__builtin_ctz(lo) >> 3) : 4 + (__builtin_ctz(hi) >> 3);
+        break;
+      }
+      p += 8;
+    }
+    while (p < end && chars[p] != ' ') ++p;
   }
   piece_offset[v] = p;
 }
