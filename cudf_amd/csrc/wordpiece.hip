@@ -1316,8 +1316,8 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(ColVi
 // megabytes would take milliseconds while the rest of the device is idle.  Without a word limit the tokens of a row
 // are simply those of its words in order, so such a row can be cut at spaces into pieces that are tokenized as
 // rows of their own; the list offsets of the original rows are then those of their first pieces.
-constexpr int64_t kLongRow  = 64 * 1024;  // rows beyond this many bytes are cut
-constexpr int64_t kRowPiece = 32 * 1024;  // into pieces of about this many
+constexpr int64_t kLongRow  = 32 * 1024;  // rows beyond this many bytes are cut
+constexpr int64_t kRowPiece = 16 * 1024;  // into pieces of about this many
 
 // pieces[r] = pieces row r is cut into (1 for rows that stay whole); *any_long = 1 when some row is cut
 __global__ void long_rows_kernel(ColView col, uint32_t* __restrict__ pieces, uint32_t* __restrict__ any_long)

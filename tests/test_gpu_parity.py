@@ -517,7 +517,7 @@ def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype):
             total += len(w) + 1
         return " ".join(words)
     rows = ["hello ab", text(70_000, 6), None, "", text(300_000, 40), "abc", "z" * 150_000, " " * 90_000 + "ab" + " " * 90_000,
-            text(1_100_000, 12), text(65_536, 3)[:65_536], text(65_537, 3)[:65_537], None, "ab cd"]
+            text(1_100_000, 12), text(32_768, 3)[:32_768], text(32_769, 3)[:32_769], None, "ab cd"]
     host = strings(rows, dtype)
     dv = nv.WordPieceVocabulary(dev(nv, strings(vocab)))
     ov = orc.Vocabulary(strings(vocab))
