@@ -1174,8 +1174,9 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView
 }
 
 // ------------------------------------------------------------------ emit pass
-// Expands the word arena into the child column.  A wavefront takes 64 consecutive rows at a time
-// (lanes <-> rows for the descriptors), then walks ALL their words flat, lanes <-> words: because the
+// Expands the word arena into the child column.  A wavefront takes a block of consecutive rows at a time (at most
+// 64, fewer where rows have many tokens: emit_blocks_kernel; lanes <-> rows for the descriptors), then walks ALL
+// their words flat, lanes <-> words: because the
 // list offsets are a prefix sum in row order, the tokens of consecutive words are consecutive in the
 // child even across row boundaries, so only the block's first offset is needed.  Each word finds its
 // row by binary search in the block's word-count prefix (LDS).
@@ -1189,7 +1190,8 @@ struct EmitLds {
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
                                                                      const uint32_t* __restrict__ arena,
                                                                      const int32_t* __restrict__ nwords, OovResult* __restrict__ results,
-                                                                     const int32_t* __restrict__ offsets, int32_t* __restrict__ out, int block_rows,
+                                                                     const int32_t* __restrict__ offsets, int32_t* __restrict__ out,
+                                                                     const int32_t* __restrict__ block_first, int64_t nblocks,
                                                                      uint32_t* __restrict__ again, uint32_t* __restrict__ again_count)
 {
   // block_rows (1..64) rows per wavefront at a time: fewer when rows are long, so that the walks stay
@@ -1198,8 +1200,6 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
   int const lane        = lane_id();
   int const wave        = threadIdx.x / kWave;
   EmitLds& lds          = lds_all[wave];
-  int64_t const rows    = col.size;
-  int64_t const nblocks = (rows + block_rows - 1) / block_rows;
   int64_t const nwave   = static_cast<int64_t>(gridDim.x) * kTokWaves;
   auto lds_sync = [] {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1207,14 +1207,16 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
   for (int64_t blk = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave; blk < nblocks; blk += nwave) {
-    int64_t const r  = blk * block_rows + lane;
-    uint32_t W       = 0;
-    int64_t slot0    = 0;
-    if (lane < block_rows && r < rows) {
+    // rows [first, next) of the block: at most kWave
+    int32_t const first = block_first[blk], next = block_first[blk + 1];
+    int64_t const r     = static_cast<int64_t>(first) + lane;
+    uint32_t W          = 0;
+    int64_t slot0       = 0;
+    if (lane < next - first) {
       W     = static_cast<uint32_t>(nwords[r]);
       slot0 = arena_pos(col, first_offset, r);
     }
-    int32_t const base   = offsets[blk * block_rows];
+    int32_t const base   = offsets[first];
     uint32_t const incl  = wave_inclusive_scan(W);
     uint32_t const total = wave_bcast(incl, kWave - 1);
     lds.word_prefix[lane] = incl - W;
@@ -1309,6 +1311,26 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(ColVi
     int32_t* const d = out + results[q].tok[0];
     tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t j, int32_t id) { d[j] = id; });
   }
+}
+
+// The blocks of rows of the emit pass: block b begins with the first row r for which offsets[r] + kEmitRowWeight * r
+// reaches b * kEmitBlockWork, so a block holds at most kEmitBlockWork / kEmitRowWeight = 64 rows and, unless it is a
+// single row, fewer than kEmitBlockWork tokens, however uneven the rows are.  block_first has nblocks + 1 entries.
+constexpr int64_t kEmitRowWeight = 128;
+constexpr int64_t kEmitBlockWork = kEmitRowWeight * kWave;
+__global__ void emit_blocks_kernel(const int32_t* __restrict__ offsets, int64_t rows, int64_t nblocks, int32_t* __restrict__ block_first)
+{
+  int64_t const b = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (b > nblocks) return;
+  int64_t lo = 0, hi = rows;  // the first row in [0, rows] with that much work before it
+  if (b == nblocks) lo = rows;
+  int64_t const target = b * kEmitBlockWork;
+  while (lo < hi) {
+    int64_t const mid = (lo + hi) >> 1;
+    if (static_cast<int64_t>(offsets[mid]) + kEmitRowWeight * mid < target) lo = mid + 1;
+    else hi = mid;
+  }
+  block_first[b] = static_cast<int32_t>(lo);
 }
 
 // ------------------------------------------------------------------ very long rows
@@ -1874,16 +1896,21 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
         return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
       }
       ProfileScope ps("wordpiece_emit_kernel", stream);
-      // about 4096 words (at 5.6 bytes each) per walk, judged by the mean row; where the rows are the pieces of very
-      // long rows (among ordinary rows, so the mean says little) a walk takes one row at a time
-      int64_t const mean_bytes = (last_offset - first_offset) / rows + 1;
-      int block_rows           = may_cut_rows ? kWave : 1;
-      while (block_rows > 1 && block_rows * mean_bytes > 4096 * 56 / 10) block_rows >>= 1;
-      int64_t const emit_blocks = (static_cast<int64_t>(rows) + block_rows * kTokWaves - 1) / (block_rows * kTokWaves);
+      // the blocks of rows that a wavefront walks at a time: evened out by tokens (see emit_blocks_kernel)
+      int64_t const emit_work   = static_cast<int64_t>(total) + kEmitRowWeight * rows;
+      int64_t const nblocks     = (emit_work + kEmitBlockWork - 1) / kEmitBlockWork;
+      Temp block_first(mr, static_cast<size_t>(nblocks + 1) * sizeof(int32_t));
+      if (!block_first.ok()) {
+        nvtext_amd_list_column_free(out, stream_, mr_);
+        return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+      }
+      hipLaunchKernelGGL(emit_blocks_kernel, dim3(static_cast<unsigned>((nblocks + 1 + 255) / 256)), dim3(256), 0, stream, out->offsets,
+                         static_cast<int64_t>(rows), nblocks, block_first.as<int32_t>());
+      int64_t const emit_blocks = (nblocks + kTokWaves - 1) / kTokWaves;
       unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
                          arena, nwords, results, out->offsets,
-                         static_cast<int32_t*>(out->child), block_rows, longer, qsize + 1);
+                         static_cast<int32_t*>(out->child), block_first.as<int32_t>(), nblocks, longer, qsize + 1);
       // (the list of longer words has served its purpose by now: its memory takes the list of words to do again,
       // at most one entry per queued word)
       hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
