@@ -1066,6 +1066,7 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(ColView c
                                                                     OovResult* __restrict__ results, int32_t* __restrict__ counts,
                                                                     uint32_t* __restrict__ longer)
 {
+  if (*queue_size > queue_capacity) return;  // the queue was too small: the host repeats the passes with a larger one
   uint32_t const total  = min(*queue_size, queue_capacity);
   uint32_t const nwave  = gridDim.x * (kOovThreads / kWave);
   uint32_t const wave   = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
@@ -1145,6 +1146,7 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView
 {
   __shared__ uint32_t windows[kStage / 4][kOovThreads];
   uint32_t* const win    = &windows[0][threadIdx.x];
+  if (*queue_size > queue_capacity) return;  // (see wordpiece_oov_kernel)
   uint32_t const total   = min(*queue_size, queue_capacity);
   uint32_t const nwave   = gridDim.x * (kOovThreads / kWave);
   uint32_t const wave    = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
