@@ -175,12 +175,11 @@ def test_config4_minhash64_full_size(nv, orc):
     _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, ranges, "C4")
 
 
-@gpu
-def test_config5_utf8_pipeline_full_size(nv, orc):
+def _utf8_pipeline(nv, orc, w, token_ranges, normalize_ranges, minhash_ranges, what):
+    """tokenize, normalize_characters and minhash64 of the whole column `w.rows`; exact against the oracle on the given
+    row ranges, each also run as a slice of the column and compared with the matching part of the whole result."""
     import torch
-    w = datagen.config5()
     p = w.params
-    assert w.rows.size == 8_000_000 and w.rows.offsets.dtype == np.int64
     d = nv.DeviceStringsColumn.from_host(w.rows)
     dv = nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(w.vocab))
     ov = orc.Vocabulary(w.vocab)
@@ -189,12 +188,12 @@ def test_config5_utf8_pipeline_full_size(nv, orc):
     assert np.all(np.diff(offs) >= 0) and int(offs[-1]) == full.child_size
     child = _child(full)
     # exact against the oracle on row ranges, each also as a slice of the whole
-    for lo, hi in [(0, 1_000_000), (3_999_999, 4_600_001), (7_400_000, 8_000_000)]:
+    for lo, hi in token_ranges:
         hs = w.rows.slice(lo, hi)
         exp = orc.wordpiece_tokenize(hs, ov, p["max_words_per_row"], nthreads=16)
         got = nv.wordpiece_tokenize(d.slice(lo, hi, hs.null_count), dv, p["max_words_per_row"])
-        _same(got.to_host(), exp, f"C5 tokenize rows {lo}:{hi}")
-        assert torch.equal(_child(got), child[int(offs[lo]): int(offs[hi])]), f"C5 tokenize: slice {lo}:{hi} of the whole"
+        _same(got.to_host(), exp, f"{what} tokenize rows {lo}:{hi}")
+        assert torch.equal(_child(got), child[int(offs[lo]): int(offs[hi])]), f"{what} tokenize: slice {lo}:{hi} of the whole"
         assert np.array_equal(exp.offsets.astype(np.int64) + int(offs[lo]), offs[lo: hi + 1].astype(np.int64))
     del full, child
     torch.cuda.empty_cache()
@@ -207,15 +206,77 @@ def test_config5_utf8_pipeline_full_size(nv, orc):
     assert whole.offsets.dtype == torch.int64 and whole.size == w.rows.size
     woff = whole.offsets.cpu().numpy()
     assert woff[0] == 0 and np.all(np.diff(woff) >= 0) and int(woff[-1]) == whole.chars.numel() > 0x7FFFFFFF
-    for lo, hi in [(0, 400_000), (3_999_999, 4_300_001), (7_700_000, 8_000_000)]:
+    for lo, hi in normalize_ranges:
         hs = w.rows.slice(lo, hi)
         exp = normalize_py.normalize_characters_native(hs, True, [t.encode() for t in tokens], nthreads=16)
         got = nv.normalize_characters(d.slice(lo, hi, hs.null_count), normalizer)
         gh = got.to_host()
-        assert np.array_equal(gh.offsets, exp.offsets) and np.array_equal(gh.chars, exp.chars), f"C5 normalize rows {lo}:{hi}"
-        assert torch.equal(got.chars, whole.chars[int(woff[lo]): int(woff[hi])]), f"C5 normalize: slice {lo}:{hi} of the whole"
+        assert np.array_equal(gh.offsets, exp.offsets) and np.array_equal(gh.chars, exp.chars), f"{what} normalize rows {lo}:{hi}"
+        assert torch.equal(got.chars, whole.chars[int(woff[lo]): int(woff[hi])]), f"{what} normalize: slice {lo}:{hi} of the whole"
         assert np.array_equal(exp.offsets.astype(np.int64) + int(woff[lo]), woff[lo: hi + 1])
     del whole
     torch.cuda.empty_cache()
     a, b, da, db = _params(nv, p)
-    _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, [(0, 20_000), (6_000_000, 6_010_000)], "C5 minhash64")
+    _minhash_properties(nv, nv.minhash64, orc.minhash64, w, d, da, db, a, b, minhash_ranges, what + " minhash64")
+    return d
+
+
+@gpu
+def test_config5_utf8_pipeline_full_size(nv, orc):
+    w = datagen.config5()
+    assert w.rows.size == 8_000_000 and w.rows.offsets.dtype == np.int64
+    _utf8_pipeline(nv, orc, w, [(0, 1_000_000), (3_999_999, 4_600_001), (7_400_000, 8_000_000)],
+                   [(0, 400_000), (3_999_999, 4_300_001), (7_700_000, 8_000_000)], [(0, 20_000), (6_000_000, 6_010_000)], "C5")
+
+
+@gpu
+def test_utf8_pipeline_on_more_than_4_gib_of_chars(nv, orc):
+    """The same pipeline on a column a third larger than C5: its chars pass 2^32 bytes (byte offsets that need more than
+    32 bits) and its words pass 2^31 slots of the tokenizer's word table.  The row ranges checked against the oracle
+    straddle that place and lie beyond it."""
+    w = datagen.config5(1.3)
+    rows, off = w.rows.size, w.rows.offsets
+    assert off.dtype == np.int64 and int(off[-1]) > (1 << 32) + (1 << 29)
+    at = int(np.searchsorted(off, 1 << 32))  # the first row that begins at or beyond 4 GiB
+    assert 200_000 < at < rows - 600_000
+    d = _utf8_pipeline(nv, orc, w, [(at - 200_000, at + 200_000), (rows - 500_000, rows)],
+                       [(at - 100_000, at + 100_000), (rows - 300_000, rows)], [(at - 5_000, at + 5_000), (rows - 10_000, rows)],
+                       "C5 x1.3")
+    # minhash (uint32) and jaccard_index of rows r / r + 1 across the same place and at the end
+    a, b = datagen.make_params(32, 32, 7)
+    for lo, hi in [(at - 20_000, at + 20_000), (rows - 20_001, rows - 1)]:
+        h1, h2 = w.rows.slice(lo, hi), w.rows.slice(lo + 1, hi + 1)
+        d1, d2 = d.slice(lo, hi, 0), d.slice(lo + 1, hi + 1, 0)
+        _same(nv.minhash(d1, 3, a, b, 6).to_host(), orc.minhash(h1, 3, a, b, 6, nthreads=16), f"C5 x1.3 minhash rows {lo}:{hi}")
+        got, exp = nv.jaccard_index(d1, d2, 5).to_host(), orc.jaccard_index(h1, h2, 5, nthreads=16)
+        assert got.size == exp.size and got.null_count == exp.null_count == 0
+        assert np.array_equal(got.values.view(np.uint32), exp.values.view(np.uint32)), f"C5 x1.3 jaccard rows {lo}:{hi}"
+
+
+@gpu
+@pytest.mark.parametrize("rows", [4096, 40])
+def test_tokenize_reports_more_tokens_than_a_list_column_holds(nv, rows):
+    """2^31 one-letter words and a few more: the child would pass INT32_MAX entries, which the reference reports as
+    std::overflow_error (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:331-335).  With 4096 rows each is a
+    megabyte, with 40 each is a hundred megabytes; either way the rows are tokenized in pieces, so the error
+    comes from the call over the pieces.  The library must give everything back and go on working afterwards."""
+    import torch
+    per_row = (1 << 31) // rows + 1                      # words per row
+    chars = np.tile(np.frombuffer(b"a ", np.uint8), per_row * rows)
+    offsets = np.arange(rows + 1, dtype=np.int64) * (2 * per_row)
+    host = HostStringsColumn(chars, offsets, None, rows, 0, 0)
+    dv = nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(["[UNK]", "a", "b"])))
+    d = nv.DeviceStringsColumn.from_host(host)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    with pytest.raises(OverflowError, match="exceeds the column size limit"):
+        nv.wordpiece_tokenize(d, dv, 0)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    # one row less stays below the limit: the same call succeeds and every word is the token of "a"
+    fewer = nv.wordpiece_tokenize(d.slice(0, rows - 1, 0), dv, 0)
+    assert fewer.child_size == per_row * (rows - 1)
+    child = _child(fewer)
+    assert int(child.min()) == 1 and int(child.max()) == 1
+    offs = fewer.offsets.view(torch.int32)[:rows].cpu().numpy()
+    assert np.array_equal(offs.astype(np.int64), np.arange(rows, dtype=np.int64) * per_row)
