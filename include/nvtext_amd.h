@@ -197,7 +197,8 @@ nvtext_amd_status nvtext_amd_minhash64_ngrams(const nvtext_amd_list_strings_colu
  * For every row r: A, B = the sets of non-zero MurmurHash3_x86_32(seed 0) values of the `width`-character
  * windows of input1[r], input2[r] (the window rule of nvtext_amd_minhash); result[r] = |A n B| / |A u B| as
  * float32 (0 when both sets are empty).  A row that is null in either input is null in the result (its value
- * is unspecified); the result has a null mask only if an input has nulls.  Synchronises the stream once. */
+ * is unspecified); the result has a null mask only if an input has nulls.  Synchronises the stream once.
+ * Limit: two rows of one pair may have 2^32 / 3 bytes together (1.43 GB); beyond that NVTEXT_AMD_OVERFLOW. */
 nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* input1,
                                            const nvtext_amd_strings_column* input2,
                                            int32_t width,

@@ -280,3 +280,87 @@ def test_tokenize_reports_more_tokens_than_a_list_column_holds(nv, rows):
     assert int(child.min()) == 1 and int(child.max()) == 1
     offs = fewer.offsets.view(torch.int32)[:rows].cpu().numpy()
     assert np.array_equal(offs.astype(np.int64), np.arange(rows, dtype=np.int64) * per_row)
+
+
+@gpu
+def test_rows_of_gigabytes(nv, orc):
+    """A row of 2.1 GB (2047 copies of a megabyte of text: near the 2^31 - 1 bytes a row may have) and one of 0.3 GB
+    among short rows.  What the oracle says of one copy fixes the result: the tokens and the normalized bytes of
+    the row are those of the copy, repeated (a copy ends with a space), and its windows are those of the copy
+    continued by its own first width - 1 bytes."""
+    import torch
+    from oracle import normalize_py
+    w = datagen.config2(0.004)
+    text = w.rows.chars
+    def block(at):
+        b = text[at: at + (1 << 20)].copy()
+        b[-1] = 0x20
+        assert b[0] != 0x20
+        return b
+    A, B = block(0), block(1 << 21)
+    kA, kB, width = 2047, 300, 5
+    small = [np.frombuffer(b"hello ab", np.uint8), np.frombuffer(b"ab", np.uint8)]
+    parts = [small[0], np.tile(A, kA), np.tile(B, kB), small[1]]
+    sizes = [len(parts[0]), len(parts[1]), 0, len(parts[2]), len(parts[3])]          # row 2 is null
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    host = HostStringsColumn(np.concatenate(parts), offsets, np.array([0b11011], np.uint32), 5, 0, 1)
+    assert int(offsets[2] - offsets[1]) == kA << 20 > (1 << 31) - (1 << 21)
+    d = nv.DeviceStringsColumn.from_host(host)
+    def one(chars):
+        return HostStringsColumn(np.ascontiguousarray(chars), np.array([0, len(chars)], np.int64), None, 1, 0, 0)
+    copies = [(one(small[0]), 1), (one(A), kA), None, (one(B), kB), (one(small[1]), 1)]
+    wrapped = [one(small[0]), one(np.concatenate([A, A[:width - 1]])), None, one(np.concatenate([B, B[:width - 1]])), one(small[1])]
+
+    # wordpiece_tokenize: without a word limit (the long rows are tokenized in pieces), and with one
+    dv = nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(w.vocab))
+    ov = orc.Vocabulary(w.vocab)
+    for max_words in (0, 1000):
+        exp = [np.zeros(0, np.int32) if c is None else
+               (np.tile(orc.wordpiece_tokenize(c[0], ov, 0, nthreads=1).child, c[1]) if max_words == 0
+                else orc.wordpiece_tokenize(c[0], ov, max_words, nthreads=1).child) for c in copies]
+        got = nv.wordpiece_tokenize(d, dv, max_words)
+        assert got.size == 5 and got.null_count == 1
+        offs = got.offsets.view(torch.int32)[:6].cpu().numpy()
+        assert np.array_equal(offs, np.concatenate([[0], np.cumsum([len(e) for e in exp])])), f"max_words={max_words}"
+        child = _child(got)
+        for r in range(5):
+            assert torch.equal(child[int(offs[r]): int(offs[r + 1])].cpu(), torch.from_numpy(exp[r])), f"tokens of row {r}, max_words={max_words}"
+        del got, child
+    torch.cuda.empty_cache()
+
+    # minhash, minhash64
+    for fn, ofn, bits in ((nv.minhash, orc.minhash, 32), (nv.minhash64, orc.minhash64, 64)):
+        a, b = datagen.make_params(8, bits, 5)
+        got = fn(d, 9, a, b, width).to_host()
+        assert np.array_equal(got.offsets, [0, 8, 16, 16, 24, 32]) and got.null_count == 1
+        for r, c in enumerate(wrapped):
+            if c is not None:
+                at = int(got.offsets[r])
+                assert np.array_equal(got.child[at: at + 8], ofn(c, 9, a, b, width, nthreads=1).child), f"minhash{bits} of row {r}"
+
+    # normalize_characters
+    norm = nv.normalize_characters(d, nv.CharacterNormalizer(True, None))
+    noff = norm.offsets.cpu().numpy()
+    for r, c in enumerate(copies):
+        lo, hi = int(noff[r]), int(noff[r + 1])
+        if c is None:
+            assert lo == hi
+            continue
+        e = torch.from_numpy(normalize_py.normalize_characters_native(c[0], True, [], nthreads=1).chars)
+        assert hi - lo == len(e) * c[1], f"normalized size of row {r}"
+        assert bool((norm.chars[lo:hi].view(c[1], len(e)).cpu() == e).all()), f"normalized bytes of row {r}"
+    del norm
+    torch.cuda.empty_cache()
+
+    # jaccard_index: 300 copies of B against 300 copies of A share what the two copies (continued) share; a pair of
+    # more than 2^32 / 3 bytes together is refused
+    other = HostStringsColumn(np.concatenate([small[0], np.tile(A, kB), small[0]]),
+                              np.array([0, 8, 8 + (kB << 20), 16 + (kB << 20)], np.int64), None, 3, 0, 0)
+    d2 = nv.DeviceStringsColumn.from_host(other)
+    got = nv.jaccard_index(d.slice(2, 5, 1), d2, width).to_host()
+    assert got.size == 3 and got.null_count == 1 and list(got.validity()) == [False, True, True]
+    exp = orc.jaccard_index(wrapped[3], wrapped[1], width, nthreads=1)
+    assert got.values.view(np.uint32)[1] == exp.values.view(np.uint32)[0]
+    assert got.values[2] == orc.jaccard_index(one(small[1]), one(small[0]), width, nthreads=1).values[0]
+    with pytest.raises(OverflowError, match="row pair is too long"):
+        nv.jaccard_index(d.slice(1, 2, 0), d.slice(1, 2, 0), width)
