@@ -364,3 +364,32 @@ def test_rows_of_gigabytes(nv, orc):
     assert got.values[2] == orc.jaccard_index(one(small[1]), one(small[0]), width, nthreads=1).values[0]
     with pytest.raises(OverflowError, match="row pair is too long"):
         nv.jaccard_index(d.slice(1, 2, 0), d.slice(1, 2, 0), width)
+
+
+@gpu
+def test_minhash_ngrams_on_a_child_of_more_than_4_gib(nv, orc):
+    """LIST<STRING> rows whose strings child holds 4.7 GB (int64 child offsets): the rows whose elements lie across
+    byte 2^32 of the child, and the last ones, against the oracle; each range also as a slice of the whole."""
+    import torch
+    from cudf_amd.arrow_host import HostListStringsColumn
+    rng = np.random.default_rng(5)
+    chars = np.tile(rng.integers(97, 123, 1 << 26, dtype=np.uint8), 70)
+    each, per_row = 47, 37                       # bytes per element, elements per row
+    elements = len(chars) // each
+    rows = elements // per_row
+    child = HostStringsColumn(chars, np.arange(elements + 1, dtype=np.int64) * each, None, elements, 0, 0)
+    host = HostListStringsColumn(np.arange(rows + 1, dtype=np.int32) * per_row, child, None, rows, 0, 0)
+    assert int(child.offsets[rows * per_row]) > (1 << 32) + (1 << 28)
+    d = nv.DeviceListStringsColumn.from_host(host)
+    at = (1 << 32) // (each * per_row)           # the row that holds byte 2^32
+    for fn, ofn, bits in ((nv.minhash_ngrams, orc.minhash_ngrams, 32), (nv.minhash64_ngrams, orc.minhash64_ngrams, 64)):
+        a, b = datagen.make_params(16, bits, 3)
+        whole = fn(d, 4, 11, a, b)
+        assert whole.size == rows and whole.child_size == rows * 16
+        child_all = _child(whole).view(rows, 16)
+        for lo, hi in [(at - 3000, at + 3000), (rows - 6000, rows)]:
+            exp = ofn(host.slice(lo, hi), 4, 11, a, b, nthreads=16)
+            got = fn(d.slice(lo, hi, 0), 4, 11, a, b)
+            _same(got.to_host(), exp, f"ngrams{bits} rows {lo}:{hi}")
+            assert torch.equal(_child(got).view(hi - lo, 16), child_all[lo:hi]), f"ngrams{bits}: slice {lo}:{hi} of the whole"
+        del whole, child_all
