@@ -578,3 +578,56 @@ def test_cpp_api_program():
     p = subprocess.run([exe], capture_output=True, text=True, timeout=110)
     assert p.returncode == 0, p.stdout + p.stderr
     assert "ALL PASSED" in p.stdout
+
+
+# ----------------------------------------------------------------------------- the caller's stream
+def test_every_operation_on_streams_of_the_caller(nv, orc):
+    """Everything so far ran on the default stream.  Here the inputs are uploaded and the operations issued on two
+    streams the caller made (which do not synchronise with the default stream), calls alternating between them; a
+    kernel or copy that the library put on another stream than the one it was given would race with the upload or
+    with the result's download."""
+    import torch
+    from cudf_amd import datagen
+    from oracle import normalize_py
+    w = datagen.config5(0.02)  # 160k UTF-8 rows, int64 offsets, 250k-entry vocabulary
+    host, p = w.rows, w.params
+    a32, b32 = datagen.make_params(32, 32, 1)
+    a64, b64 = datagen.make_params(32, 64, 2)
+    lists = datagen.words_as_lists(datagen.config3(0.005).rows)
+    h1, h2 = host.slice(0, host.size - 1), host.slice(1, host.size)
+    ov = orc.Vocabulary(w.vocab)
+    expected = {
+        "tokens": orc.wordpiece_tokenize(host, ov, p["max_words_per_row"], nthreads=8),
+        "minhash": orc.minhash(host, 3, a32, b32, 5, nthreads=8),
+        "minhash64": orc.minhash64(host, 4, a64, b64, 7, nthreads=8),
+        "ngrams": orc.minhash_ngrams(lists, 3, 5, a32, b32, nthreads=8),
+        "normalized": normalize_py.normalize_characters_native(host, True, [b"[CLS]"], nthreads=8),
+        "jaccard": orc.jaccard_index(h1, h2, 5, nthreads=8),
+    }
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [{}, {}]
+    for turn in range(2):
+        for k, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                if turn == 0:
+                    d = dev(nv, host)
+                    got[k]["d"] = d
+                    got[k]["vocab"] = nv.WordPieceVocabulary(dev(nv, w.vocab))
+                    got[k]["normalizer"] = nv.CharacterNormalizer(True, dev(nv, strings(["[CLS]"])))
+                    got[k]["minhash"] = nv.minhash(d, 3, a32, b32, 5)
+                    got[k]["minhash64"] = nv.minhash64(d, 4, a64, b64, 7)
+                    got[k]["ngrams"] = nv.minhash_ngrams(nv.DeviceListStringsColumn.from_host(lists), 3, 5, a32, b32)
+                else:
+                    d = got[k]["d"]
+                    got[k]["tokens"] = nv.wordpiece_tokenize(d, got[k]["vocab"], p["max_words_per_row"])
+                    got[k]["normalized"] = nv.normalize_characters(d, got[k]["normalizer"])
+                    got[k]["jaccard"] = nv.jaccard_index(d.slice(0, host.size - 1, 0), d.slice(1, host.size, 0), 5)
+    for k, s in enumerate(streams):
+        with torch.cuda.stream(s):
+            for name in ("tokens", "minhash", "minhash64", "ngrams"):
+                assert_same(got[k][name].to_host(), expected[name], f"{name} on stream {k}")
+            n = got[k]["normalized"].to_host()
+            assert np.array_equal(n.offsets, expected["normalized"].offsets) and np.array_equal(n.chars, expected["normalized"].chars), f"normalized on stream {k}"
+            j = got[k]["jaccard"].to_host()
+            assert np.array_equal(j.values.view(np.uint32), expected["jaccard"].values.view(np.uint32)), f"jaccard on stream {k}"
+    torch.cuda.synchronize()
