@@ -32,9 +32,16 @@ class _TorchAllocator:
 
     def __init__(self):
         self.live: Dict[int, object] = {}
+        # for tests of the library's error paths: when set to n, the n + 1-th request from now and all later ones
+        # are refused until it is set to None again
+        self.fail_after: Optional[int] = None
         torch = _torch()
 
         def _alloc(ctx, nbytes, stream):
+            if self.fail_after is not None:
+                if self.fail_after == 0:
+                    return None
+                self.fail_after -= 1
             try:
                 t = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda")
             except Exception:  # out of memory -> NULL, reported as ALLOC_FAILED

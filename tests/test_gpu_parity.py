@@ -631,3 +631,76 @@ def test_every_operation_on_streams_of_the_caller(nv, orc):
             j = got[k]["jaccard"].to_host()
             assert np.array_equal(j.values.view(np.uint32), expected["jaccard"].values.view(np.uint32)), f"jaccard on stream {k}"
     torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- a failing allocator
+def test_allocation_failures_are_reported_and_leak_nothing(nv, orc):
+    """The caller's allocator refuses the n-th request of a call and every later one, for every n until the call
+    succeeds.  Each failed call reports NVTEXT_AMD_ALLOC_FAILED (MemoryError in this binding) and has given back what
+    it had been given; the call that succeeds has the oracle's result."""
+    from oracle import normalize_py
+    from cudf_amd import datagen
+    rng = np.random.default_rng(3)
+    vocab = strings(["[UNK]", "hello", "world", "##s", "a", "b", "##b", "ab"])
+    words = ["hello", "worlds", "a", "abb", "zzz", "b"]
+    rows = [None if i % 7 == 3 else " ".join(rng.choice(words, int(rng.integers(0, 30)))) for i in range(2000)]
+    rows[11] = " ".join(rng.choice(words, 12_000))   # beyond 32 KiB: cut into pieces when there is no word limit
+    rows[12] = rows[11][:30_000]                      # a pair for jaccard_index' set in global memory
+    host = strings(rows, np.int64)
+    d = dev(nv, host)
+    dv, ov = nv.WordPieceVocabulary(dev(nv, vocab)), orc.Vocabulary(vocab)
+    a32, b32 = datagen.make_params(20, 32, 1)
+    a64, b64 = datagen.make_params(20, 64, 2)
+    lists = gc.list_strings([None if i % 5 == 2 else [str(w) for w in rng.choice(words, int(rng.integers(0, 9)))] for i in range(300)])
+    dl = nv.DeviceListStringsColumn.from_host(lists)
+    h1, h2 = host.slice(0, host.size - 1), host.slice(1, host.size)
+    d1, d2 = d.slice(0, host.size - 1, h1.null_count), d.slice(1, host.size, h2.null_count)
+    normalizer = nv.CharacterNormalizer(True, None)
+
+    def lists_equal(got, exp, what):
+        assert_same(got.to_host(), exp, what)
+
+    def strings_equal(got, exp, what):
+        g = got.to_host()
+        assert np.array_equal(g.offsets, exp.offsets) and np.array_equal(g.chars, exp.chars), what
+        assert np.array_equal(g.validity(), exp.validity()), what
+
+    def floats_equal(got, exp, what):
+        g, v = got.to_host(), exp.validity()
+        assert g.null_count == exp.null_count and np.array_equal(g.validity(), v), what
+        assert np.array_equal(g.values.view(np.uint32)[v], exp.values.view(np.uint32)[v]), what
+
+    calls = [
+        ("tokenize", lambda: nv.wordpiece_tokenize(d, dv, 0), lambda: orc.wordpiece_tokenize(host, ov, 0, nthreads=4), lists_equal),
+        ("tokenize, word limit", lambda: nv.wordpiece_tokenize(d, dv, 5), lambda: orc.wordpiece_tokenize(host, ov, 5, nthreads=4), lists_equal),
+        ("minhash", lambda: nv.minhash(d, 1, a32, b32, 4), lambda: orc.minhash(host, 1, a32, b32, 4, nthreads=4), lists_equal),
+        ("minhash64", lambda: nv.minhash64(d, 1, a64, b64, 4), lambda: orc.minhash64(host, 1, a64, b64, 4, nthreads=4), lists_equal),
+        ("minhash_ngrams", lambda: nv.minhash_ngrams(dl, 2, 1, a32, b32), lambda: orc.minhash_ngrams(lists, 2, 1, a32, b32), lists_equal),
+        ("minhash64_ngrams", lambda: nv.minhash64_ngrams(dl, 2, 1, a64, b64), lambda: orc.minhash64_ngrams(lists, 2, 1, a64, b64), lists_equal),
+        ("normalize", lambda: nv.normalize_characters(d, normalizer),
+         lambda: normalize_py.normalize_characters_native(host, True, [], nthreads=4), strings_equal),
+        ("jaccard", lambda: nv.jaccard_index(d1, d2, 5), lambda: orc.jaccard_index(h1, h2, 5, nthreads=4), floats_equal),
+    ]
+    mr = nv._mr()
+    held = len(mr.live)
+    try:
+        for name, call, expect, same in calls:
+            refused = 0
+            for n in range(40):
+                mr.fail_after = n
+                try:
+                    got = call()
+                except MemoryError:
+                    refused += 1
+                    assert len(mr.live) == held, f"{name}: buffers kept after the failure of request {n}"
+                    continue
+                finally:
+                    mr.fail_after = None
+                assert len(mr.live) == held, f"{name}: buffers kept after success"
+                same(got, expect(), name)
+                break
+            else:
+                raise AssertionError(f"{name} still fails with 40 requests granted")
+            assert refused >= 2, f"{name}: only {refused} requests seen"
+    finally:
+        mr.fail_after = None
