@@ -704,3 +704,64 @@ def test_allocation_failures_are_reported_and_leak_nothing(nv, orc):
             assert refused >= 2, f"{name}: only {refused} requests seen"
     finally:
         mr.fail_after = None
+
+
+# ----------------------------------------------------------------------------- several host threads
+def test_host_threads_share_a_vocabulary_and_a_normalizer(nv, orc):
+    """Four host threads, each with a stream of its own, call the operations at the same time on the same input
+    columns, vocabulary and normalizer (which are immutable once made); every result is the oracle's."""
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    from cudf_amd import datagen
+    from oracle import normalize_py
+    w = datagen.config5(0.01)
+    host, p = w.rows, w.params
+    a32, b32 = datagen.make_params(16, 32, 1)
+    a64, b64 = datagen.make_params(16, 64, 2)
+    h1, h2 = host.slice(0, host.size - 1), host.slice(1, host.size)
+    ov = orc.Vocabulary(w.vocab)
+    exp_tokens = orc.wordpiece_tokenize(host, ov, p["max_words_per_row"], nthreads=8)
+    exp_mh = orc.minhash(host, 3, a32, b32, 5, nthreads=8)
+    exp_mh64 = orc.minhash64(host, 4, a64, b64, 7, nthreads=8)
+    exp_norm = normalize_py.normalize_characters_native(host, True, [], nthreads=8)
+    exp_j = orc.jaccard_index(h1, h2, 5, nthreads=8)
+    d = dev(nv, host)
+    dv = nv.WordPieceVocabulary(dev(nv, w.vocab))
+    normalizer = nv.CharacterNormalizer(True, None)
+    d1, d2 = d.slice(0, host.size - 1, 0), d.slice(1, host.size, 0)
+    torch.cuda.synchronize()
+
+    def worker(k):
+        out = []
+        with torch.cuda.stream(torch.cuda.Stream()):
+            for turn in range(3):
+                order = [(turn + k + i) % 5 for i in range(5)]
+                for what in order:
+                    if what == 0:
+                        out.append(("tokens", nv.wordpiece_tokenize(d, dv, p["max_words_per_row"]).to_host()))
+                    elif what == 1:
+                        out.append(("minhash", nv.minhash(d, 3, a32, b32, 5).to_host()))
+                    elif what == 2:
+                        out.append(("minhash64", nv.minhash64(d, 4, a64, b64, 7).to_host()))
+                    elif what == 3:
+                        out.append(("normalized", nv.normalize_characters(d, normalizer).to_host()))
+                    else:
+                        out.append(("jaccard", nv.jaccard_index(d1, d2, 5).to_host()))
+        return out
+
+    with ThreadPoolExecutor(4) as pool:
+        results = list(pool.map(worker, range(4)))
+    for k, out in enumerate(results):
+        assert len(out) == 15
+        for name, got in out:
+            what = f"{name} from thread {k}"
+            if name == "tokens":
+                assert_same(got, exp_tokens, what)
+            elif name == "minhash":
+                assert_same(got, exp_mh, what)
+            elif name == "minhash64":
+                assert_same(got, exp_mh64, what)
+            elif name == "normalized":
+                assert np.array_equal(got.offsets, exp_norm.offsets) and np.array_equal(got.chars, exp_norm.chars), what
+            else:
+                assert np.array_equal(got.values.view(np.uint32), exp_j.values.view(np.uint32)), what
