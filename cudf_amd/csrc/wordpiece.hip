@@ -1185,12 +1185,11 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView
 // their words flat, lanes <-> words: because the
 // list offsets are a prefix sum in row order, the tokens of consecutive words are consecutive in the
 // child even across row boundaries, so only the block's first offset is needed.  Each word finds its
-// row by binary search in the block's word-count prefix (LDS).
+// row by binary search in the block's word-count prefix (LDS); its lane then writes its tokens (one, or the up to
+// kOovKeep that the out-of-vocabulary pass left in its result record) behind those of the lanes below it.
 struct EmitLds {
   uint32_t word_prefix[kWave + 1];  // words before row k of the block
   int64_t slot0[kWave];             // arena slot of word 0 of row k
-  uint32_t first_token[kWave + 1];  // of the 64 words in flight: (token count << 16) | index of the word's first token
-  uint32_t value[kWave];            // their arena values
 };
 
 __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
@@ -1240,10 +1239,15 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
         if (lds.word_prefix[lo + step] <= j) lo += step;
       return arena[lds.slot0[lo] + (j - lds.word_prefix[lo])];
     };
-    // tokens of flat word j whose arena value is v: one, or what the out-of-vocabulary pass found
-    auto count_of = [&](uint32_t j, uint32_t v) -> uint32_t {
+    // tokens of flat word j whose arena value is v: one, or what the out-of-vocabulary pass found (its whole
+    // result record is fetched here, once)
+    auto count_of = [&](uint32_t j, uint32_t v, uint4& ra, uint4& rb) -> uint32_t {
       if (j >= total) return 0u;
-      return ((v & kOovMark) != 0 && v != 0xFFFFFFFFu) ? results[v & ~kOovMark].count : 1u;
+      if ((v & kOovMark) == 0 || v == 0xFFFFFFFFu) return 1u;
+      const uint4* const src = reinterpret_cast<const uint4*>(results + (v & ~kOovMark));
+      ra = src[0];
+      rb = src[1];
+      return rb.w;  // OovResult: seven tokens, then the count
     };
 
     int32_t* const dst = out + base;
@@ -1251,48 +1255,40 @@ __global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col
     // three stages in flight: arena value two rounds ahead, token count one round ahead, the round being written
     uint32_t v_nxt = load_value(lane);
     uint32_t v_far = load_value(kWave + lane);
-    uint32_t c_nxt = count_of(lane, v_nxt);
+    uint4 a_nxt = make_uint4(0u, 0u, 0u, 0u), b_nxt = a_nxt;
+    uint32_t c_nxt = count_of(lane, v_nxt, a_nxt, b_nxt);
     for (uint32_t j0 = 0; j0 < total; j0 += kWave) {
       uint32_t const value = v_nxt, cnt = c_nxt;
+      uint4 const ra = a_nxt, rb = b_nxt;
       v_nxt = v_far;
-      c_nxt = count_of(j0 + kWave + lane, v_nxt);
+      c_nxt = count_of(j0 + kWave + lane, v_nxt, a_nxt, b_nxt);
       v_far = load_value(j0 + 2 * kWave + lane);
       uint32_t const here   = min(total - j0, static_cast<uint32_t>(kWave));  // words of this round (every word has >= 1 token)
       uint32_t const incl2  = wave_inclusive_scan(cnt);
       uint32_t const tokens = wave_bcast(incl2, kWave - 1);
       bool const marked     = static_cast<uint32_t>(lane) < here && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
-      if (tokens == here && ballot64(marked) == 0) {
-        // one token per word and none from the queue: the arena values are the tokens
-        if (static_cast<uint32_t>(lane) < here) dst[done + lane] = static_cast<int32_t>(value);
+      // lanes <-> words: every lane writes its word's tokens behind those of the words below it, token k of all
+      // words at a time (a word from the queue has up to kOovKeep of them in its record)
+      int32_t* const mine = dst + done + (incl2 - cnt);
+      if (marked && cnt > kOovKeep) {
+        // more pieces than a result record keeps (seldom): noted for wordpiece_retokenize_kernel, with the
+        // place of the word's first token in the child left where its tokens would have been
+        uint32_t const q = value & ~kOovMark;
+        again[atomicAdd(again_count, 1u)] = q;
+        results[q].tok[0]                 = base + static_cast<int32_t>(done + (incl2 - cnt));
       } else {
-        // lanes <-> tokens: each finds its word among the 64 by binary search over the words' first-token indices
-        lds.first_token[lane] = (cnt << 16) | (incl2 - cnt);
-        if (lane == kWave - 1) lds.first_token[kWave] = tokens;
-        lds.value[lane] = value;
-        lds_sync();
-        for (uint32_t t = lane; t < tokens; t += kWave) {
-          uint32_t lo = 0;
-#pragma unroll
-          for (uint32_t step = kWave / 2; step > 0; step >>= 1)
-            if ((lds.first_token[lo + step] & 0xFFFFu) <= t) lo += step;
-          uint32_t const ft = lds.first_token[lo];
-          uint32_t const v  = lds.value[lo];
-          uint32_t const k  = t - (ft & 0xFFFFu);
-          uint32_t const c  = ft >> 16;
-          bool const oov    = (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
-          if (!oov) {
-            dst[done + t] = static_cast<int32_t>(v);
-          } else if (c <= kOovKeep) {
-            dst[done + t] = results[v & ~kOovMark].tok[k];
-          } else if (k == 0) {
-            // more pieces than a result record keeps (seldom): noted for wordpiece_retokenize_kernel, with the
-            // place of the word's first token in the child left where its tokens would have been
-            uint32_t const q = v & ~kOovMark;
-            again[atomicAdd(again_count, 1u)] = q;
-            results[q].tok[0]                 = base + static_cast<int32_t>(done + t);
+        uint32_t const mc = static_cast<uint32_t>(lane) < here ? cnt : 0u;
+        if (mc > 0u) mine[0] = static_cast<int32_t>(marked ? ra.x : value);
+        if (ballot64(mc > 1u) != 0) {
+          if (mc > 1u) mine[1] = static_cast<int32_t>(ra.y);
+          if (mc > 2u) mine[2] = static_cast<int32_t>(ra.z);
+          if (ballot64(mc > 3u) != 0) {
+            if (mc > 3u) mine[3] = static_cast<int32_t>(ra.w);
+            if (mc > 4u) mine[4] = static_cast<int32_t>(rb.x);
+            if (mc > 5u) mine[5] = static_cast<int32_t>(rb.y);
+            if (mc > 6u) mine[6] = static_cast<int32_t>(rb.z);
           }
         }
-        lds_sync();
       }
       done += tokens;
     }
