@@ -26,9 +26,9 @@ VALU_PEAK_TOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 lanes x 2.4 GHz: one 32
 # raw readings are in profiles/hbm_traffic_pmc_all_workloads.md.  Counters cannot be read from inside this
 # process, so the line reports these figures only for the workload they were measured on.
 MEASURED_TRAFFIC_C2 = {
-    "wordpiece_probe_kernel": (1763900000, 1970600000),
-    "wordpiece_oov_kernel": (866100000, 1367300000),
-    "wordpiece_emit_kernel": (2440700000, 856600000),
+    "wordpiece_probe_kernel": (1766100000, 1970100000),
+    "wordpiece_oov_kernel": (866200000, 1367300000),
+    "wordpiece_emit_kernel": (2368800000, 862800000),
 }
 
 
