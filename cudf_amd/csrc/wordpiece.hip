@@ -32,6 +32,7 @@
 #include "common.cuh"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -118,29 +119,10 @@ struct nvtext_amd_wordpiece_vocabulary {
 namespace nvtext_amd {
 namespace {
 
-constexpr int kTokWaves     = 4;
+constexpr int kTokWaves     = 2;
 constexpr int kTokThreads   = kTokWaves * kWave;
-constexpr int kGroups       = 4;     // rows a wavefront walks at the same time, 16 lanes each
-constexpr int kGroupLanes   = kWave / kGroups;
-constexpr int kChunk        = 16 * kGroupLanes;  // bytes per group step (16 per lane) = 256
-constexpr int kRing         = 2 * kChunk;        // per group: the current chunk and the one before it
 constexpr int32_t kNone     = std::numeric_limits<int32_t>::min();
-constexpr int kOovKeep      = 7;     // tokens stored per queued word; longer results are redone at emit time
-constexpr uint32_t kOovMark = 0x80000000u;  // word-arena value 0x80000000 | queue index (never 0xFFFFFFFF = id -1)
-
-struct OovEntry {
-  int32_t row;     // -1: unused entry
-  uint32_t delta;  // byte offset of the word inside its row
-  uint32_t widx;   // index of the word inside its row (its word-arena slot)
-  uint32_t len;    // bytes in the word (1..199)
-  uint32_t head[4];  // the word's first 16 bytes, zero padded: most words are tokenized without reading the chars again
-};
-struct OovResult {
-  int32_t tok[kOovKeep];
-  uint32_t count;  // tokens of the word (may exceed kOovKeep)
-};
-static_assert(sizeof(OovEntry) == 32 && sizeof(OovResult) == 32, "queue records are two 16-byte stores");
-
+constexpr int kOovKeep      = 7;     // tokens of an out-of-vocabulary word that are kept while it is tokenized
 // ------------------------------------------------------------------ where candidate keys live
 // Each source offers byte(k) and key8(p, len, &k0, &k1): bytes [p, p+8) as two dwords, zero padded past len.
 __device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& hi)
@@ -151,17 +133,18 @@ __device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& 
   hi &= nhi >= 4 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << (8 * nhi));
 }
 
-// A word inside a group's 512-byte LDS ring of the probe pass: byte k of the word is ring byte (start + k) & 511.
-struct RingWord {
-  const uint32_t* ring;
+// A word inside the bytes a wavefront has staged in LDS: `bytes` points at the staged dwords, `start` is the
+// byte index of the word's first byte in them.  Everything a word of fewer than kMaxWord bytes can touch is staged.
+struct TileWord {
+  const uint32_t* bytes;
   uint32_t start;
-  __device__ __forceinline__ uint32_t byte(uint32_t k) const { return reinterpret_cast<const uint8_t*>(ring)[(start + k) & (kRing - 1)]; }
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const { return reinterpret_cast<const uint8_t*>(bytes)[start + k]; }
   __device__ __forceinline__ void key8(uint32_t p, uint32_t len, uint32_t* k0, uint32_t* k1) const
   {
-    uint32_t const o  = (start + p) & (kRing - 1);
+    uint32_t const o  = start + p;
     uint32_t const i  = o >> 2;
     uint32_t const sh = (o & 3u) * 8u;
-    uint32_t const d0 = ring[i], d1 = ring[(i + 1) & (kRing / 4 - 1)], d2 = ring[(i + 2) & (kRing / 4 - 1)];
+    uint32_t const d0 = bytes[i], d1 = bytes[i + 1], d2 = bytes[i + 2];
     uint32_t lo       = __builtin_amdgcn_alignbit(d1, d0, sh);
     uint32_t hi       = __builtin_amdgcn_alignbit(d2, d1, sh);
     trim_key8(len, lo, hi);
@@ -175,7 +158,7 @@ struct RingWord {
     uint32_t const sh = (start & 3u) * 8u;
     uint32_t d[5];
 #pragma unroll
-    for (uint32_t j = 0; j < 5; ++j) d[j] = ring[(i + j) & (kRing / 4 - 1)];
+    for (uint32_t j = 0; j < 5; ++j) d[j] = bytes[i + j];
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) k[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
   }
@@ -196,45 +179,6 @@ struct GlobalWord {
     uint32_t const d2   = need > 8 ? a[2] : 0u;
     uint32_t lo         = __builtin_amdgcn_alignbit(d1, d0, mis * 8u);
     uint32_t hi         = __builtin_amdgcn_alignbit(d2, d1, mis * 8u);
-    trim_key8(len, lo, hi);
-    *k0 = lo;
-    *k1 = hi;
-  }
-};
-
-constexpr uint32_t kStage      = 64;   // bytes of each queued word kept in LDS (from a 16-byte aligned base)
-constexpr uint32_t kOovThreads = 256;
-
-// A queued word whose first kStage - mis bytes sit in LDS; later bytes come from memory.  The windows of
-// the workgroup are interleaved dword by dword (dword j of thread t at [j][t]), so that the lanes of a
-// wavefront reading "their" dword j hit 64 different banks instead of one.
-struct StagedWord {
-  const uint32_t* win;  // dword 0 of this lane's window; dword j is win[j * kOovThreads]
-  const uint8_t* p;     // the word in global memory
-  uint32_t mis;         // offset of the word inside the window
-  __device__ __forceinline__ uint32_t dword(uint32_t j) const { return win[j * kOovThreads]; }
-  __device__ __forceinline__ uint32_t byte(uint32_t k) const
-  {
-    uint32_t const o = mis + k;
-    return o < kStage ? (dword(o >> 2) >> (8 * (o & 3u))) & 0xffu : p[k];
-  }
-  __device__ __forceinline__ void key8(uint32_t off, uint32_t len, uint32_t* k0, uint32_t* k1) const
-  {
-    uint32_t const o = mis + off;
-    uint32_t lo, hi;
-    if (o + 12 <= kStage) {
-      uint32_t const i  = o >> 2;
-      uint32_t const sh = (o & 3u) * 8u;
-      uint32_t const d0 = dword(i), d1 = dword(i + 1), d2 = dword(i + 2);
-      lo                = __builtin_amdgcn_alignbit(d1, d0, sh);
-      hi                = __builtin_amdgcn_alignbit(d2, d1, sh);
-    } else {
-      lo = hi = 0;
-      for (uint32_t k = 0; k < 8 && k < len; ++k) {
-        uint32_t const b = byte(off + k);
-        if (k < 4) lo |= b << (8 * k); else hi |= b << (8 * (k - 4));
-      }
-    }
     trim_key8(len, lo, hi);
     *k0 = lo;
     *k1 = hi;
@@ -345,6 +289,34 @@ __device__ __forceinline__ int32_t lookup(VocabTable const& t, uint32_t kind, W 
   return finish_probe(t, pr, s0, s1, w, p, len);
 }
 
+// The general lookup, kept out of line: the callers have straight-line code for the common outcomes and come here
+// for the rest (keys in the pool, buckets that keys have been carried past).
+template <typename W>
+__device__ __forceinline__ int32_t lookup_slow(VocabTable const& t, uint32_t kind, W w, uint32_t p, uint32_t len)
+{
+  uint32_t r0, r1;
+  w.key8(p, min(len, 8u), &r0, &r1);
+  return lookup(t, kind, w, p, len, r0, r1);
+}
+
+// Sixteen bytes held in registers as a key source.
+struct RegWord {
+  uint32_t r[4];
+  __device__ __forceinline__ uint32_t byte(uint32_t k) const
+  {
+    uint32_t const d = k >> 2;
+    uint32_t const v = d == 0 ? r[0] : d == 1 ? r[1] : d == 2 ? r[2] : r[3];
+    return (v >> (8 * (k & 3u))) & 0xffu;
+  }
+  __device__ __forceinline__ void key8(uint32_t p, uint32_t len, uint32_t* k0, uint32_t* k1) const
+  {
+    uint32_t lo = p == 0 ? r[0] : r[2], hi = p == 0 ? r[1] : r[3];  // p is 0 or 8
+    trim_key8(len, lo, hi);
+    *k0 = lo;
+    *k1 = hi;
+  }
+};
+
 // What the two home slots say about a key of l bytes without any further memory access:
 // 1 = found (*id set), 0 = absent, 2 = undecided (a key of more than 8 bytes has the right tag, or keys have been
 // carried past this bucket and the search goes on in the next one).  Straight-line code.
@@ -379,30 +351,6 @@ __device__ __forceinline__ uint32_t verdict_16(VocabTable const& t, Probe const&
   return on ? 2u : 0u;
 }
 
-// ------------------------------------------------------------------ wavefront helpers of the probe pass
-template <int CTRL, int ROW_MASK, int OLD>
-__device__ __forceinline__ uint32_t dpp_old(uint32_t v)
-{
-  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(OLD, static_cast<int>(v), CTRL, ROW_MASK, 0xf, false));
-}
-
-__device__ __forceinline__ uint32_t wave_scan_max(uint32_t v)
-{
-  v = max(v, dpp_zero<0x111, 0xf>(v));
-  v = max(v, dpp_zero<0x112, 0xf>(v));
-  v = max(v, dpp_zero<0x114, 0xf>(v));
-  v = max(v, dpp_zero<0x118, 0xf>(v));
-  v = max(v, dpp_zero<0x142, 0xa>(v));
-  v = max(v, dpp_zero<0x143, 0xc>(v));
-  return v;
-}
-
-// value of the lane below (lane 0 gets FIRST)
-template <int FIRST>
-__device__ __forceinline__ uint32_t from_lane_below(uint32_t v)
-{
-  return dpp_old<0x138, 0xf, FIRST>(v);  // wave_shr:1
-}
 
 // Bit 7 of every byte of x that equals ' ' (exact: no carries cross bytes).
 __device__ __forceinline__ uint32_t space_bytes(uint32_t x)
@@ -412,347 +360,6 @@ __device__ __forceinline__ uint32_t space_bytes(uint32_t x)
 }
 // Gathers bits 7, 15, 23, 31 into bits 0..3.
 __device__ __forceinline__ uint32_t gather_byte_flags(uint32_t z) { return (((z >> 7) * 0x00204081u) >> 21) & 0xFu; }
-
-// Row r owns the word-arena slots [arena_pos(r), arena_pos(r+1)): at least floor(bytes/2) + 1, and a
-// row cannot hold more words than that.
-__device__ __forceinline__ int64_t arena_pos(ColView const& col, int64_t first_offset, int64_t r) { return ((col.off(r) - first_offset) >> 1) + r; }
-
-struct ProbeLds {
-  alignas(16) uint32_t bytes[kGroups][kRing / 4];  // per group: the bytes of the current chunk and the one before it, as in memory
-  uint32_t word[kGroups * kChunk / 2 + 2];         // per word ending in this step: (length, clamped to kMaxWord) << 16 | offset of its last byte in the chunk
-  alignas(16) uint32_t group[kGroups][8];          // per group: first word slot, words that count, chunk base, words so far, row start in its block, row, arena slot of the row
-};
-
-// Where a row sits relative to 16-byte aligned memory.  Coordinates count bytes from `base` and fit 32 bits
-// (a row is below 2 GiB).
-struct RowCtx {
-  const uint4* base;  // aligned address at or below the row's first byte
-  uint32_t mis;       // row start inside that block
-  uint32_t aend;      // row end (mis + row bytes)
-  // the 16 bytes at coordinate a0 (a multiple of 16) as they are in memory, if any of them belongs to the row
-  __device__ __forceinline__ uint4 load_raw(uint32_t a0) const
-  {
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (a0 < aend && a0 + 16 > mis) v = load_stream(base + (a0 >> 4));
-    return v;
-  }
-  // which of the 16 bytes at coordinate a0 belong to the row (bit k = byte a0 + k)
-  __device__ __forceinline__ uint32_t inside(uint32_t a0) const
-  {
-    uint32_t const lo = mis > a0 ? min(mis - a0, 16u) : 0u;
-    uint32_t const hi = aend > a0 ? min(aend - a0, 16u) : 0u;
-    return ((1u << hi) - 1u) & ~((1u << lo) - 1u);
-  }
-  // the byte at coordinate a (any alignment); ' ' outside the row
-  __device__ __forceinline__ uint32_t byte_at(uint32_t a) const
-  {
-    if (a < mis || a >= aend) return 0x20u;
-    return reinterpret_cast<const uint8_t*>(base)[a];
-  }
-};
-
-__device__ __forceinline__ RowCtx make_row_ctx(ColView const& col, int64_t o, int64_t n)
-{
-  const uint8_t* row = col.chars + o;
-  RowCtx c;
-  c.mis  = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u);
-  c.base = reinterpret_cast<const uint4*>(row - c.mis);
-  c.aend = c.mis + static_cast<uint32_t>(n);
-  return c;
-}
-
-// ------------------------------------------------------------------ probe pass
-// DPP moves inside a row of 16 lanes; lanes without a source keep `old`.
-template <int CTRL>
-__device__ __forceinline__ uint32_t dpp_row(uint32_t old, uint32_t v)
-{
-  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(old), static_cast<int>(v), CTRL, 0xf, 0xf, false));
-}
-// inclusive max-scan inside each group of 16 lanes
-__device__ __forceinline__ uint32_t group_scan_max(uint32_t v)
-{
-  v = max(v, dpp_row<0x111>(0u, v));  // row_shr:1
-  v = max(v, dpp_row<0x112>(0u, v));  // row_shr:2
-  v = max(v, dpp_row<0x114>(0u, v));  // row_shr:4
-  v = max(v, dpp_row<0x118>(0u, v));  // row_shr:8
-  return v;
-}
-__device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return static_cast<uint32_t>(__shfl(static_cast<int>(v), src_lane)); }
-
-// Persistent wavefronts.  Each group of 16 lanes walks its own row in 256-byte chunks (16 bytes per lane),
-// so a wavefront has four rows in flight; the words the four groups find in a step are pooled and probed
-// with lanes <-> words.  The next chunk of every group (the rest of its row, else the start of its next
-// row, whose offsets were fetched a row earlier) is requested before the probes of the current step.
-// For row r and its word k (slot = arena_pos(r) + k): arena[slot] = the token, or an out-of-vocabulary
-// marker carrying the queue index; nwords[r] = counts[r] = words kept.
-__global__ void __launch_bounds__(kTokThreads, 7) wordpiece_probe_kernel(ColView col, VocabTable table, int32_t max_words, int64_t first_offset,
-                                                                      int64_t last_offset, uint32_t* __restrict__ arena,
-                                                                      int32_t* __restrict__ nwords, int32_t* __restrict__ counts,
-                                                                      OovEntry* __restrict__ queue, uint32_t queue_capacity, uint32_t queue_block,
-                                                                      uint32_t* __restrict__ queue_size)
-{
-  __shared__ ProbeLds lds_all[kTokWaves];
-  int const lane       = lane_id();
-  int const wave       = threadIdx.x / kWave;
-  int const g          = lane / kGroupLanes;  // my group
-  int const gl         = lane % kGroupLanes;  // my lane inside it
-  int const g_first    = g * kGroupLanes;
-  int const g_last     = g_first + kGroupLanes - 1;
-  ProbeLds& lds        = lds_all[wave];
-  int64_t const rows   = col.size;
-  uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue range
-  uint32_t my_block       = min(queue_block, 128u);  // entries reserved at a time: doubled up to queue_block when ranges fill fast
-  uint32_t steps_in_range = 0;                       // steps of the loop below since the range was reserved
-
-  // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
-  // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
-  auto word_cap = [&](int64_t row, int64_t bytes) -> uint32_t {
-    if (max_words <= 0) return static_cast<uint32_t>(std::numeric_limits<int32_t>::max());
-    return col.valid(row) ? static_cast<uint32_t>(min(static_cast<int64_t>(max_words), bytes / 2)) : 0u;
-  };
-
-  // ---- the rows of a group: consecutive ones, [r, r_end), that hold its share of the column's WORK, a row counting
-  // as its bytes plus one chunk (which is about what walking it costs; rows without bytes must count, or a long run
-  // of them would fall to one group).  Group k of G begins with the first row at or after k/G of the total.  With a
-  // share of the rows instead (every G-th row) the groups with the longest rows walked a seventh more chunks than the
-  // average group, and the pass waited for them.  r_end is found together with r: two searches over the offsets in
-  // step, 22 dependent reads for 4M rows.
-  uint32_t r = 0, r_end = 0;
-  {
-    uint32_t const groups = gridDim.x * kTokWaves * kGroups;
-    uint32_t const k      = (blockIdx.x * kTokWaves + wave) * kGroups + g;
-    auto work_before = [&](int64_t row) -> int64_t { return col.off(row) - first_offset + row * static_cast<int64_t>(kChunk); };
-    // (work < 2^48 and groups < 2^16: the products fit)
-    int64_t const work = last_offset - first_offset + rows * static_cast<int64_t>(kChunk);
-    int64_t const t0   = work / groups * k + work % groups * k / groups;
-    int64_t const t1   = work / groups * (k + 1) + work % groups * (k + 1) / groups;
-    // number of rows 0..rows with less work before them than t, which is the first row at or after t
-    uint32_t below0 = 0, below1 = 0;
-    uint32_t step   = 1;
-    while (step <= static_cast<uint32_t>(rows)) step <<= 1;  // rows + 1 entries; rows < 2^31
-    for (; step > 0; step >>= 1) {
-      uint32_t const p0 = below0 + step, p1 = below1 + step;
-      int64_t const v0  = p0 <= static_cast<uint32_t>(rows) + 1u ? work_before(static_cast<int64_t>(p0) - 1) : std::numeric_limits<int64_t>::max();
-      int64_t const v1  = p1 <= static_cast<uint32_t>(rows) + 1u ? work_before(static_cast<int64_t>(p1) - 1) : std::numeric_limits<int64_t>::max();
-      if (v0 < t0) below0 = p0;
-      if (v1 < t1) below1 = p1;
-    }
-    r     = min(below0, static_cast<uint32_t>(rows));
-    r_end = k + 1 == groups ? static_cast<uint32_t>(rows) : min(below1, static_cast<uint32_t>(rows));
-    if (k == 0) r = 0;
-  }
-  // ---- per-group state (the same value in all 16 lanes of a group).  Kept small: the row being walked is known by its
-  // RowCtx alone (its first byte's address gives back its offset; the next row begins where it ends), the row after
-  // it by its end.
-  int64_t e_nxt = 0;
-  uint32_t cap  = 0;
-  RowCtx ctx;
-  {
-    int64_t o = 0, n = 0;
-    if (r < r_end) {
-      o   = col.off(r);
-      n   = col.off(r + 1) - o;
-      cap = word_cap(r, n);
-    }
-    ctx = make_row_ctx(col, o, n);
-  }
-  if (r + 1 < r_end) e_nxt = col.off(static_cast<int64_t>(r) + 2);
-  uint32_t cbase   = 0;
-  uint32_t wdone   = 0;     // words kept so far in this row
-  uint32_t carry_start = 0; // 1-based coordinate of the start of the word running into the chunk
-  uint32_t prev_space  = 1; // the byte before the chunk is a space (or the row starts here)
-  // the chunk about to be processed: my sixteen bytes and (last lane of the group) the byte after the chunk
-  uint4 mine_cur    = make_uint4(0u, 0u, 0u, 0u);
-  uint32_t tail_cur = 0x20u;
-  if (r < r_end) {
-    mine_cur = ctx.load_raw(16 * gl);
-    if (gl == kGroupLanes - 1) tail_cur = ctx.byte_at(kChunk);
-  }
-
-  while (ballot64(r < r_end) != 0) {
-    ++steps_in_range;
-    bool const has_row  = r < r_end;
-    bool const chunk_ok = has_row && cbase < ctx.aend && wdone < cap;
-
-    // ---- bytes -> word ends (lanes <-> bytes, per group)
-    uint32_t ends = 0, starts = 0, xs = 0;
-    uint32_t const a0 = cbase + 16u * gl;
-    if (chunk_ok) *reinterpret_cast<uint4*>(&lds.bytes[g][(a0 & (kRing - 1)) >> 2]) = mine_cur;
-    {
-      uint4 const mine  = mine_cur;
-      // spaces, and everything outside the row counts as one
-      uint32_t const sp = (gather_byte_flags(space_bytes(mine.x)) | (gather_byte_flags(space_bytes(mine.y)) << 4) |
-                           (gather_byte_flags(space_bytes(mine.z)) << 8) | (gather_byte_flags(space_bytes(mine.w)) << 12) | ~ctx.inside(a0)) &
-                          0xFFFFu;
-      // is the byte before my sixteen a space, and the byte after them
-      uint32_t const before = dpp_row<0x111>(prev_space, sp >> 15);                       // row_shr:1
-      uint32_t const after  = dpp_row<0x101>(tail_cur == 0x20u ? 1u : 0u, sp & 1u);        // row_shl:1
-      uint32_t const word   = ~sp & 0xFFFFu;
-      starts                = word & ((sp << 1) | before);         // a word byte after a space
-      ends                  = word & ((sp >> 1) | (after << 15));  // a word byte before a space
-      if (!chunk_ok) ends = starts = 0;
-      // start of the word that runs into my bytes: the last start in the lanes below, else the carry
-      uint32_t const my_last = starts ? a0 + (32u - __builtin_clz(starts)) : 0u;
-      uint32_t const is      = group_scan_max(my_last);
-      xs                     = max(dpp_row<0x111>(0u, is), carry_start);
-      if (chunk_ok) {
-        carry_start = max(carry_start, shfl_u32(is, g_last));
-        prev_space  = shfl_u32(sp >> 15, g_last);
-      }
-    }
-    uint32_t const ne   = __builtin_popcount(ends);
-    uint32_t const incl = wave_inclusive_scan(ne);
-    // first word slot of every group and the total
-    uint32_t const gb1 = wave_bcast(incl, 15), gb2 = wave_bcast(incl, 31), gb3 = wave_bcast(incl, 47), total = wave_bcast(incl, 63);
-    uint32_t const my_gbase  = g == 0 ? 0u : g == 1 ? gb1 : g == 2 ? gb2 : gb3;
-    uint32_t const my_gtotal = (g == 0 ? gb1 : g == 1 ? gb2 : g == 2 ? gb3 : total) - my_gbase;
-    uint32_t slot            = incl - ne;
-    for (uint32_t em = ends; em; em &= em - 1) {
-      uint32_t const p  = __builtin_ctz(em);
-      uint32_t const sb = starts & ((2u << p) - 1u);
-      uint32_t const st = sb ? a0 + (32u - __builtin_clz(sb)) : xs;  // 1-based
-      uint32_t const wl = a0 + p + 1u - st + 1u;
-      lds.word[slot]    = (min(wl, kMaxWord) << 16) | (16u * gl + p);
-      ++slot;
-    }
-    // words of this chunk that count (the row's word limit may cut them short)
-    uint32_t const allowed = chunk_ok ? min(my_gtotal, cap - wdone) : 0u;
-    uint32_t const wd_after = wdone + allowed;
-    uint32_t const r_now    = r;
-    if (gl == 0) {
-      int64_t const o_cur    = reinterpret_cast<const uint8_t*>(ctx.base) + ctx.mis - col.chars;
-      int64_t const row_slot = ((o_cur - first_offset) >> 1) + r;
-      *reinterpret_cast<uint4*>(&lds.group[g][0]) = make_uint4(my_gbase, allowed, cbase, wdone);
-      *reinterpret_cast<uint4*>(&lds.group[g][4]) =
-        make_uint4(ctx.mis, static_cast<uint32_t>(r), static_cast<uint32_t>(row_slot), static_cast<uint32_t>(static_cast<uint64_t>(row_slot) >> 32));
-    }
-
-    // ---- what this group looks at next; request it now so it arrives while the probes run
-    bool const row_done = has_row && !(chunk_ok && cbase + kChunk < ctx.aend && wd_after < cap);
-    if (has_row) {
-      if (!row_done) {
-        cbase += kChunk;
-        wdone = wd_after;
-      } else {
-        // the next row begins where this one ends
-        int64_t const o_new = reinterpret_cast<const uint8_t*>(ctx.base) + ctx.aend - col.chars;
-        int64_t const n_new = r + 1 < r_end ? e_nxt - o_new : 0;
-        ++r;
-        ctx   = make_row_ctx(col, o_new, n_new);
-        cbase = 0;
-        wdone = 0;
-        carry_start = 0;
-        prev_space  = 1;
-        if (r < r_end) cap = word_cap(r, n_new);
-        if (r + 1 < r_end) e_nxt = col.off(static_cast<int64_t>(r) + 2);
-      }
-      if (r < r_end) {
-        mine_cur = ctx.load_raw(cbase + 16 * gl);
-        tail_cur = gl == kGroupLanes - 1 ? ctx.byte_at(cbase + kChunk) : 0x20u;
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-    // ---- probes (lanes <-> words, all groups pooled)
-    for (uint32_t w0 = 0; w0 < total; w0 += kWave) {
-      uint32_t const ws = w0 + lane;  // word slot
-      int const gw      = (ws >= gb1) + (ws >= gb2) + (ws >= gb3);
-      uint4 const ga    = *reinterpret_cast<const uint4*>(&lds.group[gw][0]);  // first slot, allowed, chunk base, words so far
-      uint4 const gb    = *reinterpret_cast<const uint4*>(&lds.group[gw][4]);  // row start in its block, row, arena slot of the row
-      uint32_t const idx = ws - ga.x;
-      bool const active  = ws < total && idx < ga.y;
-      bool miss       = false;
-      uint32_t value  = 0, wl = 0, wstart = 0;
-      uint32_t head[4] = {0u, 0u, 0u, 0u};
-      if (active) {
-        uint32_t const rec = lds.word[ws];
-        wl     = rec >> 16;
-        wstart = ga.z + (rec & 0xFFFFu) + 1u - wl;  // coordinate of the word's first byte
-        if (wl >= kMaxWord) {
-          value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
-        } else {
-          int32_t id = kNone;
-          RingWord const rw_{lds.bytes[gw], wstart & (kRing - 1)};
-          rw_.head16(head);
-          trim_key8(wl, head[0], head[1]);
-          trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
-          if (wl <= table.max_len[0]) {
-            // hash of the first two blocks without a loop; longer words go on from there
-            Probe pr;
-            pr.k0 = head[0];
-            pr.k1 = head[1];
-            uint32_t h        = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
-            uint32_t const h2 = key_hash_block(h, head[2], head[3]);
-            h                 = wl > 8 ? h2 : h;
-            if (wl > 16) {
-              for (uint32_t done = 16; done < wl; done += 8) {
-                uint32_t b0, b1;
-                rw_.key8(done, wl - done, &b0, &b1);
-                h = key_hash_block(h, b0, b1);
-              }
-            }
-            uint32_t b;
-            pr.want   = slot_word0(h, 0, wl, &b);
-            pr.bucket = b & table.bucket_mask;
-            uint4 const s0 = table.slots[2 * pr.bucket];
-            uint4 const s1 = table.slots[2 * pr.bucket + 1];
-            uint32_t v = verdict(pr, s0, s1, wl, &id);
-            if (v == 2u && wl > 8 && wl <= 16) v = verdict_16(table, pr, s0, s1, head, &id);
-            if (v == 2u) id = finish_probe(table, pr, s0, s1, rw_, 0u, wl);
-            else if (v == 0u) id = kNone;
-          }
-          miss  = id == kNone;
-          value = static_cast<uint32_t>(id);
-        }
-      }
-      uint64_t const mm = ballot64(miss);
-      if (mm) {
-        uint32_t const nm   = static_cast<uint32_t>(__builtin_popcountll(mm));
-        uint32_t const room = q_lim - q_pos;  // left of the reserved range: filled up before the next one is begun,
-        uint32_t fresh      = 0;              // so that unused entries only ever follow a wavefront's last word
-        if (nm > room) {                      // my_block >= 64 >= nm
-          // a range that lasted only a few steps is followed by one twice as long: atomics on the one counter
-          // run at about 150 M/s for the whole device, and unused entries cost the next pass time
-          if (steps_in_range < 8u && my_block < queue_block) my_block <<= 1;
-          steps_in_range = 0;
-          if (lane == 0) fresh = atomicAdd(queue_size, my_block);
-          fresh = wave_bcast(fresh, 0);
-        }
-        if (miss) {
-          uint32_t const rank = lanes_below(mm);
-          uint32_t const q    = rank < room ? q_pos + rank : fresh + (rank - room);
-          if (q < queue_capacity) {
-            uint4* const dst = reinterpret_cast<uint4*>(queue + q);
-            store_stream(dst, make_uint4(gb.y, wstart - gb.x, ga.w + idx, wl));
-            store_stream(dst + 1, make_uint4(head[0], head[1], head[2], head[3]));
-          }
-          value = kOovMark | q;
-        }
-        if (nm > room) {
-          q_pos = fresh + (nm - room);
-          q_lim = fresh + my_block;
-        } else {
-          q_pos += nm;
-        }
-      }
-      if (active) {
-        int64_t const s = static_cast<int64_t>((static_cast<uint64_t>(gb.w) << 32) | gb.z) + ga.w + idx;
-        store_stream(arena + s, value);
-      }
-    }
-    if (row_done && gl == 0) {
-      // one token per word; the out-of-vocabulary pass adds what its words give beyond that
-      nwords[r_now] = static_cast<int32_t>(wd_after);
-      counts[r_now] = static_cast<int32_t>(wd_after);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-  }
-  for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
-    if (q < queue_capacity) queue[q] = OovEntry{-1, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
-}
 
 // ------------------------------------------------------------------ out-of-vocabulary pass
 // Greedy longest-match-first tokenization (cpp/src/text/wordpiece_tokenize.cu:349-407) of a word whose
@@ -890,27 +497,19 @@ __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W con
   return st.count;
 }
 
-// Brings the first bytes of the `len`-byte word at p into this lane's LDS window with 16-byte aligned
-// loads (only blocks that overlap the word).  *ascii = no byte of the word has bit 7 set (judged on the
-// whole blocks, so it may be false for a plain word next to other text; never true wrongly).
-__device__ __forceinline__ uint32_t stage_word(const uint8_t* p, uint32_t len, uint32_t* win, bool* ascii)
+// The same, out of line, for the callers' rare cases: the number of tokens of a word staged in LDS, and the tokens
+// of a word in memory written to dst[0 .. cnt) (cnt = the number counted before).
+__device__ __forceinline__ uint32_t count_oov_tokens(VocabTable const& t, const uint32_t* bytes, uint32_t start, uint32_t len)
 {
-  uint32_t const mis    = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 15u);
-  const uint4* a        = reinterpret_cast<const uint4*>(p - mis);
-  uint32_t const need   = (mis + len + 15u) >> 4;
-  uint32_t const blocks = min(kStage / 16, need);
-  uint32_t seen         = 0;
-  for (uint32_t i = 0; i < blocks; ++i) {
-    uint4 const v = a[i];
-    seen |= v.x | v.y | v.z | v.w;
-    win[(4 * i + 0) * kOovThreads] = v.x;
-    win[(4 * i + 1) * kOovThreads] = v.y;
-    win[(4 * i + 2) * kOovThreads] = v.z;
-    win[(4 * i + 3) * kOovThreads] = v.w;
-  }
-  *ascii = (seen & 0x80808080u) == 0 && need <= kStage / 16;
-  return mis;
+  return tokenize_oov_word(t, TileWord{bytes, start}, len, [](uint32_t, int32_t) {});
 }
+__device__ __forceinline__ void write_oov_tokens(VocabTable const& t, const uint8_t* p, uint32_t len, uint32_t* dst, uint32_t cnt)
+{
+  tokenize_oov_word(t, GlobalWord{p}, len, [&](uint32_t j, int32_t id) {
+    if (j < cnt) dst[j] = static_cast<uint32_t>(id);
+  });
+}
+
 
 // Bit 7 of every byte of x that is a UTF-8 continuation byte (10xxxxxx); exact, no carries cross bytes.
 __device__ __forceinline__ uint32_t continuation_bytes(uint32_t x)
@@ -1023,7 +622,8 @@ struct ShortWord {
       uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
       uint32_t va    = verdict(pa, a0, a1, la, &ida);
       if (va == 2u) {  // the general lookup (keys in the pool, overflowing buckets)
-        ida = finish_probe(t, pa, a0, a1, *this, 0u, la);
+        RegWord const rw{{r[0], r[1], r[2], r[3]}};
+        ida = lookup_slow(t, kind, rw, 0u, la);
         va  = ida == kNone ? 0u : 1u;
       }
       hit_a = va == 1u;
@@ -1054,364 +654,685 @@ struct ShortWord {
   }
 };
 
-// One lane per queued word, and a lane that finishes its word takes the next one: every wavefront owns a
-// contiguous part of the queue and, every eighth trip, lets its idle lanes store their result and pick up
-// new entries, so lanes with short words do not wait for the longest word of a batch.  Words of up to 16
-// bytes (whole in their queue record) run in registers; the few longer ones are set aside for the kernel
-// below: their queue indices go to longer[first entry of the part ...], their number to
-// longer[queue_capacity + wavefront].
-// results[q] = the word's first kOovKeep tokens and its token count; counts[row] += count - 1.
-__global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
-                                                                    const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
-                                                                    OovResult* __restrict__ results, int32_t* __restrict__ counts,
-                                                                    uint32_t* __restrict__ longer)
+// ------------------------------------------------------------------ the tile pass
+// The column's bytes, from the 16-byte aligned address at or below its first byte, are cut into tiles of TILE
+// bytes without regard to rows; kRangeTiles consecutive tiles form a range.  A wavefront takes one range at a
+// time and walks its tiles in order, so that the rows that start in them are met in order too.
+constexpr int kRangeTiles    = 16;
+constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
+constexpr uint32_t kQueueCap = 256;  // out-of-vocabulary words that wait in LDS
+constexpr uint32_t kTokCap   = 256;  // their tokens (per unit)
+constexpr int kStragglers    = 24;   // a unit's out-of-vocabulary words may go on into the next unit's once fewer lanes than this are busy
+// lds.word[k] after its word has been looked up: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or
+//   kOovMark | count << 16 | index of its tokens in lds.tokens          (1 <= count <= kOovKeep), or
+//   kOovMark | kOovRedo | count << 21 | length << 13 | start            (tokens not kept: tokenized again when written)
+constexpr uint32_t kOovMark = 0x80000000u;
+constexpr uint32_t kOovRedo = 0x40000000u;
+
+template <int TILE>
+struct TileLds {
+  static constexpr int kBlocks = TILE / 16;
+  alignas(16) uint32_t bytes[(16 + TILE + 16 * kOverBlocks) / 4 + 4];  // tile position x at byte 16 + x; key reads run a few bytes past a word
+  uint32_t bound[kBlocks + kOverBlocks + 1];  // per block: bit i = a row starts at byte i; bit 16 + i = the words that a row's limit drops begin / stop here
+  uint32_t masks[kBlocks];                    // per block: bit i = a word starts at byte i, bit 16 + i = a word ends at byte i
+  uint32_t prefix[kBlocks + 1];               // word starts before the block | word ends before the block << 16
+  static constexpr uint32_t kWordCap = TILE / 4;
+  uint32_t word[2][kWordCap];                 // per word of a unit: start | end << 16, then its token (see kOovMark), then the tokens before it
+  uint32_t tokens[2][kTokCap];
+  uint16_t queue[kQueueCap];
+};
+
+struct TileArgs {
+  ColView col;
+  VocabTable table;
+  const uint4* abase;      // 16-byte aligned address at or below the first byte of the view; coordinates count bytes from here
+  int64_t first_offset;    // offsets[0] of the view
+  int64_t cend;            // coordinate past the view's last byte
+  int64_t ntiles;
+  uint32_t cbeg;           // coordinate of the view's first byte (0..15)
+  uint32_t nranges;
+  int32_t max_words;
+  uint32_t range_cap;      // arena slots of a range
+  const uint32_t* range_first_row;
+  uint32_t* arena;         // tokens of range g from arena[g * range_cap], densely, in order
+  uint32_t* range_count;   // tokens of range g
+  int32_t* offsets_out;    // per row: tokens of its range before the row
+  uint32_t* counter;       // next range to hand out
+  uint32_t* overflow;      // set when a range has more tokens than range_cap
+};
+
+__device__ __forceinline__ void wave_lds_sync()
 {
-  if (*queue_size > queue_capacity) return;  // the queue was too small: the host repeats the passes with a larger one
-  uint32_t const total  = min(*queue_size, queue_capacity);
-  uint32_t const nwave  = gridDim.x * (kOovThreads / kWave);
-  uint32_t const wave   = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
-  uint32_t const chunk  = (total + nwave - 1) / nwave;
-  uint32_t const q_begin = min(total, wave * chunk);
-  uint32_t next          = q_begin;                          // wave-uniform cursor into this wavefront's part
-  uint32_t const q_end   = min(total, next + chunk);
-  uint32_t n_longer      = 0;                                // entries of this part set aside (wave-uniform)
-  int const lane         = lane_id();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
-  int32_t tok[kOovKeep];
-  auto keep_token = [&](uint32_t j, int32_t id) {
-#pragma unroll
-    for (int k = 0; k < kOovKeep; ++k)
-      if (j == static_cast<uint32_t>(k)) tok[k] = id;
-  };
-  auto deliver = [&](uint32_t q, int32_t row, uint32_t count) {
-    uint4* const dst = reinterpret_cast<uint4*>(results + q);
-    store_stream(dst, make_uint4(static_cast<uint32_t>(tok[0]), static_cast<uint32_t>(tok[1]), static_cast<uint32_t>(tok[2]), static_cast<uint32_t>(tok[3])));
-    store_stream(dst + 1, make_uint4(static_cast<uint32_t>(tok[4]), static_cast<uint32_t>(tok[5]), static_cast<uint32_t>(tok[6]), count));
-    if (count > 1) atomicAdd(&counts[row], static_cast<int32_t>(count - 1));  // the probe pass has counted one token per word
-  };
+// bit i = byte i of the sixteen is a space
+__device__ __forceinline__ uint32_t space_mask16(uint4 const& v)
+{
+  return gather_byte_flags(space_bytes(v.x)) | (gather_byte_flags(space_bytes(v.y)) << 4) | (gather_byte_flags(space_bytes(v.z)) << 8) |
+         (gather_byte_flags(space_bytes(v.w)) << 12);
+}
 
-  {
+// bit i = coordinate g0 + i lies outside [lo, hi)
+__device__ __forceinline__ uint32_t outside_mask16(int64_t g0, int64_t lo, int64_t hi)
+{
+  int64_t const a  = lo - g0, b = hi - g0;
+  uint32_t const l = a <= 0 ? 0u : a >= 16 ? 16u : static_cast<uint32_t>(a);
+  uint32_t const h = b <= 0 ? 0u : b >= 16 ? 16u : static_cast<uint32_t>(b);
+  return ~(((1u << h) - 1u) & ~((1u << l) - 1u)) & 0xFFFFu;
+}
+
+// Words that start in coordinates [from, to) (bytes outside count as spaces), counted by the whole wavefront, 1 KiB
+// a step; stops once `limit` is reached.  Same value in every lane.
+__device__ __forceinline__ uint32_t count_word_starts(const uint4* abase, int64_t from, int64_t to, uint32_t limit)
+{
+  int const lane      = lane_id();
+  uint32_t total      = 0;
+  uint32_t prev_space = 1;
+  for (int64_t g = from & ~static_cast<int64_t>(15); g < to && total < limit; g += 16 * kWave) {
+    int64_t const g0 = g + 16 * lane;
+    uint4 v          = make_uint4(0u, 0u, 0u, 0u);
+    if (g0 < to && g0 + 16 > from) v = abase[g0 >> 4];
+    uint32_t const sp     = (space_mask16(v) | outside_mask16(g0, from, to)) & 0xFFFFu;
+    uint32_t const before = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(prev_space), static_cast<int>(sp >> 15), 0x138, 0xf, 0xf, false));
+    uint32_t const starts = ~sp & ((sp << 1) | before) & 0xFFFFu;
+    total += wave_bcast(wave_inclusive_scan(static_cast<uint32_t>(__builtin_popcount(starts))), kWave - 1);
+    prev_space = wave_bcast(sp >> 15, kWave - 1);
+  }
+  return total;
+}
+
+// range_first_row[g] = the first row (0..rows) that starts at or after the first byte of range g
+__global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32_t cbeg, int64_t range_bytes, uint32_t nranges,
+                                       uint32_t* __restrict__ range_first_row)
+{
+  uint32_t const g = blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= nranges) return;
+  int64_t const target = static_cast<int64_t>(g) * range_bytes;
+  uint32_t lo = 0, hi = static_cast<uint32_t>(col.size);
+  while (lo < hi) {
+    uint32_t const mid = lo + ((hi - lo) >> 1);
+    if (col.off(mid) - first_offset + cbeg < target) lo = mid + 1;
+    else hi = mid;
+  }
+  range_first_row[g] = lo;
+}
+
+// One tile at a time per wavefront: stage its bytes (and the 256 after it) in LDS; mark the row starts in it; find
+// word starts and ends (lanes <-> 16-byte blocks: spaces by SWAR, row starts as extra separators); with a word limit,
+// drop the words past each row's limit; list the words (word k pairs start k with end k); look all of them up (lanes
+// <-> words, one probe each); tokenize the ones that are not in the vocabulary (lanes <-> such words, a lane that
+// finishes takes the next one); then place the tokens (a wave scan of the words' token counts) and write them to the
+// range's arena, and give every row that starts in the tile the number of tokens before it.
+#ifdef WP_PHASE_TIMING
+#define WP_PHASE(i)                                         \
+  {                                                         \
+    uint64_t const now_ = __builtin_amdgcn_s_memtime();     \
+    phase_t[i] += now_ - phase_last;                        \
+    phase_last = now_;                                      \
+  }
+#else
+#define WP_PHASE(i)
+#endif
+
+template <int TILE>
+__global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs a)
+{
+#ifdef WP_PHASE_TIMING
+  uint64_t phase_t[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  uint64_t phase_last  = __builtin_amdgcn_s_memtime();
+#endif
+  constexpr int kBlocks       = TILE / 16;
+  constexpr int kSubs         = kBlocks / kWave;
+  constexpr uint32_t kWordCap = TileLds<TILE>::kWordCap;
+  static_assert(kBlocks % kWave == 0, "whole wavefronts of blocks");
+  __shared__ TileLds<TILE> lds_all[kTokWaves];
+  TileLds<TILE>& lds  = lds_all[threadIdx.x / kWave];
+  int const lane      = lane_id();
+  uint32_t const rows = static_cast<uint32_t>(a.col.size);
+  int64_t const cbeg  = a.cbeg, cend = a.cend;
+  VocabTable const& table = a.table;
+  auto coord = [&](uint32_t r) -> int64_t { return a.col.off(r) - a.first_offset + cbeg; };
+  // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
+  // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
+  auto word_cap = [&](uint32_t r, int64_t bytes) -> uint32_t {
+    return a.col.valid(r) ? static_cast<uint32_t>(min(static_cast<int64_t>(a.max_words), bytes / 2)) : 0u;
+  };
+  const uint8_t* const lds_byte = reinterpret_cast<const uint8_t*>(lds.bytes);
+  enum { kQueueFull = 0, kUnitDone = 1, kRangeDone = 2 };
+
+  for (;;) {
+    uint32_t range = 0;
+    if (lane == 0) range = atomicAdd(a.counter, 1u);
+    range = wave_bcast(range, 0);
+    if (range >= a.nranges) break;
+    int64_t t           = static_cast<int64_t>(range) * kRangeTiles;
+    int64_t const t_end = min(t + kRangeTiles, a.ntiles);
+    uint32_t r_cur      = a.range_first_row[range];
+    uint32_t cursor     = 0;  // tokens of this range so far
+    uint32_t open_left  = 0;  // words the row that runs into the tile may still have (with a word limit)
+    uint32_t* const region = a.arena + static_cast<int64_t>(range) * a.range_cap;
+    bool spill             = false;
+    if (a.max_words > 0 && r_cur > 0) {
+      uint32_t const ro  = r_cur - 1;
+      int64_t const c0   = coord(ro), c1 = coord(ro + 1);
+      uint32_t const cap = word_cap(ro, c1 - c0);
+      uint32_t const used = cap ? count_word_starts(a.abase, c0, t * TILE, cap) : 0u;
+      open_left           = cap - min(cap, used);
+    }
+
+    // A unit is the words of a tile (of a tile with more than kWordCap words: that many of them at a time).  Two are in
+    // flight: the one whose words are being looked up, and the one before it, whose last out-of-vocabulary words
+    // are still being tokenized by the lanes that took them; its tokens are written once those are done.  So the
+    // words that take many steps share their steps with the next unit's words instead of idling the other lanes.
+    // -- the tile being looked up
+    bool tile_open = false, unit_open = false;
+    int64_t tb     = 0;
+    uint32_t nw = 0, ne = 0, inside0 = 0;  // words that start in the tile, words that end in it, the tile begins inside a word
+    uint32_t r_first = 0, r_end = 0;       // the rows that start in it
+    uint32_t w_lo = 0, w_hi = 0, nwc = 0;  // the unit: words [w_lo, w_hi) of the tile
+    uint32_t par = 0;                      // which half of lds.word / lds.tokens it uses
+    uint32_t k0 = 0, qn = 0, q_next = 0;   // words looked up so far; queue entries written / taken
+    bool edge = false;
+    // -- the unit before it
+    bool pend = false;
+    int64_t p_tb = 0;
+    uint32_t p_par = 0, p_nwc = 0, p_wlo = 0, p_nw = 0, p_rfirst = 0, p_rend = 0;
+    // -- the lanes' out-of-vocabulary words
     ShortWord sw;
-    sw.done    = true;
-    bool busy  = false;  // this lane holds a word (finished or not)
-    uint32_t q = 0;
-    int32_t row = -1;
-    for (uint32_t trip = 0;; ++trip) {
-      if ((trip & 7u) == 0) {
-        if (busy && sw.done) {
-          deliver(q, row, sw.count);
-          busy = false;
+    sw.done  = true;
+    sw.count = 0;
+    bool busy = false;
+    uint32_t mine = 0, mine_par = 0;  // my word: lds.word[mine_par][mine]
+    int32_t tok[kOovKeep];
+    uint32_t tok_used0 = 0, tok_used1 = 0;  // tokens kept in lds.tokens[0], [1]
+    auto keep_token = [&](uint32_t j, int32_t id) {
+#pragma unroll
+      for (int i = 0; i < kOovKeep; ++i)
+        if (j == static_cast<uint32_t>(i)) tok[i] = id;
+    };
+
+    for (;;) {
+      int reason = kRangeDone;
+      if (!unit_open) {
+        if (!tile_open && t < t_end) {
+          // ================================================================ a new tile
+          tb                   = t * TILE;
+          bool const last_tile = t + 1 == a.ntiles;
+          edge                 = tb < 16 + cbeg || tb + TILE + 16 * kOverBlocks > cend;  // some staged byte lies outside the view
+          // ---- stage the bytes
+          for (int j = lane - 1; j < kBlocks + kOverBlocks; j += kWave) {
+            int64_t const g0 = tb + 16 * j;
+            uint4 v          = make_uint4(0u, 0u, 0u, 0u);
+            if (g0 + 16 > cbeg && g0 < cend) v = load_stream(a.abase + (g0 >> 4));
+            *reinterpret_cast<uint4*>(&lds.bytes[4 * (j + 1)]) = v;
+          }
+          for (int i = lane; i < kBlocks + kOverBlocks + 1; i += kWave) lds.bound[i] = 0;
+          wave_lds_sync();
+          WP_PHASE(0)
+
+          // ---- the rows that start in the tile: [r_first, r_end)
+          r_first = r_cur;
+          for (;;) {
+            uint32_t const r = r_cur + lane;
+            int64_t const p  = r <= rows ? coord(r) - tb : std::numeric_limits<int64_t>::max();
+            bool const in    = r < rows && (last_tile || p < TILE);
+            if (p < TILE + 16 * kOverBlocks) atomicOr(&lds.bound[p >> 4], 1u << (p & 15));
+            uint32_t const n = static_cast<uint32_t>(__builtin_popcountll(ballot64(in)));
+            r_cur += n;
+            if (n < kWave) break;
+          }
+          r_end = r_cur;
+          wave_lds_sync();
+          WP_PHASE(1)
+
+          // ---- word starts and ends
+          {
+            uint32_t base = 0;
+#pragma unroll
+            for (int s = 0; s < kSubs; ++s) {
+              int const b     = s * kWave + lane;
+              uint4 const v   = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
+              uint32_t sp     = space_mask16(v);
+              uint32_t before = lds_byte[16 + 16 * b - 1] == 0x20u, after = lds_byte[16 + 16 * b + 16] == 0x20u;
+              if (edge) {
+                int64_t const g0 = tb + 16 * b;
+                sp |= outside_mask16(g0, cbeg, cend);
+                before |= (g0 - 1 < cbeg || g0 - 1 >= cend);
+                after |= (g0 + 16 < cbeg || g0 + 16 >= cend);
+              }
+              uint32_t const bd = lds.bound[b] & 0xFFFFu;
+              after |= lds.bound[b + 1] & 1u;
+              uint32_t const word   = ~sp & 0xFFFFu;
+              uint32_t const starts = word & ((sp << 1) | before | bd);
+              uint32_t const ends   = word & ((sp >> 1) | (after << 15) | (bd >> 1));
+              if (s == 0) inside0 = wave_bcast(word & ~starts & 1u, 0);
+              lds.masks[b]          = starts | (ends << 16);
+              uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
+              uint32_t const incl   = wave_inclusive_scan(cnt);
+              lds.prefix[b]         = base + incl - cnt;
+              base += wave_bcast(incl, kWave - 1);
+            }
+            if (lane == 0) lds.prefix[kBlocks] = base;
+            nw = base & 0xFFFFu;
+            ne = base >> 16;
+          }
+          wave_lds_sync();
+          WP_PHASE(2)
+
+          // word starts at positions below x (0 <= x)
+          auto words_before = [&](uint32_t x) -> uint32_t {
+            if (x >= TILE) return nw;
+            uint32_t const b = x >> 4;
+            return (lds.prefix[b] & 0xFFFFu) + static_cast<uint32_t>(__builtin_popcount(lds.masks[b] & ((1u << (x & 15u)) - 1u)));
+          };
+          // position of word start k (k < nw)
+          auto word_start = [&](uint32_t k) -> uint32_t {
+            uint32_t b = 0;
+#pragma unroll
+            for (uint32_t step = kBlocks / 2; step > 0; step >>= 1)
+              if ((lds.prefix[b + step] & 0xFFFFu) <= k) b += step;
+            uint32_t m = lds.masks[b] & 0xFFFFu;
+            for (uint32_t j = k - (lds.prefix[b] & 0xFFFFu); j > 0; --j) m &= m - 1u;
+            return 16u * b + static_cast<uint32_t>(__builtin_ctz(m | 0x10000u));
+          };
+
+          // ---- a word limit: the words of a row past its limit are dropped.  The first such word and the row's end
+          // are marked; a prefix parity over the marks gives the bytes whose word starts and ends go.
+          if (a.max_words > 0) {
+            bool cut = false;
+            auto drop_from = [&](uint32_t k, int64_t e) {  // from word start k up to position e
+              uint32_t const at = word_start(k);
+              atomicXor(&lds.bound[at >> 4], 0x10000u << (at & 15u));
+              if (e < TILE) atomicXor(&lds.bound[e >> 4], 0x10000u << (e & 15));
+              cut = true;
+            };
+            for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
+              uint32_t const r = r_first + i + lane;
+              if (r < r_end) {
+                int64_t const c0 = coord(r), c1 = coord(r + 1);
+                if (c1 > c0) {
+                  int64_t const p = c0 - tb, e = c1 - tb;  // (p < TILE: the rows past the last tile's end are empty)
+                  uint32_t const cap = word_cap(r, c1 - c0);
+                  uint32_t const wp  = words_before(static_cast<uint32_t>(p));
+                  uint32_t const we  = words_before(e < TILE ? static_cast<uint32_t>(e) : static_cast<uint32_t>(TILE));
+                  if (wp + cap < we) drop_from(wp + cap, e);
+                }
+              }
+            }
+            // the row that runs into the tile
+            int64_t const e0   = r_first < r_end ? coord(r_first) - tb : static_cast<int64_t>(TILE);
+            uint32_t const we0 = words_before(e0 < TILE ? static_cast<uint32_t>(e0) : static_cast<uint32_t>(TILE));
+            if (lane == 0 && open_left < we0) drop_from(open_left, e0);
+            // and the row that runs out of it
+            if (r_first < r_end) {
+              uint32_t const rl   = r_end - 1;
+              int64_t const c0    = coord(rl), c1 = coord(rl + 1);
+              int64_t const p     = c0 - tb;
+              uint32_t const cap  = word_cap(rl, c1 - c0);
+              uint32_t const used = nw - words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
+              open_left           = cap - min(cap, used);
+            } else {
+              open_left -= min(open_left, nw);
+            }
+            if (ballot64(cut) != 0) {
+              wave_lds_sync();
+              uint32_t base = 0, carry = 0;
+#pragma unroll
+              for (int s = 0; s < kSubs; ++s) {
+                int const b      = s * kWave + lane;
+                uint32_t const m = lds.masks[b];
+                uint32_t px      = lds.bound[b] >> 16;
+                px ^= px << 1;
+                px ^= px << 2;
+                px ^= px << 4;
+                px ^= px << 8;
+                px &= 0xFFFFu;
+                uint64_t const odd  = ballot64((px >> 15) != 0);
+                uint32_t const flip = (lanes_below(odd) & 1u) ^ carry;
+                carry ^= static_cast<uint32_t>(__builtin_popcountll(odd)) & 1u;
+                uint32_t const dead   = flip ? (~px & 0xFFFFu) : px;
+                uint32_t const starts = m & 0xFFFFu & ~dead, ends = (m >> 16) & ~dead;
+                lds.masks[b]          = starts | (ends << 16);
+                uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
+                uint32_t const incl   = wave_inclusive_scan(cnt);
+                lds.prefix[b]         = base + incl - cnt;
+                base += wave_bcast(incl, kWave - 1);
+              }
+              if (lane == 0) lds.prefix[kBlocks] = base;
+              nw = base & 0xFFFFu;
+              ne = base >> 16;
+              wave_lds_sync();
+            }
+          }
+          // ---- every row that starts in the tile notes the word it begins at (marked as not final), until that
+          // word's tokens have been placed
+          for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
+            uint32_t const r = r_first + i + lane;
+            if (r < r_end) {
+              int64_t const p  = coord(r) - tb;
+              a.offsets_out[r] = static_cast<int32_t>(0x80000000u | words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE)));
+            }
+          }
+          tile_open = true;
+          w_lo      = 0;
+          WP_PHASE(3)
         }
-        uint64_t const idle = ballot64(!busy);
-        if (idle != 0 && next < q_end) {  // refill
-          uint32_t const mine = next + lanes_below(idle);
-          next += static_cast<uint32_t>(__builtin_popcountll(idle));
-          bool is_longer = false;
-          if (!busy && mine < q_end) {
-            const uint4* const src = reinterpret_cast<const uint4*>(queue + mine);
-            uint4 const a = load_stream(src), b = load_stream(src + 1);
-            if (static_cast<int32_t>(a.x) >= 0) {  // (-1 marks the unused tail of a reserved queue range)
-              if (a.w <= 16) {
-                q   = mine;
-                row = static_cast<int32_t>(a.x);
-                uint32_t const head[4] = {b.x, b.y, b.z, b.w};
-                sw.begin(table, head, a.w);
-                busy = true;
-              } else {
-                is_longer = true;
+        if (tile_open) {
+          // ================================================================ a new unit: words [w_lo, w_hi) of the tile
+          w_hi = min(nw, w_lo + kWordCap);
+          nwc  = w_hi - w_lo;
+          uint16_t* const word16 = reinterpret_cast<uint16_t*>(lds.word[par]);
+          // start k pairs with end k (after the end of the word that ran into the tile)
+#pragma unroll
+          for (int s = 0; s < kSubs; ++s) {
+            int const b       = s * kWave + lane;
+            uint32_t const m  = lds.masks[b];
+            uint32_t const pf = lds.prefix[b];
+            uint32_t ks       = pf & 0xFFFFu;
+            int32_t ke        = static_cast<int32_t>(pf >> 16) - static_cast<int32_t>(inside0);
+            for (uint32_t st = m & 0xFFFFu; st; st &= st - 1u, ++ks)
+              if (ks >= w_lo && ks < w_hi) word16[2 * (ks - w_lo)] = static_cast<uint16_t>(16 * b + __builtin_ctz(st));
+            for (uint32_t en = m >> 16; en; en &= en - 1u, ++ke)
+              if (ke >= static_cast<int32_t>(w_lo) && ke < static_cast<int32_t>(w_hi)) word16[2 * (ke - w_lo) + 1] = static_cast<uint16_t>(16 * b + __builtin_ctz(en));
+          }
+          if (w_hi == nw && nwc > 0 && nw + inside0 > ne) {
+            // the last word ends past the tile: at the byte before the first space, row start or end of the view
+            uint32_t sep = 0;
+            if (lane < kOverBlocks) {
+              int const b   = kBlocks + lane;
+              uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
+              sep           = space_mask16(v) | (lds.bound[b] & 0xFFFFu);
+              if (edge) sep |= outside_mask16(tb + 16 * b, cbeg, cend);
+            }
+            uint64_t const sm = ballot64(sep != 0);
+            uint32_t endpos   = TILE + 16 * kOverBlocks - 1;
+            if (sm != 0) {
+              int const fl = __builtin_ctzll(sm);
+              endpos       = TILE + 16 * fl + __builtin_ctz(wave_bcast(sep, fl)) - 1;
+            }
+            if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
+          }
+          if (par) tok_used1 = 0;
+          else tok_used0 = 0;
+          k0        = 0;
+          unit_open = true;
+          wave_lds_sync();
+          WP_PHASE(4)
+        }
+      }
+      if (unit_open) {
+        // ================================================================ look the words up; the ones that are not in
+        // the vocabulary wait in the queue
+        uint32_t* const uw = lds.word[par];
+        while (k0 < nwc && qn + kWave <= kQueueCap) {
+          uint32_t const k  = k0 + lane;
+          bool miss         = false;
+          if (k < nwc) {
+            uint32_t const rec = uw[k];
+            uint32_t const s   = rec & 0xFFFFu;
+            uint32_t const wl  = (rec >> 16) - s + 1u;
+            uint32_t value;
+            if (wl >= kMaxWord) {
+              value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+            } else {
+              int32_t id = kNone;
+              TileWord const tw{lds.bytes, 16u + s};
+              uint32_t head[4];
+              tw.head16(head);
+              trim_key8(wl, head[0], head[1]);
+              trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
+              if (wl <= table.max_len[0]) {
+                Probe pr;
+                pr.k0 = head[0];
+                pr.k1 = head[1];
+                uint32_t h        = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
+                uint32_t const h2 = key_hash_block(h, head[2], head[3]);
+                h                 = wl > 8 ? h2 : h;  // (not the hash of a word of more than 16 bytes: those go to the general lookup)
+                uint32_t bk;
+                pr.want   = slot_word0(h, 0, wl, &bk);
+                pr.bucket = bk & table.bucket_mask;
+                uint4 const s0 = table.slots[2 * pr.bucket];
+                uint4 const s1 = table.slots[2 * pr.bucket + 1];
+                uint32_t vd = wl > 16 ? 2u : verdict(pr, s0, s1, wl, &id);
+                if (vd == 2u && wl > 8 && wl <= 16) vd = verdict_16(table, pr, s0, s1, head, &id);
+                if (vd == 2u) id = lookup_slow(table, 0u, tw, 0u, wl);
+                else if (vd == 0u) id = kNone;
+              }
+              miss  = id == kNone;
+              value = static_cast<uint32_t>(id);
+            }
+            if (!miss) uw[k] = value;
+          }
+          uint64_t const mm = ballot64(miss);
+          if (miss) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k);
+          qn += static_cast<uint32_t>(__builtin_popcountll(mm));
+          k0 += kWave;
+        }
+        reason = k0 >= nwc ? kUnitDone : kQueueFull;
+        wave_lds_sync();
+        WP_PHASE(5)
+      }
+
+      // ================================================================ the out-of-vocabulary words, one lane each; a lane
+      // that finishes stores its result and takes the next word from the queue.  Words of up to 16 bytes run in
+      // registers; the few longer ones are set aside (queue[0 .. n_long)) and only counted here.
+      {
+        // stores the tokens of the words finished by this step
+        auto deliver = [&](bool fin, uint32_t cnt) {
+          uint32_t const keep   = fin && cnt <= kOovKeep ? cnt : 0u;
+          uint32_t const packed = mine_par ? keep << 16 : keep;
+          uint32_t const incl   = wave_inclusive_scan(packed);
+          uint32_t const ex     = incl - packed;
+          uint32_t const tot    = wave_bcast(incl, kWave - 1);
+          uint32_t const off    = mine_par ? tok_used1 + (ex >> 16) : tok_used0 + (ex & 0xFFFFu);
+          tok_used0 += tot & 0xFFFFu;
+          tok_used1 += tot >> 16;
+          if (fin) {
+            uint32_t* const slot = &lds.word[mine_par][mine];
+            if (keep > 0 && off + keep <= kTokCap) {
+#pragma unroll
+              for (int i = 0; i < kOovKeep; ++i)
+                if (static_cast<uint32_t>(i) < keep) lds.tokens[mine_par][off + i] = static_cast<uint32_t>(tok[i]);
+              *slot = kOovMark | (cnt << 16) | off;
+            } else {
+              uint32_t const rec = *slot;
+              uint32_t const s   = rec & 0xFFFFu;
+              *slot              = kOovMark | kOovRedo | (cnt << 21) | (((rec >> 16) - s + 1u) << 13) | s;
+            }
+          }
+        };
+        uint32_t n_long = 0;
+        for (;;) {
+          bool const fin      = busy && sw.done;
+          uint64_t const finm = ballot64(fin);
+          if (finm != 0 || q_next < qn) {
+            if (finm != 0) {
+              deliver(fin, sw.count);
+              if (fin) busy = false;
+            }
+            uint64_t const idle = ballot64(!busy);
+            uint32_t const left = qn - q_next;
+            if (left > 0 && idle != 0) {
+              uint32_t const rank = lanes_below(idle);
+              bool is_long        = false;
+              uint32_t k          = 0;
+              if (!busy && rank < left) {
+                k                  = lds.queue[q_next + rank];
+                uint32_t const rec = lds.word[par][k];
+                uint32_t const s   = rec & 0xFFFFu;
+                uint32_t const wl  = (rec >> 16) - s + 1u;
+                if (wl <= 16) {
+                  TileWord const tw{lds.bytes, 16u + s};
+                  uint32_t head[4];
+                  tw.head16(head);
+                  trim_key8(wl, head[0], head[1]);
+                  trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
+                  sw.begin(table, head, wl);
+                  busy     = true;
+                  mine     = k;
+                  mine_par = par;
+                } else {
+                  is_long = true;
+                }
+              }
+              q_next += min(static_cast<uint32_t>(__builtin_popcountll(idle)), left);
+              uint64_t const lm = ballot64(is_long);
+              if (lm != 0) {
+                wave_lds_sync();  // (the queue entries just read lie at or past n_long)
+                if (is_long) lds.queue[n_long + lanes_below(lm)] = static_cast<uint16_t>(k);
+                n_long += static_cast<uint32_t>(__builtin_popcountll(lm));
               }
             }
           }
-          uint64_t const lm = ballot64(is_longer);
-          if (lm != 0) {
-            if (is_longer) longer[q_begin + n_longer + lanes_below(lm)] = mine;
-            n_longer += static_cast<uint32_t>(__builtin_popcountll(lm));
+          uint64_t const bm = ballot64(busy);
+          if (q_next >= qn) {
+            if (bm == 0 || reason == kQueueFull) break;
+            if (reason == kUnitDone && ballot64(busy && mine_par != par) == 0 && __builtin_popcountll(bm) < kStragglers) break;
+          }
+#ifdef WP_PHASE_TIMING
+          phase_t[9] += 1;
+#endif
+          if (busy && !sw.done) sw.step(table, keep_token);
+        }
+        if (n_long > 0) {
+          wave_lds_sync();
+          for (uint32_t base = 0; base < n_long; base += kWave) {
+            if (base + lane < n_long) {
+              uint32_t const k   = lds.queue[base + lane];
+              uint32_t const rec = lds.word[par][k];
+              uint32_t const s   = rec & 0xFFFFu;
+              uint32_t const wl  = (rec >> 16) - s + 1u;
+              uint32_t const cnt = count_oov_tokens(table, lds.bytes, 16u + s, wl);
+              lds.word[par][k]   = kOovMark | kOovRedo | (cnt << 21) | (wl << 13) | s;
+            }
           }
         }
-        if (ballot64(busy) == 0 && next >= q_end) break;
+        qn     = 0;
+        q_next = 0;
+        wave_lds_sync();
+        WP_PHASE(6)
       }
-      if (busy && !sw.done) sw.step(table, keep_token);
-    }
-  }
+      if (reason == kQueueFull) continue;
 
-  if (lane == 0) longer[queue_capacity + wave] = n_longer;
-}
-
-// The queued words of more than 16 bytes, which the kernel above has set aside (same grid, same parts):
-// one lane per word, bytes staged from the chars into the lane's LDS window, the general state machine.
-__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
-                                                                         const uint32_t* __restrict__ queue_size, uint32_t queue_capacity,
-                                                                         OovResult* __restrict__ results, int32_t* __restrict__ counts,
-                                                                         const uint32_t* __restrict__ longer)
-{
-  __shared__ uint32_t windows[kStage / 4][kOovThreads];
-  uint32_t* const win    = &windows[0][threadIdx.x];
-  if (*queue_size > queue_capacity) return;  // (see wordpiece_oov_kernel)
-  uint32_t const total   = min(*queue_size, queue_capacity);
-  uint32_t const nwave   = gridDim.x * (kOovThreads / kWave);
-  uint32_t const wave    = blockIdx.x * (kOovThreads / kWave) + threadIdx.x / kWave;
-  uint32_t const chunk   = (total + nwave - 1) / nwave;
-  uint32_t const q_begin = min(total, wave * chunk);
-  uint32_t const n_longer = longer[queue_capacity + wave];
-  uint32_t const lane    = static_cast<uint32_t>(lane_id());
-  for (uint32_t base = 0; base < n_longer; base += kWave) {
-    if (base + lane < n_longer) {
-      uint32_t const q = longer[q_begin + base + lane];
-      OovEntry const e = queue[q];
-      const uint8_t* p = col.chars + col.off(e.row) + e.delta;
-      bool ascii;
-      StagedWord w{win, p, 0};
-      w.mis = stage_word(p, e.len, win, &ascii);
-      OovResult res;
-      OovStepper<StagedWord> st;
-      st.begin(table, w, e.len, ascii);
-      while (!st.done) {
-        st.step(table, w, [&](uint32_t j, int32_t id) {
+      // ================================================================ the unit before: place and write its tokens
+      if (pend) {
+        uint32_t* const uw       = lds.word[p_par];
+        const uint32_t* const ut = lds.tokens[p_par];
+        uint32_t done            = 0;  // tokens of the unit so far
+        for (uint32_t j0 = 0; j0 < p_nwc; j0 += kWave) {
+          uint32_t const k   = j0 + lane;
+          bool const active  = k < p_nwc;
+          uint32_t const v   = active ? uw[k] : 0u;
+          bool const marked  = active && (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
+          bool const redo    = marked && (v & kOovRedo) != 0;
+          uint32_t const cnt = !active ? 0u : !marked ? 1u : redo ? (v >> 21) & 0xFFu : (v >> 16) & 0xFFu;
+          uint32_t const incl = wave_inclusive_scan(cnt);
+          uint32_t const ex   = incl - cnt;
+          uint32_t const tot  = wave_bcast(incl, kWave - 1);
+          if (cursor + done + tot > a.range_cap) spill = true;
+          if (!spill) {
+            uint32_t* const dst = region + (cursor + done + ex);
+            if (redo) {
+              // tokens that were not kept (more than kOovKeep, a word of more than 16 bytes, no room left in LDS):
+              // tokenized again, into place
+              write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + p_tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
+            } else if (active) {
+              uint32_t const off = v & 0xFFFFu;
+              dst[0]             = marked ? ut[off] : v;
 #pragma unroll
-          for (int k = 0; k < kOovKeep; ++k)
-            if (j == static_cast<uint32_t>(k)) res.tok[k] = id;
-        });
-      }
-      res.count  = st.count;
-      results[q] = res;
-      if (st.count > 1) atomicAdd(&counts[e.row], static_cast<int32_t>(st.count - 1));
-    }
-  }
-}
-
-// ------------------------------------------------------------------ emit pass
-// Expands the word arena into the child column.  A wavefront takes a block of consecutive rows at a time (at most
-// 64, fewer where rows have many tokens: emit_blocks_kernel; lanes <-> rows for the descriptors), then walks ALL
-// their words flat, lanes <-> words: because the
-// list offsets are a prefix sum in row order, the tokens of consecutive words are consecutive in the
-// child even across row boundaries, so only the block's first offset is needed.  Each word finds its
-// row by binary search in the block's word-count prefix (LDS); its lane then writes its tokens (one, or the up to
-// kOovKeep that the out-of-vocabulary pass left in its result record) behind those of the lanes below it.
-struct EmitLds {
-  uint32_t word_prefix[kWave + 1];  // words before row k of the block
-  int64_t slot0[kWave];             // arena slot of word 0 of row k
-};
-
-__global__ void __launch_bounds__(kTokThreads) wordpiece_emit_kernel(ColView col, VocabTable table, int64_t first_offset,
-                                                                     const uint32_t* __restrict__ arena,
-                                                                     const int32_t* __restrict__ nwords, OovResult* __restrict__ results,
-                                                                     const int32_t* __restrict__ offsets, int32_t* __restrict__ out,
-                                                                     const int32_t* __restrict__ block_first, int64_t nblocks,
-                                                                     uint32_t* __restrict__ again, uint32_t* __restrict__ again_count)
-{
-  // block_rows (1..64) rows per wavefront at a time: fewer when rows are long, so that the walks stay
-  // short and there are enough of them to fill the device
-  __shared__ EmitLds lds_all[kTokWaves];
-  int const lane        = lane_id();
-  int const wave        = threadIdx.x / kWave;
-  EmitLds& lds          = lds_all[wave];
-  int64_t const nwave   = static_cast<int64_t>(gridDim.x) * kTokWaves;
-  auto lds_sync = [] {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  };
-  for (int64_t blk = static_cast<int64_t>(blockIdx.x) * kTokWaves + wave; blk < nblocks; blk += nwave) {
-    // rows [first, next) of the block: at most kWave
-    int32_t const first = block_first[blk], next = block_first[blk + 1];
-    int64_t const r     = static_cast<int64_t>(first) + lane;
-    uint32_t W          = 0;
-    int64_t slot0       = 0;
-    if (lane < next - first) {
-      W     = static_cast<uint32_t>(nwords[r]);
-      slot0 = arena_pos(col, first_offset, r);
-    }
-    int32_t const base   = offsets[first];
-    uint32_t const incl  = wave_inclusive_scan(W);
-    uint32_t const total = wave_bcast(incl, kWave - 1);
-    lds.word_prefix[lane] = incl - W;
-    if (lane == kWave - 1) lds.word_prefix[kWave] = total;
-    lds.slot0[lane] = slot0;
-    lds_sync();
-
-    // the arena entry of flat word j: row k = last row with word_prefix[k] <= j (rows without words are skipped
-    // because their prefix equals the next row's)
-    auto load_value = [&](uint32_t j) -> uint32_t {
-      if (j >= total) return 0u;
-      uint32_t lo = 0;
-#pragma unroll
-      for (uint32_t step = kWave / 2; step > 0; step >>= 1)
-        if (lds.word_prefix[lo + step] <= j) lo += step;
-      return arena[lds.slot0[lo] + (j - lds.word_prefix[lo])];
-    };
-    // tokens of flat word j whose arena value is v: one, or what the out-of-vocabulary pass found (its whole
-    // result record is fetched here, once)
-    auto count_of = [&](uint32_t j, uint32_t v, uint4& ra, uint4& rb) -> uint32_t {
-      if (j >= total) return 0u;
-      if ((v & kOovMark) == 0 || v == 0xFFFFFFFFu) return 1u;
-      const uint4* const src = reinterpret_cast<const uint4*>(results + (v & ~kOovMark));
-      ra = src[0];
-      rb = src[1];
-      return rb.w;  // OovResult: seven tokens, then the count
-    };
-
-    int32_t* const dst = out + base;
-    uint32_t done      = 0;  // tokens written so far in this block
-    // three stages in flight: arena value two rounds ahead, token count one round ahead, the round being written
-    uint32_t v_nxt = load_value(lane);
-    uint32_t v_far = load_value(kWave + lane);
-    uint4 a_nxt = make_uint4(0u, 0u, 0u, 0u), b_nxt = a_nxt;
-    uint32_t c_nxt = count_of(lane, v_nxt, a_nxt, b_nxt);
-    for (uint32_t j0 = 0; j0 < total; j0 += kWave) {
-      uint32_t const value = v_nxt, cnt = c_nxt;
-      uint4 const ra = a_nxt, rb = b_nxt;
-      v_nxt = v_far;
-      c_nxt = count_of(j0 + kWave + lane, v_nxt, a_nxt, b_nxt);
-      v_far = load_value(j0 + 2 * kWave + lane);
-      uint32_t const here   = min(total - j0, static_cast<uint32_t>(kWave));  // words of this round (every word has >= 1 token)
-      uint32_t const incl2  = wave_inclusive_scan(cnt);
-      uint32_t const tokens = wave_bcast(incl2, kWave - 1);
-      bool const marked     = static_cast<uint32_t>(lane) < here && (value & kOovMark) != 0 && value != 0xFFFFFFFFu;
-      // lanes <-> words: every lane writes its word's tokens behind those of the words below it, token k of all
-      // words at a time (a word from the queue has up to kOovKeep of them in its record)
-      int32_t* const mine = dst + done + (incl2 - cnt);
-      if (marked && cnt > kOovKeep) {
-        // more pieces than a result record keeps (seldom): noted for wordpiece_retokenize_kernel, with the
-        // place of the word's first token in the child left where its tokens would have been
-        uint32_t const q = value & ~kOovMark;
-        again[atomicAdd(again_count, 1u)] = q;
-        results[q].tok[0]                 = base + static_cast<int32_t>(done + (incl2 - cnt));
-      } else {
-        uint32_t const mc = static_cast<uint32_t>(lane) < here ? cnt : 0u;
-        if (mc > 0u) mine[0] = static_cast<int32_t>(marked ? ra.x : value);
-        if (ballot64(mc > 1u) != 0) {
-          if (mc > 1u) mine[1] = static_cast<int32_t>(ra.y);
-          if (mc > 2u) mine[2] = static_cast<int32_t>(ra.z);
-          if (ballot64(mc > 3u) != 0) {
-            if (mc > 3u) mine[3] = static_cast<int32_t>(ra.w);
-            if (mc > 4u) mine[4] = static_cast<int32_t>(rb.x);
-            if (mc > 5u) mine[5] = static_cast<int32_t>(rb.y);
-            if (mc > 6u) mine[6] = static_cast<int32_t>(rb.z);
+              for (uint32_t j = 1; j < kOovKeep; ++j) {
+                if (ballot64(marked && j < cnt) == 0) break;
+                if (marked && j < cnt) dst[j] = ut[off + j];
+              }
+            }
+          }
+          if (active) uw[k] = done + ex;
+          done += tot;
+        }
+        wave_lds_sync();
+        WP_PHASE(7)
+        // the rows that start in its tile at one of its words (or, for the last words of the tile, after them): the
+        // tokens of the range before them
+        bool const p_last = p_wlo + p_nwc == p_nw;
+        for (uint32_t i = 0; p_rfirst + i < p_rend; i += kWave) {
+          uint32_t const r = p_rfirst + i + lane;
+          if (r < p_rend) {
+            uint32_t const v = static_cast<uint32_t>(a.offsets_out[r]);
+            if ((v & 0x80000000u) != 0) {
+              uint32_t const k = v & 0x7FFFFFFFu;
+              if (k >= p_wlo && k < p_wlo + p_nwc) a.offsets_out[r] = static_cast<int32_t>(cursor + uw[k - p_wlo]);
+              else if (k == p_nw && p_last) a.offsets_out[r] = static_cast<int32_t>(cursor + done);
+            }
           }
         }
+        cursor += done;
+        pend = false;
+        wave_lds_sync();
+        WP_PHASE(8)
       }
-      done += tokens;
+      if (reason == kRangeDone) break;
+      // the unit just looked up waits for its last words
+      pend     = true;
+      p_tb     = tb;
+      p_par    = par;
+      p_nwc    = nwc;
+      p_wlo    = w_lo;
+      p_nw     = nw;
+      p_rfirst = r_first;
+      p_rend   = r_end;
+      par ^= 1u;
+      unit_open = false;
+      w_lo      = w_hi;
+      if (w_hi == nw) {
+        tile_open = false;
+        ++t;
+      }
     }
-    lds_sync();
+    if (lane == 0) {
+      a.range_count[range] = cursor;
+      if (spill) *a.overflow = 1u;
+    }
   }
+#ifdef WP_PHASE_TIMING
+  if (lane == 0)
+    for (int i = 0; i < 10; ++i) atomicAdd(reinterpret_cast<unsigned long long*>(a.overflow + 3) + i, static_cast<unsigned long long>(phase_t[i]));
+#endif
 }
 
-// The words that have more pieces than a result record keeps (the emit pass has listed them in again[0 .. *again_count)
-// and left the index of each one's first token in the child in its result record): tokenized again, straight into
-// place.  One lane per word; kept apart from the emit pass so that it is compiled for its common case (a third of
-// the registers, all the wavefronts a unit can hold).
-__global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(ColView col, VocabTable table, const OovEntry* __restrict__ queue,
-                                                                           const OovResult* __restrict__ results,
-                                                                           const uint32_t* __restrict__ again,
-                                                                           const uint32_t* __restrict__ again_count, int32_t* __restrict__ out)
-{
-  uint32_t const n = *again_count;
-  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
-    uint32_t const q = again[i];
-    OovEntry const e = queue[q];
-    const uint8_t* p = col.chars + col.off(e.row) + e.delta;
-    int32_t* const d = out + results[q].tok[0];
-    tokenize_oov_word(table, GlobalWord{p}, e.len, [&](uint32_t j, int32_t id) { d[j] = id; });
-  }
-}
-
-// The blocks of rows of the emit pass: block b begins with the first row r for which offsets[r] + kEmitRowWeight * r
-// reaches b * kEmitBlockWork, so a block holds at most kEmitBlockWork / kEmitRowWeight = 64 rows and, unless it is a
-// single row, fewer than kEmitBlockWork tokens, however uneven the rows are.  block_first has nblocks + 1 entries.
-constexpr int64_t kEmitRowWeight = 128;
-constexpr int64_t kEmitBlockWork = kEmitRowWeight * kWave;
-__global__ void emit_blocks_kernel(const int32_t* __restrict__ offsets, int64_t rows, int64_t nblocks, int32_t* __restrict__ block_first)
-{
-  int64_t const b = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (b > nblocks) return;
-  int64_t lo = 0, hi = rows;  // the first row in [0, rows] with that much work before it
-  if (b == nblocks) lo = rows;
-  int64_t const target = b * kEmitBlockWork;
-  while (lo < hi) {
-    int64_t const mid = (lo + hi) >> 1;
-    if (static_cast<int64_t>(offsets[mid]) + kEmitRowWeight * mid < target) lo = mid + 1;
-    else hi = mid;
-  }
-  block_first[b] = static_cast<int32_t>(lo);
-}
-
-// ------------------------------------------------------------------ very long rows
-// A row is walked by one group of lanes in the probe pass and by one wavefront in the emit pass, so a row of
-// megabytes would take milliseconds while the rest of the device is idle.  Without a word limit the tokens of a row
-// are simply those of its words in order, so such a row can be cut at spaces into pieces that are tokenized as
-// rows of their own; the list offsets of the original rows are then those of their first pieces.
-constexpr int64_t kLongRow  = 32 * 1024;  // rows beyond this many bytes are cut
-constexpr int64_t kRowPiece = 16 * 1024;  // into pieces of about this many
-
-// pieces[r] = pieces row r is cut into (1 for rows that stay whole); *any_long = 1 when some row is cut
-__global__ void long_rows_kernel(ColView col, uint32_t* __restrict__ pieces, uint32_t* __restrict__ any_long)
-{
-  int64_t const r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (r >= col.size) return;
-  int64_t const bytes = col.off(r + 1) - col.off(r);
-  bool const is_long  = bytes > kLongRow;
-  pieces[r]           = is_long ? static_cast<uint32_t>((bytes + kRowPiece - 1) / kRowPiece) : 1u;
-  if (is_long) *any_long = 1u;
-}
-
-struct PiecesOf {
-  const uint32_t* pieces;
-  __device__ uint64_t operator()(int64_t i) const { return pieces[i]; }
+struct RangeCountOf {
+  const uint32_t* counts;
+  __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
 };
 
-// piece_offset[v] = where piece v begins: piece j > 0 of a row begins at the first space at or after byte
-// j * kRowPiece of the row (the row's end if there is none), so no word is cut.  first_piece[r] = index of row r's
-// first piece, first_piece[rows] = number of pieces.
-__global__ void piece_offsets_kernel(ColView col, const uint32_t* __restrict__ first_piece, int64_t pieces, int64_t* __restrict__ piece_offset)
+// Blocks 0 .. nranges-1: the tokens of a range go from the arena to their place in the child.  The blocks after
+// them: every row's offset becomes absolute (the tokens before its range are added), and offsets[rows] the total.
+__global__ void __launch_bounds__(256) wordpiece_gather_kernel(ColView col, int64_t first_offset, uint32_t cbeg, int range_shift, uint32_t nranges,
+                                                               const uint32_t* __restrict__ arena, uint32_t range_cap,
+                                                               const uint32_t* __restrict__ range_count, const int64_t* __restrict__ range_base,
+                                                               int32_t* __restrict__ child, int32_t* __restrict__ offsets)
 {
-  int64_t const v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (v > pieces) return;
-  int64_t const rows = col.size;
-  if (v == pieces) {
-    piece_offset[v] = col.off(rows);
+  if (blockIdx.x < nranges) {
+    uint32_t const g        = blockIdx.x;
+    const uint32_t* src     = arena + static_cast<int64_t>(g) * range_cap;
+    uint32_t* dst           = reinterpret_cast<uint32_t*>(child) + range_base[g];
+    uint32_t const n        = range_count[g];
+    for (uint32_t i = threadIdx.x; i < n; i += 256) dst[i] = src[i];
     return;
   }
-  int64_t lo = 0, hi = rows - 1;  // the last row whose first piece is at or before v
-  while (lo < hi) {
-    int64_t const mid = (lo + hi + 1) >> 1;
-    if (static_cast<int64_t>(first_piece[mid]) <= v) lo = mid;
-    else hi = mid - 1;
+  int64_t const rows = col.size;
+  int64_t const r    = static_cast<int64_t>(blockIdx.x - nranges) * 256 + threadIdx.x;
+  if (r < rows) {
+    int64_t const c = col.off(r) - first_offset + cbeg;
+    uint32_t g      = static_cast<uint32_t>(c >> range_shift);
+    if (g >= nranges) g = nranges - 1;
+    offsets[r] += static_cast<int32_t>(range_base[g]);
+  } else if (r == rows) {
+    offsets[rows] = static_cast<int32_t>(range_base[nranges]);
   }
-  int64_t const j = v - first_piece[lo];
-  int64_t p       = col.off(lo);
-  if (j > 0) {
-    int64_t const end = col.off(lo + 1);
-    p += j * kRowPiece;
-    // eight bytes at a time from an aligned address (ordinary text has a space within a few bytes; a stretch
-    // without one is read to its end)
-    const uint8_t* const chars = col.chars;
-    while (p < end && (reinterpret_cast<uintptr_t>(chars + p) & 7u) != 0 && chars[p] != ' ') ++p;
-    while (p + 8 <= end && chars[p] != ' ') {
-      uint2 const w      = *reinterpret_cast<const uint2*>(chars + p);
-      uint32_t const lo  = space_bytes(w.x), hi = space_bytes(w.y);
-      if ((lo | hi) != 0) {
-        p += lo ? (__builtin_ctz(lo) >> 3) : 4 + (__builtin_ctz(hi) >> 3);
-        break;
-      }
-      p += 8;
-    }
-    while (p < end && chars[p] != ' ') ++p;
-  }
-  piece_offset[v] = p;
 }
-
-// offsets[r] = piece_token_offsets[first_piece[r]] for r in 0..rows
-__global__ void row_offsets_of_pieces_kernel(const int32_t* __restrict__ piece_token_offsets, const uint32_t* __restrict__ first_piece,
-                                             int64_t rows, int32_t* __restrict__ offsets)
-{
-  int64_t const r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (r <= rows) offsets[r] = piece_token_offsets[first_piece[r]];
-}
-
-struct CountOf {
-  const int32_t* counts;
-  __device__ uint64_t operator()(int64_t i) const { return static_cast<uint64_t>(counts[i]); }
-};
 
 // ------------------------------------------------------------------ vocabulary construction (host)
 struct HostSlot {
@@ -1645,21 +1566,9 @@ void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
 
 int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* v) { return v ? v->table.unk_id : -1; }
 
-// may_cut_rows: very long rows may be cut into pieces that are tokenized as rows (false in the call that does the pieces)
-static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
-                                       int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out,
-                                       bool may_cut_rows);
-
 nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
                                                 int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_,
                                                 nvtext_amd_list_column* out)
-{
-  return tokenize_rows(input, vocabulary, max_words_per_row, stream_, mr_, out, true);
-}
-
-static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
-                                       int32_t max_words_per_row, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out,
-                                       bool may_cut_rows)
 {
   using namespace nvtext_amd;
   if (!input || !vocabulary || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
@@ -1672,6 +1581,10 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
   Mr mr{mr_, stream};
   int32_t const rows = input->size;
   out->child_type    = NVTEXT_AMD_TYPE_INT32;
+  auto give_up = [&](nvtext_amd_status st, const char* what) {
+    nvtext_amd_list_column_free(out, stream_, mr_);
+    return fail(st, what);
+  };
 
   if (rows == input->null_count) {  // wordpiece_tokenize.cu:849-853
     if (rows == 0) return NVTEXT_AMD_SUCCESS;  // canonical empty list column: no rows, no offsets
@@ -1683,13 +1596,10 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
     out->offsets       = static_cast<int32_t*>(mr.allocate(out->offsets_bytes));
     out->null_mask_bytes = mask_alloc_bytes(rows);
     out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
-    if (!out->offsets || !out->null_mask) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_ALLOC_FAILED, "allocation failed");
-    }
+    if (!out->offsets || !out->null_mask) return give_up(NVTEXT_AMD_ALLOC_FAILED, "allocation failed");
     launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, rows + 1, stream);
     launch_fill_u32(out->null_mask, 0u, static_cast<int64_t>(out->null_mask_bytes / 4), stream);
-    NVTEXT_HIP_TRY(hipGetLastError());
+    if (hipGetLastError() != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, "kernel launch failed");
     return NVTEXT_AMD_SUCCESS;
   }
 
@@ -1702,34 +1612,13 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
   if (input->null_mask) {
     out->null_mask_bytes = mask_alloc_bytes(rows);
     out->null_mask       = static_cast<uint32_t*>(mr.allocate(out->null_mask_bytes));
-    if (!out->null_mask) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
-    }
+    if (!out->null_mask) return give_up(NVTEXT_AMD_ALLOC_FAILED, "mask allocation failed");
     launch_copy_bitmask(out->null_mask, input->null_mask, input->offset, rows, stream);
   }
 
   ColView const v = make_view(*input);
-  // Without a word limit very long rows are cut into pieces (see long_rows_kernel): are there any?  The answer
-  // comes back with the two offsets read below.
-  bool const look_for_long_rows = may_cut_rows && max_words_per_row == 0;
-  size_t const cut_bytes[3]     = {look_for_long_rows ? static_cast<size_t>(rows) * sizeof(uint32_t) : 0,
-                                   look_for_long_rows ? (static_cast<size_t>(rows) + 1) * sizeof(uint32_t) : 0, look_for_long_rows ? 256u : 0u};
-  TempParts<3> const cut_temps(mr, cut_bytes);
-  uint32_t* const pieces      = cut_temps.part<uint32_t>(0);
-  uint32_t* const first_piece = cut_temps.part<uint32_t>(1);
-  uint32_t* const any_long    = cut_temps.part<uint32_t>(2);
-  uint32_t has_long           = 0;
-  if (look_for_long_rows) {
-    if (!cut_temps.ok()) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-    }
-    launch_fill_u32(any_long, 0u, 1, stream);
-    hipLaunchKernelGGL(long_rows_kernel, dim3(static_cast<unsigned>((rows + 255) / 256)), dim3(256), 0, stream, v, pieces, any_long);
-  }
-  // first and last offset of the view (the reference reads the same two scalars,
-  // cpp/src/strings/utilities.cu:180-190); they size the token arena
+  // first and last offset of the view (the reference reads the same two scalars, cpp/src/strings/utilities.cu:180-190):
+  // the bytes between them are what is tokenized
   size_t const ow = input->offsets_is_int64 ? 8 : 4;
   int64_t first_offset = 0, last_offset = 0;
   {
@@ -1737,12 +1626,8 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
     const uint8_t* d_off  = static_cast<const uint8_t*>(input->offsets) + static_cast<size_t>(input->offset) * ow;
     hipError_t e          = hipMemcpyAsync(buf, d_off, ow, hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipMemcpyAsync(buf + 8, d_off + static_cast<size_t>(rows) * ow, ow, hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess && look_for_long_rows) e = hipMemcpyAsync(&has_long, any_long, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
-    }
+    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
     if (ow == 8) {
       std::memcpy(&first_offset, buf, 8);
       std::memcpy(&last_offset, buf + 8, 8);
@@ -1754,174 +1639,120 @@ static nvtext_amd_status tokenize_rows(const nvtext_amd_strings_column* input, c
       last_offset  = b32;
     }
   }
-  if (last_offset < first_offset) {
-    nvtext_amd_list_column_free(out, stream_, mr_);
-    return fail(NVTEXT_AMD_INVALID_ARGUMENT, "offsets are not monotone");
-  }
-  if (has_long != 0) {
-    // the pieces as a strings column of their own over the same chars (int64 offsets, no mask: validity is not
-    // consulted without a word limit), tokenized by this same function; then the rows' offsets from their first pieces
-    auto give_up = [&](nvtext_amd_status st, const char* what) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(st, what);
-    };
-    Temp scan_tmp(mr, scan_temp_bytes(rows));
-    if (!scan_tmp.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-    device_exclusive_scan(PiecesOf{pieces}, static_cast<int64_t>(rows), first_piece, scan_tmp.as<uint64_t>(), stream);
-    uint64_t n_pieces = 0;
-    hipError_t e      = hipMemcpyAsync(&n_pieces, scan_tmp.as<uint64_t>() + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
-    if (n_pieces > static_cast<uint64_t>(std::numeric_limits<int32_t>::max()) - 1) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
-    Temp piece_offset(mr, (static_cast<size_t>(n_pieces) + 1) * sizeof(int64_t));
-    if (!piece_offset.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-    hipLaunchKernelGGL(piece_offsets_kernel, dim3(static_cast<unsigned>((n_pieces + 1 + 255) / 256)), dim3(256), 0, stream, v, first_piece,
-                       static_cast<int64_t>(n_pieces), piece_offset.as<int64_t>());
-    nvtext_amd_strings_column cut{};
-    cut.chars            = input->chars;
-    cut.offsets          = piece_offset.ptr;
-    cut.offsets_is_int64 = 1;
-    cut.size             = static_cast<int32_t>(n_pieces);
-    nvtext_amd_list_column of_pieces{};
-    nvtext_amd_status const st = tokenize_rows(&cut, vocabulary, 0, stream_, mr_, &of_pieces, false);
-    if (st != NVTEXT_AMD_SUCCESS) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return st;
-    }
-    hipLaunchKernelGGL(row_offsets_of_pieces_kernel, dim3(static_cast<unsigned>((rows + 1 + 255) / 256)), dim3(256), 0, stream, of_pieces.offsets,
-                       first_piece, static_cast<int64_t>(rows), out->offsets);
-    out->child       = of_pieces.child;  // the tokens are the pieces' tokens, in the same order
-    out->child_size  = of_pieces.child_size;
-    out->child_bytes = of_pieces.child_bytes;
-    of_pieces.child  = nullptr;
-    of_pieces.child_bytes = 0;
-    nvtext_amd_list_column_free(&of_pieces, stream_, mr_);
-    NVTEXT_HIP_TRY(hipGetLastError());
+  if (last_offset < first_offset) return give_up(NVTEXT_AMD_INVALID_ARGUMENT, "offsets are not monotone");
+  if (last_offset == first_offset) {  // rows without bytes: no tokens
+    launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, rows + 1, stream);
+    if (hipGetLastError() != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, "kernel launch failed");
     return NVTEXT_AMD_SUCCESS;
   }
-  // word arena: one slot per possible word; row r gets floor(bytes/2) + 1 slots
-  size_t const arena_slots = static_cast<size_t>((last_offset - first_offset) >> 1) + static_cast<size_t>(rows) + 1;
-  // queue of words whose whole-word probe missed.  Sized for a generous share of the input; if a run
-  // overflows it the exact size is known afterwards and the passes are repeated once.
+
+  constexpr int kTile         = 2048;
+  constexpr int64_t kRange    = static_cast<int64_t>(kTile) * kRangeTiles;
+  constexpr int kRangeShift   = 15;
+  static_assert((int64_t{1} << kRangeShift) == kRange, "a range is 2^kRangeShift bytes");
+  const uint8_t* const first_byte = v.chars + first_offset;
+  uint32_t const cbeg             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(first_byte) & 15u);
+  int64_t const cend              = cbeg + (last_offset - first_offset);
+  int64_t const ntiles            = (cend + kTile - 1) / kTile;
+  int64_t const nranges64         = (ntiles + kRangeTiles - 1) / kRangeTiles;
+  if (nranges64 > 0x7FFFFFF0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+  uint32_t const nranges = static_cast<uint32_t>(nranges64);
+
   int device = 0, cus = 256;
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-  // persistent kernels: as many workgroups as can be resident at once
-  auto resident = [&](const void* kernel, int threads) -> int64_t {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 4;
-    return static_cast<int64_t>(per_cu) * cus;
-  };
-  unsigned const row_blocks = static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(rows) + kTokWaves * kGroups - 1) / (kTokWaves * kGroups),
-                                                                      resident(reinterpret_cast<const void*>(wordpiece_probe_kernel), kTokThreads)));
-  // Each wavefront reserves queue entries a range at a time (one atomic per range), at most `queue_block` of them:
-  // it starts with short ranges and doubles them while they fill within a few steps, because atomics on one
-  // address are slow (about 150 M/s) and the unused tail of each wavefront's last range, half a range on
-  // average, is time lost in the pass that reads the queue.
-  uint64_t const waves = static_cast<uint64_t>(row_blocks) * kTokWaves;
-  uint32_t queue_block = 64;
-  while (queue_block < 1024 && static_cast<uint64_t>(queue_block) * waves * 64 < static_cast<uint64_t>(last_offset - first_offset)) queue_block <<= 1;
-  uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 4) + waves * queue_block + 4096;
-  size_t const temp_bytes[5] = {arena_slots * sizeof(uint32_t), static_cast<size_t>(rows) * sizeof(int32_t),
-                                static_cast<size_t>(rows) * sizeof(int32_t), scan_temp_bytes(rows), 256};
-  TempParts<5> const temps(mr, temp_bytes);
-  uint32_t* const arena    = temps.part<uint32_t>(0);
-  int32_t* const nwords    = temps.part<int32_t>(1);
-  int32_t* const counts    = temps.part<int32_t>(2);
-  uint64_t* const scan_tmp = temps.part<uint64_t>(3);
-  uint32_t* const qsize    = temps.part<uint32_t>(4);
-  if (!temps.ok()) {
-    nvtext_amd_list_column_free(out, stream_, mr_);
-    return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-  }
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(wordpiece_tile_kernel<kTile>), kTokThreads, 0) != hipSuccess || per_cu < 1)
+    per_cu = 2;
+  unsigned const tile_grid =
+    static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, static_cast<int64_t>(per_cu) * cus));
+
+  TileArgs args{};
+  args.col          = v;
+  args.table        = vocabulary->table;
+  args.abase        = reinterpret_cast<const uint4*>(first_byte - cbeg);
+  args.first_offset = first_offset;
+  args.cend         = cend;
+  args.ntiles       = ntiles;
+  args.cbeg         = cbeg;
+  args.nranges      = nranges;
+  args.max_words    = max_words_per_row;
+
   uint64_t total = 0;
   for (int attempt = 0;; ++attempt) {
-    if (queue_capacity > 0x7FFFFFFEull) queue_capacity = 0x7FFFFFFEull;
-    uint32_t const qcap = static_cast<uint32_t>(queue_capacity);
-    // (third part: queue indices of the words of more than 16 bytes, then one count per wavefront of the out-of-vocabulary pass)
-    int64_t const oov_blocks    = resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads);
-    size_t const queue_bytes[3] = {static_cast<size_t>(qcap) * sizeof(OovEntry), static_cast<size_t>(qcap) * sizeof(OovResult),
-                                   (static_cast<size_t>(qcap) + static_cast<size_t>(oov_blocks) * (kOovThreads / kWave)) * sizeof(uint32_t)};
-    TempParts<3> const queue_temps(mr, queue_bytes);
-    OovEntry* const queue    = queue_temps.part<OovEntry>(0);
-    OovResult* const results = queue_temps.part<OovResult>(1);
-    uint32_t* const longer   = queue_temps.part<uint32_t>(2);
-    if (!queue_temps.ok()) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-    }
-    launch_fill_u32(qsize, 0u, 2, stream);  // queue size; words the emit pass hands on
+    // Arena slots per range.  A range of ordinary text has a token per five or six bytes; the first attempt leaves
+    // room for three per eight.  A range with more (rows or words of a byte or two, words that fall apart into
+    // letters) makes the attempt fail, and the second has room for the most a range can give: a token per byte, plus
+    // those of a word that begins in its last bytes.
+    uint32_t const range_cap   = attempt == 0 ? static_cast<uint32_t>(kRange * 3 / 8) : static_cast<uint32_t>(kRange + 256);
+    size_t const temp_bytes[6] = {static_cast<size_t>(nranges) * range_cap * sizeof(uint32_t),
+                                  static_cast<size_t>(nranges) * sizeof(uint32_t),
+                                  static_cast<size_t>(nranges) * sizeof(uint32_t),
+                                  (static_cast<size_t>(nranges) + 1) * sizeof(int64_t),
+                                  scan_temp_bytes(nranges),
+                                  256};
+    TempParts<6> const temps(mr, temp_bytes);
+    if (!temps.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
+    uint32_t* const arena     = temps.part<uint32_t>(0);
+    uint32_t* const first_row = temps.part<uint32_t>(1);
+    uint32_t* const counts    = temps.part<uint32_t>(2);
+    int64_t* const bases      = temps.part<int64_t>(3);
+    uint64_t* const scan_tmp  = temps.part<uint64_t>(4);
+    uint32_t* const flags     = temps.part<uint32_t>(5);  // range counter, overflow flag
+    args.range_cap       = range_cap;
+    args.range_first_row = first_row;
+    args.arena           = arena;
+    args.range_count     = counts;
+    args.offsets_out     = out->offsets;
+    args.counter         = flags;
+    args.overflow        = flags + 1;
+    launch_fill_u32(flags, 0u, 64, stream);
+    hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
     {
-      ProfileScope ps("wordpiece_probe_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_probe_kernel, dim3(row_blocks), dim3(kTokThreads), 0, stream, v, vocabulary->table, max_words_per_row,
-                         first_offset, last_offset, arena, nwords, counts, queue, qcap,
-                         queue_block, qsize);
+      ProfileScope ps("wordpiece_tile_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_tile_kernel<kTile>, dim3(tile_grid), dim3(kTokThreads), 0, stream, args);
     }
-    {
-      ProfileScope ps("wordpiece_oov_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue, qsize, qcap, results, counts, longer);
-    }
-    {
-      ProfileScope ps("wordpiece_oov_long_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(oov_blocks)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue, qsize, qcap, results, counts, longer);
-    }
-    // int32 list offsets; the total decides the child size (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
-    device_exclusive_scan(CountOf{counts}, static_cast<int64_t>(rows), out->offsets, scan_tmp, stream);
-    uint32_t queued = 0;
-    hipError_t e    = hipMemcpyAsync(&total, scan_tmp + scan_tiles(rows), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(&queued, qsize, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+    // where the tokens of each range go; the total decides the child size
+    // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
+    device_exclusive_scan(RangeCountOf{counts}, static_cast<int64_t>(nranges), bases, scan_tmp, stream);
+    uint32_t overflow = 0;
+    hipError_t e      = hipMemcpyAsync(&total, scan_tmp + scan_tiles(nranges), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(&overflow, flags + 1, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+#ifdef WP_PHASE_TIMING
+    {
+      unsigned long long ph[10];
+      (void)hipMemcpy(ph, flags + 4, sizeof(ph), hipMemcpyDeviceToHost);
+      unsigned long long sum = 0;
+      for (auto x : ph) sum += x;
+      static const char* const names[10] = {"stage", "rows", "detect", "cap", "lists", "probe", "oov", "write", "rowoffs", "tail"};
+      sum -= ph[9];
+      for (int i = 0; i < 9; ++i) fprintf(stderr, "%s %.1f%%  ", names[i], 100.0 * ph[i] / (sum ? sum : 1));
+      fprintf(stderr, "trips/tile %.2f", double(ph[9]) / double(ntiles));
+      fprintf(stderr, "\n");
     }
-    if (queued > qcap) {  // the queue was too small: repeat once with the exact size
-      if (attempt > 0 || queued > 0x7FFFFFFEu) {
-        nvtext_amd_list_column_free(out, stream_, mr_);
-        return fail(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
-      }
-      queue_capacity = queued;
+#endif
+    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) return give_up(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
+    if (overflow != 0) {
+      if (attempt > 0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
       continue;
-    }
-    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) {
-      nvtext_amd_list_column_free(out, stream_, mr_);
-      return fail(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
     }
     out->child_size  = static_cast<int64_t>(total);
     out->child_bytes = static_cast<size_t>(total) * sizeof(int32_t);
     if (total) {
       out->child = mr.allocate(out->child_bytes);
-      if (!out->child) {
-        nvtext_amd_list_column_free(out, stream_, mr_);
-        return fail(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
-      }
-      ProfileScope ps("wordpiece_emit_kernel", stream);
-      // the blocks of rows that a wavefront walks at a time: evened out by tokens (see emit_blocks_kernel)
-      int64_t const emit_work   = static_cast<int64_t>(total) + kEmitRowWeight * rows;
-      int64_t const nblocks     = (emit_work + kEmitBlockWork - 1) / kEmitBlockWork;
-      Temp block_first(mr, static_cast<size_t>(nblocks + 1) * sizeof(int32_t));
-      if (!block_first.ok()) {
-        nvtext_amd_list_column_free(out, stream_, mr_);
-        return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
-      }
-      hipLaunchKernelGGL(emit_blocks_kernel, dim3(static_cast<unsigned>((nblocks + 1 + 255) / 256)), dim3(256), 0, stream, out->offsets,
-                         static_cast<int64_t>(rows), nblocks, block_first.as<int32_t>());
-      int64_t const emit_blocks = (nblocks + kTokWaves - 1) / kTokWaves;
-      unsigned const emit_grid  = static_cast<unsigned>(std::min<int64_t>(emit_blocks, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
-      hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, v, vocabulary->table, first_offset,
-                         arena, nwords, results, out->offsets,
-                         static_cast<int32_t*>(out->child), block_first.as<int32_t>(), nblocks, longer, qsize + 1);
-      // (the list of longer words has served its purpose by now: its memory takes the list of words to do again,
-      // at most one entry per queued word)
-      hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, v, vocabulary->table,
-                         queue, results, longer, qsize + 1,
-                         static_cast<int32_t*>(out->child));
+      if (!out->child) return give_up(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
+    }
+    {
+      ProfileScope ps("wordpiece_gather_kernel", stream);
+      unsigned const row_blocks = static_cast<unsigned>((static_cast<int64_t>(rows) + 1 + 255) / 256);
+      hipLaunchKernelGGL(wordpiece_gather_kernel, dim3(nranges + row_blocks), dim3(256), 0, stream, v, first_offset, cbeg, kRangeShift, nranges, arena,
+                         range_cap, counts, bases, static_cast<int32_t*>(out->child), out->offsets);
     }
     break;
   }
-  NVTEXT_HIP_TRY(hipGetLastError());
+  if (hipGetLastError() != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, "kernel launch failed");
   return NVTEXT_AMD_SUCCESS;
 }
 
