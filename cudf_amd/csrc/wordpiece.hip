@@ -62,13 +62,15 @@ __host__ __device__ __forceinline__ uint32_t key_hash_block(uint32_t h, uint32_t
   return h ^ (h >> 15);
 }
 
-// slot.x = (tag23 << 9) | (kind << 8) | len   (0 = empty; len in 1..199)
+// slot.x = (tag15 << 17) | (carried8 << 9) | (kind << 8) | len   (0 = empty; len in 1..199).  carried8, in slot 0 of a bucket only:
+//          one of eight bits per key that has been carried past this bucket (which bit: carried_bit() of the key's hash)
 // slot.y = token id; in slot 0 of a bucket, bit 31 says that some key has been carried past this bucket
 //          (kSearchOn: a key that is not in a bucket without the bit is not in the table)
 // slot.z, slot.w = the key itself when len <= 8 (zero padded), else (byte offset of the key in the pool, 0);
 // the pool holds the keys of more than 8 bytes, each zero padded to a multiple of 8 at an 8-byte aligned offset
 // Bucket b = slots[2b], slots[2b+1]; a bucket fills slot 0 first, overflow goes to the next bucket.
 constexpr uint32_t kSearchOn = 0x80000000u;
+constexpr uint32_t kCarried  = 0x0001FE00u;
 struct VocabTable {
   const uint4* slots;
   const uint8_t* pool;
@@ -99,8 +101,11 @@ __host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t h, uint32_t kin
 {
   uint32_t const x = mix32(h + kind * 0x7F4A7C15u);
   *bucket          = x;
-  return (x & 0xFFFFFE00u) | (kind << 8) | len;
+  return (x & 0xFFFE0000u) | (kind << 8) | len;
 }
+// The bit that a key with hash h sets in the carried8 field of the buckets it is carried past: a key that is not in
+// its home bucket and does not find its bit there is not in the table.
+__host__ __device__ __forceinline__ uint32_t carried_bit(uint32_t h) { return 0x200u << ((h * 0x9E3779B1u) >> 29); }
 
 }  // namespace
 }  // namespace nvtext_amd
@@ -188,7 +193,8 @@ struct GlobalWord {
 // A candidate key, ready to be probed: its first block (trimmed), tag word and home bucket.
 struct Probe {
   uint32_t k0, k1;  // key bytes [0, 8), zero padded
-  uint32_t want;    // slot.x of a matching slot
+  uint32_t want;    // slot.x of a matching slot (without the carried8 field)
+  uint32_t fp;      // carried_bit() of the key
   uint32_t bucket;  // home bucket (already masked)
 };
 
@@ -216,6 +222,7 @@ __device__ __forceinline__ Probe make_probe(VocabTable const& t, uint32_t kind, 
   if (len > 8) h = hash_long_key(w, p, len, h);
   uint32_t b;
   pr.want   = slot_word0(h, kind, len, &b);
+  pr.fp     = carried_bit(h);
   pr.bucket = b & t.bucket_mask;
   return pr;
 }
@@ -237,7 +244,7 @@ __device__ __forceinline__ bool pool_key_equal(VocabTable const& t, uint32_t poo
 template <typename W>
 __device__ __forceinline__ int check_slot(VocabTable const& t, uint4 const& s, Probe const& pr, W const& w, uint32_t p, uint32_t len, int32_t* id)
 {
-  if (s.x == pr.want) {
+  if ((s.x & ~kCarried) == pr.want) {
     bool const same = len <= 8 ? (s.z == pr.k0 && s.w == pr.k1) : pool_key_equal(t, s.z, w, p, len);
     if (same) {
       *id = static_cast<int32_t>(s.y & ~kSearchOn);
@@ -322,12 +329,12 @@ struct RegWord {
 // carried past this bucket and the search goes on in the next one).  Straight-line code.
 __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
 {
-  bool const tag0  = s0.x == pr.want, tag1 = s1.x == pr.want;
+  bool const tag0  = (s0.x & ~kCarried) == pr.want, tag1 = s1.x == pr.want;
   bool const is0   = tag0 && s0.z == pr.k0 && s0.w == pr.k1;
   bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
   bool const small = l <= 8;
   bool const found = small && (is0 || is1);
-  bool const more  = (!small && (tag0 || tag1)) || (!found && (s0.y & kSearchOn) != 0);
+  bool const more  = (!small && (tag0 || tag1)) || (!found && (s0.x & pr.fp) != 0);
   *id              = static_cast<int32_t>((is0 ? s0.y : s1.y) & ~kSearchOn);
   return found ? 1u : more ? 2u : 0u;
 }
@@ -338,8 +345,8 @@ __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, ui
 __device__ __forceinline__ uint32_t verdict_16(VocabTable const& t, Probe const& pr, uint4 const& s0, uint4 const& s1, const uint32_t (&k)[4],
                                                int32_t* id)
 {
-  bool const tag0 = s0.x == pr.want, tag1 = s1.x == pr.want;
-  bool const on   = (s0.y & kSearchOn) != 0;
+  bool const tag0 = (s0.x & ~kCarried) == pr.want, tag1 = s1.x == pr.want;
+  bool const on   = (s0.x & pr.fp) != 0;
   if (tag0 && tag1) return 2u;
   if (!tag0 && !tag1) return on ? 2u : 0u;
   const uint2* const e = reinterpret_cast<const uint2*>(t.pool + (tag0 ? s0.z : s1.z));
@@ -422,11 +429,12 @@ struct OovStepper {
     lens = len - start >= 3 ? t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
   }
 
-  __device__ __forceinline__ void begin(VocabTable const& t, W const& w, uint32_t len_, bool ascii_)
+  // probed: the whole word has been looked up and is known to be absent
+  __device__ __forceinline__ void begin(VocabTable const& t, W const& w, uint32_t len_, bool ascii_, bool probed)
   {
     len = len_; start = 0; e = len_; count = 0;
     ascii = ascii_;
-    fresh = false;  // the whole word is known to be absent: begin by shortening it
+    fresh = !probed;  // a word known to be absent begins by being shortened
     done  = false;
     w.key8(0, min(len, 8u), &raw0, &raw1);
     load_filter(t, 0);
@@ -487,12 +495,13 @@ struct OovStepper {
   }
 };
 
-// Runs one word to completion (used where out-of-vocabulary words are rare).  Returns the token count.
+// Runs one word, which has not been looked up whole, to completion (used where such words are rare).  Returns the
+// token count.
 template <typename W, typename Emit>
 __device__ __forceinline__ uint32_t tokenize_oov_word(VocabTable const& t, W const& w, uint32_t len, Emit emit)
 {
   OovStepper<W> st;
-  st.begin(t, w, len, false);
+  st.begin(t, w, len, false, false);
   while (!st.done) st.step(t, w, emit);
   return st.count;
 }
@@ -530,44 +539,70 @@ struct ShortWord {
   int32_t id1, id2;  // ids of the piece's first byte and first two bytes as keys (kNone: no such key)
   bool done;
 
+  // What a piece needs to know before any of its candidates is looked up: which lengths of three bytes and more
+  // can exist for its first three bytes, and the ids of its first byte and first two bytes as keys.
+  struct Opening {
+    uint32_t lens;
+    int32_t id1, id2;
+  };
+
   __device__ __forceinline__ uint32_t byte(uint32_t k) const
   {
     uint32_t const d = k >> 2;
     uint32_t const v = d == 0 ? r[0] : d == 1 ? r[1] : d == 2 ? r[2] : r[3];
     return (v >> (8 * (k & 3u))) & 0xffu;
   }
-  __device__ __forceinline__ void key8(uint32_t p, uint32_t len, uint32_t* k0, uint32_t* k1) const
+  // bytes [p, p + 4) of the rest of the word (p < 16)
+  __device__ __forceinline__ uint32_t dword_at(uint32_t p) const
   {
-    // only called with p = 8 by the generic probe code (keys of 9 to 16 bytes)
-    uint32_t lo = p == 0 ? r[0] : r[2], hi = p == 0 ? r[1] : r[3];
-    trim_key8(len, lo, hi);
-    *k0 = lo;
-    *k1 = hi;
+    uint32_t const d  = p >> 2;
+    uint32_t const lo = d == 0 ? r[0] : d == 1 ? r[1] : d == 2 ? r[2] : r[3];
+    uint32_t const hi = d == 0 ? r[1] : d == 1 ? r[2] : d == 2 ? r[3] : 0u;
+    return __builtin_amdgcn_alignbit(hi, lo, (p & 3u) * 8u);
   }
 
-  // Candidate lengths of the piece at start: on a character boundary, no longer than the rest of the word
-  // or the longest key, and not ruled out by the length filter of the piece's first three bytes.
-  __device__ __forceinline__ void open_piece(VocabTable const& t, uint32_t kind)
+  // Requests the opening of the piece that would start p bytes on (key space `kind`).  The reads are made whatever p
+  // is (bytes past the word are zeros, every index is inside its table); what they give only counts for the p
+  // that the word goes on from.  first_ids: the ids of the one-byte keys, [kind * 256 + byte], in LDS.
+  __device__ __forceinline__ Opening request(VocabTable const& t, const int32_t* first_ids, uint32_t kind, uint32_t p) const
   {
-    uint32_t const lens = rem >= 3 ? t.lens[length_filter_index(kind, r[0] & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
-    uint32_t const lim  = min(min(rem, t.max_len[kind]), 16u);
-    cand                = (bnd >> 1) & ((1u << lim) - 1u) & ((lens << 2) | 3u);
-    id1                 = t.short_ids[2 * 65536 + kind * 256 + (r[0] & 0xFFu)];
-    id2                 = rem >= 2 ? t.short_ids[kind * 65536 + (r[0] & 0xFFFFu)] : kNone;
+    uint32_t const b    = dword_at(p);
+    uint32_t const left = rem - min(p, rem);
+    Opening o;
+    uint32_t const lens = t.lens[length_filter_index(kind, b & 0x00FFFFFFu) & t.lens_mask];
+    int32_t const two   = t.short_ids[kind * 65536 + (b & 0xFFFFu)];
+    o.id1               = first_ids[kind * 256 + (b & 0xFFu)];
+    o.lens              = left >= 3 ? lens : 0xFFFFFFFFu;
+    o.id2               = left >= 2 ? two : kNone;
+    return o;
   }
 
-  __device__ __forceinline__ void begin(VocabTable const& t, const uint32_t (&head)[4], uint32_t len)
+  // The piece at start begins: its candidate lengths are those on a character boundary, no longer than the rest of
+  // the word or the longest key, and not ruled out by the length filter of its first three bytes.
+  __device__ __forceinline__ void open_piece(VocabTable const& t, uint32_t kind, Opening const& o)
+  {
+    uint32_t const lim = min(min(rem, t.max_len[kind]), 16u);
+    cand               = (bnd >> 1) & ((1u << lim) - 1u) & ((o.lens << 2) | 3u);
+    id1                = o.id1;
+    id2                = o.id2;
+  }
+
+  // probed: the whole word has been looked up and is known to be absent
+  // ascii (the same in every lane): no byte of any of the lanes' words has bit 7 set
+  __device__ __forceinline__ void begin(VocabTable const& t, const int32_t* first_ids, const uint32_t (&head)[4], uint32_t len, bool probed, bool ascii)
   {
 #pragma unroll
     for (int k = 0; k < 4; ++k) r[k] = head[k];
     rem   = len;
     count = 0;
     done  = false;
-    uint32_t const cont = gather_byte_flags(continuation_bytes(r[0])) | (gather_byte_flags(continuation_bytes(r[1])) << 4) |
-                          (gather_byte_flags(continuation_bytes(r[2])) << 8) | (gather_byte_flags(continuation_bytes(r[3])) << 12);
+    uint32_t cont = 0;
+    if (!ascii)
+      cont = gather_byte_flags(continuation_bytes(r[0])) | (gather_byte_flags(continuation_bytes(r[1])) << 4) |
+             (gather_byte_flags(continuation_bytes(r[2])) << 8) | (gather_byte_flags(continuation_bytes(r[3])) << 12);
     bnd = (~cont & ((1u << len) - 1u)) | (1u << len);
-    open_piece(t, 0);
-    cand &= ~(1u << (len - 1));  // the whole word is known to be absent
+    open_piece(t, 0, request(t, first_ids, 0, 0));
+    if (probed) cand &= ~(1u << (len - 1));
   }
 
   __device__ __forceinline__ Probe probe_of(VocabTable const& t, uint32_t kind, uint32_t l) const
@@ -583,6 +618,7 @@ struct ShortWord {
     h                 = l > 8 ? h2 : h;
     uint32_t b;
     pr.want   = slot_word0(h, kind, l, &b);
+    pr.fp     = carried_bit(h);
     pr.bucket = b & t.bucket_mask;
     return pr;
   }
@@ -604,24 +640,30 @@ struct ShortWord {
     bnd >>= l;
   }
 
-  // One trip: probes the longest remaining candidate of three bytes and more; when none of those is left, the
-  // candidates of two bytes and of one byte are settled from the ids fetched when the piece was opened, without
-  // hashing or further reads.  (The length filter leaves few candidates: a piece that has any has 1.4 on average,
-  // so a second probe in the same trip would mostly be wasted work.)
+  // One trip: looks up the longest remaining candidate of three bytes and more; when none of those is left, the
+  // candidates of two bytes and of one byte are settled from the ids the opening gave, without hashing or further
+  // reads.  (The length filter leaves few candidates: a piece that has any has 1.4 on average, so a second lookup in
+  // the same trip would mostly be wasted work; and requesting, in the same breath, the openings of the pieces that
+  // could come next costs more in scattered reads than the waits it saves: measured, 18 % slower.)
   template <typename Emit>
-  __device__ __forceinline__ void step(VocabTable const& t, Emit&& emit)
+  __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, Emit&& emit)
   {
     uint32_t const kind   = count ? 1u : 0u;
     uint32_t const longer = cand & ~3u;
     bool const has_a      = longer != 0;
     uint32_t const la     = 32u - static_cast<uint32_t>(__builtin_clz(has_a ? longer : 4u));
-    bool hit_a            = false;
-    int32_t ida           = kNone;
+    Probe pa;
+    uint4 a0 = make_uint4(0u, 0u, 0u, 0u), a1 = a0;
     if (has_a) {
-      Probe const pa = probe_of(t, kind, la);
-      uint4 const a0 = t.slots[2 * pa.bucket], a1 = t.slots[2 * pa.bucket + 1];
-      uint32_t va    = verdict(pa, a0, a1, la, &ida);
-      if (va == 2u) {  // the general lookup (keys in the pool, overflowing buckets)
+      pa = probe_of(t, kind, la);
+      a0 = t.slots[2 * pa.bucket];
+      a1 = t.slots[2 * pa.bucket + 1];
+    }
+    bool hit_a  = false;
+    int32_t ida = kNone;
+    if (has_a) {
+      uint32_t va = verdict(pa, a0, a1, la, &ida);
+      if (va == 2u) {  // the general lookup (keys in the pool, keys carried past their bucket)
         RegWord const rw{{r[0], r[1], r[2], r[3]}};
         ida = lookup_slow(t, kind, rw, 0u, la);
         va  = ida == kNone ? 0u : 1u;
@@ -649,7 +691,7 @@ struct ShortWord {
     cand  = longer_left | (cand & 3u);
     if (hit && !done) {
       advance(len);  // next piece: the rest of the word (381-395)
-      open_piece(t, 1);
+      open_piece(t, 1, request(t, first_ids, 1u, 0u));
     }
   }
 };
@@ -661,7 +703,7 @@ struct ShortWord {
 constexpr int kRangeTiles    = 16;
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueCap = 256;  // out-of-vocabulary words that wait in LDS
-constexpr uint32_t kTokCap   = 256;  // their tokens (per unit)
+constexpr uint32_t kTokCap   = 192;  // their tokens (per unit)
 constexpr int kStragglers    = 24;   // a unit's out-of-vocabulary words may go on into the next unit's once fewer lanes than this are busy
 // lds.word[k] after its word has been looked up: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or
 //   kOovMark | count << 16 | index of its tokens in lds.tokens          (1 <= count <= kOovKeep), or
@@ -680,6 +722,7 @@ struct TileLds {
   uint32_t word[2][kWordCap];                 // per word of a unit: start | end << 16, then its token (see kOovMark), then the tokens before it
   uint32_t tokens[2][kTokCap];
   uint16_t queue[kQueueCap];
+  uint32_t tok_used[2];                       // tokens kept in tokens[0], [1]
 };
 
 struct TileArgs {
@@ -773,6 +816,8 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
     phase_t[i] += now_ - phase_last;                        \
     phase_last = now_;                                      \
   }
+#elif defined(WP_MARK)
+#define WP_PHASE(i) asm volatile("; WPMARK " #i);
 #else
 #define WP_PHASE(i)
 #endif
@@ -802,6 +847,10 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
   };
   const uint8_t* const lds_byte = reinterpret_cast<const uint8_t*>(lds.bytes);
   enum { kQueueFull = 0, kUnitDone = 1, kRangeDone = 2 };
+  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
+  __shared__ int32_t first_ids[512];
+  for (int i = threadIdx.x; i < 512; i += kTokThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
+  __syncthreads();
 
   for (;;) {
     uint32_t range = 0;
@@ -835,7 +884,7 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
     uint32_t w_lo = 0, w_hi = 0, nwc = 0;  // the unit: words [w_lo, w_hi) of the tile
     uint32_t par = 0;                      // which half of lds.word / lds.tokens it uses
     uint32_t k0 = 0, qn = 0, q_next = 0;   // words looked up so far; queue entries written / taken
-    bool edge = false;
+    bool edge = false, ascii = false;  // some staged byte lies outside the view; no staged byte has bit 7 set
     // -- the unit before it
     bool pend = false;
     int64_t p_tb = 0;
@@ -847,7 +896,6 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
     bool busy = false;
     uint32_t mine = 0, mine_par = 0;  // my word: lds.word[mine_par][mine]
     int32_t tok[kOovKeep];
-    uint32_t tok_used0 = 0, tok_used1 = 0;  // tokens kept in lds.tokens[0], [1]
     auto keep_token = [&](uint32_t j, int32_t id) {
 #pragma unroll
       for (int i = 0; i < kOovKeep; ++i)
@@ -891,10 +939,16 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
           // ---- word starts and ends
           {
             uint32_t base = 0;
+            uint32_t seen = 0;
+            if (lane < kOverBlocks) {
+              uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (kBlocks + lane + 1)]);
+              seen          = v.x | v.y | v.z | v.w;
+            }
 #pragma unroll
             for (int s = 0; s < kSubs; ++s) {
               int const b     = s * kWave + lane;
               uint4 const v   = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
+              seen |= v.x | v.y | v.z | v.w;
               uint32_t sp     = space_mask16(v);
               uint32_t before = lds_byte[16 + 16 * b - 1] == 0x20u, after = lds_byte[16 + 16 * b + 16] == 0x20u;
               if (edge) {
@@ -916,8 +970,9 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
               base += wave_bcast(incl, kWave - 1);
             }
             if (lane == 0) lds.prefix[kBlocks] = base;
-            nw = base & 0xFFFFu;
-            ne = base >> 16;
+            nw    = base & 0xFFFFu;
+            ne    = base >> 16;
+            ascii = ballot64((seen & 0x80808080u) != 0) == 0;
           }
           wave_lds_sync();
           WP_PHASE(2)
@@ -1055,8 +1110,7 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
             }
             if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
           }
-          if (par) tok_used1 = 0;
-          else tok_used0 = 0;
+          if (lane == 0) lds.tok_used[par] = 0;
           k0        = 0;
           unit_open = true;
           wave_lds_sync();
@@ -1068,46 +1122,42 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
         // the vocabulary wait in the queue
         uint32_t* const uw = lds.word[par];
         while (k0 < nwc && qn + kWave <= kQueueCap) {
-          uint32_t const k  = k0 + lane;
-          bool miss         = false;
+          uint32_t const k = k0 + lane;
+          uint32_t defer   = 0;  // 1: not in the vocabulary; 2: not decided here (more than 8 bytes; a key that may have been carried past its bucket)
           if (k < nwc) {
             uint32_t const rec = uw[k];
             uint32_t const s   = rec & 0xFFFFu;
             uint32_t const wl  = (rec >> 16) - s + 1u;
-            uint32_t value;
             if (wl >= kMaxWord) {
-              value = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+              uw[k] = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
+            } else if (wl > 8) {
+              defer = 2;
             } else {
-              int32_t id = kNone;
-              TileWord const tw{lds.bytes, 16u + s};
-              uint32_t head[4];
-              tw.head16(head);
-              trim_key8(wl, head[0], head[1]);
-              trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
+              uint32_t const o  = 16u + s;
+              uint32_t const sh = (o & 3u) * 8u;
+              uint32_t const d0 = lds.bytes[o >> 2], d1 = lds.bytes[(o >> 2) + 1], d2 = lds.bytes[(o >> 2) + 2];
+              Probe pr;
+              pr.k0 = __builtin_amdgcn_alignbit(d1, d0, sh);
+              pr.k1 = __builtin_amdgcn_alignbit(d2, d1, sh);
+              trim_key8(wl, pr.k0, pr.k1);
+              int32_t id  = kNone;
+              uint32_t vd = 0;
               if (wl <= table.max_len[0]) {
-                Probe pr;
-                pr.k0 = head[0];
-                pr.k1 = head[1];
-                uint32_t h        = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
-                uint32_t const h2 = key_hash_block(h, head[2], head[3]);
-                h                 = wl > 8 ? h2 : h;  // (not the hash of a word of more than 16 bytes: those go to the general lookup)
+                uint32_t const h = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
                 uint32_t bk;
                 pr.want   = slot_word0(h, 0, wl, &bk);
+                pr.fp     = carried_bit(h);
                 pr.bucket = bk & table.bucket_mask;
                 uint4 const s0 = table.slots[2 * pr.bucket];
                 uint4 const s1 = table.slots[2 * pr.bucket + 1];
-                uint32_t vd = wl > 16 ? 2u : verdict(pr, s0, s1, wl, &id);
-                if (vd == 2u && wl > 8 && wl <= 16) vd = verdict_16(table, pr, s0, s1, head, &id);
-                if (vd == 2u) id = lookup_slow(table, 0u, tw, 0u, wl);
-                else if (vd == 0u) id = kNone;
+                vd = verdict(pr, s0, s1, wl, &id);
               }
-              miss  = id == kNone;
-              value = static_cast<uint32_t>(id);
+              if (vd == 1u) uw[k] = static_cast<uint32_t>(id);
+              else defer = vd == 2u ? 2u : 1u;
             }
-            if (!miss) uw[k] = value;
           }
-          uint64_t const mm = ballot64(miss);
-          if (miss) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k);
+          uint64_t const mm = ballot64(defer != 0);
+          if (defer != 0) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k | (defer == 2u ? 0x8000u : 0u));
           qn += static_cast<uint32_t>(__builtin_popcountll(mm));
           k0 += kWave;
         }
@@ -1122,15 +1172,9 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
       {
         // stores the tokens of the words finished by this step
         auto deliver = [&](bool fin, uint32_t cnt) {
-          uint32_t const keep   = fin && cnt <= kOovKeep ? cnt : 0u;
-          uint32_t const packed = mine_par ? keep << 16 : keep;
-          uint32_t const incl   = wave_inclusive_scan(packed);
-          uint32_t const ex     = incl - packed;
-          uint32_t const tot    = wave_bcast(incl, kWave - 1);
-          uint32_t const off    = mine_par ? tok_used1 + (ex >> 16) : tok_used0 + (ex & 0xFFFFu);
-          tok_used0 += tot & 0xFFFFu;
-          tok_used1 += tot >> 16;
           if (fin) {
+            uint32_t const keep  = cnt <= kOovKeep ? cnt : 0u;
+            uint32_t const off   = keep > 0 ? atomicAdd(&lds.tok_used[mine_par], keep) : 0u;
             uint32_t* const slot = &lds.word[mine_par][mine];
             if (keep > 0 && off + keep <= kTokCap) {
 #pragma unroll
@@ -1161,7 +1205,7 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
               uint32_t k          = 0;
               if (!busy && rank < left) {
                 k                  = lds.queue[q_next + rank];
-                uint32_t const rec = lds.word[par][k];
+                uint32_t const rec = lds.word[par][k & 0x7FFFu];
                 uint32_t const s   = rec & 0xFFFFu;
                 uint32_t const wl  = (rec >> 16) - s + 1u;
                 if (wl <= 16) {
@@ -1170,9 +1214,9 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
                   tw.head16(head);
                   trim_key8(wl, head[0], head[1]);
                   trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
-                  sw.begin(table, head, wl);
+                  sw.begin(table, first_ids, head, wl, (k & 0x8000u) == 0, ascii);
                   busy     = true;
-                  mine     = k;
+                  mine     = k & 0x7FFFu;
                   mine_par = par;
                 } else {
                   is_long = true;
@@ -1195,13 +1239,13 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
 #ifdef WP_PHASE_TIMING
           phase_t[9] += 1;
 #endif
-          if (busy && !sw.done) sw.step(table, keep_token);
+          if (busy && !sw.done) sw.step(table, first_ids, keep_token);
         }
         if (n_long > 0) {
           wave_lds_sync();
           for (uint32_t base = 0; base < n_long; base += kWave) {
             if (base + lane < n_long) {
-              uint32_t const k   = lds.queue[base + lane];
+              uint32_t const k   = lds.queue[base + lane] & 0x7FFFu;  // (words of more than 16 bytes have not been looked up whole)
               uint32_t const rec = lds.word[par][k];
               uint32_t const s   = rec & 0xFFFFu;
               uint32_t const wl  = (rec >> 16) - s + 1u;
@@ -1222,6 +1266,23 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
         uint32_t* const uw       = lds.word[p_par];
         const uint32_t* const ut = lds.tokens[p_par];
         uint32_t done            = 0;  // tokens of the unit so far
+        // The tokens are put together in LDS in their final order and leave in whole runs, one dword per lane, because
+        // scattered stores cost the memory pipeline a cycle per lane.  The room for that is the staged bytes of the tile
+        // being looked up, which are free once the last of its words has been taken from the queue.
+        constexpr uint32_t kOutCap = sizeof(lds.bytes) / sizeof(uint32_t);
+        uint32_t* const out        = lds.bytes;
+        bool const may_stage       = reason == kRangeDone || w_hi == nw;
+        uint32_t flush_base = cursor, staged = 0;  // out[0 .. staged) are the tokens from flush_base on
+        auto flush = [&] {
+          if (staged == 0) return;
+          wave_lds_sync();
+          if (flush_base + staged > a.range_cap) spill = true;
+          if (!spill)
+            for (uint32_t i = lane; i < staged; i += kWave) region[flush_base + i] = out[i];
+          wave_lds_sync();
+          flush_base += staged;
+          staged = 0;
+        };
         for (uint32_t j0 = 0; j0 < p_nwc; j0 += kWave) {
           uint32_t const k   = j0 + lane;
           bool const active  = k < p_nwc;
@@ -1232,26 +1293,44 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
           uint32_t const incl = wave_inclusive_scan(cnt);
           uint32_t const ex   = incl - cnt;
           uint32_t const tot  = wave_bcast(incl, kWave - 1);
-          if (cursor + done + tot > a.range_cap) spill = true;
-          if (!spill) {
-            uint32_t* const dst = region + (cursor + done + ex);
-            if (redo) {
-              // tokens that were not kept (more than kOovKeep, a word of more than 16 bytes, no room left in LDS):
-              // tokenized again, into place
-              write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + p_tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
-            } else if (active) {
-              uint32_t const off = v & 0xFFFFu;
-              dst[0]             = marked ? ut[off] : v;
+          uint32_t const off  = v & 0xFFFFu;
+          if (may_stage && ballot64(redo) == 0) {
+            if (staged + tot > kOutCap) flush();  // (tot <= 64 * kOovKeep < kOutCap)
+            if (active) {
+              uint32_t* const dst = out + staged + ex;
+              dst[0]              = marked ? ut[off] : v;
 #pragma unroll
               for (uint32_t j = 1; j < kOovKeep; ++j) {
                 if (ballot64(marked && j < cnt) == 0) break;
                 if (marked && j < cnt) dst[j] = ut[off + j];
               }
             }
+            staged += tot;
+          } else {
+            // straight to memory: while the staged bytes are still in use (a tile of more words than a unit holds),
+            // and the rounds with a word whose tokens were not kept (more than kOovKeep, a word of more than 16 bytes,
+            // no room left in LDS), which is tokenized again, into place
+            flush();
+            if (cursor + done + tot > a.range_cap) spill = true;
+            if (!spill) {
+              uint32_t* const dst = region + (cursor + done + ex);
+              if (redo) {
+                write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + p_tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
+              } else if (active) {
+                dst[0] = marked ? ut[off] : v;
+#pragma unroll
+                for (uint32_t j = 1; j < kOovKeep; ++j) {
+                  if (ballot64(marked && j < cnt) == 0) break;
+                  if (marked && j < cnt) dst[j] = ut[off + j];
+                }
+              }
+            }
+            flush_base = cursor + done + tot;
           }
           if (active) uw[k] = done + ex;
           done += tot;
         }
+        flush();
         wave_lds_sync();
         WP_PHASE(7)
         // the rows that start in its tile at one of its words (or, for the last words of the tile, after them): the
@@ -1360,7 +1439,7 @@ uint32_t host_hash(const uint8_t* key, uint32_t len)
 
 bool host_same(HostSlot const& s, uint32_t w0, const std::vector<uint8_t>& pool, const uint8_t* key, uint32_t len, uint32_t k0, uint32_t k1)
 {
-  if (s.x != w0) return false;
+  if ((s.x & ~kCarried) != w0) return false;
   return len <= 8 ? (s.z == k0 && s.w == k1) : (std::memcmp(pool.data() + s.z, key, len) == 0);
 }
 
@@ -1368,7 +1447,9 @@ void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::
                  uint32_t len, uint32_t pool_off, int32_t id)
 {
   uint32_t b;
-  uint32_t const w0 = slot_word0(host_hash(key, len), kind, len, &b);
+  uint32_t const hh = host_hash(key, len);
+  uint32_t const w0 = slot_word0(hh, kind, len, &b);
+  uint32_t const fp = carried_bit(hh);
   uint32_t k0 = 0, k1 = 0;
   if (len <= 8) host_key8(key, len, &k0, &k1);
   for (;;) {
@@ -1386,6 +1467,7 @@ void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::
       if (host_same(s, w0, pool, key, len, k0, k1)) return;
     }
     slots[2 * static_cast<size_t>(b)].y |= kSearchOn;  // the key is carried past this bucket
+    slots[2 * static_cast<size_t>(b)].x |= fp;
     ++b;
   }
 }
