@@ -124,7 +124,7 @@ struct nvtext_amd_wordpiece_vocabulary {
 namespace nvtext_amd {
 namespace {
 
-constexpr int kTokWaves     = 2;
+constexpr int kTokWaves     = 4;
 constexpr int kTokThreads   = kTokWaves * kWave;
 constexpr int32_t kNone     = std::numeric_limits<int32_t>::min();
 constexpr int kOovKeep      = 7;     // tokens of an out-of-vocabulary word that are kept while it is tokenized
@@ -330,8 +330,8 @@ struct RegWord {
 __device__ __forceinline__ uint32_t verdict(Probe const& pr, uint4 const& s0, uint4 const& s1, uint32_t l, int32_t* id)
 {
   bool const tag0  = (s0.x & ~kCarried) == pr.want, tag1 = s1.x == pr.want;
-  bool const is0   = tag0 && s0.z == pr.k0 && s0.w == pr.k1;
-  bool const is1   = tag1 && s1.z == pr.k0 && s1.w == pr.k1;
+  bool const is0   = tag0 & (s0.z == pr.k0) & (s0.w == pr.k1);  // (no short cuts: the slots are read whole, at once)
+  bool const is1   = tag1 & (s1.z == pr.k0) & (s1.w == pr.k1);
   bool const small = l <= 8;
   bool const found = small && (is0 || is1);
   bool const more  = (!small && (tag0 || tag1)) || (!found && (s0.x & pr.fp) != 0);
@@ -645,6 +645,9 @@ struct ShortWord {
   // reads.  (The length filter leaves few candidates: a piece that has any has 1.4 on average, so a second lookup in
   // the same trip would mostly be wasted work; and requesting, in the same breath, the openings of the pieces that
   // could come next costs more in scattered reads than the waits it saves: measured, 18 % slower.)
+  // (Measured and left out: requesting, in the same breath, the openings of the pieces that could come next, so that no
+  // trip waits twice: 18 % slower, the scattered reads cost more than the waits they save; settling pieces that need
+  // no lookup several to a trip: fewer trips, each slower by more.)
   template <typename Emit>
   __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, Emit&& emit)
   {
@@ -659,32 +662,27 @@ struct ShortWord {
       a0 = t.slots[2 * pa.bucket];
       a1 = t.slots[2 * pa.bucket + 1];
     }
-    bool hit_a  = false;
-    int32_t ida = kNone;
-    if (has_a) {
-      uint32_t va = verdict(pa, a0, a1, la, &ida);
-      if (va == 2u) {  // the general lookup (keys in the pool, keys carried past their bucket)
-        RegWord const rw{{r[0], r[1], r[2], r[3]}};
-        ida = lookup_slow(t, kind, rw, 0u, la);
-        va  = ida == kNone ? 0u : 1u;
-      }
-      hit_a = va == 1u;
-    }
+    // where the word would go on from if this trip settles a piece: after the candidate, or, when it is the last one of
+    // three bytes and more (or there is none), after two bytes or one
     uint32_t const longer_left = has_a ? longer ^ (1u << (la - 1)) : 0u;  // after a miss
-    bool hit     = hit_a;
-    uint32_t len = la;
-    int32_t id   = ida;
-    bool unknown = false;
-    if (!hit && longer_left == 0) {
-      // two bytes, then one byte; else no prefix of the word matched (375-379), or a later piece has no match and
-      // the word collapses (396-404): either way a single unknown token
-      bool const two = (cand & 2u) != 0 && id2 != kNone;
-      bool const one = (cand & 1u) != 0 && id1 != kNone;
-      hit            = two || one;
-      len            = two ? 2u : 1u;
-      id             = two ? id2 : id1;
-      unknown        = !hit;
+    bool const two             = (cand & 2u) != 0 && id2 != kNone;
+    bool const one             = (cand & 1u) != 0 && id1 != kNone;
+    uint32_t const short_len   = two ? 2u : 1u;
+    int32_t ida = kNone;
+    uint32_t va = has_a ? verdict(pa, a0, a1, la, &ida) : 0u;
+    if (va == 2u) {  // the general lookup (keys in the pool, keys carried past their bucket)
+      RegWord const rw{{r[0], r[1], r[2], r[3]}};
+      ida = lookup_slow(t, kind, rw, 0u, la);
+      va  = ida == kNone ? 0u : 1u;
     }
+    bool const hit_a = has_a && va == 1u;
+    // two bytes, then one byte; else no prefix of the word matched (375-379), or a later piece has no match and the
+    // word collapses (396-404): either way a single unknown token
+    bool const settle  = !hit_a && longer_left == 0;
+    bool const hit     = hit_a || (settle && (two || one));
+    bool const unknown = settle && !(two || one);
+    uint32_t const len = hit_a ? la : short_len;
+    int32_t const id   = hit_a ? ida : two ? id2 : id1;
     if (hit || unknown) emit(unknown ? 0u : count, unknown ? t.unk_id : id);
     count = unknown ? 1u : count + (hit ? 1u : 0u);
     done  = unknown || (hit && len == rem);
@@ -703,8 +701,7 @@ struct ShortWord {
 constexpr int kRangeTiles    = 16;
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueCap = 256;  // out-of-vocabulary words that wait in LDS
-constexpr uint32_t kTokCap   = 192;  // their tokens (per unit)
-constexpr int kStragglers    = 24;   // a unit's out-of-vocabulary words may go on into the next unit's once fewer lanes than this are busy
+constexpr uint32_t kTokCap   = 256;  // their tokens
 // lds.word[k] after its word has been looked up: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or
 //   kOovMark | count << 16 | index of its tokens in lds.tokens          (1 <= count <= kOovKeep), or
 //   kOovMark | kOovRedo | count << 21 | length << 13 | start            (tokens not kept: tokenized again when written)
@@ -719,10 +716,11 @@ struct TileLds {
   uint32_t masks[kBlocks];                    // per block: bit i = a word starts at byte i, bit 16 + i = a word ends at byte i
   uint32_t prefix[kBlocks + 1];               // word starts before the block | word ends before the block << 16
   static constexpr uint32_t kWordCap = TILE / 4;
-  uint32_t word[2][kWordCap];                 // per word of a unit: start | end << 16, then its token (see kOovMark), then the tokens before it
-  uint32_t tokens[2][kTokCap];
+  uint32_t word_guard[1];                     // (takes the end of the word that ran into the tile)
+  uint32_t word[kWordCap];                    // per word: start | end << 16, then its token (see kOovMark), then the tokens before it
+  uint32_t tokens[kTokCap];
   uint16_t queue[kQueueCap];
-  uint32_t tok_used[2];                       // tokens kept in tokens[0], [1]
+  uint32_t tok_used;                          // tokens kept in `tokens`
 };
 
 struct TileArgs {
@@ -822,8 +820,8 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
 #define WP_PHASE(i)
 #endif
 
-template <int TILE>
-__global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs a)
+template <int TILE, bool IS64, bool LIMIT>
+__global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs a)
 {
 #ifdef WP_PHASE_TIMING
   uint64_t phase_t[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -834,21 +832,25 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
   constexpr uint32_t kWordCap = TileLds<TILE>::kWordCap;
   static_assert(kBlocks % kWave == 0, "whole wavefronts of blocks");
   __shared__ TileLds<TILE> lds_all[kTokWaves];
+  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
+  __shared__ int32_t first_ids[512];
   TileLds<TILE>& lds  = lds_all[threadIdx.x / kWave];
   int const lane      = lane_id();
   uint32_t const rows = static_cast<uint32_t>(a.col.size);
   int64_t const cbeg  = a.cbeg, cend = a.cend;
   VocabTable const& table = a.table;
-  auto coord = [&](uint32_t r) -> int64_t { return a.col.off(r) - a.first_offset + cbeg; };
+  int64_t const cadj      = cbeg - a.first_offset;
+  auto coord = [&](uint32_t r) -> int64_t {
+    int64_t const i = static_cast<int64_t>(r) + a.col.offset;
+    return (IS64 ? static_cast<const int64_t*>(a.col.offsets)[i] : static_cast<int64_t>(static_cast<const int32_t*>(a.col.offsets)[i])) + cadj;
+  };
   // wordpiece_tokenize.cu:776-781: with a word limit, null rows have no words and the limit is
   // min(max_words, size_bytes / 2); without one, validity is not consulted (503-568).
   auto word_cap = [&](uint32_t r, int64_t bytes) -> uint32_t {
     return a.col.valid(r) ? static_cast<uint32_t>(min(static_cast<int64_t>(a.max_words), bytes / 2)) : 0u;
   };
   const uint8_t* const lds_byte = reinterpret_cast<const uint8_t*>(lds.bytes);
-  enum { kQueueFull = 0, kUnitDone = 1, kRangeDone = 2 };
-  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
-  __shared__ int32_t first_ids[512];
+  uint16_t* const word16        = reinterpret_cast<uint16_t*>(lds.word);
   for (int i = threadIdx.x; i < 512; i += kTokThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
   __syncthreads();
 
@@ -864,7 +866,7 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
     uint32_t open_left  = 0;  // words the row that runs into the tile may still have (with a word limit)
     uint32_t* const region = a.arena + static_cast<int64_t>(range) * a.range_cap;
     bool spill             = false;
-    if (a.max_words > 0 && r_cur > 0) {
+    if (LIMIT && r_cur > 0) {
       uint32_t const ro  = r_cur - 1;
       int64_t const c0   = coord(ro), c1 = coord(ro + 1);
       uint32_t const cap = word_cap(ro, c1 - c0);
@@ -872,215 +874,185 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
       open_left           = cap - min(cap, used);
     }
 
-    // A unit is the words of a tile (of a tile with more than kWordCap words: that many of them at a time).  Two are in
-    // flight: the one whose words are being looked up, and the one before it, whose last out-of-vocabulary words
-    // are still being tokenized by the lanes that took them; its tokens are written once those are done.  So the
-    // words that take many steps share their steps with the next unit's words instead of idling the other lanes.
-    // -- the tile being looked up
-    bool tile_open = false, unit_open = false;
-    int64_t tb     = 0;
-    uint32_t nw = 0, ne = 0, inside0 = 0;  // words that start in the tile, words that end in it, the tile begins inside a word
-    uint32_t r_first = 0, r_end = 0;       // the rows that start in it
-    uint32_t w_lo = 0, w_hi = 0, nwc = 0;  // the unit: words [w_lo, w_hi) of the tile
-    uint32_t par = 0;                      // which half of lds.word / lds.tokens it uses
-    uint32_t k0 = 0, qn = 0, q_next = 0;   // words looked up so far; queue entries written / taken
-    bool edge = false, ascii = false;  // some staged byte lies outside the view; no staged byte has bit 7 set
-    // -- the unit before it
-    bool pend = false;
-    int64_t p_tb = 0;
-    uint32_t p_par = 0, p_nwc = 0, p_wlo = 0, p_nw = 0, p_rfirst = 0, p_rend = 0;
-    // -- the lanes' out-of-vocabulary words
-    ShortWord sw;
-    sw.done  = true;
-    sw.count = 0;
-    bool busy = false;
-    uint32_t mine = 0, mine_par = 0;  // my word: lds.word[mine_par][mine]
-    int32_t tok[kOovKeep];
-    auto keep_token = [&](uint32_t j, int32_t id) {
-#pragma unroll
-      for (int i = 0; i < kOovKeep; ++i)
-        if (j == static_cast<uint32_t>(i)) tok[i] = id;
-    };
+    for (; t < t_end; ++t) {
+      int64_t const tb     = t * TILE;
+      bool const last_tile = t + 1 == a.ntiles;
+      bool const edge      = tb < 16 + cbeg || tb + TILE + 16 * kOverBlocks > cend;  // some staged byte lies outside the view
 
-    for (;;) {
-      int reason = kRangeDone;
-      if (!unit_open) {
-        if (!tile_open && t < t_end) {
-          // ================================================================ a new tile
-          tb                   = t * TILE;
-          bool const last_tile = t + 1 == a.ntiles;
-          edge                 = tb < 16 + cbeg || tb + TILE + 16 * kOverBlocks > cend;  // some staged byte lies outside the view
-          // ---- stage the bytes
-          for (int j = lane - 1; j < kBlocks + kOverBlocks; j += kWave) {
-            int64_t const g0 = tb + 16 * j;
-            uint4 v          = make_uint4(0u, 0u, 0u, 0u);
-            if (g0 + 16 > cbeg && g0 < cend) v = load_stream(a.abase + (g0 >> 4));
-            *reinterpret_cast<uint4*>(&lds.bytes[4 * (j + 1)]) = v;
-          }
-          for (int i = lane; i < kBlocks + kOverBlocks + 1; i += kWave) lds.bound[i] = 0;
-          wave_lds_sync();
-          WP_PHASE(0)
+      // ---- stage the bytes
+      for (int j = lane - 1; j < kBlocks + kOverBlocks; j += kWave) {
+        int64_t const g0 = tb + 16 * j;
+        uint4 v          = make_uint4(0u, 0u, 0u, 0u);
+        if (!edge || (g0 + 16 > cbeg && g0 < cend)) v = load_stream(a.abase + (g0 >> 4));
+        *reinterpret_cast<uint4*>(&lds.bytes[4 * (j + 1)]) = v;
+      }
+      for (int i = lane; i < kBlocks + kOverBlocks + 1; i += kWave) lds.bound[i] = 0;
+      wave_lds_sync();
+      WP_PHASE(0)
 
-          // ---- the rows that start in the tile: [r_first, r_end)
-          r_first = r_cur;
-          for (;;) {
-            uint32_t const r = r_cur + lane;
-            int64_t const p  = r <= rows ? coord(r) - tb : std::numeric_limits<int64_t>::max();
-            bool const in    = r < rows && (last_tile || p < TILE);
-            if (p < TILE + 16 * kOverBlocks) atomicOr(&lds.bound[p >> 4], 1u << (p & 15));
-            uint32_t const n = static_cast<uint32_t>(__builtin_popcountll(ballot64(in)));
-            r_cur += n;
-            if (n < kWave) break;
-          }
-          r_end = r_cur;
-          wave_lds_sync();
-          WP_PHASE(1)
+      // ---- the rows that start in the tile: [r_first, r_end)
+      uint32_t const r_first = r_cur;
+      for (;;) {
+        uint32_t const r = r_cur + lane;
+        int64_t const p  = r <= rows ? coord(r) - tb : std::numeric_limits<int64_t>::max();
+        bool const in    = r < rows && (last_tile || p < TILE);
+        if (p < TILE + 16 * kOverBlocks) atomicOr(&lds.bound[p >> 4], 1u << (p & 15));
+        uint32_t const n = static_cast<uint32_t>(__builtin_popcountll(ballot64(in)));
+        r_cur += n;
+        if (n < kWave) break;
+      }
+      uint32_t const r_end = r_cur;
+      wave_lds_sync();
+      WP_PHASE(1)
 
-          // ---- word starts and ends
-          {
-            uint32_t base = 0;
-            uint32_t seen = 0;
-            if (lane < kOverBlocks) {
-              uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (kBlocks + lane + 1)]);
-              seen          = v.x | v.y | v.z | v.w;
-            }
-#pragma unroll
-            for (int s = 0; s < kSubs; ++s) {
-              int const b     = s * kWave + lane;
-              uint4 const v   = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
-              seen |= v.x | v.y | v.z | v.w;
-              uint32_t sp     = space_mask16(v);
-              uint32_t before = lds_byte[16 + 16 * b - 1] == 0x20u, after = lds_byte[16 + 16 * b + 16] == 0x20u;
-              if (edge) {
-                int64_t const g0 = tb + 16 * b;
-                sp |= outside_mask16(g0, cbeg, cend);
-                before |= (g0 - 1 < cbeg || g0 - 1 >= cend);
-                after |= (g0 + 16 < cbeg || g0 + 16 >= cend);
-              }
-              uint32_t const bd = lds.bound[b] & 0xFFFFu;
-              after |= lds.bound[b + 1] & 1u;
-              uint32_t const word   = ~sp & 0xFFFFu;
-              uint32_t const starts = word & ((sp << 1) | before | bd);
-              uint32_t const ends   = word & ((sp >> 1) | (after << 15) | (bd >> 1));
-              if (s == 0) inside0 = wave_bcast(word & ~starts & 1u, 0);
-              lds.masks[b]          = starts | (ends << 16);
-              uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
-              uint32_t const incl   = wave_inclusive_scan(cnt);
-              lds.prefix[b]         = base + incl - cnt;
-              base += wave_bcast(incl, kWave - 1);
-            }
-            if (lane == 0) lds.prefix[kBlocks] = base;
-            nw    = base & 0xFFFFu;
-            ne    = base >> 16;
-            ascii = ballot64((seen & 0x80808080u) != 0) == 0;
-          }
-          wave_lds_sync();
-          WP_PHASE(2)
-
-          // word starts at positions below x (0 <= x)
-          auto words_before = [&](uint32_t x) -> uint32_t {
-            if (x >= TILE) return nw;
-            uint32_t const b = x >> 4;
-            return (lds.prefix[b] & 0xFFFFu) + static_cast<uint32_t>(__builtin_popcount(lds.masks[b] & ((1u << (x & 15u)) - 1u)));
-          };
-          // position of word start k (k < nw)
-          auto word_start = [&](uint32_t k) -> uint32_t {
-            uint32_t b = 0;
-#pragma unroll
-            for (uint32_t step = kBlocks / 2; step > 0; step >>= 1)
-              if ((lds.prefix[b + step] & 0xFFFFu) <= k) b += step;
-            uint32_t m = lds.masks[b] & 0xFFFFu;
-            for (uint32_t j = k - (lds.prefix[b] & 0xFFFFu); j > 0; --j) m &= m - 1u;
-            return 16u * b + static_cast<uint32_t>(__builtin_ctz(m | 0x10000u));
-          };
-
-          // ---- a word limit: the words of a row past its limit are dropped.  The first such word and the row's end
-          // are marked; a prefix parity over the marks gives the bytes whose word starts and ends go.
-          if (a.max_words > 0) {
-            bool cut = false;
-            auto drop_from = [&](uint32_t k, int64_t e) {  // from word start k up to position e
-              uint32_t const at = word_start(k);
-              atomicXor(&lds.bound[at >> 4], 0x10000u << (at & 15u));
-              if (e < TILE) atomicXor(&lds.bound[e >> 4], 0x10000u << (e & 15));
-              cut = true;
-            };
-            for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
-              uint32_t const r = r_first + i + lane;
-              if (r < r_end) {
-                int64_t const c0 = coord(r), c1 = coord(r + 1);
-                if (c1 > c0) {
-                  int64_t const p = c0 - tb, e = c1 - tb;  // (p < TILE: the rows past the last tile's end are empty)
-                  uint32_t const cap = word_cap(r, c1 - c0);
-                  uint32_t const wp  = words_before(static_cast<uint32_t>(p));
-                  uint32_t const we  = words_before(e < TILE ? static_cast<uint32_t>(e) : static_cast<uint32_t>(TILE));
-                  if (wp + cap < we) drop_from(wp + cap, e);
-                }
-              }
-            }
-            // the row that runs into the tile
-            int64_t const e0   = r_first < r_end ? coord(r_first) - tb : static_cast<int64_t>(TILE);
-            uint32_t const we0 = words_before(e0 < TILE ? static_cast<uint32_t>(e0) : static_cast<uint32_t>(TILE));
-            if (lane == 0 && open_left < we0) drop_from(open_left, e0);
-            // and the row that runs out of it
-            if (r_first < r_end) {
-              uint32_t const rl   = r_end - 1;
-              int64_t const c0    = coord(rl), c1 = coord(rl + 1);
-              int64_t const p     = c0 - tb;
-              uint32_t const cap  = word_cap(rl, c1 - c0);
-              uint32_t const used = nw - words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
-              open_left           = cap - min(cap, used);
-            } else {
-              open_left -= min(open_left, nw);
-            }
-            if (ballot64(cut) != 0) {
-              wave_lds_sync();
-              uint32_t base = 0, carry = 0;
-#pragma unroll
-              for (int s = 0; s < kSubs; ++s) {
-                int const b      = s * kWave + lane;
-                uint32_t const m = lds.masks[b];
-                uint32_t px      = lds.bound[b] >> 16;
-                px ^= px << 1;
-                px ^= px << 2;
-                px ^= px << 4;
-                px ^= px << 8;
-                px &= 0xFFFFu;
-                uint64_t const odd  = ballot64((px >> 15) != 0);
-                uint32_t const flip = (lanes_below(odd) & 1u) ^ carry;
-                carry ^= static_cast<uint32_t>(__builtin_popcountll(odd)) & 1u;
-                uint32_t const dead   = flip ? (~px & 0xFFFFu) : px;
-                uint32_t const starts = m & 0xFFFFu & ~dead, ends = (m >> 16) & ~dead;
-                lds.masks[b]          = starts | (ends << 16);
-                uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
-                uint32_t const incl   = wave_inclusive_scan(cnt);
-                lds.prefix[b]         = base + incl - cnt;
-                base += wave_bcast(incl, kWave - 1);
-              }
-              if (lane == 0) lds.prefix[kBlocks] = base;
-              nw = base & 0xFFFFu;
-              ne = base >> 16;
-              wave_lds_sync();
-            }
-          }
-          // ---- every row that starts in the tile notes the word it begins at (marked as not final), until that
-          // word's tokens have been placed
-          for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
-            uint32_t const r = r_first + i + lane;
-            if (r < r_end) {
-              int64_t const p  = coord(r) - tb;
-              a.offsets_out[r] = static_cast<int32_t>(0x80000000u | words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE)));
-            }
-          }
-          tile_open = true;
-          w_lo      = 0;
-          WP_PHASE(3)
+      // ---- word starts and ends
+      uint32_t nw = 0, ne = 0, inside0 = 0;  // words that start in the tile, words that end in it, the tile begins inside a word
+      bool ascii = false;                    // no staged byte has bit 7 set
+      {
+        uint32_t base = 0;
+        uint32_t seen = 0;
+        if (lane < kOverBlocks) {
+          uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (kBlocks + lane + 1)]);
+          seen          = v.x | v.y | v.z | v.w;
         }
-        if (tile_open) {
-          // ================================================================ a new unit: words [w_lo, w_hi) of the tile
-          w_hi = min(nw, w_lo + kWordCap);
-          nwc  = w_hi - w_lo;
-          uint16_t* const word16 = reinterpret_cast<uint16_t*>(lds.word[par]);
-          // start k pairs with end k (after the end of the word that ran into the tile)
+#pragma unroll
+        for (int s = 0; s < kSubs; ++s) {
+          int const b     = s * kWave + lane;
+          uint4 const v   = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
+          seen |= v.x | v.y | v.z | v.w;
+          uint32_t sp     = space_mask16(v);
+          uint32_t before = lds_byte[16 + 16 * b - 1] == 0x20u, after = lds_byte[16 + 16 * b + 16] == 0x20u;
+          if (edge) {
+            int64_t const g0 = tb + 16 * b;
+            sp |= outside_mask16(g0, cbeg, cend);
+            before |= (g0 - 1 < cbeg || g0 - 1 >= cend);
+            after |= (g0 + 16 < cbeg || g0 + 16 >= cend);
+          }
+          uint32_t const bd = lds.bound[b] & 0xFFFFu;
+          after |= lds.bound[b + 1] & 1u;
+          uint32_t const word   = ~sp & 0xFFFFu;
+          uint32_t const starts = word & ((sp << 1) | before | bd);
+          uint32_t const ends   = word & ((sp >> 1) | (after << 15) | (bd >> 1));
+          if (s == 0) inside0 = wave_bcast(word & ~starts & 1u, 0);
+          lds.masks[b]          = starts | (ends << 16);
+          uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
+          uint32_t const incl   = wave_inclusive_scan(cnt);
+          lds.prefix[b]         = base + incl - cnt;
+          base += wave_bcast(incl, kWave - 1);
+        }
+        if (lane == 0) lds.prefix[kBlocks] = base;
+        nw    = base & 0xFFFFu;
+        ne    = base >> 16;
+        ascii = ballot64((seen & 0x80808080u) != 0) == 0;
+      }
+      wave_lds_sync();
+      WP_PHASE(2)
+
+      // word starts at positions below x (0 <= x)
+      auto words_before = [&](uint32_t x) -> uint32_t {
+        if (x >= TILE) return nw;
+        uint32_t const b = x >> 4;
+        return (lds.prefix[b] & 0xFFFFu) + static_cast<uint32_t>(__builtin_popcount(lds.masks[b] & ((1u << (x & 15u)) - 1u)));
+      };
+
+      // ---- a word limit: the words of a row past its limit are dropped.  The first such word and the row's end are
+      // marked; a prefix parity over the marks gives the bytes whose word starts and ends go.
+      if (LIMIT) {
+        // position of word start k (k < nw)
+        auto word_start = [&](uint32_t k) -> uint32_t {
+          uint32_t b = 0;
+#pragma unroll
+          for (uint32_t step = kBlocks / 2; step > 0; step >>= 1)
+            if ((lds.prefix[b + step] & 0xFFFFu) <= k) b += step;
+          uint32_t m = lds.masks[b] & 0xFFFFu;
+          for (uint32_t j = k - (lds.prefix[b] & 0xFFFFu); j > 0; --j) m &= m - 1u;
+          return 16u * b + static_cast<uint32_t>(__builtin_ctz(m | 0x10000u));
+        };
+        bool cut = false;
+        auto drop_from = [&](uint32_t k, int64_t e) {  // from word start k up to position e
+          uint32_t const at = word_start(k);
+          atomicXor(&lds.bound[at >> 4], 0x10000u << (at & 15u));
+          if (e < TILE) atomicXor(&lds.bound[e >> 4], 0x10000u << (e & 15));
+          cut = true;
+        };
+        for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
+          uint32_t const r = r_first + i + lane;
+          if (r < r_end) {
+            int64_t const c0 = coord(r), c1 = coord(r + 1);
+            if (c1 > c0) {
+              int64_t const p = c0 - tb, e = c1 - tb;  // (p < TILE: the rows past the last tile's end are empty)
+              uint32_t const cap = word_cap(r, c1 - c0);
+              uint32_t const wp  = words_before(static_cast<uint32_t>(p));
+              uint32_t const we  = words_before(e < TILE ? static_cast<uint32_t>(e) : static_cast<uint32_t>(TILE));
+              if (wp + cap < we) drop_from(wp + cap, e);
+            }
+          }
+        }
+        // the row that runs into the tile
+        int64_t const e0   = r_first < r_end ? coord(r_first) - tb : static_cast<int64_t>(TILE);
+        uint32_t const we0 = words_before(e0 < TILE ? static_cast<uint32_t>(e0) : static_cast<uint32_t>(TILE));
+        if (lane == 0 && open_left < we0) drop_from(open_left, e0);
+        // and the row that runs out of it
+        if (r_first < r_end) {
+          uint32_t const rl   = r_end - 1;
+          int64_t const c0    = coord(rl), c1 = coord(rl + 1);
+          int64_t const p     = c0 - tb;
+          uint32_t const cap  = word_cap(rl, c1 - c0);
+          uint32_t const used = nw - words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
+          open_left           = cap - min(cap, used);
+        } else {
+          open_left -= min(open_left, nw);
+        }
+        if (ballot64(cut) != 0) {
+          wave_lds_sync();
+          uint32_t base = 0, carry = 0;
+#pragma unroll
+          for (int s = 0; s < kSubs; ++s) {
+            int const b      = s * kWave + lane;
+            uint32_t const m = lds.masks[b];
+            uint32_t px      = lds.bound[b] >> 16;
+            px ^= px << 1;
+            px ^= px << 2;
+            px ^= px << 4;
+            px ^= px << 8;
+            px &= 0xFFFFu;
+            uint64_t const odd  = ballot64((px >> 15) != 0);
+            uint32_t const flip = (lanes_below(odd) & 1u) ^ carry;
+            carry ^= static_cast<uint32_t>(__builtin_popcountll(odd)) & 1u;
+            uint32_t const dead   = flip ? (~px & 0xFFFFu) : px;
+            uint32_t const starts = m & 0xFFFFu & ~dead, ends = (m >> 16) & ~dead;
+            lds.masks[b]          = starts | (ends << 16);
+            uint32_t const cnt    = static_cast<uint32_t>(__builtin_popcount(starts)) | (static_cast<uint32_t>(__builtin_popcount(ends)) << 16);
+            uint32_t const incl   = wave_inclusive_scan(cnt);
+            lds.prefix[b]         = base + incl - cnt;
+            base += wave_bcast(incl, kWave - 1);
+          }
+          if (lane == 0) lds.prefix[kBlocks] = base;
+          nw = base & 0xFFFFu;
+          ne = base >> 16;
+          wave_lds_sync();
+        }
+      }
+      WP_PHASE(3)
+
+      // ---- the words, at most kWordCap at a time (only a tile of one-byte rows has more)
+      uint32_t done = 0;  // tokens of this tile so far
+      for (uint32_t w_lo = 0;; w_lo += kWordCap) {
+        uint32_t const w_hi = min(nw, w_lo + kWordCap);
+        uint32_t const nwc  = w_hi - w_lo;
+        // start k pairs with end k (after the end of the word that ran into the tile)
+        if (nw <= kWordCap) {
+#pragma unroll
+          for (int s = 0; s < kSubs; ++s) {
+            int const b       = s * kWave + lane;
+            uint32_t const m  = lds.masks[b];
+            uint32_t const pf = lds.prefix[b];
+            uint32_t ks       = pf & 0xFFFFu;
+            uint32_t ke       = (pf >> 16) - inside0;  // (the end without a start comes first: it goes to slot -1, which is the entry before lds.word)
+            for (uint32_t st = m & 0xFFFFu; st; st &= st - 1u, ++ks) word16[2 * ks] = static_cast<uint16_t>(16 * b + __builtin_ctz(st));
+            for (uint32_t en = m >> 16; en; en &= en - 1u, ++ke) word16[2 * static_cast<int32_t>(ke) + 1] = static_cast<uint16_t>(16 * b + __builtin_ctz(en));
+          }
+        } else {
 #pragma unroll
           for (int s = 0; s < kSubs; ++s) {
             int const b       = s * kWave + lane;
@@ -1093,199 +1065,168 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
             for (uint32_t en = m >> 16; en; en &= en - 1u, ++ke)
               if (ke >= static_cast<int32_t>(w_lo) && ke < static_cast<int32_t>(w_hi)) word16[2 * (ke - w_lo) + 1] = static_cast<uint16_t>(16 * b + __builtin_ctz(en));
           }
-          if (w_hi == nw && nwc > 0 && nw + inside0 > ne) {
-            // the last word ends past the tile: at the byte before the first space, row start or end of the view
-            uint32_t sep = 0;
-            if (lane < kOverBlocks) {
-              int const b   = kBlocks + lane;
-              uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
-              sep           = space_mask16(v) | (lds.bound[b] & 0xFFFFu);
-              if (edge) sep |= outside_mask16(tb + 16 * b, cbeg, cend);
-            }
-            uint64_t const sm = ballot64(sep != 0);
-            uint32_t endpos   = TILE + 16 * kOverBlocks - 1;
-            if (sm != 0) {
-              int const fl = __builtin_ctzll(sm);
-              endpos       = TILE + 16 * fl + __builtin_ctz(wave_bcast(sep, fl)) - 1;
-            }
-            if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
-          }
-          if (lane == 0) lds.tok_used[par] = 0;
-          k0        = 0;
-          unit_open = true;
-          wave_lds_sync();
-          WP_PHASE(4)
         }
-      }
-      if (unit_open) {
-        // ================================================================ look the words up; the ones that are not in
-        // the vocabulary wait in the queue
-        uint32_t* const uw = lds.word[par];
-        while (k0 < nwc && qn + kWave <= kQueueCap) {
-          uint32_t const k = k0 + lane;
-          uint32_t defer   = 0;  // 1: not in the vocabulary; 2: not decided here (more than 8 bytes; a key that may have been carried past its bucket)
-          if (k < nwc) {
-            uint32_t const rec = uw[k];
+        if (w_hi == nw && nwc > 0 && nw + inside0 > ne) {
+          // the last word ends past the tile: at the byte before the first space, row start or end of the view
+          uint32_t sep = 0;
+          if (lane < kOverBlocks) {
+            int const b   = kBlocks + lane;
+            uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
+            sep           = space_mask16(v) | (lds.bound[b] & 0xFFFFu);
+            if (edge) sep |= outside_mask16(tb + 16 * b, cbeg, cend);
+          }
+          uint64_t const sm = ballot64(sep != 0);
+          uint32_t endpos   = TILE + 16 * kOverBlocks - 1;
+          if (sm != 0) {
+            int const fl = __builtin_ctzll(sm);
+            endpos       = TILE + 16 * fl + __builtin_ctz(wave_bcast(sep, fl)) - 1;
+          }
+          if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
+        }
+        if (lane == 0) lds.tok_used = 0;
+        wave_lds_sync();
+        WP_PHASE(4)
+
+        // ---- look the words up; the ones that are not in the vocabulary, or not decided here, go to the queue
+        uint32_t* const uw = lds.word;
+        for (uint32_t k0 = 0;;) {
+          uint32_t qn = 0;
+          while (k0 < nwc && qn + kWave <= kQueueCap) {
+            uint32_t const k   = k0 + lane;
+            bool const active  = k < nwc;
+            uint32_t const rec = uw[active ? k : 0u];
             uint32_t const s   = rec & 0xFFFFu;
             uint32_t const wl  = (rec >> 16) - s + 1u;
-            if (wl >= kMaxWord) {
-              uw[k] = static_cast<uint32_t>(table.unk_id);  // wordpiece_tokenize.cu:442-445, 738-741
-            } else if (wl > 8) {
-              defer = 2;
-            } else {
-              uint32_t const o  = 16u + s;
-              uint32_t const sh = (o & 3u) * 8u;
-              uint32_t const d0 = lds.bytes[o >> 2], d1 = lds.bytes[(o >> 2) + 1], d2 = lds.bytes[(o >> 2) + 2];
-              Probe pr;
-              pr.k0 = __builtin_amdgcn_alignbit(d1, d0, sh);
-              pr.k1 = __builtin_amdgcn_alignbit(d2, d1, sh);
-              trim_key8(wl, pr.k0, pr.k1);
-              int32_t id  = kNone;
-              uint32_t vd = 0;
-              if (wl <= table.max_len[0]) {
-                uint32_t const h = key_hash_block(key_hash_init(wl), pr.k0, pr.k1);
-                uint32_t bk;
-                pr.want   = slot_word0(h, 0, wl, &bk);
-                pr.fp     = carried_bit(h);
-                pr.bucket = bk & table.bucket_mask;
-                uint4 const s0 = table.slots[2 * pr.bucket];
-                uint4 const s1 = table.slots[2 * pr.bucket + 1];
-                vd = verdict(pr, s0, s1, wl, &id);
-              }
-              if (vd == 1u) uw[k] = static_cast<uint32_t>(id);
-              else defer = vd == 2u ? 2u : 1u;
-            }
+            // straight-line code: every lane reads a bucket (of whatever its first bytes are), and what it makes of it
+            // depends on the word's length afterwards
+            uint32_t const o  = 16u + s;
+            uint32_t const sh = (o & 3u) * 8u;
+            uint32_t const d0 = lds.bytes[o >> 2], d1 = lds.bytes[(o >> 2) + 1], d2 = lds.bytes[(o >> 2) + 2];
+            Probe pr;
+            pr.k0 = __builtin_amdgcn_alignbit(d1, d0, sh);
+            pr.k1 = __builtin_amdgcn_alignbit(d2, d1, sh);
+            uint32_t const wl8 = min(wl, 8u);
+            trim_key8(wl8, pr.k0, pr.k1);
+            uint32_t const h = key_hash_block(key_hash_init(wl8), pr.k0, pr.k1);
+            uint32_t bk;
+            pr.want   = slot_word0(h, 0, wl8, &bk);
+            pr.fp     = carried_bit(h);
+            pr.bucket = bk & table.bucket_mask;
+            uint4 const s0 = table.slots[2 * pr.bucket];
+            uint4 const s1 = table.slots[2 * pr.bucket + 1];
+            int32_t id        = kNone;
+            uint32_t const vd = verdict(pr, s0, s1, wl8, &id);
+            bool const too_long = wl >= kMaxWord;  // wordpiece_tokenize.cu:442-445, 738-741: one unknown token
+            bool const found    = wl <= 8 && vd == 1u;
+            // 1: not in the vocabulary; 2: not decided here (more than 8 bytes; a key that may have been carried past its bucket)
+            uint32_t const defer = !active || too_long || found ? 0u : (wl > 8 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
+            if (active && (too_long || found)) uw[k] = too_long ? static_cast<uint32_t>(table.unk_id) : static_cast<uint32_t>(id);
+            uint64_t const mm = ballot64(defer != 0);
+            if (defer != 0) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k | (defer == 2u ? 0x8000u : 0u));
+            qn += static_cast<uint32_t>(__builtin_popcountll(mm));
+            k0 += kWave;
           }
-          uint64_t const mm = ballot64(defer != 0);
-          if (defer != 0) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k | (defer == 2u ? 0x8000u : 0u));
-          qn += static_cast<uint32_t>(__builtin_popcountll(mm));
-          k0 += kWave;
-        }
-        reason = k0 >= nwc ? kUnitDone : kQueueFull;
-        wave_lds_sync();
-        WP_PHASE(5)
-      }
-
-      // ================================================================ the out-of-vocabulary words, one lane each; a lane
-      // that finishes stores its result and takes the next word from the queue.  Words of up to 16 bytes run in
-      // registers; the few longer ones are set aside (queue[0 .. n_long)) and only counted here.
-      {
-        // stores the tokens of the words finished by this step
-        auto deliver = [&](bool fin, uint32_t cnt) {
-          if (fin) {
-            uint32_t const keep  = cnt <= kOovKeep ? cnt : 0u;
-            uint32_t const off   = keep > 0 ? atomicAdd(&lds.tok_used[mine_par], keep) : 0u;
-            uint32_t* const slot = &lds.word[mine_par][mine];
-            if (keep > 0 && off + keep <= kTokCap) {
+          WP_PHASE(5)
+          if (qn > 0) {
+            wave_lds_sync();
+            // ---- the queued words, one lane each; a lane that finishes stores its result and takes the next word.
+            // Words of up to 16 bytes run in registers; longer ones are set aside (queue[0 .. n_long)) for the loop below.
+            uint32_t q_next = 0, n_long = 0;
+            ShortWord sw;
+            sw.done   = true;
+            sw.count  = 0;
+            bool busy = false;
+            uint32_t mine = 0;  // my word
+            int32_t tok[kOovKeep];
+            auto keep_token = [&](uint32_t j, int32_t id) {
 #pragma unroll
               for (int i = 0; i < kOovKeep; ++i)
-                if (static_cast<uint32_t>(i) < keep) lds.tokens[mine_par][off + i] = static_cast<uint32_t>(tok[i]);
-              *slot = kOovMark | (cnt << 16) | off;
-            } else {
-              uint32_t const rec = *slot;
-              uint32_t const s   = rec & 0xFFFFu;
-              *slot              = kOovMark | kOovRedo | (cnt << 21) | (((rec >> 16) - s + 1u) << 13) | s;
-            }
-          }
-        };
-        uint32_t n_long = 0;
-        for (;;) {
-          bool const fin      = busy && sw.done;
-          uint64_t const finm = ballot64(fin);
-          if (finm != 0 || q_next < qn) {
-            if (finm != 0) {
-              deliver(fin, sw.count);
-              if (fin) busy = false;
-            }
-            uint64_t const idle = ballot64(!busy);
-            uint32_t const left = qn - q_next;
-            if (left > 0 && idle != 0) {
-              uint32_t const rank = lanes_below(idle);
-              bool is_long        = false;
-              uint32_t k          = 0;
-              if (!busy && rank < left) {
-                k                  = lds.queue[q_next + rank];
-                uint32_t const rec = lds.word[par][k & 0x7FFFu];
-                uint32_t const s   = rec & 0xFFFFu;
-                uint32_t const wl  = (rec >> 16) - s + 1u;
-                if (wl <= 16) {
-                  TileWord const tw{lds.bytes, 16u + s};
-                  uint32_t head[4];
-                  tw.head16(head);
-                  trim_key8(wl, head[0], head[1]);
-                  trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
-                  sw.begin(table, first_ids, head, wl, (k & 0x8000u) == 0, ascii);
-                  busy     = true;
-                  mine     = k & 0x7FFFu;
-                  mine_par = par;
+                if (j == static_cast<uint32_t>(i)) tok[i] = id;
+            };
+            for (;;) {
+              if (busy && sw.done) {
+                // my word is finished: its tokens go to lds.tokens (if there are at most kOovKeep, and room)
+                uint32_t const cnt  = sw.count;
+                uint32_t const keep = cnt <= kOovKeep ? cnt : 0u;
+                uint32_t const off  = keep > 0 ? atomicAdd(&lds.tok_used, keep) : 0u;
+                if (keep > 0 && off + keep <= kTokCap) {
+#pragma unroll
+                  for (int i = 0; i < kOovKeep; ++i)
+                    if (static_cast<uint32_t>(i) < keep) lds.tokens[off + i] = static_cast<uint32_t>(tok[i]);
+                  uw[mine] = kOovMark | (cnt << 16) | off;
                 } else {
-                  is_long = true;
+                  uint32_t const rec = uw[mine];
+                  uint32_t const s   = rec & 0xFFFFu;
+                  uw[mine]           = kOovMark | kOovRedo | (cnt << 21) | (((rec >> 16) - s + 1u) << 13) | s;
+                }
+                busy = false;
+              }
+              uint32_t const left = qn - q_next;
+              if (left > 0) {
+                uint64_t const idle = ballot64(!busy);
+                if (idle != 0) {
+                  uint32_t const rank = lanes_below(idle);
+                  bool is_long        = false;
+                  uint32_t k          = 0;
+                  if (!busy && rank < left) {
+                    k                  = lds.queue[q_next + rank];
+                    uint32_t const rec = uw[k & 0x7FFFu];
+                    uint32_t const s   = rec & 0xFFFFu;
+                    uint32_t const wl  = (rec >> 16) - s + 1u;
+                    if (wl <= 16) {
+                      TileWord const tw{lds.bytes, 16u + s};
+                      uint32_t head[4];
+                      tw.head16(head);
+                      trim_key8(wl, head[0], head[1]);
+                      trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
+                      sw.begin(table, first_ids, head, wl, (k & 0x8000u) == 0, ascii);
+                      busy = true;
+                      mine = k & 0x7FFFu;
+                    } else {
+                      is_long = true;
+                    }
+                  }
+                  q_next += min(static_cast<uint32_t>(__builtin_popcountll(idle)), left);
+                  uint64_t const lm = ballot64(is_long);
+                  if (lm != 0) {
+                    wave_lds_sync();  // (the queue entries just read lie at or past n_long)
+                    if (is_long) lds.queue[n_long + lanes_below(lm)] = static_cast<uint16_t>(k);
+                    n_long += static_cast<uint32_t>(__builtin_popcountll(lm));
+                  }
                 }
               }
-              q_next += min(static_cast<uint32_t>(__builtin_popcountll(idle)), left);
-              uint64_t const lm = ballot64(is_long);
-              if (lm != 0) {
-                wave_lds_sync();  // (the queue entries just read lie at or past n_long)
-                if (is_long) lds.queue[n_long + lanes_below(lm)] = static_cast<uint16_t>(k);
-                n_long += static_cast<uint32_t>(__builtin_popcountll(lm));
+              if (ballot64(busy) == 0) {
+                if (q_next >= qn) break;
+                continue;
+              }
+#ifdef WP_PHASE_TIMING
+              phase_t[9] += 1;
+#endif
+              if (busy && !sw.done) sw.step(table, first_ids, keep_token);
+            }
+            if (n_long > 0) {
+              wave_lds_sync();
+              for (uint32_t base = 0; base < n_long; base += kWave) {
+                if (base + lane < n_long) {
+                  uint32_t const k   = lds.queue[base + lane] & 0x7FFFu;  // (words of more than 16 bytes have not been looked up whole)
+                  uint32_t const rec = uw[k];
+                  uint32_t const s   = rec & 0xFFFFu;
+                  uint32_t const wl  = (rec >> 16) - s + 1u;
+                  uint32_t const cnt = count_oov_tokens(table, lds.bytes, 16u + s, wl);
+                  uw[k]              = kOovMark | kOovRedo | (cnt << 21) | (wl << 13) | s;
+                }
               }
             }
+            wave_lds_sync();
+            WP_PHASE(6)
           }
-          uint64_t const bm = ballot64(busy);
-          if (q_next >= qn) {
-            if (bm == 0 || reason == kQueueFull) break;
-            if (reason == kUnitDone && ballot64(busy && mine_par != par) == 0 && __builtin_popcountll(bm) < kStragglers) break;
-          }
-#ifdef WP_PHASE_TIMING
-          phase_t[9] += 1;
-#endif
-          if (busy && !sw.done) sw.step(table, first_ids, keep_token);
+          if (k0 >= nwc) break;
         }
-        if (n_long > 0) {
-          wave_lds_sync();
-          for (uint32_t base = 0; base < n_long; base += kWave) {
-            if (base + lane < n_long) {
-              uint32_t const k   = lds.queue[base + lane] & 0x7FFFu;  // (words of more than 16 bytes have not been looked up whole)
-              uint32_t const rec = lds.word[par][k];
-              uint32_t const s   = rec & 0xFFFFu;
-              uint32_t const wl  = (rec >> 16) - s + 1u;
-              uint32_t const cnt = count_oov_tokens(table, lds.bytes, 16u + s, wl);
-              lds.word[par][k]   = kOovMark | kOovRedo | (cnt << 21) | (wl << 13) | s;
-            }
-          }
-        }
-        qn     = 0;
-        q_next = 0;
-        wave_lds_sync();
-        WP_PHASE(6)
-      }
-      if (reason == kQueueFull) continue;
 
-      // ================================================================ the unit before: place and write its tokens
-      if (pend) {
-        uint32_t* const uw       = lds.word[p_par];
-        const uint32_t* const ut = lds.tokens[p_par];
-        uint32_t done            = 0;  // tokens of the unit so far
-        // The tokens are put together in LDS in their final order and leave in whole runs, one dword per lane, because
-        // scattered stores cost the memory pipeline a cycle per lane.  The room for that is the staged bytes of the tile
-        // being looked up, which are free once the last of its words has been taken from the queue.
-        constexpr uint32_t kOutCap = sizeof(lds.bytes) / sizeof(uint32_t);
-        uint32_t* const out        = lds.bytes;
-        bool const may_stage       = reason == kRangeDone || w_hi == nw;
-        uint32_t flush_base = cursor, staged = 0;  // out[0 .. staged) are the tokens from flush_base on
-        auto flush = [&] {
-          if (staged == 0) return;
-          wave_lds_sync();
-          if (flush_base + staged > a.range_cap) spill = true;
-          if (!spill)
-            for (uint32_t i = lane; i < staged; i += kWave) region[flush_base + i] = out[i];
-          wave_lds_sync();
-          flush_base += staged;
-          staged = 0;
-        };
-        for (uint32_t j0 = 0; j0 < p_nwc; j0 += kWave) {
+        // ---- place and write the tokens
+        for (uint32_t j0 = 0; j0 < nwc; j0 += kWave) {
           uint32_t const k   = j0 + lane;
-          bool const active  = k < p_nwc;
+          bool const active  = k < nwc;
           uint32_t const v   = active ? uw[k] : 0u;
           bool const marked  = active && (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
           bool const redo    = marked && (v & kOovRedo) != 0;
@@ -1293,82 +1234,46 @@ __global__ void __launch_bounds__(kTokThreads, 4) wordpiece_tile_kernel(TileArgs
           uint32_t const incl = wave_inclusive_scan(cnt);
           uint32_t const ex   = incl - cnt;
           uint32_t const tot  = wave_bcast(incl, kWave - 1);
-          uint32_t const off  = v & 0xFFFFu;
-          if (may_stage && ballot64(redo) == 0) {
-            if (staged + tot > kOutCap) flush();  // (tot <= 64 * kOovKeep < kOutCap)
-            if (active) {
-              uint32_t* const dst = out + staged + ex;
-              dst[0]              = marked ? ut[off] : v;
+          if (cursor + done + tot > a.range_cap) spill = true;
+          if (!spill) {
+            uint32_t* const dst = region + (cursor + done + ex);
+            if (ballot64(redo) != 0 && redo) {
+              // tokens that were not kept (more than kOovKeep, a word of more than 16 bytes, no room left in LDS):
+              // tokenized again, into place
+              write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
+            }
+            if (active && !redo) {
+              uint32_t const off = v & 0xFFFFu;
+              dst[0]             = marked ? lds.tokens[off] : v;
 #pragma unroll
               for (uint32_t j = 1; j < kOovKeep; ++j) {
                 if (ballot64(marked && j < cnt) == 0) break;
-                if (marked && j < cnt) dst[j] = ut[off + j];
+                if (marked && j < cnt) dst[j] = lds.tokens[off + j];
               }
             }
-            staged += tot;
-          } else {
-            // straight to memory: while the staged bytes are still in use (a tile of more words than a unit holds),
-            // and the rounds with a word whose tokens were not kept (more than kOovKeep, a word of more than 16 bytes,
-            // no room left in LDS), which is tokenized again, into place
-            flush();
-            if (cursor + done + tot > a.range_cap) spill = true;
-            if (!spill) {
-              uint32_t* const dst = region + (cursor + done + ex);
-              if (redo) {
-                write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + p_tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
-              } else if (active) {
-                dst[0] = marked ? ut[off] : v;
-#pragma unroll
-                for (uint32_t j = 1; j < kOovKeep; ++j) {
-                  if (ballot64(marked && j < cnt) == 0) break;
-                  if (marked && j < cnt) dst[j] = ut[off + j];
-                }
-              }
-            }
-            flush_base = cursor + done + tot;
           }
           if (active) uw[k] = done + ex;
           done += tot;
         }
-        flush();
         wave_lds_sync();
         WP_PHASE(7)
-        // the rows that start in its tile at one of its words (or, for the last words of the tile, after them): the
+
+        // ---- the rows that start in the tile at one of these words (or, with the tile's last words, after them): the
         // tokens of the range before them
-        bool const p_last = p_wlo + p_nwc == p_nw;
-        for (uint32_t i = 0; p_rfirst + i < p_rend; i += kWave) {
-          uint32_t const r = p_rfirst + i + lane;
-          if (r < p_rend) {
-            uint32_t const v = static_cast<uint32_t>(a.offsets_out[r]);
-            if ((v & 0x80000000u) != 0) {
-              uint32_t const k = v & 0x7FFFFFFFu;
-              if (k >= p_wlo && k < p_wlo + p_nwc) a.offsets_out[r] = static_cast<int32_t>(cursor + uw[k - p_wlo]);
-              else if (k == p_nw && p_last) a.offsets_out[r] = static_cast<int32_t>(cursor + done);
-            }
+        for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
+          uint32_t const r = r_first + i + lane;
+          if (r < r_end) {
+            int64_t const p  = coord(r) - tb;
+            uint32_t const k = words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
+            if (k >= w_lo && k < w_hi) a.offsets_out[r] = static_cast<int32_t>(cursor + uw[k - w_lo]);
+            else if (k == nw && w_hi == nw) a.offsets_out[r] = static_cast<int32_t>(cursor + done);
           }
         }
-        cursor += done;
-        pend = false;
         wave_lds_sync();
-        WP_PHASE(8)
+        if (w_hi == nw) break;
       }
-      if (reason == kRangeDone) break;
-      // the unit just looked up waits for its last words
-      pend     = true;
-      p_tb     = tb;
-      p_par    = par;
-      p_nwc    = nwc;
-      p_wlo    = w_lo;
-      p_nw     = nw;
-      p_rfirst = r_first;
-      p_rend   = r_end;
-      par ^= 1u;
-      unit_open = false;
-      w_lo      = w_hi;
-      if (w_hi == nw) {
-        tile_open = false;
-        ++t;
-      }
+      cursor += done;
+      WP_PHASE(8)
     }
     if (lane == 0) {
       a.range_count[range] = cursor;
@@ -1744,7 +1649,11 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
   int per_cu = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(wordpiece_tile_kernel<kTile>), kTokThreads, 0) != hipSuccess || per_cu < 1)
+  bool const is64  = input->offsets_is_int64 != 0;
+  bool const limit = max_words_per_row > 0;
+  void (*const tile_kernel)(TileArgs) = is64 ? (limit ? wordpiece_tile_kernel<kTile, true, true> : wordpiece_tile_kernel<kTile, true, false>)
+                                             : (limit ? wordpiece_tile_kernel<kTile, false, true> : wordpiece_tile_kernel<kTile, false, false>);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(tile_kernel), kTokThreads, 0) != hipSuccess || per_cu < 1)
     per_cu = 2;
   unsigned const tile_grid =
     static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, static_cast<int64_t>(per_cu) * cus));
@@ -1792,7 +1701,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
     {
       ProfileScope ps("wordpiece_tile_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_tile_kernel<kTile>, dim3(tile_grid), dim3(kTokThreads), 0, stream, args);
+      hipLaunchKernelGGL(tile_kernel, dim3(tile_grid), dim3(kTokThreads), 0, stream, args);
     }
     // where the tokens of each range go; the total decides the child size
     // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
