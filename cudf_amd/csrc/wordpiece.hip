@@ -534,7 +534,8 @@ struct ShortWord {
   uint32_t r[4];   // bytes [start, start + 16) of the word, zero padded
   uint32_t rem;    // bytes from start to the end of the word
   uint32_t bnd;    // bit i: start + i is a character boundary (bit rem is set)
-  uint32_t cand;   // lengths still to try for the piece at start (bit l - 1), longest first
+  uint32_t cand;   // lengths still to try for the piece at start (bit l - 1), longest first, once the length filter has been applied
+  uint32_t lens;   // the length filter word of the piece's opening (all ones once applied)
   uint32_t count;  // tokens so far
   int32_t id1, id2;  // ids of the piece's first byte and first two bytes as keys (kNone: no such key)
   bool done;
@@ -579,10 +580,12 @@ struct ShortWord {
 
   // The piece at start begins: its candidate lengths are those on a character boundary, no longer than the rest of
   // the word or the longest key, and not ruled out by the length filter of its first three bytes.
+  // (What the opening holds is not looked at here but when the next trip begins: by then its reads have arrived.)
   __device__ __forceinline__ void open_piece(VocabTable const& t, uint32_t kind, Opening const& o)
   {
     uint32_t const lim = min(min(rem, t.max_len[kind]), 16u);
-    cand               = (bnd >> 1) & ((1u << lim) - 1u) & ((o.lens << 2) | 3u);
+    cand               = (bnd >> 1) & ((1u << lim) - 1u);
+    lens               = o.lens;
     id1                = o.id1;
     id2                = o.id2;
   }
@@ -651,7 +654,9 @@ struct ShortWord {
   template <typename Emit>
   __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, Emit&& emit)
   {
-    uint32_t const kind   = count ? 1u : 0u;
+    uint32_t const kind = count ? 1u : 0u;
+    cand &= (lens << 2) | 3u;
+    lens                  = 0xFFFFFFFFu;
     uint32_t const longer = cand & ~3u;
     bool const has_a      = longer != 0;
     uint32_t const la     = 32u - static_cast<uint32_t>(__builtin_clz(has_a ? longer : 4u));
@@ -670,7 +675,13 @@ struct ShortWord {
     uint32_t const short_len   = two ? 2u : 1u;
     int32_t ida = kNone;
     uint32_t va = has_a ? verdict(pa, a0, a1, la, &ida) : 0u;
-    if (va == 2u) {  // the general lookup (keys in the pool, keys carried past their bucket)
+    if (va == 2u && la > 8) {  // a key of 9 to 16 bytes with the right tag: its bytes decide
+      uint32_t k[4] = {r[0], r[1], r[2], r[3]};
+      trim_key8(8u, k[0], k[1]);
+      trim_key8(la - 8u, k[2], k[3]);
+      va = verdict_16(t, pa, a0, a1, k, &ida);
+    }
+    if (va == 2u) {  // the general lookup (keys of more than 16 bytes, keys carried past their bucket)
       RegWord const rw{{r[0], r[1], r[2], r[3]}};
       ida = lookup_slow(t, kind, rw, 0u, la);
       va  = ida == kNone ? 0u : 1u;
@@ -1098,28 +1109,33 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
             uint32_t const s   = rec & 0xFFFFu;
             uint32_t const wl  = (rec >> 16) - s + 1u;
             // straight-line code: every lane reads a bucket (of whatever its first bytes are), and what it makes of it
-            // depends on the word's length afterwards
-            uint32_t const o  = 16u + s;
-            uint32_t const sh = (o & 3u) * 8u;
-            uint32_t const d0 = lds.bytes[o >> 2], d1 = lds.bytes[(o >> 2) + 1], d2 = lds.bytes[(o >> 2) + 2];
+            // depends on the word's length afterwards; only a key of 9 to 16 bytes with the right tag needs a second
+            // read, of the key's bytes
+            TileWord const tw{lds.bytes, 16u + s};
+            uint32_t head[4];
+            tw.head16(head);
+            uint32_t const wl16 = min(wl, 16u);
+            trim_key8(wl16, head[0], head[1]);
+            trim_key8(wl16 > 8 ? wl16 - 8u : 0u, head[2], head[3]);
             Probe pr;
-            pr.k0 = __builtin_amdgcn_alignbit(d1, d0, sh);
-            pr.k1 = __builtin_amdgcn_alignbit(d2, d1, sh);
-            uint32_t const wl8 = min(wl, 8u);
-            trim_key8(wl8, pr.k0, pr.k1);
-            uint32_t const h = key_hash_block(key_hash_init(wl8), pr.k0, pr.k1);
+            pr.k0             = head[0];
+            pr.k1             = head[1];
+            uint32_t const h1 = key_hash_block(key_hash_init(wl16), pr.k0, pr.k1);
+            uint32_t const h2 = key_hash_block(h1, head[2], head[3]);
+            uint32_t const h  = wl16 > 8 ? h2 : h1;
             uint32_t bk;
-            pr.want   = slot_word0(h, 0, wl8, &bk);
+            pr.want   = slot_word0(h, 0, wl16, &bk);
             pr.fp     = carried_bit(h);
             pr.bucket = bk & table.bucket_mask;
             uint4 const s0 = table.slots[2 * pr.bucket];
             uint4 const s1 = table.slots[2 * pr.bucket + 1];
-            int32_t id        = kNone;
-            uint32_t const vd = verdict(pr, s0, s1, wl8, &id);
+            int32_t id  = kNone;
+            uint32_t vd = verdict(pr, s0, s1, wl16, &id);
+            if (vd == 2u && wl > 8 && wl <= 16) vd = verdict_16(table, pr, s0, s1, head, &id);
             bool const too_long = wl >= kMaxWord;  // wordpiece_tokenize.cu:442-445, 738-741: one unknown token
-            bool const found    = wl <= 8 && vd == 1u;
-            // 1: not in the vocabulary; 2: not decided here (more than 8 bytes; a key that may have been carried past its bucket)
-            uint32_t const defer = !active || too_long || found ? 0u : (wl > 8 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
+            bool const found    = wl <= 16 && vd == 1u;
+            // 1: not in the vocabulary; 2: not decided here (more than 16 bytes; a key that may have been carried past its bucket)
+            uint32_t const defer = !active || too_long || found ? 0u : (wl > 16 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
             if (active && (too_long || found)) uw[k] = too_long ? static_cast<uint32_t>(table.unk_id) : static_cast<uint32_t>(id);
             uint64_t const mm = ballot64(defer != 0);
             if (defer != 0) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k | (defer == 2u ? 0x8000u : 0u));
@@ -1200,9 +1216,12 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
                 continue;
               }
 #ifdef WP_PHASE_TIMING
-              phase_t[9] += 1;
+              uint64_t const t_before = __builtin_amdgcn_s_memtime();
 #endif
               if (busy && !sw.done) sw.step(table, first_ids, keep_token);
+#ifdef WP_PHASE_TIMING
+              phase_t[9] += __builtin_amdgcn_s_memtime() - t_before;
+#endif
             }
             if (n_long > 0) {
               wave_lds_sync();
@@ -1719,6 +1738,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       for (auto x : ph) sum += x;
       static const char* const names[10] = {"stage", "rows", "detect", "cap", "lists", "probe", "oov", "write", "rowoffs", "tail"};
       sum -= ph[9];
+      fprintf(stderr, "[step share of all %.1f%%] ", 100.0 * ph[9] / (sum ? sum : 1));
       for (int i = 0; i < 9; ++i) fprintf(stderr, "%s %.1f%%  ", names[i], 100.0 * ph[i] / (sum ? sum : 1));
       fprintf(stderr, "trips/tile %.2f", double(ph[9]) / double(ntiles));
       fprintf(stderr, "\n");

@@ -405,6 +405,77 @@ def test_wordpiece_random_vs_oracle(nv, orc, max_words, dtype):
     assert exp.child.size > (5000 if max_words == 7 else 50000)
 
 
+def _tile_kernel_launches(nv, fn):
+    """Runs fn() with the library's kernel timing on; returns its result and the number of tile-pass launches."""
+    from cudf_amd import _capi
+    import torch
+    _capi.profile_enable(True)
+    _capi.profile_read()
+    try:
+        out = fn()
+        torch.cuda.synchronize()
+        names = [n for n, _ in _capi.profile_read()]
+    finally:
+        _capi.profile_enable(False)
+    return out, sum(1 for n in names if n == "wordpiece_tile_kernel")
+
+
+@pytest.mark.parametrize("max_words", [0, 5, 100000])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("shape", ["few rows", "many rows"])
+def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shape, dtype, max_words):
+    """Text whose ranges give more than three tokens per eight bytes (here two-letter words that are not in the
+    vocabulary and fall apart into letters: two tokens per three bytes) does not fit the arena of the first
+    attempt: the call has to notice, run the tile pass again with room for a token per byte, and give the same
+    result as the oracle (greedy rule: cpp/src/text/wordpiece_tokenize.cu:349-407).  A million such words, in
+    a few long rows and in many short ones; the two launches are read off the library's kernel timing."""
+    rng = np.random.default_rng(5)
+    letters = "abcdefgh"
+    vocab = ["[UNK]"] + list(letters) + ["##" + c for c in letters] + ["abcdefgh"]
+    words = ["".join(rng.choice(list(letters), 2)) for _ in range(4096)]
+    per_row = 125000 if shape == "few rows" else 7
+    nrows = 8 if shape == "few rows" else 150000
+    rows = [" ".join(words[int(j) % 4096] for j in rng.integers(0, 4096, per_row)) for _ in range(nrows)]
+    rows[1] = None
+    rows[2] = ""
+    host = strings(rows, dtype)
+    hv = strings(vocab)
+    dcol, dvoc = dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv))
+    got, launches = _tile_kernel_launches(nv, lambda: nv.wordpiece_tokenize(dcol, dvoc, max_words))
+    exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), max_words, nthreads=8)
+    assert_same(got.to_host(), exp, f"{shape}, max_words={max_words}")
+    if max_words != 5 or shape == "many rows":
+        assert launches == 2, launches  # (five words of a long row are too few tokens to fill anything)
+        assert exp.child.size > 1_000_000
+    # ordinary text right afterwards: one launch, nothing left over from the call before
+    plain = strings(["abcdefgh " * 2000] * 50, dtype)
+    got, launches = _tile_kernel_launches(nv, lambda: nv.wordpiece_tokenize(dev(nv, plain), dvoc, max_words))
+    assert launches == 1
+    assert_same(got.to_host(), orc.wordpiece_tokenize(plain, orc.Vocabulary(hv), max_words, nthreads=8), "plain text afterwards")
+
+
+def test_wordpiece_rows_of_one_byte_and_tiles_of_more_words_than_a_unit(nv, orc):
+    """Every byte a row of its own (row starts separate words as spaces do: cpp/src/text/wordpiece_tokenize.cu:515-523), so a
+    tile of 2048 bytes holds 2048 words, four times what is looked up at a time, and a token per byte; then the
+    same bytes as words of one letter between spaces (1024 words per tile).  With a word limit a one-byte row has
+    room for no word at all (limit = bytes / 2, :780)."""
+    rng = np.random.default_rng(6)
+    letters = "abcdefgh"
+    vocab = ["[UNK]"] + list(letters) + ["##" + c for c in letters]
+    hv = strings(vocab)
+    dvoc, ovoc = nv.WordPieceVocabulary(dev(nv, hv)), orc.Vocabulary(hv)
+    n = 300_000
+    chars = rng.choice(list(letters + "xy"), n)
+    for dtype in (np.int32, np.int64):
+        one_byte_rows = strings(list(chars), dtype)
+        spaced = strings([" ".join(chars[i:i + 5000]) for i in range(0, n, 5000)] + ["x", " ", ""], dtype)
+        for host in (one_byte_rows, spaced):
+            for max_words in (0, 3):
+                got = nv.wordpiece_tokenize(dev(nv, host), dvoc, max_words).to_host()
+                assert_same(got, orc.wordpiece_tokenize(host, ovoc, max_words, nthreads=8), f"max_words={max_words}")
+    assert orc.wordpiece_tokenize(one_byte_rows, ovoc, 0, nthreads=8).child.size == n
+
+
 def test_wordpiece_utf8_vs_oracle(nv, orc):
     rng = np.random.default_rng(99)
     base = list("abcdeé漢字ñ語😀")
