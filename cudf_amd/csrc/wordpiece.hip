@@ -705,19 +705,38 @@ struct ShortWord {
   }
 };
 
-// ------------------------------------------------------------------ the tile pass
+// ------------------------------------------------------------------ the passes
 // The column's bytes, from the 16-byte aligned address at or below its first byte, are cut into tiles of TILE
-// bytes without regard to rows; kRangeTiles consecutive tiles form a range.  A wavefront takes one range at a
-// time and walks its tiles in order, so that the rows that start in them are met in order too.
+// bytes without regard to rows; kRangeTiles consecutive tiles form a range.
+//   * word pass: a wavefront takes one range at a time and walks its tiles in order, so that the rows that start in
+//     them are met in order too.  Per tile: find the words, look each one up whole.  Every word gets one slot of the
+//     range's part of the word arena, in order: its token, or a marker with the index of its entry in the queue of
+//     words that are not in the vocabulary as they stand.
+//   * out-of-vocabulary pass: one lane per queued word; the result takes the place of the queue entry.
+//   * emit pass: a wavefront per range expands the word slots into the tokens and gives every row that starts in the
+//     range its list offset.
 constexpr int kRangeTiles    = 16;
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
-constexpr uint32_t kQueueCap = 256;  // out-of-vocabulary words that wait in LDS
-constexpr uint32_t kTokCap   = 256;  // their tokens
-// lds.word[k] after its word has been looked up: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or
-//   kOovMark | count << 16 | index of its tokens in lds.tokens          (1 <= count <= kOovKeep), or
-//   kOovMark | kOovRedo | count << 21 | length << 13 | start            (tokens not kept: tokenized again when written)
+constexpr uint32_t kQueueChunk = 256;  // queue entries a wavefront of the word pass reserves at a time
+// A word slot: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or kOovMark | index of the word's queue entry
+// (never 0xFFFFFFFF: the queue has fewer than 2^31 - 1 entries).
 constexpr uint32_t kOovMark = 0x80000000u;
-constexpr uint32_t kOovRedo = 0x40000000u;
+
+// A queued word (32 bytes).  The out-of-vocabulary pass puts the word's result in its place: up to kOovKeep tokens and
+// their number; for a word with more tokens, only the number (the emit pass tokenizes it again, into place, from where
+// and how long the word is, which stay).
+struct OovEntry {
+  uint32_t head[4];    // the word's first 16 bytes, zero padded: most words are tokenized without reading the chars again
+  uint32_t len_flags;  // bytes in the word (1..199) | kUnprobed; 0: an unused entry
+  uint32_t range;      // the range the word begins in
+  uint32_t coord[2];   // coordinate of its first byte (low, high)
+};
+struct OovResult {
+  int32_t tok[kOovKeep];  // count <= kOovKeep: the tokens.  More: tok[4..6] = len_flags, range, coord[0] of the entry; tok[3] = coord[1]
+  uint32_t count;
+};
+static_assert(sizeof(OovEntry) == 32 && sizeof(OovResult) == 32, "a queue record is two 16-byte stores");
+constexpr uint32_t kUnprobed = 0x100u;  // the word has not been looked up whole (more than 16 bytes; a key that may have been carried past its bucket)
 
 template <int TILE>
 struct TileLds {
@@ -728,10 +747,7 @@ struct TileLds {
   uint32_t prefix[kBlocks + 1];               // word starts before the block | word ends before the block << 16
   static constexpr uint32_t kWordCap = TILE / 4;
   uint32_t word_guard[1];                     // (takes the end of the word that ran into the tile)
-  uint32_t word[kWordCap];                    // per word: start | end << 16, then its token (see kOovMark), then the tokens before it
-  uint32_t tokens[kTokCap];
-  uint16_t queue[kQueueCap];
-  uint32_t tok_used;                          // tokens kept in `tokens`
+  uint32_t word[kWordCap];                    // per word: start | end << 16
 };
 
 struct TileArgs {
@@ -744,13 +760,17 @@ struct TileArgs {
   uint32_t cbeg;           // coordinate of the view's first byte (0..15)
   uint32_t nranges;
   int32_t max_words;
-  uint32_t range_cap;      // arena slots of a range
+  uint32_t range_cap;      // word slots of a range
   const uint32_t* range_first_row;
-  uint32_t* arena;         // tokens of range g from arena[g * range_cap], densely, in order
-  uint32_t* range_count;   // tokens of range g
-  int32_t* offsets_out;    // per row: tokens of its range before the row
+  uint32_t* arena;         // the word slots of range g from arena[g * range_cap], densely, in order
+  uint32_t* range_words;   // words of range g
+  uint32_t* range_tokens;  // tokens of range g (here: of its words that are in the vocabulary; the next pass adds the others')
+  int32_t* offsets_out;    // per row: words of its range before the row
+  OovEntry* queue;
+  uint32_t queue_cap;
+  uint32_t* queue_size;    // entries reserved so far
   uint32_t* counter;       // next range to hand out
-  uint32_t* overflow;      // set when a range has more tokens than range_cap
+  uint32_t* overflow;      // set when a range has more words than range_cap
 };
 
 __device__ __forceinline__ void wave_lds_sync()
@@ -796,14 +816,15 @@ __device__ __forceinline__ uint32_t count_word_starts(const uint4* abase, int64_
   return total;
 }
 
-// range_first_row[g] = the first row (0..rows) that starts at or after the first byte of range g
+// range_first_row[g] = the first row (0..rows) that starts at or after the first byte of range g; [nranges] = rows
 __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32_t cbeg, int64_t range_bytes, uint32_t nranges,
                                        uint32_t* __restrict__ range_first_row)
 {
   uint32_t const g = blockIdx.x * blockDim.x + threadIdx.x;
-  if (g >= nranges) return;
+  if (g > nranges) return;
   int64_t const target = static_cast<int64_t>(g) * range_bytes;
   uint32_t lo = 0, hi = static_cast<uint32_t>(col.size);
+  if (g == nranges) lo = hi;
   while (lo < hi) {
     uint32_t const mid = lo + ((hi - lo) >> 1);
     if (col.off(mid) - first_offset + cbeg < target) lo = mid + 1;
@@ -812,12 +833,6 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
   range_first_row[g] = lo;
 }
 
-// One tile at a time per wavefront: stage its bytes (and the 256 after it) in LDS; mark the row starts in it; find
-// word starts and ends (lanes <-> 16-byte blocks: spaces by SWAR, row starts as extra separators); with a word limit,
-// drop the words past each row's limit; list the words (word k pairs start k with end k); look all of them up (lanes
-// <-> words, one probe each); tokenize the ones that are not in the vocabulary (lanes <-> such words, a lane that
-// finishes takes the next one); then place the tokens (a wave scan of the words' token counts) and write them to the
-// range's arena, and give every row that starts in the tile the number of tokens before it.
 #ifdef WP_PHASE_TIMING
 #define WP_PHASE(i)                                         \
   {                                                         \
@@ -831,8 +846,13 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
 #define WP_PHASE(i)
 #endif
 
+// One tile at a time per wavefront: stage its bytes (and the 256 after it) in LDS; mark the row starts in it; find
+// word starts and ends (lanes <-> 16-byte blocks: spaces by SWAR, row starts as extra separators); with a word limit,
+// drop the words past each row's limit; list the words (word k pairs start k with end k); look all of them up (lanes
+// <-> words, one probe each) and write their slots; give every row that starts in the tile the number of words of the
+// range before it.
 template <int TILE, bool IS64, bool LIMIT>
-__global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs a)
+__global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs a)
 {
 #ifdef WP_PHASE_TIMING
   uint64_t phase_t[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -843,8 +863,6 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
   constexpr uint32_t kWordCap = TileLds<TILE>::kWordCap;
   static_assert(kBlocks % kWave == 0, "whole wavefronts of blocks");
   __shared__ TileLds<TILE> lds_all[kTokWaves];
-  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
-  __shared__ int32_t first_ids[512];
   TileLds<TILE>& lds  = lds_all[threadIdx.x / kWave];
   int const lane      = lane_id();
   uint32_t const rows = static_cast<uint32_t>(a.col.size);
@@ -862,8 +880,7 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
   };
   const uint8_t* const lds_byte = reinterpret_cast<const uint8_t*>(lds.bytes);
   uint16_t* const word16        = reinterpret_cast<uint16_t*>(lds.word);
-  for (int i = threadIdx.x; i < 512; i += kTokThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
-  __syncthreads();
+  uint32_t q_pos = 0, q_lim = 0;  // this wavefront's reserved queue entries [q_pos, q_lim)
 
   for (;;) {
     uint32_t range = 0;
@@ -873,7 +890,8 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
     int64_t t           = static_cast<int64_t>(range) * kRangeTiles;
     int64_t const t_end = min(t + kRangeTiles, a.ntiles);
     uint32_t r_cur      = a.range_first_row[range];
-    uint32_t cursor     = 0;  // tokens of this range so far
+    uint32_t cursor     = 0;  // words of this range so far
+    uint32_t known      = 0;  // of them, in the vocabulary (or too long: one unknown token each)
     uint32_t open_left  = 0;  // words the row that runs into the tile may still have (with a word limit)
     uint32_t* const region = a.arena + static_cast<int64_t>(range) * a.range_cap;
     bool spill             = false;
@@ -885,27 +903,43 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
       open_left           = cap - min(cap, used);
     }
 
+    // the bytes of a tile, the 16 before them and the 256 after them, as 16-byte blocks: block j of lane l is l - 1 + 64 j
+    constexpr int kStageLoads = (kBlocks + kOverBlocks + 1 + kWave - 1) / kWave;
+    uint4 ahead[kStageLoads];
+    auto request_tile = [&](int64_t tile) {
+      int64_t const tile_begin = tile * TILE;
+#pragma unroll
+      for (int i = 0; i < kStageLoads; ++i) {
+        int64_t const g0 = tile_begin + 16 * (lane - 1 + i * kWave);
+        ahead[i]         = make_uint4(0u, 0u, 0u, 0u);
+        if (g0 + 16 > cbeg && g0 < cend) ahead[i] = load_stream(a.abase + (g0 >> 4));
+      }
+    };
+    request_tile(t);
     for (; t < t_end; ++t) {
       int64_t const tb     = t * TILE;
       bool const last_tile = t + 1 == a.ntiles;
       bool const edge      = tb < 16 + cbeg || tb + TILE + 16 * kOverBlocks > cend;  // some staged byte lies outside the view
 
-      // ---- stage the bytes
-      for (int j = lane - 1; j < kBlocks + kOverBlocks; j += kWave) {
-        int64_t const g0 = tb + 16 * j;
-        uint4 v          = make_uint4(0u, 0u, 0u, 0u);
-        if (!edge || (g0 + 16 > cbeg && g0 < cend)) v = load_stream(a.abase + (g0 >> 4));
-        *reinterpret_cast<uint4*>(&lds.bytes[4 * (j + 1)]) = v;
+      // ---- stage the bytes (requested while the tile before was being worked on), and request the next tile's
+#pragma unroll
+      for (int i = 0; i < kStageLoads; ++i) {
+        int const j = lane - 1 + i * kWave;
+        if (j < kBlocks + kOverBlocks) *reinterpret_cast<uint4*>(&lds.bytes[4 * (j + 1)]) = ahead[i];
       }
+      if (t + 1 < t_end) request_tile(t + 1);
       for (int i = lane; i < kBlocks + kOverBlocks + 1; i += kWave) lds.bound[i] = 0;
       wave_lds_sync();
       WP_PHASE(0)
 
       // ---- the rows that start in the tile: [r_first, r_end)
       uint32_t const r_first = r_cur;
+      int64_t crow           = 0;  // where row r_first + lane begins (kept for the passes over the rows below)
       for (;;) {
         uint32_t const r = r_cur + lane;
-        int64_t const p  = r <= rows ? coord(r) - tb : std::numeric_limits<int64_t>::max();
+        int64_t const c  = r <= rows ? coord(r) : std::numeric_limits<int64_t>::max();
+        int64_t const p  = r <= rows ? c - tb : c;
+        if (r_cur == r_first) crow = c;
         bool const in    = r < rows && (last_tile || p < TILE);
         if (p < TILE + 16 * kOverBlocks) atomicOr(&lds.bound[p >> 4], 1u << (p & 15));
         uint32_t const n = static_cast<uint32_t>(__builtin_popcountll(ballot64(in)));
@@ -918,19 +952,12 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
 
       // ---- word starts and ends
       uint32_t nw = 0, ne = 0, inside0 = 0;  // words that start in the tile, words that end in it, the tile begins inside a word
-      bool ascii = false;                    // no staged byte has bit 7 set
       {
         uint32_t base = 0;
-        uint32_t seen = 0;
-        if (lane < kOverBlocks) {
-          uint4 const v = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (kBlocks + lane + 1)]);
-          seen          = v.x | v.y | v.z | v.w;
-        }
 #pragma unroll
         for (int s = 0; s < kSubs; ++s) {
           int const b     = s * kWave + lane;
           uint4 const v   = *reinterpret_cast<const uint4*>(&lds.bytes[4 * (b + 1)]);
-          seen |= v.x | v.y | v.z | v.w;
           uint32_t sp     = space_mask16(v);
           uint32_t before = lds_byte[16 + 16 * b - 1] == 0x20u, after = lds_byte[16 + 16 * b + 16] == 0x20u;
           if (edge) {
@@ -952,9 +979,8 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
           base += wave_bcast(incl, kWave - 1);
         }
         if (lane == 0) lds.prefix[kBlocks] = base;
-        nw    = base & 0xFFFFu;
-        ne    = base >> 16;
-        ascii = ballot64((seen & 0x80808080u) != 0) == 0;
+        nw = base & 0xFFFFu;
+        ne = base >> 16;
       }
       wave_lds_sync();
       WP_PHASE(2)
@@ -988,8 +1014,12 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
         };
         for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
           uint32_t const r = r_first + i + lane;
+          // (the first 64 rows' beginnings are at hand; a row ends where the next begins)
+          int64_t c_next = static_cast<int64_t>((static_cast<uint64_t>(static_cast<uint32_t>(__shfl_down(static_cast<int>(static_cast<uint64_t>(crow) >> 32), 1))) << 32) |
+                                                static_cast<uint32_t>(__shfl_down(static_cast<int>(static_cast<uint32_t>(crow)), 1)));
           if (r < r_end) {
-            int64_t const c0 = coord(r), c1 = coord(r + 1);
+            int64_t const c0 = i == 0 ? crow : coord(r);
+            int64_t const c1 = i == 0 && lane < kWave - 1 ? c_next : coord(r + 1);
             if (c1 > c0) {
               int64_t const p = c0 - tb, e = c1 - tb;  // (p < TILE: the rows past the last tile's end are empty)
               uint32_t const cap = word_cap(r, c1 - c0);
@@ -1000,13 +1030,15 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
           }
         }
         // the row that runs into the tile
-        int64_t const e0   = r_first < r_end ? coord(r_first) - tb : static_cast<int64_t>(TILE);
+        int64_t const e0   = r_first < r_end ? static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(crow), 0)) - tb : static_cast<int64_t>(TILE);
         uint32_t const we0 = words_before(e0 < TILE ? static_cast<uint32_t>(e0) : static_cast<uint32_t>(TILE));
         if (lane == 0 && open_left < we0) drop_from(open_left, e0);
         // and the row that runs out of it
         if (r_first < r_end) {
           uint32_t const rl   = r_end - 1;
-          int64_t const c0    = coord(rl), c1 = coord(rl + 1);
+          uint32_t const il   = rl - r_first;
+          int64_t const c0    = il < kWave ? static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(crow), static_cast<int>(il))) : coord(rl);
+          int64_t const c1    = il + 1 < kWave ? static_cast<int64_t>(wave_bcast64(static_cast<uint64_t>(crow), static_cast<int>(il + 1))) : coord(rl + 1);
           int64_t const p     = c0 - tb;
           uint32_t const cap  = word_cap(rl, c1 - c0);
           uint32_t const used = nw - words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
@@ -1044,10 +1076,17 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
           wave_lds_sync();
         }
       }
+      // ---- the rows that start in the tile: the words of the range before them
+      for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
+        uint32_t const r = r_first + i + lane;
+        if (r < r_end) {
+          int64_t const p  = (i == 0 ? crow : coord(r)) - tb;
+          a.offsets_out[r] = static_cast<int32_t>(cursor + words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE)));
+        }
+      }
       WP_PHASE(3)
 
-      // ---- the words, at most kWordCap at a time (only a tile of one-byte rows has more)
-      uint32_t done = 0;  // tokens of this tile so far
+      // ---- the words, at most kWordCap at a time (only a tile of one- and two-byte rows or words has more)
       for (uint32_t w_lo = 0;; w_lo += kWordCap) {
         uint32_t const w_hi = min(nw, w_lo + kWordCap);
         uint32_t const nwc  = w_hi - w_lo;
@@ -1094,248 +1133,413 @@ __global__ void __launch_bounds__(kTokThreads, 5) wordpiece_tile_kernel(TileArgs
           }
           if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
         }
-        if (lane == 0) lds.tok_used = 0;
         wave_lds_sync();
         WP_PHASE(4)
 
         // ---- look the words up; the ones that are not in the vocabulary, or not decided here, go to the queue
-        uint32_t* const uw = lds.word;
-        for (uint32_t k0 = 0;;) {
-          uint32_t qn = 0;
-          while (k0 < nwc && qn + kWave <= kQueueCap) {
-            uint32_t const k   = k0 + lane;
-            bool const active  = k < nwc;
-            uint32_t const rec = uw[active ? k : 0u];
-            uint32_t const s   = rec & 0xFFFFu;
-            uint32_t const wl  = (rec >> 16) - s + 1u;
-            // straight-line code: every lane reads a bucket (of whatever its first bytes are), and what it makes of it
-            // depends on the word's length afterwards; only a key of 9 to 16 bytes with the right tag needs a second
-            // read, of the key's bytes
-            TileWord const tw{lds.bytes, 16u + s};
-            uint32_t head[4];
-            tw.head16(head);
-            uint32_t const wl16 = min(wl, 16u);
-            trim_key8(wl16, head[0], head[1]);
-            trim_key8(wl16 > 8 ? wl16 - 8u : 0u, head[2], head[3]);
-            Probe pr;
-            pr.k0             = head[0];
-            pr.k1             = head[1];
-            uint32_t const h1 = key_hash_block(key_hash_init(wl16), pr.k0, pr.k1);
-            uint32_t const h2 = key_hash_block(h1, head[2], head[3]);
-            uint32_t const h  = wl16 > 8 ? h2 : h1;
-            uint32_t bk;
-            pr.want   = slot_word0(h, 0, wl16, &bk);
-            pr.fp     = carried_bit(h);
-            pr.bucket = bk & table.bucket_mask;
-            uint4 const s0 = table.slots[2 * pr.bucket];
-            uint4 const s1 = table.slots[2 * pr.bucket + 1];
-            int32_t id  = kNone;
-            uint32_t vd = verdict(pr, s0, s1, wl16, &id);
-            if (vd == 2u && wl > 8 && wl <= 16) vd = verdict_16(table, pr, s0, s1, head, &id);
-            bool const too_long = wl >= kMaxWord;  // wordpiece_tokenize.cu:442-445, 738-741: one unknown token
-            bool const found    = wl <= 16 && vd == 1u;
-            // 1: not in the vocabulary; 2: not decided here (more than 16 bytes; a key that may have been carried past its bucket)
-            uint32_t const defer = !active || too_long || found ? 0u : (wl > 16 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
-            if (active && (too_long || found)) uw[k] = too_long ? static_cast<uint32_t>(table.unk_id) : static_cast<uint32_t>(id);
-            uint64_t const mm = ballot64(defer != 0);
-            if (defer != 0) lds.queue[qn + lanes_below(mm)] = static_cast<uint16_t>(k | (defer == 2u ? 0x8000u : 0u));
-            qn += static_cast<uint32_t>(__builtin_popcountll(mm));
-            k0 += kWave;
-          }
-          WP_PHASE(5)
-          if (qn > 0) {
-            wave_lds_sync();
-            // ---- the queued words, one lane each; a lane that finishes stores its result and takes the next word.
-            // Words of up to 16 bytes run in registers; longer ones are set aside (queue[0 .. n_long)) for the loop below.
-            uint32_t q_next = 0, n_long = 0;
-            ShortWord sw;
-            sw.done   = true;
-            sw.count  = 0;
-            bool busy = false;
-            uint32_t mine = 0;  // my word
-            int32_t tok[kOovKeep];
-            auto keep_token = [&](uint32_t j, int32_t id) {
-#pragma unroll
-              for (int i = 0; i < kOovKeep; ++i)
-                if (j == static_cast<uint32_t>(i)) tok[i] = id;
-            };
-            for (;;) {
-              if (busy && sw.done) {
-                // my word is finished: its tokens go to lds.tokens (if there are at most kOovKeep, and room)
-                uint32_t const cnt  = sw.count;
-                uint32_t const keep = cnt <= kOovKeep ? cnt : 0u;
-                uint32_t const off  = keep > 0 ? atomicAdd(&lds.tok_used, keep) : 0u;
-                if (keep > 0 && off + keep <= kTokCap) {
-#pragma unroll
-                  for (int i = 0; i < kOovKeep; ++i)
-                    if (static_cast<uint32_t>(i) < keep) lds.tokens[off + i] = static_cast<uint32_t>(tok[i]);
-                  uw[mine] = kOovMark | (cnt << 16) | off;
-                } else {
-                  uint32_t const rec = uw[mine];
-                  uint32_t const s   = rec & 0xFFFFu;
-                  uw[mine]           = kOovMark | kOovRedo | (cnt << 21) | (((rec >> 16) - s + 1u) << 13) | s;
-                }
-                busy = false;
-              }
-              uint32_t const left = qn - q_next;
-              if (left > 0) {
-                uint64_t const idle = ballot64(!busy);
-                if (idle != 0) {
-                  uint32_t const rank = lanes_below(idle);
-                  bool is_long        = false;
-                  uint32_t k          = 0;
-                  if (!busy && rank < left) {
-                    k                  = lds.queue[q_next + rank];
-                    uint32_t const rec = uw[k & 0x7FFFu];
-                    uint32_t const s   = rec & 0xFFFFu;
-                    uint32_t const wl  = (rec >> 16) - s + 1u;
-                    if (wl <= 16) {
-                      TileWord const tw{lds.bytes, 16u + s};
-                      uint32_t head[4];
-                      tw.head16(head);
-                      trim_key8(wl, head[0], head[1]);
-                      trim_key8(wl > 8 ? wl - 8u : 0u, head[2], head[3]);
-                      sw.begin(table, first_ids, head, wl, (k & 0x8000u) == 0, ascii);
-                      busy = true;
-                      mine = k & 0x7FFFu;
-                    } else {
-                      is_long = true;
-                    }
-                  }
-                  q_next += min(static_cast<uint32_t>(__builtin_popcountll(idle)), left);
-                  uint64_t const lm = ballot64(is_long);
-                  if (lm != 0) {
-                    wave_lds_sync();  // (the queue entries just read lie at or past n_long)
-                    if (is_long) lds.queue[n_long + lanes_below(lm)] = static_cast<uint16_t>(k);
-                    n_long += static_cast<uint32_t>(__builtin_popcountll(lm));
-                  }
-                }
-              }
-              if (ballot64(busy) == 0) {
-                if (q_next >= qn) break;
-                continue;
-              }
-#ifdef WP_PHASE_TIMING
-              uint64_t const t_before = __builtin_amdgcn_s_memtime();
-#endif
-              if (busy && !sw.done) sw.step(table, first_ids, keep_token);
-#ifdef WP_PHASE_TIMING
-              phase_t[9] += __builtin_amdgcn_s_memtime() - t_before;
-#endif
-            }
-            if (n_long > 0) {
-              wave_lds_sync();
-              for (uint32_t base = 0; base < n_long; base += kWave) {
-                if (base + lane < n_long) {
-                  uint32_t const k   = lds.queue[base + lane] & 0x7FFFu;  // (words of more than 16 bytes have not been looked up whole)
-                  uint32_t const rec = uw[k];
-                  uint32_t const s   = rec & 0xFFFFu;
-                  uint32_t const wl  = (rec >> 16) - s + 1u;
-                  uint32_t const cnt = count_oov_tokens(table, lds.bytes, 16u + s, wl);
-                  uw[k]              = kOovMark | kOovRedo | (cnt << 21) | (wl << 13) | s;
-                }
-              }
-            }
-            wave_lds_sync();
-            WP_PHASE(6)
-          }
-          if (k0 >= nwc) break;
-        }
-
-        // ---- place and write the tokens
-        for (uint32_t j0 = 0; j0 < nwc; j0 += kWave) {
-          uint32_t const k   = j0 + lane;
+        if (cursor + nwc > a.range_cap) spill = true;
+        for (uint32_t k0 = 0; k0 < nwc; k0 += kWave) {
+          uint32_t const k   = k0 + lane;
           bool const active  = k < nwc;
-          uint32_t const v   = active ? uw[k] : 0u;
-          bool const marked  = active && (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
-          bool const redo    = marked && (v & kOovRedo) != 0;
-          uint32_t const cnt = !active ? 0u : !marked ? 1u : redo ? (v >> 21) & 0xFFu : (v >> 16) & 0xFFu;
-          uint32_t const incl = wave_inclusive_scan(cnt);
-          uint32_t const ex   = incl - cnt;
-          uint32_t const tot  = wave_bcast(incl, kWave - 1);
-          if (cursor + done + tot > a.range_cap) spill = true;
-          if (!spill) {
-            uint32_t* const dst = region + (cursor + done + ex);
-            if (ballot64(redo) != 0 && redo) {
-              // tokens that were not kept (more than kOovKeep, a word of more than 16 bytes, no room left in LDS):
-              // tokenized again, into place
-              write_oov_tokens(table, reinterpret_cast<const uint8_t*>(a.abase) + tb + (v & 0x1FFFu), (v >> 13) & 0xFFu, dst, cnt);
+          uint32_t const rec = lds.word[active ? k : 0u];
+          uint32_t const s   = rec & 0xFFFFu;
+          uint32_t const wl  = (rec >> 16) - s + 1u;
+          // straight-line code: every lane reads a bucket (of whatever its first bytes are), and what it makes of it
+          // depends on the word's length afterwards; only a key of 9 to 16 bytes with the right tag needs a second
+          // read, of the key's bytes
+          TileWord const tw{lds.bytes, 16u + s};
+          uint32_t head[4];
+          tw.head16(head);
+          uint32_t const wl16 = min(wl, 16u);
+          trim_key8(wl16, head[0], head[1]);
+          trim_key8(wl16 > 8 ? wl16 - 8u : 0u, head[2], head[3]);
+          Probe pr;
+          pr.k0             = head[0];
+          pr.k1             = head[1];
+          uint32_t const h1 = key_hash_block(key_hash_init(wl16), pr.k0, pr.k1);
+          uint32_t const h2 = key_hash_block(h1, head[2], head[3]);
+          uint32_t const h  = wl16 > 8 ? h2 : h1;
+          uint32_t bk;
+          pr.want   = slot_word0(h, 0, wl16, &bk);
+          pr.fp     = carried_bit(h);
+          pr.bucket = bk & table.bucket_mask;
+          uint4 const s0 = table.slots[2 * pr.bucket];
+          uint4 const s1 = table.slots[2 * pr.bucket + 1];
+          int32_t id  = kNone;
+          uint32_t vd = verdict(pr, s0, s1, wl16, &id);
+          if (vd == 2u && wl > 8 && wl <= 16) vd = verdict_16(table, pr, s0, s1, head, &id);
+          bool const too_long = wl >= kMaxWord;  // wordpiece_tokenize.cu:442-445, 738-741: one unknown token
+          bool const found    = wl <= 16 && vd == 1u;
+          // 1: not in the vocabulary; 2: not decided here (more than 16 bytes; a key that may have been carried past its bucket)
+          uint32_t const defer = !active || too_long || found ? 0u : (wl > 16 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
+          uint32_t value       = too_long ? static_cast<uint32_t>(table.unk_id) : static_cast<uint32_t>(id);
+          uint64_t const mm    = ballot64(defer != 0);
+          if (mm != 0) {
+            uint32_t const nm   = static_cast<uint32_t>(__builtin_popcountll(mm));
+            uint32_t const room = q_lim - q_pos;  // left of the reserved entries: used up before the next ones are begun
+            uint32_t fresh      = 0;
+            if (nm > room) {
+              if (lane == 0) fresh = atomicAdd(a.queue_size, kQueueChunk);
+              fresh = wave_bcast(fresh, 0);
             }
-            if (active && !redo) {
-              uint32_t const off = v & 0xFFFFu;
-              dst[0]             = marked ? lds.tokens[off] : v;
-#pragma unroll
-              for (uint32_t j = 1; j < kOovKeep; ++j) {
-                if (ballot64(marked && j < cnt) == 0) break;
-                if (marked && j < cnt) dst[j] = lds.tokens[off + j];
+            if (defer != 0) {
+              uint32_t const rank = lanes_below(mm);
+              uint32_t const q    = rank < room ? q_pos + rank : fresh + (rank - room);
+              if (q < a.queue_cap) {
+                int64_t const at = tb + s;
+                uint4* const dst = reinterpret_cast<uint4*>(a.queue + q);
+                store_stream(dst, make_uint4(head[0], head[1], head[2], head[3]));
+                store_stream(dst + 1, make_uint4(wl | (defer == 2u ? kUnprobed : 0u), range, static_cast<uint32_t>(at), static_cast<uint32_t>(static_cast<uint64_t>(at) >> 32)));
               }
+              value = kOovMark | q;
+            }
+            if (nm > room) {
+              q_pos = fresh + (nm - room);
+              q_lim = fresh + kQueueChunk;
+            } else {
+              q_pos += nm;
             }
           }
-          if (active) uw[k] = done + ex;
-          done += tot;
+          known += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && defer == 0)));
+          if (active && !spill) region[cursor + k] = value;
         }
+        cursor += nwc;
         wave_lds_sync();
-        WP_PHASE(7)
-
-        // ---- the rows that start in the tile at one of these words (or, with the tile's last words, after them): the
-        // tokens of the range before them
-        for (uint32_t i = 0; r_first + i < r_end; i += kWave) {
-          uint32_t const r = r_first + i + lane;
-          if (r < r_end) {
-            int64_t const p  = coord(r) - tb;
-            uint32_t const k = words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE));
-            if (k >= w_lo && k < w_hi) a.offsets_out[r] = static_cast<int32_t>(cursor + uw[k - w_lo]);
-            else if (k == nw && w_hi == nw) a.offsets_out[r] = static_cast<int32_t>(cursor + done);
-          }
-        }
-        wave_lds_sync();
+        WP_PHASE(5)
         if (w_hi == nw) break;
       }
-      cursor += done;
-      WP_PHASE(8)
     }
     if (lane == 0) {
-      a.range_count[range] = cursor;
+      a.range_words[range]  = cursor;
+      a.range_tokens[range] = known;
       if (spill) *a.overflow = 1u;
     }
   }
+  // the reserved entries that no word took
+  for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
+    if (q < a.queue_cap) a.queue[q].len_flags = 0;
 #ifdef WP_PHASE_TIMING
   if (lane == 0)
-    for (int i = 0; i < 10; ++i) atomicAdd(reinterpret_cast<unsigned long long*>(a.overflow + 3) + i, static_cast<unsigned long long>(phase_t[i]));
+    for (int i = 0; i < 10; ++i) atomicAdd(reinterpret_cast<unsigned long long*>(a.overflow + 7) + i, static_cast<unsigned long long>(phase_t[i]));
 #endif
 }
 
-struct RangeCountOf {
+// ------------------------------------------------------------------ out-of-vocabulary pass
+// One lane per queued word, and a lane that finishes its word stores the result and takes the next one.  A wavefront
+// takes kOovBlock queue entries at a time (one atomic), brings them into LDS 64 at a time with whole-record reads (the
+// next 64 are requested while these are worked on) and lets its idle lanes take entries from there every trip.  Words
+// of up to 16 bytes, whole in their queue record, run in registers; the few longer ones are set aside and done, one
+// lane each, by the general state machine over the chars in memory, 64 and more at a time or at the end.
+constexpr uint32_t kOovBlock = 256;
+constexpr int kRefillAt      = 32;
+constexpr int kOovWaves      = 4;
+constexpr int kOovThreads    = kOovWaves * kWave;
+struct OovLds {
+  alignas(16) uint4 staged[kWave][2];  // 64 queue entries
+};
+
+__global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTable table, const uint4* abase, OovEntry* __restrict__ queue,
+                                                                    const uint32_t* __restrict__ queue_size, uint32_t queue_cap,
+                                                                    uint32_t* __restrict__ range_tokens, uint32_t* __restrict__ counter,
+                                                                    uint32_t* __restrict__ longer, uint32_t* __restrict__ longer_count)
+{
+  __shared__ OovLds lds_all[kOovWaves];
+  __shared__ int32_t first_ids[512];  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
+  for (int i = threadIdx.x; i < 512; i += kOovThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
+  __syncthreads();
+  if (*queue_size > queue_cap) return;  // the queue was too small: the host repeats the passes with a larger one
+  uint32_t const total = *queue_size;
+  OovLds& lds          = lds_all[threadIdx.x / kWave];
+  int const lane       = lane_id();
+
+  ShortWord sw;
+  sw.done   = true;
+  sw.count  = 0;
+  bool busy = false;
+  uint32_t mine = 0, mine_range = 0;  // my word's queue entry and range
+  uint32_t acc_range = 0, acc_count = 0;
+  int32_t tok[kOovKeep];
+  auto keep_token = [&](uint32_t j, int32_t id) {
+#pragma unroll
+    for (int i = 0; i < kOovKeep; ++i)
+      if (j == static_cast<uint32_t>(i)) tok[i] = id;
+  };
+  // the result takes the place of the entry
+  auto deliver = [&](uint32_t q, uint32_t range, uint32_t count, uint4 const& entry_tail) {
+    uint4* const dst = reinterpret_cast<uint4*>(queue + q);
+    if (count <= kOovKeep) {
+      store_stream(dst, make_uint4(static_cast<uint32_t>(tok[0]), static_cast<uint32_t>(tok[1]), static_cast<uint32_t>(tok[2]), static_cast<uint32_t>(tok[3])));
+      store_stream(dst + 1, make_uint4(static_cast<uint32_t>(tok[4]), static_cast<uint32_t>(tok[5]), static_cast<uint32_t>(tok[6]), count));
+    } else {
+      // more tokens than a record keeps: where and how long the word is stays, for the emit pass
+      store_stream(dst, make_uint4(0u, 0u, 0u, entry_tail.w));
+      store_stream(dst + 1, make_uint4(entry_tail.x, entry_tail.y, entry_tail.z, count));
+    }
+    // the tokens of a range are added up per lane as long as its words are of the same range (the queue holds the words
+    // of a range side by side): an atomic per word is what this pass would spend a third of its time on
+    if (range != acc_range) {
+      if (acc_count != 0) atomicAdd(&range_tokens[acc_range], acc_count);
+      acc_range = range;
+      acc_count = 0;
+    }
+    acc_count += count;
+  };
+  uint4 mine_tail = make_uint4(0u, 0u, 0u, 0u);  // the second half of my word's entry
+
+  // the queue entries being fetched: [f_base, f_base + f_n), one per lane; they come from the block [.., q_end) that
+  // this wavefront has taken, and a new block is taken when that one is used up
+  uint32_t next_fetch = 0, q_end = 0, f_base = 0, f_n = 0;
+  bool no_more = false;
+  uint4 pa = make_uint4(0u, 0u, 0u, 0u), pb = pa;
+  auto start_fetch = [&] {
+    f_n = 0;
+    if (next_fetch >= q_end && !no_more) {
+      uint32_t block = 0;
+      if (lane == 0) block = atomicAdd(counter, 1u);
+      block                  = wave_bcast(block, 0);
+      uint64_t const b_begin = static_cast<uint64_t>(block) * kOovBlock;
+      if (b_begin >= total) {
+        no_more = true;
+      } else {
+        next_fetch = static_cast<uint32_t>(b_begin);
+        q_end      = static_cast<uint32_t>(min(b_begin + kOovBlock, static_cast<uint64_t>(total)));
+      }
+    }
+    if (next_fetch < q_end) {
+      f_base = next_fetch;
+      f_n    = min(static_cast<uint32_t>(kWave), q_end - next_fetch);
+      next_fetch += f_n;
+      if (static_cast<uint32_t>(lane) < f_n) {
+        const uint4* const src = reinterpret_cast<const uint4*>(queue + f_base + lane);
+        pa = load_stream(src);
+        pb = load_stream(src + 1);
+      }
+    }
+  };
+  uint32_t st_base = 0, st_next = 0, st_end = 0;  // the staged entries still to be taken are queue[st_base + st_next .. st_base + st_end)
+  start_fetch();
+  for (;;) {
+    // Lanes that have finished wait until kRefillAt of them are free (or nobody is working): storing results and
+    // taking new words is code that the whole wavefront runs through, whether for one lane or for sixty-four.
+    uint64_t const working = ballot64(busy && !sw.done);
+    if (kWave - __builtin_popcountll(working) >= kRefillAt || working == 0) {
+      if (busy && sw.done) {
+        deliver(mine, mine_range, sw.count, mine_tail);
+        busy = false;
+      }
+      if (st_next >= st_end && f_n > 0) {
+        // the staged entries are used up: the fetched ones take their place, and the next are requested
+        wave_lds_sync();
+        lds.staged[lane][0] = pa;
+        lds.staged[lane][1] = pb;
+        st_base = f_base;
+        st_next = 0;
+        st_end  = f_n;
+        wave_lds_sync();
+        start_fetch();
+      }
+      uint32_t const left = st_end - st_next;
+      if (left > 0) {
+        uint64_t const idle = ballot64(!busy);
+        if (idle != 0) {
+          uint32_t const rank = lanes_below(idle);
+          bool is_long        = false;
+          uint32_t at         = 0;
+          // no byte of any word taken now has bit 7 set: every position of theirs is a character boundary
+          bool const taking = !busy && rank < left;
+          uint4 const ha    = lds.staged[taking ? st_next + rank : 0u][0];
+          bool const ascii  = ballot64(taking && ((ha.x | ha.y | ha.z | ha.w) & 0x80808080u) != 0) == 0;
+          if (taking) {
+            at            = st_next + rank;
+            uint4 const a = ha, b = lds.staged[at][1];
+            uint32_t const wl = b.x & 0xFFu;
+            if (wl != 0) {  // (0: an entry that no word took)
+              if (wl <= 16) {
+                uint32_t const head[4] = {a.x, a.y, a.z, a.w};
+                sw.begin(table, first_ids, head, wl, (b.x & kUnprobed) == 0, ascii);
+                busy       = true;
+                mine       = st_base + at;
+                mine_range = b.y;
+                mine_tail  = b;
+              } else {
+                is_long = true;
+              }
+            }
+          }
+          st_next += min(static_cast<uint32_t>(__builtin_popcountll(idle)), left);
+          uint64_t const lm = ballot64(is_long);
+          if (lm != 0) {
+            // words of more than 16 bytes: listed for the kernel that does those
+            uint32_t first = 0;
+            if (lane == 0) first = atomicAdd(longer_count, static_cast<uint32_t>(__builtin_popcountll(lm)));
+            first = wave_bcast(first, 0);
+            if (is_long) longer[first + lanes_below(lm)] = st_base + at;
+          }
+        }
+      }
+    }
+    bool const drained = st_next >= st_end && f_n == 0;
+    if (ballot64(busy && !sw.done) == 0) {
+      if (drained && ballot64(busy) == 0) break;
+      continue;
+    }
+    if (busy && !sw.done) sw.step(table, first_ids, keep_token);
+  }
+  if (acc_count != 0) atomicAdd(&range_tokens[acc_range], acc_count);
+}
+
+// The queued words of more than 16 bytes, which the kernel above has listed: one lane per word, the general state
+// machine over the chars in memory.
+__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(VocabTable table, const uint4* abase, OovEntry* __restrict__ queue,
+                                                                         const uint32_t* __restrict__ queue_size, uint32_t queue_cap,
+                                                                         const uint32_t* __restrict__ longer, const uint32_t* __restrict__ longer_count,
+                                                                         uint32_t* __restrict__ range_tokens)
+{
+  if (*queue_size > queue_cap) return;  // (see wordpiece_oov_kernel)
+  uint32_t const n = *longer_count;
+  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
+    uint32_t const q   = longer[i];
+    OovEntry const e   = queue[q];
+    uint32_t const wl  = e.len_flags & 0xFFu;
+    int64_t const at   = static_cast<int64_t>((static_cast<uint64_t>(e.coord[1]) << 32) | e.coord[0]);
+    int32_t tok[kOovKeep];
+    uint32_t const cnt = tokenize_oov_word(table, GlobalWord{reinterpret_cast<const uint8_t*>(abase) + at}, wl, [&](uint32_t j, int32_t id) {
+#pragma unroll
+      for (int k = 0; k < kOovKeep; ++k)
+        if (j == static_cast<uint32_t>(k)) tok[k] = id;
+    });
+    uint4* const dst = reinterpret_cast<uint4*>(queue + q);
+    if (cnt <= kOovKeep) {
+      dst[0] = make_uint4(static_cast<uint32_t>(tok[0]), static_cast<uint32_t>(tok[1]), static_cast<uint32_t>(tok[2]), static_cast<uint32_t>(tok[3]));
+      dst[1] = make_uint4(static_cast<uint32_t>(tok[4]), static_cast<uint32_t>(tok[5]), static_cast<uint32_t>(tok[6]), cnt);
+    } else {
+      dst[0] = make_uint4(0u, 0u, 0u, e.coord[1]);
+      dst[1] = make_uint4(e.len_flags, e.range, e.coord[0], cnt);
+    }
+    atomicAdd(&range_tokens[e.range], cnt);
+  }
+}
+
+// ------------------------------------------------------------------ emit pass
+// A wavefront takes a range: walks its word slots 64 at a time, in order; a word from the queue has its tokens (or
+// their number) in its queue record; a wave scan of the token counts places the tokens, and every lane writes its own
+// word's.  The rows that start in the range (the word pass left each the number of the range's words before it) are
+// walked alongside: a row that begins at one of the 64 words gets that word's place as its list offset.
+__global__ void __launch_bounds__(kTokThreads, 8) wordpiece_emit_kernel(uint32_t nranges, const uint32_t* __restrict__ arena, uint32_t range_cap,
+                                                                     const uint32_t* __restrict__ range_words, const int64_t* __restrict__ range_base,
+                                                                     const uint32_t* __restrict__ range_first_row, OovEntry* __restrict__ queue,
+                                                                     int32_t* __restrict__ offsets, int32_t* __restrict__ child, uint32_t* __restrict__ counter,
+                                                                     uint32_t* __restrict__ again, uint32_t* __restrict__ again_count)
+{
+  int const lane = lane_id();
+  for (;;) {
+    uint32_t range = 0;
+    if (lane == 0) range = atomicAdd(counter, 1u);
+    range = wave_bcast(range, 0);
+    if (range >= nranges) break;
+    const uint32_t* const slots = arena + static_cast<int64_t>(range) * range_cap;
+    uint32_t const nwords       = range_words[range];
+    int64_t const base          = range_base[range];
+    int32_t* const dst0         = child + base;
+    uint32_t r_win              = range_first_row[range];  // the 64 rows being placed: r_win + lane, the first row_used of them done
+    uint32_t const r_end        = range_first_row[range + 1];
+    uint32_t row_used           = 0;
+    uint32_t done               = 0;  // tokens of the range so far
+    // the words of the range before my row
+    uint32_t row_k = r_win + lane < r_end ? static_cast<uint32_t>(offsets[r_win + lane]) : 0xFFFFFFFFu;
+    // three stages in flight: the slot two rounds ahead, the queue record of a word from the queue one round ahead, the
+    // round being written (the pass is bound by the latency of its reads)
+    auto load_slot = [&](uint32_t k) -> uint32_t { return k < nwords ? slots[k] : 0u; };
+    auto load_record = [&](uint32_t k, uint32_t v, uint4& ra, uint4& rb) {
+      if (k < nwords && (v & kOovMark) != 0 && v != 0xFFFFFFFFu) {
+        const uint4* const src = reinterpret_cast<const uint4*>(queue + (v & ~kOovMark));
+        ra = src[0];
+        rb = src[1];
+      }
+    };
+    uint32_t v_nxt = load_slot(lane), v_far = load_slot(kWave + lane);
+    uint4 a_nxt = make_uint4(0u, 0u, 0u, 0u), b_nxt = a_nxt;
+    load_record(lane, v_nxt, a_nxt, b_nxt);
+    for (uint32_t j0 = 0; j0 < nwords; j0 += kWave) {
+      uint32_t const k  = j0 + lane;
+      bool const active = k < nwords;
+      uint32_t const v  = v_nxt;
+      uint4 const ra = a_nxt, rb = b_nxt;
+      v_nxt = v_far;
+      load_record(k + kWave, v_nxt, a_nxt, b_nxt);
+      v_far = load_slot(k + 2 * kWave);
+      bool const marked   = active && (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
+      uint32_t const cnt  = !active ? 0u : marked ? rb.w : 1u;
+      uint32_t const incl = wave_inclusive_scan(cnt);
+      uint32_t const ex   = incl - cnt;
+      uint32_t const tot  = wave_bcast(incl, kWave - 1);
+      int32_t* const dst  = dst0 + done + ex;
+      bool const more     = marked && cnt > kOovKeep;
+      if (more) {
+        // more tokens than a record keeps (seldom): noted for wordpiece_retokenize_kernel, with the place of the word's
+        // first token in the child left in its record
+        uint32_t const q                 = v & ~kOovMark;
+        again[atomicAdd(again_count, 1u)] = q;
+        queue[q].head[0]                 = static_cast<uint32_t>(base + done + ex);
+      } else if (active) {
+        dst[0] = static_cast<int32_t>(marked ? ra.x : v);
+        if (ballot64(marked && cnt > 1u) != 0) {
+          if (marked && cnt > 1u) dst[1] = static_cast<int32_t>(ra.y);
+          if (marked && cnt > 2u) dst[2] = static_cast<int32_t>(ra.z);
+          if (ballot64(marked && cnt > 3u) != 0) {
+            if (marked && cnt > 3u) dst[3] = static_cast<int32_t>(ra.w);
+            if (marked && cnt > 4u) dst[4] = static_cast<int32_t>(rb.x);
+            if (marked && cnt > 5u) dst[5] = static_cast<int32_t>(rb.y);
+            if (marked && cnt > 6u) dst[6] = static_cast<int32_t>(rb.z);
+          }
+        }
+      }
+      // rows that begin at one of these words (or, in the last round, after the last word: the lanes past it
+      // hold the round's total)
+      for (;;) {
+        bool const mine  = lane >= static_cast<int>(row_used) && row_k < j0 + kWave;  // (row_k >= j0: the rows are in order)
+        uint32_t const e = static_cast<uint32_t>(__shfl(static_cast<int>(ex), static_cast<int>((row_k - j0) & 63u)));
+        if (mine) offsets[r_win + lane] = static_cast<int32_t>(base + done + e);
+        row_used += static_cast<uint32_t>(__builtin_popcountll(ballot64(mine)));
+        if (row_used < kWave) break;
+        // all 64 are placed: the next 64
+        r_win += kWave;
+        row_used = 0;
+        row_k    = r_win + lane < r_end ? static_cast<uint32_t>(offsets[r_win + lane]) : 0xFFFFFFFFu;
+      }
+      done += tot;
+    }
+    // the rows after the range's last word; after the last range's, the end of the last row
+    for (; r_win < r_end; r_win += kWave, row_used = 0)
+      if (lane >= static_cast<int>(row_used) && r_win + lane < r_end) offsets[r_win + lane] = static_cast<int32_t>(base + done);
+    if (range + 1 == nranges && lane == 0) offsets[r_end] = static_cast<int32_t>(base + done);
+  }
+}
+
+// The words that have more tokens than a queue record keeps (the emit pass has listed them in again[0 .. *again_count)
+// and left the index of each one's first token in the child in its record, beside where and how long the word is):
+// tokenized again, straight into place.  One lane per word; kept apart from the emit pass so that that is compiled for
+// its common case.
+__global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(VocabTable table, const uint4* abase, const OovEntry* __restrict__ queue,
+                                                                           const uint32_t* __restrict__ again, const uint32_t* __restrict__ again_count,
+                                                                           int32_t* __restrict__ child)
+{
+  uint32_t const n = *again_count;
+  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
+    OovEntry const e   = queue[again[i]];  // head[0] = place in the child, head[3] = coord[1], len_flags, range, coord[0] as they were; coord[1] = the count
+    uint32_t const cnt = e.coord[1];
+    int64_t const at   = static_cast<int64_t>((static_cast<uint64_t>(e.head[3]) << 32) | e.coord[0]);
+    int32_t* const d   = child + e.head[0];
+    tokenize_oov_word(table, GlobalWord{reinterpret_cast<const uint8_t*>(abase) + at}, e.len_flags & 0xFFu, [&](uint32_t j, int32_t id) {
+      if (j < cnt) d[j] = id;
+    });
+  }
+}
+
+struct RangeTokensOf {
   const uint32_t* counts;
   __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
 };
-
-// Blocks 0 .. nranges-1: the tokens of a range go from the arena to their place in the child.  The blocks after
-// them: every row's offset becomes absolute (the tokens before its range are added), and offsets[rows] the total.
-__global__ void __launch_bounds__(256) wordpiece_gather_kernel(ColView col, int64_t first_offset, uint32_t cbeg, int range_shift, uint32_t nranges,
-                                                               const uint32_t* __restrict__ arena, uint32_t range_cap,
-                                                               const uint32_t* __restrict__ range_count, const int64_t* __restrict__ range_base,
-                                                               int32_t* __restrict__ child, int32_t* __restrict__ offsets)
-{
-  if (blockIdx.x < nranges) {
-    uint32_t const g        = blockIdx.x;
-    const uint32_t* src     = arena + static_cast<int64_t>(g) * range_cap;
-    uint32_t* dst           = reinterpret_cast<uint32_t*>(child) + range_base[g];
-    uint32_t const n        = range_count[g];
-    for (uint32_t i = threadIdx.x; i < n; i += 256) dst[i] = src[i];
-    return;
-  }
-  int64_t const rows = col.size;
-  int64_t const r    = static_cast<int64_t>(blockIdx.x - nranges) * 256 + threadIdx.x;
-  if (r < rows) {
-    int64_t const c = col.off(r) - first_offset + cbeg;
-    uint32_t g      = static_cast<uint32_t>(c >> range_shift);
-    if (g >= nranges) g = nranges - 1;
-    offsets[r] += static_cast<int32_t>(range_base[g]);
-  } else if (r == rows) {
-    offsets[rows] = static_cast<int32_t>(range_base[nranges]);
-  }
-}
 
 // ------------------------------------------------------------------ vocabulary construction (host)
 struct HostSlot {
@@ -1654,8 +1858,6 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
 
   constexpr int kTile         = 2048;
   constexpr int64_t kRange    = static_cast<int64_t>(kTile) * kRangeTiles;
-  constexpr int kRangeShift   = 15;
-  static_assert((int64_t{1} << kRangeShift) == kRange, "a range is 2^kRangeShift bytes");
   const uint8_t* const first_byte = v.chars + first_offset;
   uint32_t const cbeg             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(first_byte) & 15u);
   int64_t const cend              = cbeg + (last_offset - first_offset);
@@ -1667,15 +1869,21 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   int device = 0, cus = 256;
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-  int per_cu = 0;
+  // persistent kernels: as many workgroups as can be resident at once
+  auto resident = [&](const void* kernel, int threads) -> int64_t {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 2;
+    return static_cast<int64_t>(per_cu) * cus;
+  };
   bool const is64  = input->offsets_is_int64 != 0;
   bool const limit = max_words_per_row > 0;
-  void (*const tile_kernel)(TileArgs) = is64 ? (limit ? wordpiece_tile_kernel<kTile, true, true> : wordpiece_tile_kernel<kTile, true, false>)
-                                             : (limit ? wordpiece_tile_kernel<kTile, false, true> : wordpiece_tile_kernel<kTile, false, false>);
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(tile_kernel), kTokThreads, 0) != hipSuccess || per_cu < 1)
-    per_cu = 2;
-  unsigned const tile_grid =
-    static_cast<unsigned>(std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, static_cast<int64_t>(per_cu) * cus));
+  void (*const word_kernel)(TileArgs) = is64 ? (limit ? wordpiece_word_kernel<kTile, true, true> : wordpiece_word_kernel<kTile, true, false>)
+                                             : (limit ? wordpiece_word_kernel<kTile, false, true> : wordpiece_word_kernel<kTile, false, false>);
+  unsigned const word_grid = static_cast<unsigned>(
+    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(word_kernel), kTokThreads)));
+  unsigned const oov_grid  = static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads));
+  unsigned const emit_grid = static_cast<unsigned>(
+    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
 
   TileArgs args{};
   args.col          = v;
@@ -1688,67 +1896,91 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   args.nranges      = nranges;
   args.max_words    = max_words_per_row;
 
+  // Word slots per range and queue entries.  A range of ordinary text has a word per five or six bytes, and about a
+  // word in forty of a large column is not in the vocabulary; the first attempt has room for five words per sixteen
+  // bytes and queues a word per 32 bytes.  A column with more (rows or words of a byte or two; text in another
+  // language than the vocabulary's) makes the attempt fail, and the second has what the first found to be needed:
+  // room for a word per byte, the exact number of queue entries.
+  uint32_t range_cap      = static_cast<uint32_t>(kRange * 5 / 16);
+  uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 5) + static_cast<uint64_t>(word_grid) * kTokWaves * kQueueChunk + 4096;
   uint64_t total = 0;
   for (int attempt = 0;; ++attempt) {
-    // Arena slots per range.  A range of ordinary text has a token per five or six bytes; the first attempt leaves
-    // room for three per eight.  A range with more (rows or words of a byte or two, words that fall apart into
-    // letters) makes the attempt fail, and the second has room for the most a range can give: a token per byte, plus
-    // those of a word that begins in its last bytes.
-    uint32_t const range_cap   = attempt == 0 ? static_cast<uint32_t>(kRange * 3 / 8) : static_cast<uint32_t>(kRange + 256);
-    size_t const temp_bytes[6] = {static_cast<size_t>(nranges) * range_cap * sizeof(uint32_t),
+    if (queue_capacity > 0x7FFFFFF0ull) queue_capacity = 0x7FFFFFF0ull;
+    uint32_t const qcap        = static_cast<uint32_t>(queue_capacity);
+    size_t const temp_bytes[9] = {static_cast<size_t>(nranges) * range_cap * sizeof(uint32_t),
+                                  (static_cast<size_t>(nranges) + 1) * sizeof(uint32_t),
                                   static_cast<size_t>(nranges) * sizeof(uint32_t),
                                   static_cast<size_t>(nranges) * sizeof(uint32_t),
                                   (static_cast<size_t>(nranges) + 1) * sizeof(int64_t),
                                   scan_temp_bytes(nranges),
-                                  256};
-    TempParts<6> const temps(mr, temp_bytes);
+                                  256,
+                                  static_cast<size_t>(qcap) * sizeof(OovEntry),
+                                  static_cast<size_t>(qcap) * sizeof(uint32_t)};
+    TempParts<9> const temps(mr, temp_bytes);
     if (!temps.ok()) return give_up(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
     uint32_t* const arena     = temps.part<uint32_t>(0);
     uint32_t* const first_row = temps.part<uint32_t>(1);
-    uint32_t* const counts    = temps.part<uint32_t>(2);
-    int64_t* const bases      = temps.part<int64_t>(3);
-    uint64_t* const scan_tmp  = temps.part<uint64_t>(4);
-    uint32_t* const flags     = temps.part<uint32_t>(5);  // range counter, overflow flag
+    uint32_t* const words     = temps.part<uint32_t>(2);
+    uint32_t* const tokens    = temps.part<uint32_t>(3);
+    int64_t* const bases      = temps.part<int64_t>(4);
+    uint64_t* const scan_tmp  = temps.part<uint64_t>(5);
+    uint32_t* const flags     = temps.part<uint32_t>(6);  // [0] ranges handed out by the word pass, [1] a range had more words than slots, [2] queue entries, [3] blocks handed out by the out-of-vocabulary pass, [4] ranges handed out by the emit pass, [5] words of more than 16 bytes, [6] words of more tokens than a queue record keeps
+    OovEntry* const queue     = temps.part<OovEntry>(7);
+    uint32_t* const longer    = temps.part<uint32_t>(8);  // queue indices of the words of more than 16 bytes
     args.range_cap       = range_cap;
     args.range_first_row = first_row;
     args.arena           = arena;
-    args.range_count     = counts;
+    args.range_words     = words;
+    args.range_tokens    = tokens;
     args.offsets_out     = out->offsets;
+    args.queue           = queue;
+    args.queue_cap       = qcap;
+    args.queue_size      = flags + 2;
     args.counter         = flags;
     args.overflow        = flags + 1;
     launch_fill_u32(flags, 0u, 64, stream);
-    hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
+    hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 1 + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
     {
-      ProfileScope ps("wordpiece_tile_kernel", stream);
-      hipLaunchKernelGGL(tile_kernel, dim3(tile_grid), dim3(kTokThreads), 0, stream, args);
+      ProfileScope ps("wordpiece_word_kernel", stream);
+      hipLaunchKernelGGL(word_kernel, dim3(word_grid), dim3(kTokThreads), 0, stream, args);
+    }
+    {
+      ProfileScope ps("wordpiece_oov_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(oov_grid), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue, flags + 2, qcap, tokens,
+                         flags + 3, longer, flags + 5);
+    }
+    {
+      ProfileScope ps("wordpiece_oov_long_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue,
+                         flags + 2, qcap, longer, flags + 5, tokens);
     }
     // where the tokens of each range go; the total decides the child size
     // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
-    device_exclusive_scan(RangeCountOf{counts}, static_cast<int64_t>(nranges), bases, scan_tmp, stream);
-    uint32_t overflow = 0;
+    device_exclusive_scan(RangeTokensOf{tokens}, static_cast<int64_t>(nranges), bases, scan_tmp, stream);
+    uint32_t state[3] = {0, 0, 0};
     hipError_t e      = hipMemcpyAsync(&total, scan_tmp + scan_tiles(nranges), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(&overflow, flags + 1, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(state, flags, sizeof(state), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
     if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
 #ifdef WP_PHASE_TIMING
     {
       unsigned long long ph[10];
-      (void)hipMemcpy(ph, flags + 4, sizeof(ph), hipMemcpyDeviceToHost);
+      (void)hipMemcpy(ph, flags + 8, sizeof(ph), hipMemcpyDeviceToHost);
       unsigned long long sum = 0;
       for (auto x : ph) sum += x;
-      static const char* const names[10] = {"stage", "rows", "detect", "cap", "lists", "probe", "oov", "write", "rowoffs", "tail"};
-      sum -= ph[9];
-      fprintf(stderr, "[step share of all %.1f%%] ", 100.0 * ph[9] / (sum ? sum : 1));
-      for (int i = 0; i < 9; ++i) fprintf(stderr, "%s %.1f%%  ", names[i], 100.0 * ph[i] / (sum ? sum : 1));
-      fprintf(stderr, "trips/tile %.2f", double(ph[9]) / double(ntiles));
+      static const char* const names[10] = {"stage", "rows", "detect", "cap", "lists", "probe", "-", "-", "-", "-"};
+      for (int i = 0; i < 6; ++i) fprintf(stderr, "%s %.1f%%  ", names[i], 100.0 * ph[i] / (sum ? sum : 1));
       fprintf(stderr, "\n");
     }
 #endif
-    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) return give_up(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
-    if (overflow != 0) {
-      if (attempt > 0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+    bool const words_over = state[1] != 0, queue_over = state[2] > qcap;
+    if (words_over || queue_over) {
+      if (attempt > 0 || state[2] > 0x7FFFFFF0u) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+      if (words_over) range_cap = static_cast<uint32_t>(kRange + 8);
+      queue_capacity = std::max<uint64_t>(queue_capacity, state[2]);
       continue;
     }
+    if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) return give_up(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");
     out->child_size  = static_cast<int64_t>(total);
     out->child_bytes = static_cast<size_t>(total) * sizeof(int32_t);
     if (total) {
@@ -1756,10 +1988,13 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       if (!out->child) return give_up(NVTEXT_AMD_ALLOC_FAILED, "child allocation failed");
     }
     {
-      ProfileScope ps("wordpiece_gather_kernel", stream);
-      unsigned const row_blocks = static_cast<unsigned>((static_cast<int64_t>(rows) + 1 + 255) / 256);
-      hipLaunchKernelGGL(wordpiece_gather_kernel, dim3(nranges + row_blocks), dim3(256), 0, stream, v, first_offset, cbeg, kRangeShift, nranges, arena,
-                         range_cap, counts, bases, static_cast<int32_t*>(out->child), out->offsets);
+      ProfileScope ps("wordpiece_emit_kernel", stream);
+      hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, nranges, arena, range_cap, words, bases, first_row, queue,
+                         out->offsets, static_cast<int32_t*>(out->child), flags + 4, longer, flags + 6);
+      // (the list of longer words has served its purpose by now: its memory takes the list of words to do again, at most
+      // one entry per queued word)
+      hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue,
+                         longer, flags + 6, static_cast<int32_t*>(out->child));
     }
     break;
   }

@@ -417,7 +417,7 @@ def _tile_kernel_launches(nv, fn):
         names = [n for n, _ in _capi.profile_read()]
     finally:
         _capi.profile_enable(False)
-    return out, sum(1 for n in names if n == "wordpiece_tile_kernel")
+    return out, sum(1 for n in names if n == "wordpiece_word_kernel")
 
 
 @pytest.mark.parametrize("max_words", [0, 5, 100000])
