@@ -4,9 +4,10 @@
 A step is one wordpiece_tokenize call over the whole synthetic batch of configuration C2
 (4M rows, lognormal mean 256 B, Zipf(1.1) words over a 30,522-entry vocabulary, 15 % OOV,
 int32 offsets, max_words_per_row=128), inputs resident in HBM, output allocation included.
-Prints one JSON line: input GB/s as `value`, plus Mrows/s, the roofline of the dominant
-kernel, the host-oracle baseline on a bounded sample, and the minhash / minhash64 figures
-(configurations C3 / C4 at a stated scale).
+Prints one JSON line: input GB/s as `value`, plus Mrows/s, the roofline of the whole call,
+the host-oracle baseline on a bounded sample, the minhash / minhash64 figures (configurations
+C3 / C4 at a stated scale), the UTF-8 pipeline of C5 and the reference's own benchmark shapes.
+Every leg carries the mean and the median step time and the device memory a call holds at its peak.
 """
 import argparse
 import json
@@ -19,16 +20,32 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-VALU_PEAK_TOPS = 256 * 64 * 2.4e9 / 1e12  # 256 CUs x 64 lanes x 2.4 GHz: one 32-bit integer operation per lane and cycle
 
-# HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload, from two
-# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; the commands and
-# raw readings are in profiles/hbm_traffic_pmc_all_workloads.md.  Counters cannot be read from inside this
-# process, so the line reports these figures only for the workload they were measured on.
+# Hardware counters cannot be read from inside this process.  The figures below were read off rocprofv3 --pmc runs
+# of this same program; each names the file under profiles/ that holds the command and the raw readings, and is only
+# reported for the workload it was measured on.
+#
+# HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
+# scaled by a copy kernel of known size.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md"
 MEASURED_TRAFFIC_C2 = {
-    "wordpiece_probe_kernel": (1766100000, 1970100000),
-    "wordpiece_oov_kernel": (866200000, 1367300000),
-    "wordpiece_emit_kernel": (2368800000, 862800000),
+    "wordpiece_word_kernel": (0, 0),
+    "wordpiece_oov_kernel": (0, 0),
+    "wordpiece_emit_kernel": (0, 0),
+}
+MEASURED_TRAFFIC_C5_NORMALIZE = {
+    "normalize_count_kernel": (0, 0),
+    "normalize_write_kernel": (0, 0),
+}
+# minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
+# the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
+# moves issue in fewer than 4 cycles).  The floor is the instruction sequence of the inner loop: uint32, one
+# v_mad_u64_u32 per product and one v_min3_u32 per two; uint64, three v_mad_u64_u32, and / shift / 64-bit add (2) of the
+# fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products.
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md"
+MINHASH_VALU = {
+    "C3": {"floor": 1.5, "measured": 2.0, "issue": 1.00},
+    "C4": {"floor": 8.5, "measured": 13.5, "issue": 1.00},
 }
 
 
@@ -49,6 +66,7 @@ def input_bytes(col):
 
 
 def timed_steps(fn, steps, warmup, torch):
+    """Seconds per step over exactly `steps` steps (wall clock between two synchronisations)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -57,6 +75,72 @@ def timed_steps(fn, steps, warmup, torch):
         fn()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
+
+
+def median_step_ms(fn, reps, torch):
+    """Median over `reps` single steps, each bracketed by events on the stream the library launches on."""
+    times = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return median(times)
+
+
+def peak_device_bytes(fn, torch):
+    """Device memory one call holds at its peak, results and temporaries together, beyond what was allocated before it
+    (every allocation of the library goes through torch's allocator here)."""
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    out = fn()
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - before
+    del out
+    return int(peak)
+
+
+def host_threads(orc):
+    """Threads for the host oracle and where the number comes from: every core this process may run on (affinity mask,
+    cgroup quota), and no more than the CPU share the job was given when the environment states one."""
+    n = orc.hardware_threads()
+    src = "hardware_concurrency"
+    try:
+        aff = len(os.sched_getaffinity(0))
+        if aff < n:
+            n, src = aff, "sched_getaffinity"
+    except AttributeError:
+        pass
+    try:
+        quota, period = open("/sys/fs/cgroup/cpu.max").read().split()
+        if quota != "max" and int(quota) // int(period) < n:
+            n, src = max(1, int(quota) // int(period)), "cgroup cpu.max"
+    except (OSError, ValueError):
+        pass
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    if share.isdigit() and 0 < int(share) < n:
+        n, src = int(share), "OMP_NUM_THREADS (the job's CPU share)"
+    return max(1, n), src
+
+
+def cpu_leg(orc, value, seconds, sample):
+    threads, src = host_threads(orc)
+    return {"value": value, "unit": "GB/s", "cores": threads, "cores_from": src,
+            "hardware_concurrency": orc.hardware_threads(), "kind": "port", "sample": f"{sample}, {seconds:.2f} s"}
+
+
+def measure(fn, steps, warmup, capi, torch):
+    """One leg: mean wall time per step over exactly `steps` steps, the median of at least ten single steps timed with
+    events, the library's kernels, and the device memory a call holds at its peak."""
+    sec = timed_steps(fn, steps, warmup, torch)
+    med = median_step_ms(fn, max(10, steps), torch)
+    kt = kernel_times(fn, 3, capi, torch)
+    peak = peak_device_bytes(fn, torch)
+    return sec, {"ms_per_step": round(sec * 1e3, 4), "median_ms": round(med, 4), "peak_device_bytes": peak,
+                 "kernels_ms": {k: round(v, 4) for k, v in kt.items()}}, kt
 
 
 def kernel_times(fn, reps, capi, torch):
@@ -74,6 +158,29 @@ def kernel_times(fn, reps, capi, torch):
     return {k: sum(v) / len(v) for k, v in acc.items()}
 
 
+def hbm_roofline(alg_bytes, sec, kt, traffic=None):
+    """The roofline object of an HBM-bound call: `frac` prices the algorithmic bytes against the whole call (all of
+    its kernels, its scans and its synchronisations); the longest kernel is named beside it."""
+    dom = max(kt, key=kt.get)
+    achieved = alg_bytes / sec / 1e9
+    have = traffic is not None and all(sum(v) > 0 for v in traffic.values())
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": sum(sum(v) for v in traffic.values()) if have else None,
+            "traffic_per_kernel": {k: sum(v) for k, v in traffic.items()} if have else None,
+            "traffic_source": TRAFFIC_SOURCE if have else None,
+            "algorithmic_bytes": alg_bytes, "kernel": dom, "kernel_ms": round(kt[dom], 4),
+            "kernel_frac": round(alg_bytes / (kt[dom] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
+def valu_object(name):
+    """minhash is bound by VALU issue: the share of the SIMDs' issue slots that the floor sequence of the inner loop
+    would need, floor / measured instructions per permutation x measured issue rate.  It cannot exceed 1."""
+    v = MINHASH_VALU[name]
+    return {"bound": "valu issue", "floor_inst_per_perm": v["floor"], "measured_inst_per_perm": v["measured"],
+            "valu_issue": v["issue"], "frac": round(v["floor"] / v["measured"] * min(1.0, v["issue"]), 3), "source": VALU_SOURCE}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,6 +188,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--scale", type=float, default=1.0, help="row-count multiplier of the headline workload (1.0 = 4M rows)")
     ap.add_argument("--minhash-scale", type=float, default=1.0, help="row-count multiplier of the C3/C4/C5 legs (0 = skip)")
+    ap.add_argument("--reference-shapes", type=int, default=1, help="run the reference's own benchmark shapes (0 = skip)")
     ap.add_argument("--cpu-sample-rows", type=int, default=4_000_000, help="rows of the workload given to the host oracle")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -96,6 +204,12 @@ def main():
     _capi.load()
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
+    orc = None
+    if not args.no_cpu:
+        from oracle import pyoracle as orc
+        threads, src = host_threads(orc)
+        log(f"[bench] host oracle: {threads} threads ({src}); hardware_concurrency() = {orc.hardware_threads()}")
+    side_steps = max(3, args.steps // 2)
 
     # ------------------------------------------------------------------ headline: wordpiece_tokenize on C2
     t0 = time.time()
@@ -105,48 +219,39 @@ def main():
     dcol = nvtext.DeviceStringsColumn.from_host(host)
     dvoc = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(wl.vocab))
     mw = wl.params["max_words_per_row"]
-    result = {}
+    keep = {}
 
     def step():
-        result["out"] = nvtext.wordpiece_tokenize(dcol, dvoc, mw)
+        keep["o"] = nvtext.wordpiece_tokenize(dcol, dvoc, mw)
+        return keep["o"]
 
-    sec = timed_steps(step, args.steps, args.warmup, torch)
-    out = result["out"]
-    tokens = out.child_size
+    sec, head, kt = measure(step, args.steps, args.warmup, _capi, torch)
+    tokens = keep["o"].child_size
     in_b = input_bytes(host)
     out_b = 4 * tokens + 4 * (host.size + 1) + ((host.size + 7) // 8 if host.mask is not None else 0)
-    kt = kernel_times(step, 3, _capi, torch)
-    log(f"[bench] tokenize: {sec * 1e3:.3f} ms/step, tokens={tokens}, kernels={ {k: round(v, 3) for k, v in kt.items()} }")
-    dom = max(kt, key=kt.get)  # the kernel with the longest mean duration
-    dom_ms = kt[dom]
-    achieved = (in_b + out_b) / (dom_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": sum(MEASURED_TRAFFIC_C2[dom]) if args.scale == 1.0 and dom in MEASURED_TRAFFIC_C2 else None,
-                "traffic_all_kernels": ({k: sum(v) for k, v in MEASURED_TRAFFIC_C2.items()} if args.scale == 1.0 else None),
-                "algorithmic_bytes": in_b + out_b, "kernel_ms": round(dom_ms, 4),
-                "all_kernels_ms": {k: round(v, 4) for k, v in kt.items()},
-                "frac_whole_op": round((in_b + out_b) / sec / 1e9 / HBM_PEAK_GBS, 4)}
+    log(f"[bench] tokenize: {head}, tokens={tokens}")
+    roofline = hbm_roofline(in_b + out_b, sec, kt, MEASURED_TRAFFIC_C2 if args.scale == 1.0 else None)
+    roofline["all_kernels_ms"] = head["kernels_ms"]
+    roofline["peak_bytes_per_input_byte"] = round(head["peak_device_bytes"] / in_b, 3)
 
     # ------------------------------------------------------------------ host oracle on a bounded sample (also the parity check)
     cpu = None
     parity = "skipped"
-    if not args.no_cpu:
-        from oracle import pyoracle as orc
+    if orc:
         n = min(args.cpu_sample_rows, host.size)
         sample = host.slice(0, n)
         ovoc = orc.Vocabulary(wl.vocab)
-        threads = max(1, min(orc.hardware_threads(), 16))
         t0 = time.perf_counter()
         exp = orc.wordpiece_tokenize(sample, ovoc, mw, nthreads=threads)
         cpu_s = time.perf_counter() - t0
-        cpu = {"value": round(input_bytes(sample) / cpu_s / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": f"first {n} rows of the same workload ({sample.chars_bytes / 1e6:.0f} MB), {cpu_s:.2f} s",
-               "mrows_per_s": round(n / cpu_s / 1e6, 3)}
+        cpu = cpu_leg(orc, round(input_bytes(sample) / cpu_s / 1e9, 4), cpu_s,
+                      f"first {n} rows of the same workload ({sample.chars_bytes / 1e6:.0f} MB)")
+        cpu["mrows_per_s"] = round(n / cpu_s / 1e6, 3)
         got = nvtext.wordpiece_tokenize(dcol.slice(0, n, 0), dvoc, mw).to_host()
         parity = "PASS" if got.equals(exp) else "FAIL"
         log(f"[bench] oracle: {cpu_s:.2f}s on {threads} threads; parity {parity}")
-    del dcol, out, result
+        del exp, got
+    del dcol, keep
 
     # ------------------------------------------------------------------ minhash legs (C3 uint32, C4 uint64)
     extra = {}
@@ -166,35 +271,26 @@ def main():
 
             def mstep():
                 keep["o"] = fn(dc, p["seed"], da, db, p["width"])
+                return keep["o"]
 
-            msec = timed_steps(mstep, max(3, args.steps // 2), 1, torch)
-            mk = kernel_times(mstep, 2, _capi, torch)
+            msec, leg, _ = measure(mstep, side_steps, 1, _capi, torch)
             ib = input_bytes(w.rows)
             valid = w.rows.size - w.rows.null_count
             windows = int(w.rows.chars_bytes - valid * (p["width"] - 1))  # ASCII rows longer than width
-            leg = {"workload": f"{name} x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes,
-                   "ms_per_step": round(msec * 1e3, 3), "input_GBps": round(ib / msec / 1e9, 2),
-                   "mrows_per_s": round(w.rows.size / msec / 1e6, 3),
-                   "gperm_per_s": round(windows * p["P"] / msec / 1e9, 1),
-                   "kernels_ms": {k: round(v, 3) for k, v in mk.items()}}
-            # the bound of minhash is VALU issue: algorithmic lane-operations = windows x P x C_perm (2 for uint32:
-            # multiply-add and min; 12 for uint64: three 32x32 multiply-adds, the fold mod 2^61-1, the 64-bit min)
-            c_perm = 2 if p["hash_bits"] == 32 else 12
-            ops = windows * p["P"] * c_perm
-            leg["valu"] = {"algorithmic_ops": ops, "achieved": round(ops / msec / 1e12, 2), "peak": VALU_PEAK_TOPS,
-                           "unit": "T lane-op/s", "frac": round(ops / msec / 1e12 / VALU_PEAK_TOPS, 3)}
-            if not args.no_cpu:
-                from oracle import pyoracle as orc
+            leg.update({"workload": f"{name} x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes,
+                        "input_GBps": round(ib / msec / 1e9, 2), "mrows_per_s": round(w.rows.size / msec / 1e6, 3),
+                        "gperm_per_s": round(windows * p["P"] / msec / 1e9, 1)})
+            if args.minhash_scale == 1.0:
+                leg["valu"] = valu_object(name)
+            if orc:
                 n = min(w.rows.size, 20000 if name == "C3" else 2000)
                 smp = w.rows.slice(0, n)
                 ofn = orc.minhash if name == "C3" else orc.minhash64
-                threads = max(1, min(orc.hardware_threads(), 16))
                 t0 = time.perf_counter()
                 exp = ofn(smp, p["seed"], a, b, p["width"], nthreads=threads)
                 cs = time.perf_counter() - t0
                 got = fn(dc.slice(0, n, smp.null_count), p["seed"], da, db, p["width"]).to_host()
-                leg["cpu_baseline"] = {"value": round(input_bytes(smp) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
-                                       "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+                leg["cpu_baseline"] = cpu_leg(orc, round(input_bytes(smp) / cs / 1e9, 5), cs, f"first {n} rows ({smp.chars_bytes / 1e6:.1f} MB)")
                 leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
             log(f"[bench] {name}: {leg}")
             extra["minhash" if name == "C3" else "minhash64"] = leg
@@ -217,26 +313,22 @@ def main():
 
         def nstep():
             keep["o"] = nvtext.minhash_ngrams(dl, ngrams, p["seed"], da, db)
+            return keep["o"]
 
-        nsec = timed_steps(nstep, max(3, args.steps // 2), 1, torch)
-        nk = kernel_times(nstep, 2, _capi, torch)
+        nsec, leg, _ = measure(nstep, side_steps, 1, _capi, torch)
         nb = lists.child.chars.size + (lists.child.size + 1) * lists.child.offsets.dtype.itemsize + (lists.size + 1) * 4
-        leg = {"workload": f"words of C3 x{0.25 * args.minhash_scale} as LIST<STRING>, ngrams={ngrams}, P={p['P']}", "rows": lists.size,
-               "elements": lists.child.size, "ms_per_step": round(nsec * 1e3, 3), "input_GBps": round(nb / nsec / 1e9, 2),
-               "mrows_per_s": round(lists.size / nsec / 1e6, 3), "gperm_per_s": round(lists.child.size * p["P"] / nsec / 1e9, 1),
-               "kernels_ms": {k: round(v, 3) for k, v in nk.items()}}
-        if not args.no_cpu:
-            from oracle import pyoracle as orc
+        leg.update({"workload": f"words of C3 x{0.25 * args.minhash_scale} as LIST<STRING>, ngrams={ngrams}, P={p['P']}", "rows": lists.size,
+                    "elements": lists.child.size, "input_GBps": round(nb / nsec / 1e9, 2),
+                    "mrows_per_s": round(lists.size / nsec / 1e6, 3), "gperm_per_s": round(lists.child.size * p["P"] / nsec / 1e9, 1)})
+        if orc:
             n = min(lists.size, 20000)
             smp = lists.slice(0, n)
-            threads = max(1, min(orc.hardware_threads(), 16))
             t0 = time.perf_counter()
             exp = orc.minhash_ngrams(smp, ngrams, p["seed"], a, b, nthreads=threads)
             cs = time.perf_counter() - t0
             got = nvtext.minhash_ngrams(dl.slice(0, n, smp.null_count), ngrams, p["seed"], da, db).to_host()
             sample_bytes = int(lists.child.offsets[lists.offsets[n]])
-            leg["cpu_baseline"] = {"value": round(sample_bytes / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
-                                   "sample": f"first {n} rows ({sample_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+            leg["cpu_baseline"] = cpu_leg(orc, round(sample_bytes / cs / 1e9, 5), cs, f"first {n} rows ({sample_bytes / 1e6:.1f} MB)")
             leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
         log(f"[bench] minhash_ngrams: {leg}")
         extra["minhash_ngrams"] = leg
@@ -254,24 +346,20 @@ def main():
 
         def jstep():
             keep["o"] = nvtext.jaccard_index(d1, d2, jwidth)
+            return keep["o"]
 
-        jsec = timed_steps(jstep, max(3, args.steps // 2), 1, torch)
-        jk = kernel_times(jstep, 2, _capi, torch)
+        jsec, leg, _ = measure(jstep, side_steps, 1, _capi, torch)
         jb = 2 * input_bytes(w.rows)
-        leg = {"workload": f"rows r and r+1 of C3 x{0.25 * args.minhash_scale}, width={jwidth}", "rows": n,
-               "ms_per_step": round(jsec * 1e3, 3), "input_GBps": round(jb / jsec / 1e9, 2), "mrows_per_s": round(n / jsec / 1e6, 3),
-               "kernels_ms": {k: round(v, 3) for k, v in jk.items()}}
-        if not args.no_cpu:
-            from oracle import pyoracle as orc
+        leg.update({"workload": f"rows r and r+1 of C3 x{0.25 * args.minhash_scale}, width={jwidth}", "rows": n,
+                    "input_GBps": round(jb / jsec / 1e9, 2), "mrows_per_s": round(n / jsec / 1e6, 3)})
+        if orc:
             m = min(n, 20000)
             s1, s2 = w.rows.slice(0, m), w.rows.slice(1, m + 1)
-            threads = max(1, min(orc.hardware_threads(), 16))
             t0 = time.perf_counter()
             exp = orc.jaccard_index(s1, s2, jwidth, nthreads=threads)
             cs = time.perf_counter() - t0
             got = nvtext.jaccard_index(dc.slice(0, m, 0), dc.slice(1, m + 1, 0), jwidth).to_host()
-            leg["cpu_baseline"] = {"value": round(2 * input_bytes(s1) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
-                                   "sample": f"first {m} row pairs ({2 * s1.chars_bytes / 1e6:.1f} MB), {cs:.2f} s"}
+            leg["cpu_baseline"] = cpu_leg(orc, round(2 * input_bytes(s1) / cs / 1e9, 5), cs, f"first {m} row pairs ({2 * s1.chars_bytes / 1e6:.1f} MB)")
             leg["parity"] = "PASS" if got.equals(exp) else "FAIL"
         log(f"[bench] jaccard_index: {leg}")
         extra["jaccard_index"] = leg
@@ -290,15 +378,16 @@ def main():
 
         def tstep():
             keep["o"] = nvtext.wordpiece_tokenize(dc, dv5, p["max_words_per_row"])
+            return keep["o"]
 
-        tsec = timed_steps(tstep, max(3, args.steps // 2), 1, torch)
-        tk = kernel_times(tstep, 2, _capi, torch)
+        tsec, tleg, tk = measure(tstep, side_steps, 1, _capi, torch)
         ib = input_bytes(w.rows)
+        ntok = keep["o"].child_size
+        talg = ib + 4 * ntok + 4 * (w.rows.size + 1) + ((w.rows.size + 7) // 8 if w.rows.mask is not None else 0)
+        tleg.update({"input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": ntok,
+                     "peak_bytes_per_input_byte": round(tleg["peak_device_bytes"] / ib, 3), "roofline": hbm_roofline(talg, tsec, tk)})
         leg = {"workload": f"C5 x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes, "offsets": "int64",
-               "vocab_entries": w.vocab.size,
-               "tokenize": {"ms_per_step": round(tsec * 1e3, 3), "input_GBps": round(ib / tsec / 1e9, 2),
-                            "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": keep["o"].child_size,
-                            "kernels_ms": {k: round(v, 3) for k, v in tk.items()}}}
+               "vocab_entries": w.vocab.size, "tokenize": tleg}
         keep.clear()
         # normalize_characters, the step that precedes the tokenizer in a BERT pipeline (lower-casing, five special tokens)
         special = nvtext.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(["[CLS]", "[SEP]", "[PAD]", "[MASK]", "[UNK]"]))
@@ -306,25 +395,17 @@ def main():
 
         def zstep():
             keep["o"] = nvtext.normalize_characters(dc, normalizer)
+            return keep["o"]
 
-        zsec = timed_steps(zstep, max(3, args.steps // 2), 1, torch)
-        zk = kernel_times(zstep, 2, _capi, torch)
+        zsec, zleg, zk = measure(zstep, side_steps, 1, _capi, torch)
         out_bytes = int(keep["o"].chars.numel())
-        # algorithmic bytes of a call: chars + offsets in, chars + offsets (int64 from INT32_MAX bytes on) out; priced against the longest kernel
+        # algorithmic bytes of a call: chars + offsets in, chars + offsets (int64 from INT32_MAX bytes on) out
         zalg = ib + out_bytes + (8 if out_bytes >= 0x7FFFFFFF else 4) * (w.rows.size + 1)
-        zdom = max(zk, key=zk.get)
-        leg["normalize_characters"] = {"ms_per_step": round(zsec * 1e3, 3), "input_GBps": round(ib / zsec / 1e9, 2),
-                                       "mrows_per_s": round(w.rows.size / zsec / 1e6, 3), "chars_out": out_bytes,
-                                       "kernels_ms": {k: round(v, 3) for k, v in zk.items()},
-                                       "roofline": {"bound": "hbm", "kernel": zdom, "achieved": round(zalg / (zk[zdom] * 1e-3) / 1e9, 1),
-                                                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                                    "frac": round(zalg / (zk[zdom] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                                    "algorithmic_bytes": zalg, "frac_whole_op": round(zalg / zsec / 1e9 / HBM_PEAK_GBS, 4),
-                                                    "traffic": None}}
-        if not args.no_cpu:
+        zleg.update({"input_GBps": round(ib / zsec / 1e9, 2), "mrows_per_s": round(w.rows.size / zsec / 1e6, 3), "chars_out": out_bytes,
+                     "roofline": hbm_roofline(zalg, zsec, zk, MEASURED_TRAFFIC_C5_NORMALIZE if args.minhash_scale == 1.0 else None)})
+        leg["normalize_characters"] = zleg
+        if orc:
             from oracle import normalize_py
-            from oracle import pyoracle as orc
-            threads = max(1, min(orc.hardware_threads(), 16))
             normalize_py.rule_tables()  # built once, outside the timed part (the library's tables are built at create time)
             n = min(w.rows.size, 400000)
             smp = w.rows.slice(0, n)
@@ -332,11 +413,9 @@ def main():
             exp = normalize_py.normalize_characters_native(smp, True, [b"[CLS]", b"[SEP]", b"[PAD]", b"[MASK]", b"[UNK]"], nthreads=threads)
             cs = time.perf_counter() - t0
             got = nvtext.normalize_characters(dc.slice(0, n, smp.null_count), normalizer).to_host()
-            leg["normalize_characters"]["cpu_baseline"] = {
-                "value": round(input_bytes(smp) / cs / 1e9, 5), "unit": "GB/s", "cores": threads, "kind": "port",
-                "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB), {cs:.2f} s"}
+            zleg["cpu_baseline"] = cpu_leg(orc, round(input_bytes(smp) / cs / 1e9, 5), cs, f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB)")
             same = np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets)
-            leg["normalize_characters"]["parity"] = "PASS" if same else "FAIL"
+            zleg["parity"] = "PASS" if same else "FAIL"
         keep.clear()
         a, b = datagen.make_params(p["P"], 64, p["param_seed"])
         da = torch.from_numpy(a.view(np.int64)).cuda()
@@ -344,31 +423,33 @@ def main():
 
         def m5step():
             keep["o"] = nvtext.minhash64(dc, p["seed"], da, db, p["width"])
+            return keep["o"]
 
-        msec = timed_steps(m5step, max(3, args.steps // 2), 1, torch)
-        mk = kernel_times(m5step, 2, _capi, torch)
-        leg["minhash64"] = {"ms_per_step": round(msec * 1e3, 3), "input_GBps": round(ib / msec / 1e9, 2),
-                            "mrows_per_s": round(w.rows.size / msec / 1e6, 3), "kernels_ms": {k: round(v, 3) for k, v in mk.items()}}
-        if not args.no_cpu:
-            from oracle import pyoracle as orc
+        msec, mleg, _ = measure(m5step, side_steps, 1, _capi, torch)
+        mleg.update({"input_GBps": round(ib / msec / 1e9, 2), "mrows_per_s": round(w.rows.size / msec / 1e6, 3)})
+        leg["minhash64"] = mleg
+        if orc:
             n = min(w.rows.size, 400_000)
             smp = w.rows.slice(0, n)
-            threads = max(1, min(orc.hardware_threads(), 16))
             t0 = time.perf_counter()
             exp = orc.wordpiece_tokenize(smp, orc.Vocabulary(w.vocab), p["max_words_per_row"], nthreads=threads)
             cs = time.perf_counter() - t0
             got = nvtext.wordpiece_tokenize(dc.slice(0, n, smp.null_count), dv5, p["max_words_per_row"]).to_host()
-            leg["tokenize"]["cpu_baseline"] = {"value": round(input_bytes(smp) / cs / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-                                               "sample": f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB), {cs:.2f} s"}
-            leg["tokenize"]["parity"] = "PASS" if got.equals(exp) else "FAIL"
+            tleg["cpu_baseline"] = cpu_leg(orc, round(input_bytes(smp) / cs / 1e9, 4), cs, f"first {n} rows ({smp.chars_bytes / 1e6:.0f} MB)")
+            tleg["parity"] = "PASS" if got.equals(exp) else "FAIL"
         log(f"[bench] C5: {leg}")
         extra["utf8_pipeline"] = leg
-        del dc, keep
+        del dc, dv5, keep
+
+    # ------------------------------------------------------------------ the reference's own benchmark shapes
+    if args.reference_shapes:
+        extra["reference_shapes"] = reference_shapes(args, orc, _capi, datagen, nvtext, HostStringsColumn, np, torch)
 
     line = {
         "metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline",
         "value": round(in_b / sec / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(sec * 1e3, 4), "median_ms": head["median_ms"], "peak_device_bytes": head["peak_device_bytes"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8/int32", "data": "synthetic",
         "config": {"workload": f"C2 wordpiece_tokenize x{args.scale}", "rows": host.size, "chars_bytes": host.chars_bytes,
                    "vocab_entries": wl.vocab.size, "max_words_per_row": mw, "tokens_out": tokens, "offsets": "int32"},
@@ -377,6 +458,86 @@ def main():
     }
     line.update(extra)
     print(json.dumps(line), flush=True)
+
+
+def reference_shapes(args, orc, _capi, datagen, nvtext, HostStringsColumn, np, torch):
+    """The shapes of the reference's own benchmarks, largest row counts: minhash over 60,000 rows whose lengths are normal
+    between 0 and 28,000 bytes, hash_width 12 / 24, 26 / 260 parameters, both hash widths
+    (cpp/benchmarks/text/minhash.cpp:16-62), and wordpiece_tokenize over 2,097,152 copies of a 32-word row with a
+    six-entry vocabulary, max_words 0 / 20 / 40 (cpp/benchmarks/text/subword.cpp:18-52).  Random printable ASCII stands in
+    for the reference's random strings; parity against the host oracle on the first rows of each shape."""
+    legs = {"minhash": [], "wordpiece_tokenize": []}
+    steps = max(3, args.steps // 2)
+    threads = host_threads(orc)[0] if orc else 0
+
+    rows, row_width = 60_000, 28_000
+    rng = np.random.default_rng(20231)
+    lengths = np.clip(rng.normal(row_width / 2, row_width / 6, rows), 0, row_width).astype(np.int64)
+    offsets = np.zeros(rows + 1, np.int32)
+    np.cumsum(lengths, out=offsets[1:])
+    chars = rng.integers(32, 127, int(offsets[-1]), dtype=np.uint8)
+    col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
+    dc = nvtext.DeviceStringsColumn.from_host(col)
+    ib = input_bytes(col)
+    log(f"[bench] reference minhash shape: rows={rows} chars={col.chars_bytes / 1e9:.3f} GB")
+    for bits, fn in ((32, nvtext.minhash), (64, nvtext.minhash64)):
+        signed = np.int32 if bits == 32 else np.int64
+        for nparams in (26, 260):
+            a, b = datagen.make_params(nparams, bits, 7)
+            da = torch.from_numpy(a.view(signed)).cuda()
+            db = torch.from_numpy(b.view(signed)).cuda()
+            for width in (12, 24):
+                keep = {}
+
+                def mstep():
+                    keep["o"] = fn(dc, 0, da, db, width)
+                    return keep["o"]
+
+                msec, leg, _ = measure(mstep, steps, 1, _capi, torch)
+                windows = int(np.maximum(lengths - (width - 1), (lengths > 0).astype(np.int64)).sum())
+                leg.update({"num_rows": rows, "row_width": row_width, "hash_width": width, "parameters": nparams, "hash_type": bits,
+                            "input_GBps": round(ib / msec / 1e9, 2), "gperm_per_s": round(windows * nparams / msec / 1e9, 1)})
+                if orc:
+                    n = 400 if bits == 32 else 100
+                    smp = col.slice(0, n)
+                    exp = (orc.minhash if bits == 32 else orc.minhash64)(smp, 0, a, b, width, nthreads=threads)
+                    got = fn(dc.slice(0, n, 0), 0, da, db, width).to_host()
+                    leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
+                log(f"[bench] reference minhash: {leg}")
+                legs["minhash"].append(leg)
+                del keep
+    del dc, col, chars
+
+    rows = 2_097_152
+    text = b"This is a test " * 8
+    chars = np.frombuffer(text * rows, dtype=np.uint8)
+    offsets = (np.arange(rows + 1, dtype=np.int64) * len(text)).astype(np.int32)
+    col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
+    vocab = HostStringsColumn.from_pylist(["", "[UNK]", "This", "is", "a", "test"])
+    dc = nvtext.DeviceStringsColumn.from_host(col)
+    dv = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(vocab))
+    ib = input_bytes(col)
+    for max_words in (0, 20, 40):
+        keep = {}
+
+        def tstep():
+            keep["o"] = nvtext.wordpiece_tokenize(dc, dv, max_words)
+            return keep["o"]
+
+        tsec, leg, tk = measure(tstep, steps, 1, _capi, torch)
+        ntok = keep["o"].child_size
+        leg.update({"num_rows": rows, "max_words": max_words, "chars_bytes": col.chars_bytes, "tokens_out": ntok,
+                    "input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(rows / tsec / 1e6, 2),
+                    "roofline": hbm_roofline(ib + 4 * ntok + 4 * (rows + 1), tsec, tk)})
+        if orc:
+            n = 100_000
+            exp = orc.wordpiece_tokenize(col.slice(0, n), orc.Vocabulary(vocab), max_words, nthreads=threads)
+            got = nvtext.wordpiece_tokenize(dc.slice(0, n, 0), dv, max_words).to_host()
+            leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
+        log(f"[bench] reference wordpiece_tokenize: {leg}")
+        legs["wordpiece_tokenize"].append(leg)
+        del keep
+    return legs
 
 
 if __name__ == "__main__":

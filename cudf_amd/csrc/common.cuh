@@ -27,6 +27,17 @@ nvtext_amd_status fail(nvtext_amd_status st, const char* msg);
     }                                                                                 \
   } while (0)
 
+// The same once the result has buffers: `release` hands them back before the error is returned.
+#define NVTEXT_HIP_TRY_OR(expr, release)                                              \
+  do {                                                                                \
+    hipError_t _e = (expr);                                                           \
+    if (_e != hipSuccess) {                                                           \
+      release;                                                                        \
+      std::string _m = std::string(#expr) + ": " + hipGetErrorString(_e);             \
+      return ::nvtext_amd::fail(NVTEXT_AMD_DEVICE_ERROR, _m.c_str());                 \
+    }                                                                                 \
+  } while (0)
+
 // ------------------------------------------------------------------ kernel timing (benchmarks)
 bool profiling_on();
 void profile_mark_begin(const char* name, hipStream_t stream);

@@ -16,7 +16,8 @@ struct ProfileRecord {
   hipEvent_t begin;
   hipEvent_t end;
 };
-bool g_profile_on = false;
+bool g_profile_on   = false;
+bool g_profile_open = false;  // the last profile_mark_begin made a record
 std::vector<ProfileRecord> g_profile;
 }  // namespace
 
@@ -25,14 +26,22 @@ bool profiling_on() { return g_profile_on; }
 void profile_mark_begin(const char* name, hipStream_t stream)
 {
   ProfileRecord r{name, nullptr, nullptr};
-  if (hipEventCreate(&r.begin) != hipSuccess || hipEventCreate(&r.end) != hipSuccess) return;
+  g_profile_open = false;
+  if (hipEventCreate(&r.begin) != hipSuccess) return;
+  if (hipEventCreate(&r.end) != hipSuccess) {
+    (void)hipEventDestroy(r.begin);
+    return;
+  }
   (void)hipEventRecord(r.begin, stream);
   g_profile.push_back(r);
+  g_profile_open = true;
 }
 
 void profile_mark_end(hipStream_t stream)
 {
-  if (!g_profile.empty()) (void)hipEventRecord(g_profile.back().end, stream);
+  // only the record that the matching begin made: a begin that failed leaves nothing to close
+  if (g_profile_open) (void)hipEventRecord(g_profile.back().end, stream);
+  g_profile_open = false;
 }
 
 void set_last_error(const char* msg) { g_last_error = msg ? msg : ""; }

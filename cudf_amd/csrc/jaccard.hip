@@ -69,7 +69,7 @@ __device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_
           int64_t const gpos = base + p;
           WordSrc const src{stage, mis + p};
           uint32_t hlen;
-          if (window_at(src, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen)) {
+          if (window_at(src, row + gpos, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen)) {
             uint32_t const hv = murmur3_x86_32(src, hlen, 0u);  // jaccard.cu:258: seed 0
             if (hv != 0u) set.insert(hv, which);                // 282-286: zero hashes are dropped
           }
@@ -85,7 +85,7 @@ __device__ __forceinline__ void insert_row(const uint8_t* row, int64_t n, int32_
       BoundedSrc const src{row + gpos, remaining};
       uint32_t hlen;
       uint32_t const readable = static_cast<uint32_t>(min(remaining, static_cast<int64_t>(width) * 4));
-      if (window_at(src, remaining, readable, gpos == 0, false, width, &hlen)) {
+      if (window_at(src, row + gpos, remaining, readable, gpos == 0, false, width, &hlen)) {
         uint32_t const hv = murmur3_x86_32(src, hlen, 0u);
         if (hv != 0u) set.insert(hv, which);
       }
@@ -434,10 +434,10 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
     ProfileScope ps("jaccard_global_kernel", stream);
     hipLaunchKernelGGL(jaccard_global_kernel, dim3(grid), dim3(kThreads), 0, stream, v1, v2, width, values, big.as<uint32_t>(),
                        tables.as<uint32_t>(), slots);
-    NVTEXT_HIP_TRY(hipGetLastError());
+    NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_fixed_column_free(out, stream_, mr_));
     // the tables are released in stream order when `tables` goes out of scope
   }
-  NVTEXT_HIP_TRY(hipGetLastError());
+  NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_fixed_column_free(out, stream_, mr_));
   return NVTEXT_AMD_SUCCESS;
 }
 

@@ -71,16 +71,48 @@ __device__ __forceinline__ uint64_t min_below_2_62(uint64_t m, uint64_t y)
   return r;
 }
 
-// Folds `count` compacted hashes (padded here to a multiple of 4) into m[K]; lanes <-> parameters.
+// Folds the compacted hashes first, first + 1, .. of every `stride` (the count padded to a multiple of the stride)
+// into m[K]; lanes <-> parameters.  A wavefront whose lanes all hold different parameters folds every hash
+// (first 0, stride = the hashes of one trip); with few parameters the lanes form groups that hold the same
+// parameters and fold every other trip each (see Packing).
 template <typename T, int K>
 struct Fold;
 
+// How the lanes of a wavefront share the work when there are at most 32 parameters: `groups` sets of `ppad` lanes
+// (both powers of two, groups <= 16), lane l holding parameter l % ppad and folding the trips l / ppad,
+// l / ppad + groups, ...  The sets are combined with a butterfly of minima before the results leave the registers.
+struct Packing {
+  int32_t ppad;    // lanes per set; 64 when every lane has its own parameter
+  int32_t groups;  // sets per wavefront
+  __device__ __forceinline__ int param_lane(int lane) const { return lane & (ppad - 1); }
+  __device__ __forceinline__ uint32_t first(int lane, uint32_t per_trip) const { return static_cast<uint32_t>(lane / ppad) * per_trip; }
+  __device__ __forceinline__ uint32_t stride(uint32_t per_trip) const { return static_cast<uint32_t>(groups) * per_trip; }
+  template <typename T>
+  __device__ __forceinline__ T combine(T m) const
+  {
+    for (int d = ppad; d < kWave; d <<= 1) {
+      T const other = __shfl_xor(m, d);
+      m             = min(m, other);
+    }
+    return m;
+  }
+};
+
+__host__ __device__ inline Packing packing_for(int32_t P)
+{
+  if (P > 32) return Packing{kWave, 1};
+  int32_t ppad = 4;  // at most 16 sets, so that the padding of a tile's hashes fits one wavefront-wide store
+  while (ppad < P) ppad <<= 1;
+  return Packing{ppad, kWave / ppad};
+}
+
 template <int K>
 struct Fold<uint32_t, K> {
-  static __device__ __forceinline__ void run(const uint32_t* hashes, uint32_t padded, const uint32_t (&a)[K], const uint32_t (&b)[K],
-                                             uint32_t (&m)[K])
+  static constexpr uint32_t kPerTrip = 4;
+  static __device__ __forceinline__ void run(const uint32_t* hashes, uint32_t padded, uint32_t first, uint32_t stride,
+                                             const uint32_t (&a)[K], const uint32_t (&b)[K], uint32_t (&m)[K])
   {
-    for (uint32_t i = 0; i < padded; i += 4) {
+    for (uint32_t i = first; i < padded; i += stride) {
       uint32_t const h0 = hashes[i], h1 = hashes[i + 1], h2 = hashes[i + 2], h3 = hashes[i + 3];
 #pragma unroll
       for (int k = 0; k < K; ++k) {
@@ -102,15 +134,16 @@ struct Fold<uint64_t, K> {
   // x mod p for x < 2^64: x = q*2^61 + r with q <= 7, so y = r + q <= p + 7.
   static __device__ __forceinline__ uint64_t fold_once(uint64_t x) { return (x & p) + (x >> 61); }
 
-  static __device__ __forceinline__ void run(const uint64_t* hashes, uint32_t padded, const uint64_t (&a)[K], const uint64_t (&b)[K],
-                                             uint64_t (&m)[K])
+  static constexpr uint32_t kPerTrip = 2;
+  static __device__ __forceinline__ void run(const uint64_t* hashes, uint32_t padded, uint32_t first, uint32_t stride,
+                                             const uint64_t (&a)[K], const uint64_t (&b)[K], uint64_t (&m)[K])
   {
     // Fast pass: the final "subtract p if y >= p" is left out.  y >= p needs the top dword of y to be
     // at least 0x1FFFFFFF (one chance in 2^29 per product), which is tracked with a running maximum;
     // if it ever happens the tile is folded again exactly.  Unreduced values are >= p, above every
     // reduced value, so they can never displace a correct minimum.
     uint32_t top = 0;
-    for (uint32_t i = 0; i < padded; i += 2) {
+    for (uint32_t i = first; i < padded; i += stride) {
       uint64_t const h0 = hashes[i], h1 = hashes[i + 1];
 #pragma unroll
       for (int k = 0; k < K; ++k) {
@@ -121,6 +154,7 @@ struct Fold<uint64_t, K> {
       }
     }
     if (ballot64(top >= 0x1FFFFFFFu) != 0) {
+      // every lane folds every hash here: a minimum does not mind the hashes of the other sets
       for (uint32_t i = 0; i < padded; ++i) {
         uint64_t const h = hashes[i];
 #pragma unroll
@@ -134,19 +168,25 @@ struct Fold<uint64_t, K> {
 };
 
 template <typename T, int K>
-__device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane)
+__device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane,
+                                            Packing pk = Packing{kWave, 1})
 {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (count == 0) return;
   // a duplicate never changes a minimum
-  uint32_t const padded = (count + 3u) & ~3u;
+  uint32_t const stride = K > 1 ? Fold<T, K>::kPerTrip : pk.stride(Fold<T, K>::kPerTrip);  // a power of two, at most 64
+  uint32_t const padded = (count + stride - 1u) & ~(stride - 1u);
   if (lane < static_cast<int>(padded - count)) lds.hashes[count + lane] = lds.hashes[0];
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  Fold<T, K>::run(lds.hashes, padded, a, b, m);
+  // the usual case keeps the loop counter out of the vector registers
+  if (K > 1 || pk.groups == 1)
+    Fold<T, K>::run(lds.hashes, padded, 0u, Fold<T, K>::kPerTrip, a, b, m);
+  else
+    Fold<T, K>::run(lds.hashes, padded, pk.first(lane, Fold<T, K>::kPerTrip), stride, a, b, m);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
 }
@@ -155,7 +195,7 @@ __device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, con
 // permuted hashes into m[K].  Lane l owns parameters chunk_base + l + 64*k.
 template <typename T, int K>
 __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, int64_t s_begin, int64_t s_end, T seed, int32_t width,
-                                                const T (&a)[K], const T (&b)[K], T (&m)[K], WaveLds<T>& lds, int lane)
+                                                const T (&a)[K], const T (&b)[K], T (&m)[K], WaveLds<T>& lds, int lane, Packing pk)
 {
   using H = HashTraits<T>;
   if (static_cast<int64_t>(width) * 4 <= kHalo) {
@@ -178,7 +218,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
           int64_t const gpos = base + p;
           WordSrc const src{lds.bytes, mis + p};
           uint32_t hlen;
-          valid = window_at(src, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen);
+          valid = window_at(src, row + gpos, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen);
           if (valid) {
             hv = H::hash(src, hlen, seed);
             hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
@@ -188,7 +228,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
         if (valid) lds.hashes[count + lanes_below(vm)] = hv;
         count += static_cast<uint32_t>(__builtin_popcountll(vm));
       }
-      fold_hashes<T, K>(lds, count, a, b, m, lane);
+      fold_hashes<T, K>(lds, count, a, b, m, lane, pk);
     }
   } else {
     // very wide windows: 64 starts at a time, bytes read straight from global memory
@@ -201,7 +241,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
         BoundedSrc const src{row + gpos, remaining};
         uint32_t hlen;
         uint32_t const readable = static_cast<uint32_t>(min(remaining, static_cast<int64_t>(width) * 4));
-        valid = window_at(src, remaining, readable, gpos == 0, false, width, &hlen);
+        valid = window_at(src, row + gpos, remaining, readable, gpos == 0, false, width, &hlen);
         if (valid) {
           hv = H::hash(src, hlen, seed);
           hv = hv < 1 ? T{1} : hv;
@@ -209,7 +249,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       }
       uint64_t const vm = ballot64(valid);
       if (valid) lds.hashes[lanes_below(vm)] = hv;
-      fold_hashes<T, K>(lds, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
+      fold_hashes<T, K>(lds, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane, pk);
     }
   }
 }
@@ -226,16 +266,17 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
   }
 }
 
-// One workgroup per (row, parameter chunk): the first kSpan bytes of the row.
+// One workgroup per (row, parameter chunk): the first kSpan bytes of the row.  The rows lie along x and, beyond
+// kMaxRowBlocks of them, along z (a grid holds 2^32 threads at most in one dimension).
 template <typename T, int K>
-__global__ void __launch_bounds__(kThreads) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
+__global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
                                                                 int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out)
 {
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][K * kWave];
 
-  int64_t const r = blockIdx.x;
-  if (!col.valid(r)) return;
+  int64_t const r = static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x;
+  if (r >= col.size || !col.valid(r)) return;
   int32_t const chunk_base = blockIdx.y * (K * kWave);
   int64_t const o          = col.off(r);
   int64_t const n          = col.off(r + 1) - o;
@@ -245,18 +286,20 @@ __global__ void __launch_bounds__(kThreads) minhash_rows_kernel(ColView col, T s
     for (int j = threadIdx.x; j < in_chunk; j += kThreads) dst[j] = T{0};
     return;
   }
-  int const lane = lane_id();
-  int const wave = threadIdx.x / kWave;
+  int const lane   = lane_id();
+  int const wave   = threadIdx.x / kWave;
+  Packing const pk = K == 1 ? packing_for(P) : Packing{kWave, 1};
   T a[K], b[K], m[K];
-  load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
+  load_params<T, K>(pa, pb, P, chunk_base, pk.param_lane(lane), a, b, m);
 
   int64_t const span = min(n, static_cast<int64_t>(kSpan));
   int64_t sec        = (span + kWaves - 1) / kWaves;
   sec                = (sec + kWave - 1) / kWave * kWave;
   int64_t const sb   = min(span, wave * sec);
   int64_t const se   = min(span, sb + sec);
-  if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane);
+  if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
 
+  if (K == 1) m[0] = pk.combine(m[0]);
 #pragma unroll
   for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
   __syncthreads();
@@ -282,6 +325,7 @@ __global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T 
   int32_t const in_chunk   = min(K * kWave, P - chunk_base);
   int const lane           = lane_id();
   int const wave           = threadIdx.x / kWave;
+  Packing const pk         = K == 1 ? packing_for(P) : Packing{kWave, 1};
   for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
     // last row r with extra_prefix[r] <= t
     int64_t lo = 0, hi = col.size;
@@ -294,13 +338,14 @@ __global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T 
     int64_t const o    = col.off(r);
     int64_t const n    = col.off(r + 1) - o;
     T a[K], b[K], m[K];
-    load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
+    load_params<T, K>(pa, pb, P, chunk_base, pk.param_lane(lane), a, b, m);
     int64_t const pb0  = part * kSpan;
     int64_t const pe0  = min(n, pb0 + kSpan);
     int64_t const sec  = kSpan / kWaves;
     int64_t const sb   = min(pe0, pb0 + wave * sec);
     int64_t const se   = min(pe0, sb + sec);
-    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane);
+    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
+    if (K == 1) m[0] = pk.combine(m[0]);
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
@@ -337,12 +382,15 @@ __global__ void uniform_offsets_kernel(int32_t* out, int32_t rows, int32_t P)
   if (i <= rows) out[i] = static_cast<int32_t>(i * P);
 }
 
+constexpr int32_t kMaxRowBlocks = 1 << 22;
+
 template <typename T, int K>
 void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, const int32_t* offsets,
                     const uint32_t* extra_prefix, T* child, hipStream_t stream)
 {
   int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
-  dim3 grid(static_cast<unsigned>(v.size), static_cast<unsigned>(chunks));
+  dim3 grid(static_cast<unsigned>(std::min(v.size, kMaxRowBlocks)), static_cast<unsigned>(chunks),
+            static_cast<unsigned>((v.size + kMaxRowBlocks - 1) / kMaxRowBlocks));
   {
     ProfileScope ps("minhash_rows_kernel", stream);
     hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
@@ -383,7 +431,7 @@ nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, c
   if (!out->offsets) return fail(NVTEXT_AMD_ALLOC_FAILED, "offsets allocation failed");
   if (rows == 0) {  // minhash.cu:449 then 616: zero rows, offsets = [0], empty child
     launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, 1, stream);
-    NVTEXT_HIP_TRY(hipGetLastError());
+    NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_list_column_free(out, stream_, mr_));
     return NVTEXT_AMD_SUCCESS;
   }
   out->child_size  = static_cast<int64_t>(rows - input->null_count) * P;
@@ -421,14 +469,23 @@ nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, c
 
   T* child = static_cast<T*>(out->child);
   if (out->child_size > 0) {
-    if (P > 2 * kWave)
-      launch_kernels<T, 4>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
-    else if (P > kWave)
-      launch_kernels<T, 2>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
-    else
-      launch_kernels<T, 1>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream);
+    // every chunk of 64 K parameters hashes the windows again, and a lane without a parameter still folds:
+    // the K that leaves the fewest idle parameter slots, the larger K (fewer hashing passes) on a tie
+    int best_k = 1;
+    int64_t best_slots = std::numeric_limits<int64_t>::max();
+    for (int k = 1; k <= 5; ++k) {
+      int64_t const slots = static_cast<int64_t>((P + k * kWave - 1) / (k * kWave)) * k;
+      if (slots <= best_slots) { best_slots = slots; best_k = k; }
+    }
+    switch (best_k) {
+      case 5: launch_kernels<T, 5>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
+      case 4: launch_kernels<T, 4>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
+      case 3: launch_kernels<T, 3>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
+      case 2: launch_kernels<T, 2>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
+      default: launch_kernels<T, 1>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
+    }
   }
-  NVTEXT_HIP_TRY(hipGetLastError());
+  NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_list_column_free(out, stream_, mr_));
   return NVTEXT_AMD_SUCCESS;
 }
 
@@ -492,8 +549,8 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
   constexpr bool kStageRuns = sizeof(T) == 4;
   __shared__ uint32_t run_bytes[kWaves][kStageRuns ? kNgramStageWords : 1];
 
-  int64_t const r = blockIdx.x;
-  if (!in.valid(r)) return;
+  int64_t const r = static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x;  // rows along x, then z
+  if (r >= in.size || !in.valid(r)) return;
   int32_t const chunk_base = blockIdx.y * (K * kWave);
   int64_t const first      = in.off(r);
   int64_t const n          = in.off(r + 1) - first;
@@ -574,7 +631,8 @@ void launch_ngrams(const ListView& v, int32_t ngrams, T seed, const T* a, const 
                    hipStream_t stream)
 {
   int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
-  dim3 grid(static_cast<unsigned>(v.size), static_cast<unsigned>(chunks));
+  dim3 grid(static_cast<unsigned>(std::min(v.size, kMaxRowBlocks)), static_cast<unsigned>(chunks),
+            static_cast<unsigned>((v.size + kMaxRowBlocks - 1) / kMaxRowBlocks));
   ProfileScope ps("minhash_ngrams_kernel", stream);
   hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_ngrams_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, ngrams, seed, a, b, P, offsets, child);
 }
@@ -610,7 +668,7 @@ nvtext_amd_status minhash_ngrams_impl(const nvtext_amd_list_strings_column* inpu
   if (!out->offsets) return fail(NVTEXT_AMD_ALLOC_FAILED, "offsets allocation failed");
   if (rows == 0) {  // minhash.cu:539 then 616
     launch_fill_u32(reinterpret_cast<uint32_t*>(out->offsets), 0u, 1, stream);
-    NVTEXT_HIP_TRY(hipGetLastError());
+    NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_list_column_free(out, stream_, mr_));
     return NVTEXT_AMD_SUCCESS;
   }
   out->child_size  = static_cast<int64_t>(rows - input->null_count) * P;
@@ -658,7 +716,7 @@ nvtext_amd_status minhash_ngrams_impl(const nvtext_amd_list_strings_column* inpu
     else
       launch_ngrams<T, 1>(v, ngrams, seed, a, b, P, out->offsets, child, stream);
   }
-  NVTEXT_HIP_TRY(hipGetLastError());
+  NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_list_column_free(out, stream_, mr_));
   return NVTEXT_AMD_SUCCESS;
 }
 

@@ -878,7 +878,7 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
   if (n == 0) {  // normalize.cu:504: nothing to normalize, every row is empty
     if (!allocate_offsets(false)) return release(NVTEXT_AMD_ALLOC_FAILED, "result allocation failed");
     launch_fill_u32(static_cast<uint32_t*>(out->offsets), 0u, static_cast<int64_t>(rows) + 1, stream);
-    NVTEXT_HIP_TRY(hipGetLastError());
+    NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_strings_result_free(out, stream_, mr_));
     return NVTEXT_AMD_SUCCESS;
   }
 

@@ -47,10 +47,11 @@ __device__ __forceinline__ uint32_t stage_bytes(const uint8_t* row, int64_t base
 
 // Decides whether a window starts at this position and how many bytes it hashes
 // (cpp/src/text/minhash.cu:120-133 with cpp/include/cudf/strings/string_view.cuh:67-80).
-// `remaining` = row bytes from this position on; `readable` = bytes of them reachable through src.
+// `remaining` = row bytes from this position on; `readable` = bytes of them reachable through src
+// (the whole rest of the row, or at least 4 * width bytes); `g` = this position in the row itself.
 template <typename Src>
-__device__ __forceinline__ bool window_at(Src const& src, int64_t remaining, uint32_t readable, bool first, bool all_ascii, int32_t width,
-                                          uint32_t* hlen)
+__device__ __forceinline__ bool window_at(Src const& src, const uint8_t* g, int64_t remaining, uint32_t readable, bool first, bool all_ascii,
+                                          int32_t width, uint32_t* hlen)
 {
   if (all_ascii) {
     if (remaining >= width) {
@@ -68,6 +69,17 @@ __device__ __forceinline__ bool window_at(Src const& src, int64_t remaining, uin
     left -= (w != 0);
     bytes += w;
     ++j;
+  }
+  // Well-formed text has `width` characters within 4 * width bytes.  Bytes that continue no character count for
+  // nothing, so a run of them can leave characters to find beyond what src reaches: the walk goes on in the row.
+  if (left > 0 && j < remaining) {
+    int64_t k = j;
+    while (left > 0 && k < remaining) {
+      int const w = bytes_in_utf8_byte(g[k]);
+      left -= (w != 0);
+      bytes += w;
+      ++k;
+    }
   }
   // a malformed trailing lead byte may declare more bytes than the row holds: clamp to the row
   *hlen = static_cast<uint32_t>(min(static_cast<int64_t>(bytes), remaining));

@@ -16,7 +16,8 @@ import numpy as np
 from ..arrow_host import HostListStringsColumn, HostStringsColumn
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libnvtext_datagen.so")
+# NVTEXT_DATAGEN_LIB names another build of the same source (the sanitizer build of `make SAN=1`)
+_LIB_PATH = os.environ.get("NVTEXT_DATAGEN_LIB") or os.path.join(_HERE, "libnvtext_datagen.so")
 _lib = None
 
 

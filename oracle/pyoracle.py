@@ -14,7 +14,8 @@ from typing import Optional
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libnvtext_oracle.so")
+# NVTEXT_ORACLE_LIB names another build of the same source (the sanitizer build of `make SAN=1`)
+_LIB_PATH = os.environ.get("NVTEXT_ORACLE_LIB") or os.path.join(_HERE, "libnvtext_oracle.so")
 _lib = None
 
 OK, INVALID_ARGUMENT, OVERFLOW_ERROR, LOGIC_ERROR = 0, 1, 2, 3

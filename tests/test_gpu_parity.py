@@ -78,7 +78,8 @@ def random_rows(rng, n, max_len, utf8=False, p_null=0.05, p_empty=0.05):
 
 
 @pytest.mark.parametrize("utf8", [False, True], ids=["ascii", "utf8"])
-@pytest.mark.parametrize("P,width", [(3, 4), (64, 5), (100, 2), (128, 8), (256, 5), (260, 12)])
+@pytest.mark.parametrize("P,width", [(1, 3), (3, 4), (4, 2), (5, 6), (16, 9), (26, 12), (32, 24), (33, 7), (64, 5), (100, 2), (128, 8),
+                                     (129, 4), (192, 3), (256, 5), (260, 12), (320, 24), (321, 5), (700, 6)])
 def test_minhash_random_vs_oracle(nv, orc, utf8, P, width):
     rng = np.random.default_rng(1000 + P + width + int(utf8))
     rows = random_rows(rng, 300, 700, utf8=utf8)
@@ -117,6 +118,41 @@ def test_minhash_long_rows_cross_workgroups(nv, orc):
     assert_same(nv.minhash64(col, 7, a64, b64, 5).to_host(), orc.minhash64(host, 7, a64, b64, 5, nthreads=8), "minhash64 long")
 
 
+def test_minhash_few_parameters_share_the_lanes_of_a_wavefront(nv, orc):
+    """With at most 32 parameters the lanes work in sets that each fold a part of the hashes; long rows (every wavefront
+    of a workgroup, the extra workgroups) and rows of fewer windows than sets must still give the minimum over all."""
+    rng = np.random.default_rng(26)
+    rows = random_rows(rng, 60, 3000) + ["k" * 40000, "".join(rng.choice(list("abcdefg "), 70000)), "ab", "abc", "abcd", "abcdefgh", "", None]
+    host = strings(rows)
+    col = dev(nv, host)
+    for P in (1, 2, 7, 8, 26, 31, 32):
+        a32 = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        b32 = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        assert_same(nv.minhash(col, 0, a32, b32, 12).to_host(), orc.minhash(host, 0, a32, b32, 12, nthreads=8), f"minhash P={P}")
+        a64 = rng.integers(1, 2**64, P, dtype=np.uint64)
+        b64 = rng.integers(0, 2**64, P, dtype=np.uint64)
+        assert_same(nv.minhash64(col, 0, a64, b64, 24).to_host(), orc.minhash64(host, 0, a64, b64, 24, nthreads=8), f"minhash64 P={P}")
+
+
+def test_minhash_more_rows_than_a_grid_has_workgroups(nv, orc):
+    """More rows than the launch has workgroups (the cap is 2^22, a grid holds 2^32 threads): rows share workgroups."""
+    rows = (1 << 22) + 12345
+    rng = np.random.default_rng(17)
+    lengths = rng.integers(0, 6, rows)
+    offsets = np.zeros(rows + 1, np.int32)
+    np.cumsum(lengths, out=offsets[1:])
+    chars = rng.integers(97, 123, int(offsets[-1]), dtype=np.uint8)
+    valid = rng.random(rows) > 0.01
+    from cudf_amd.arrow_host import HostStringsColumn, pack_validity
+    host = HostStringsColumn(chars, offsets, pack_validity(valid), rows, 0, int((~valid).sum()))
+    col = dev(nv, host)
+    a = np.array([3, 5], np.uint32)
+    b = np.array([1, 2], np.uint32)
+    assert_same(nv.minhash(col, 1, a, b, 3).to_host(), orc.minhash(host, 1, a, b, 3, nthreads=8), "many rows")
+    a64, b64 = a.astype(np.uint64), b.astype(np.uint64)
+    assert_same(nv.minhash64(col, 1, a64, b64, 3).to_host(), orc.minhash64(host, 1, a64, b64, 3, nthreads=8), "many rows 64")
+
+
 def test_minhash_very_wide_window(nv, orc):
     """width*4 bytes beyond the staged halo: bytes are read straight from global memory."""
     rng = np.random.default_rng(6)
@@ -127,6 +163,32 @@ def test_minhash_very_wide_window(nv, orc):
     assert_same(nv.minhash(col, 1, a, a, 40).to_host(), orc.minhash(host, 1, a, a, 40), "wide window")
     a64 = rng.integers(1, 2**64, 5, dtype=np.uint64)
     assert_same(nv.minhash64(col, 1, a64, a64, 100).to_host(), orc.minhash64(host, 1, a64, a64, 100), "wide window 64")
+
+
+def test_windows_over_runs_of_continuation_bytes(nv, orc):
+    """Bytes that continue no character count for nothing in the walk to `width` characters
+    (cpp/include/cudf/strings/string_view.cuh:67-80), so a run of them stretches a window past the 4 * width bytes that
+    well-formed text needs: the same rows at several places of the 256-position tiles, for minhash and jaccard_index."""
+    rng = np.random.default_rng(66)
+    rows = []
+    for shift in (0, 1, 100, 200, 250, 255, 256, 257, 300):
+        head = bytes(rng.integers(97, 123, shift, dtype=np.uint8))
+        for run in (4, 17, 60, 129, 300, 700):
+            rows.append(head + b"ab" + b"\x80" * run + b"cdefgh" + b"\xbf" * (run // 2) + b"ij klmnop")
+            rows.append(head + "é".encode() + b"\x9a" * run)          # the run ends the row: only the first window may be short
+            rows.append(head + b"\xe6\xbc" + b"\xa2" * run + b"xyz")
+    host = HostStringsColumn.from_pylist(rows)
+    col = dev(nv, host)
+    a = rng.integers(1, 2**32, 9, dtype=np.uint64).astype(np.uint32)
+    b = rng.integers(0, 2**32, 9, dtype=np.uint64).astype(np.uint32)
+    for width in (2, 5, 12, 40):
+        assert_same(nv.minhash(col, 3, a, b, width).to_host(), orc.minhash(host, 3, a, b, width, nthreads=4), f"minhash width {width}")
+        a64, b64 = a.astype(np.uint64) << np.uint64(7), b.astype(np.uint64)
+        assert_same(nv.minhash64(col, 3, a64, b64, width).to_host(), orc.minhash64(host, 3, a64, b64, width, nthreads=4), f"minhash64 width {width}")
+        n = len(rows) - 1
+        got = nv.jaccard_index(col.slice(0, n, 0), col.slice(1, n + 1, 0), width).to_host()
+        exp = orc.jaccard_index(host.slice(0, n), host.slice(1, n + 1), width, nthreads=4)
+        assert got.equals(exp), f"jaccard_index width {width}"
 
 
 def test_minhash64_reduction_edge(nv, orc):
