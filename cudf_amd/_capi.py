@@ -15,6 +15,7 @@ EXPORTS = [
     "nvtext_amd_last_error",
     "nvtext_amd_minhash",
     "nvtext_amd_minhash64",
+    "nvtext_amd_minhash_preallocated",
     "nvtext_amd_minhash_ngrams",
     "nvtext_amd_minhash64_ngrams",
     "nvtext_amd_jaccard_index",
@@ -166,6 +167,9 @@ def load():
     L.nvtext_amd_minhash.restype = C.c_int
     L.nvtext_amd_minhash.argtypes = [C.POINTER(StringsColumn), C.c_uint32, C.c_void_p, C.c_void_p,
                                      C.c_int64, C.c_int64] + common_tail
+    L.nvtext_amd_minhash_preallocated.restype = C.c_int
+    L.nvtext_amd_minhash_preallocated.argtypes = [C.POINTER(StringsColumn), C.c_uint32, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                                  C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     L.nvtext_amd_minhash64.restype = C.c_int
     L.nvtext_amd_minhash64.argtypes = [C.POINTER(StringsColumn), C.c_uint64, C.c_void_p, C.c_void_p,
                                        C.c_int64, C.c_int64] + common_tail

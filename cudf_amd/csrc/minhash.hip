@@ -21,6 +21,15 @@
 #include "windows.cuh"
 
 #include <limits>
+#include <mutex>
+
+// Scratch of nvtext_amd_minhash_preallocated, the entry point that allocates nothing: the extra-span counts of the
+// rows (rows + 1 values) and behind them the tile sums of the scans.  Every device holds its own copy of the array
+// for as long as the library is loaded (4.2 MB).
+constexpr int32_t kPreallocatedMaxRows = NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS;
+constexpr size_t kScratchPrefixBytes   = (static_cast<size_t>(kPreallocatedMaxRows) + 1 + 63) / 64 * 64 * sizeof(uint32_t);
+constexpr size_t kScratchScanBytes     = (static_cast<size_t>(kPreallocatedMaxRows) / nvtext_amd::kScanTile + 2) * sizeof(uint64_t);
+static __device__ __align__(256) unsigned char scratch[kScratchPrefixBytes + kScratchScanBytes];
 
 namespace nvtext_amd {
 namespace {
@@ -403,6 +412,39 @@ void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P,
   }
 }
 
+// The launches of one minhash call: the row offsets of the result, the number of extra workgroup-spans of every
+// row, then the two hashing kernels.  extra_prefix holds rows + 1 values, scan_tmp scan_temp_bytes(rows) bytes.
+template <typename T>
+void run_minhash(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, int32_t* offsets, T* child, int64_t child_size,
+                 uint32_t* extra_prefix, uint64_t* scan_tmp, hipStream_t stream)
+{
+  int32_t const rows = v.size;
+  if (v.use_mask) {
+    device_exclusive_scan(ValidTimesP{v, P}, static_cast<int64_t>(rows), offsets, scan_tmp, stream);
+  } else {
+    hipLaunchKernelGGL(uniform_offsets_kernel, dim3((rows + 1 + 255) / 256), dim3(256), 0, stream, offsets, rows, P);
+  }
+  device_exclusive_scan(ExtraParts{v}, static_cast<int64_t>(rows), extra_prefix, scan_tmp, stream);
+
+  if (child_size > 0) {
+    // every chunk of 64 K parameters hashes the windows again, and a lane without a parameter still folds:
+    // the K that leaves the fewest idle parameter slots, the larger K (fewer hashing passes) on a tie
+    int best_k = 1;
+    int64_t best_slots = std::numeric_limits<int64_t>::max();
+    for (int k = 1; k <= 5; ++k) {
+      int64_t const slots = static_cast<int64_t>((P + k * kWave - 1) / (k * kWave)) * k;
+      if (slots <= best_slots) { best_slots = slots; best_k = k; }
+    }
+    switch (best_k) {
+      case 5: launch_kernels<T, 5>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 4: launch_kernels<T, 4>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 3: launch_kernels<T, 3>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 2: launch_kernels<T, 2>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      default: launch_kernels<T, 1>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+    }
+  }
+}
+
 template <typename T>
 nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, const T* a, const T* b, int64_t a_count, int64_t b_count,
                                int32_t width, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out, int32_t type_id)
@@ -460,31 +502,8 @@ nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, c
     nvtext_amd_list_column_free(out, stream_, mr_);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "temporary allocation failed");
   }
-  if (v.use_mask) {
-    device_exclusive_scan(ValidTimesP{v, P}, static_cast<int64_t>(rows), out->offsets, scan_tmp.as<uint64_t>(), stream);
-  } else {
-    hipLaunchKernelGGL(uniform_offsets_kernel, dim3((rows + 1 + 255) / 256), dim3(256), 0, stream, out->offsets, rows, P);
-  }
-  device_exclusive_scan(ExtraParts{v}, static_cast<int64_t>(rows), extra.as<uint32_t>(), scan_tmp.as<uint64_t>(), stream);
-
-  T* child = static_cast<T*>(out->child);
-  if (out->child_size > 0) {
-    // every chunk of 64 K parameters hashes the windows again, and a lane without a parameter still folds:
-    // the K that leaves the fewest idle parameter slots, the larger K (fewer hashing passes) on a tie
-    int best_k = 1;
-    int64_t best_slots = std::numeric_limits<int64_t>::max();
-    for (int k = 1; k <= 5; ++k) {
-      int64_t const slots = static_cast<int64_t>((P + k * kWave - 1) / (k * kWave)) * k;
-      if (slots <= best_slots) { best_slots = slots; best_k = k; }
-    }
-    switch (best_k) {
-      case 5: launch_kernels<T, 5>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
-      case 4: launch_kernels<T, 4>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
-      case 3: launch_kernels<T, 3>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
-      case 2: launch_kernels<T, 2>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
-      default: launch_kernels<T, 1>(v, seed, a, b, P, width, out->offsets, extra.as<uint32_t>(), child, stream); break;
-    }
-  }
+  run_minhash<T>(v, seed, a, b, P, width, out->offsets, static_cast<T*>(out->child), out->child_size, extra.as<uint32_t>(),
+                 scan_tmp.as<uint64_t>(), stream);
   NVTEXT_HIP_TRY_OR(hipGetLastError(), nvtext_amd_list_column_free(out, stream_, mr_));
   return NVTEXT_AMD_SUCCESS;
 }
@@ -720,10 +739,72 @@ nvtext_amd_status minhash_ngrams_impl(const nvtext_amd_list_strings_column* inpu
   return NVTEXT_AMD_SUCCESS;
 }
 
+// ------------------------------------------------------------------ minhash without allocations
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// The address of this device's copy of the array (the array's name means nothing to host code).
+nvtext_amd_status scratch_of_current_device(unsigned char** out)
+{
+  int device = -1;
+  NVTEXT_HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "device index out of range");
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    NVTEXT_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[device] = p;
+  }
+  *out = static_cast<unsigned char*>(g_scratch_ptr[device]);
+  return NVTEXT_AMD_SUCCESS;
+}
+
 }  // namespace
 }  // namespace nvtext_amd
 
 extern "C" {
+
+nvtext_amd_status nvtext_amd_minhash_preallocated(const nvtext_amd_strings_column* input, uint32_t seed, const uint32_t* a, const uint32_t* b,
+                                                  int64_t a_count, int64_t b_count, int32_t width, void* stream_, int32_t* out_offsets,
+                                                  uint32_t* out_child, int64_t out_child_capacity, uint32_t* out_null_mask)
+{
+  using namespace nvtext_amd;
+  if (!input || !out_offsets) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
+  if (width < 2) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameter width should be an integer value of 2 or greater");
+  if (a_count <= 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B cannot be empty");
+  if (a_count != b_count) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B should have the same number of elements");
+  if (static_cast<uint64_t>(input->size) * static_cast<uint64_t>(a_count) >= static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
+    return fail(NVTEXT_AMD_OVERFLOW, "The number of parameters times the number of input rows exceeds the column size limit");
+  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
+  if (input->null_count > 0 && !input->null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
+  if (input->size > kPreallocatedMaxRows)
+    return fail(NVTEXT_AMD_INVALID_ARGUMENT, "more rows than nvtext_amd_minhash_preallocated takes (NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS)");
+  int32_t const rows       = input->size;
+  int32_t const P          = static_cast<int32_t>(a_count);
+  int64_t const child_size = static_cast<int64_t>(rows - input->null_count) * P;
+  if (child_size > out_child_capacity || (child_size > 0 && !out_child)) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "out_child is too small");
+  if (input->null_mask && !out_null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "the input has a null mask: out_null_mask is needed");
+
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (rows == 0) {
+    launch_fill_u32(reinterpret_cast<uint32_t*>(out_offsets), 0u, 1, stream);
+    NVTEXT_HIP_TRY(hipGetLastError());
+    return NVTEXT_AMD_SUCCESS;
+  }
+  unsigned char* base = nullptr;
+  nvtext_amd_status const st = scratch_of_current_device(&base);
+  if (st != NVTEXT_AMD_SUCCESS) return st;
+  uint32_t* const extra_prefix = reinterpret_cast<uint32_t*>(base);
+  uint64_t* const scan_tmp     = reinterpret_cast<uint64_t*>(base + kScratchPrefixBytes);
+
+  if (input->null_mask) launch_copy_bitmask(out_null_mask, input->null_mask, input->offset, rows, stream);
+  ColView const v = make_view(*input);
+  // every value of the scratch that the kernels read is written earlier in this same call: nothing to clear
+  run_minhash<uint32_t>(v, seed, a, b, P, width, out_offsets, out_child, child_size, extra_prefix, scan_tmp, stream);
+  NVTEXT_HIP_TRY(hipGetLastError());
+  return NVTEXT_AMD_SUCCESS;
+}
 
 nvtext_amd_status nvtext_amd_minhash(const nvtext_amd_strings_column* input, uint32_t seed, const uint32_t* a, const uint32_t* b, int64_t a_count,
                                      int64_t b_count, int32_t width, void* stream, const nvtext_amd_allocator* mr, nvtext_amd_list_column* out)

@@ -251,6 +251,25 @@ def minhash(input: DeviceStringsColumn, seed: int, a, b, width: int) -> DeviceLi
     return _wrap(out)
 
 
+MINHASH_PREALLOCATED_MAX_ROWS = 1048576  # NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS
+
+
+def minhash_preallocated(input: DeviceStringsColumn, seed: int, a, b, width: int, out_offsets, out_child, out_null_mask=None) -> None:
+    """nvtext_amd_minhash_preallocated: minhash into buffers of the caller (int32 tensors of size + 1 and of at least
+    (size - null_count) * len(a) values, and (size + 31) // 32 mask words when the input has a mask).  The call
+    allocates nothing on the device; the parameters must already be device tensors."""
+    L = _capi.load()
+    if not (0 <= int(seed) < 2**32):
+        raise ValueError("seed must fit uint32")
+    col = input._c()
+    st = L.nvtext_amd_minhash_preallocated(C.byref(col), int(seed), a.data_ptr() if a.numel() else None,
+                                           b.data_ptr() if b.numel() else None, a.numel(), b.numel(), int(width), _stream_handle(),
+                                           out_offsets.data_ptr(), out_child.data_ptr() if out_child.numel() else None,
+                                           out_child.numel(), out_null_mask.data_ptr() if out_null_mask is not None else None)
+    if st != _capi.SUCCESS:
+        _raise(st)
+
+
 def minhash64(input: DeviceStringsColumn, seed: int, a, b, width: int) -> DeviceListColumn:
     """nvtext::minhash64 (cpp/include/nvtext/minhash.hpp:109-116); pylibcudf minhash.pyx:88-141."""
     L = _capi.load()

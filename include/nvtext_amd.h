@@ -163,6 +163,29 @@ nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input,
                                        const nvtext_amd_allocator* mr,
                                        nvtext_amd_list_column* out);
 
+/* nvtext_amd_minhash for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid it).  It has no counterpart in the reference.  The caller brings the result buffers:
+ * out_offsets (input->size + 1 values), out_child (room for out_child_capacity values; the call needs
+ * (size - null_count) * param_count of them) and, when the input has a null mask, out_null_mask
+ * ((size + 31) / 32 words, bit i = row i of the view).  The values are those of nvtext_amd_minhash.
+ * Temporaries live in an array inside the library, one copy per device, so the call makes no allocation and
+ * releases nothing; in exchange it takes at most NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS rows (more is
+ * NVTEXT_AMD_INVALID_ARGUMENT), and two calls that overlap in time on one device race on that array: keep the
+ * calls of a device on one stream, or order them otherwise. */
+#define NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS 1048576
+nvtext_amd_status nvtext_amd_minhash_preallocated(const nvtext_amd_strings_column* input,
+                                                  uint32_t seed,
+                                                  const uint32_t* a,
+                                                  const uint32_t* b,
+                                                  int64_t a_count,
+                                                  int64_t b_count,
+                                                  int32_t width,
+                                                  void* stream,
+                                                  int32_t* out_offsets,
+                                                  uint32_t* out_child,
+                                                  int64_t out_child_capacity,
+                                                  uint32_t* out_null_mask);
+
 /* Replaces nvtext::minhash_ngrams (cpp/include/nvtext/minhash.hpp:156-163; cpp/src/text/minhash.cu:703-714).
  * The hashed items are runs of consecutive strings of a LIST<STRING> row: for element i the bytes from the
  * start of element i to the end of element min(i + ngrams, last) (adjacent elements are contiguous in the
