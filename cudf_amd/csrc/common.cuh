@@ -7,8 +7,11 @@
 #include <stdint.h>
 
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "../../include/nvtext_amd.h"
+#include "../../include/nvtext_amd_profile.h"
 
 namespace nvtext_amd {
 
@@ -64,6 +67,54 @@ struct Mr {
   hipStream_t stream;
   void* allocate(size_t bytes) const;
   void deallocate(void* p, size_t bytes) const;
+};
+
+// Device memory that an object keeps for as long as it lives.  With an allocator it comes from there and goes back
+// there on the stream of creation (a copy of the struct is kept: its ctx and that stream must outlive the object,
+// as a memory resource must outlive what it allocated); without one it is plain hipMalloc / hipFree.
+struct DeviceStore {
+  nvtext_amd_allocator alloc{};
+  bool has_alloc     = false;
+  hipStream_t stream = nullptr;
+  std::vector<std::pair<void*, size_t>> held;
+
+  void bind(const nvtext_amd_allocator* a, hipStream_t s)
+  {
+    has_alloc = a && a->allocate && a->deallocate;
+    if (has_alloc) alloc = *a;
+    stream = s;
+  }
+  void* allocate(size_t bytes)
+  {
+    void* p = nullptr;
+    if (has_alloc) {
+      p = alloc.allocate(alloc.ctx, bytes, stream);
+    } else if (hipMalloc(&p, bytes) != hipSuccess) {
+      p = nullptr;
+    }
+    if (p) held.emplace_back(p, bytes);
+    return p;
+  }
+  template <typename T>
+  bool allocate(T** out, size_t count)
+  {
+    *out = static_cast<T*>(allocate(count * sizeof(T)));
+    return *out != nullptr;
+  }
+  void release()
+  {
+    for (auto const& h : held) {
+      if (has_alloc)
+        alloc.deallocate(alloc.ctx, h.first, h.second, stream);
+      else
+        (void)hipFree(h.first);
+    }
+    held.clear();
+  }
+  DeviceStore() = default;
+  ~DeviceStore() { release(); }
+  DeviceStore(const DeviceStore&)            = delete;
+  DeviceStore& operator=(const DeviceStore&) = delete;
 };
 
 // Temporary released (stream-ordered) when it goes out of scope.

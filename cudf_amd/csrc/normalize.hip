@@ -24,6 +24,7 @@ struct nvtext_amd_character_normalizer {
   uint8_t* token_chars  = nullptr;  // device: the special tokens, sorted then lower-cased
   int32_t* token_offset = nullptr;  // device, tokens + 1
   int32_t tokens        = 0;
+  nvtext_amd::DeviceStore store;    // all of the above, from the allocator given at creation
 };
 
 namespace nvtext_amd {
@@ -697,7 +698,6 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
                                                          const nvtext_amd_allocator* mr, nvtext_amd_character_normalizer** out)
 {
   using namespace nvtext_amd;
-  (void)mr;  // the tables live as long as the object: plain hipMalloc / hipFree
   if (!out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out               = nullptr;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -780,47 +780,41 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
     nvtext_amd_character_normalizer_destroy(obj);
     return fail(e == hipErrorOutOfMemory ? NVTEXT_AMD_ALLOC_FAILED : NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
   };
-  hipError_t e = hipGetDevice(&obj->device);
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->ascii), sizeof(ascii));
-  if (e == hipSuccess) e = hipMemcpy(obj->ascii, ascii, sizeof(ascii), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->bmp), bmp.size() * sizeof(uint4));
-  if (e == hipSuccess) e = hipMemcpy(obj->bmp, bmp.data(), bmp.size() * sizeof(uint4), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->entries), entries.size() * sizeof(uint32_t));
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->second), second.size() * sizeof(uint64_t));
-  if (e == hipSuccess) e = hipMemcpy(obj->entries, entries.data(), entries.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemcpy(obj->second, second.data(), second.size() * sizeof(uint64_t), hipMemcpyHostToDevice);
-  if (e != hipSuccess) return fail_with(e);
-  if (!tokens.empty()) {
-    std::vector<int32_t> offsets(tokens.size() + 1, 0);
-    std::string chars;
-    for (size_t i = 0; i < tokens.size(); ++i) {
-      chars += tokens[i];
-      if (chars.size() > 0x7FFFFFFFull) {
-        nvtext_amd_character_normalizer_destroy(obj);
-        return fail(NVTEXT_AMD_OVERFLOW, "special tokens too large");
-      }
-      offsets[i + 1] = static_cast<int32_t>(chars.size());
+  obj->store.bind(mr, stream);
+  std::vector<int32_t> token_offsets(tokens.size() + 1, 0);
+  std::string token_chars;
+  for (size_t i = 0; i < tokens.size(); ++i) {
+    token_chars += tokens[i];
+    if (token_chars.size() > 0x7FFFFFFFull) {
+      nvtext_amd_character_normalizer_destroy(obj);
+      return fail(NVTEXT_AMD_OVERFLOW, "special tokens too large");
     }
-    e = hipMalloc(reinterpret_cast<void**>(&obj->token_offset), offsets.size() * sizeof(int32_t));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&obj->token_chars), std::max<size_t>(chars.size(), 1));
-    if (e == hipSuccess) e = hipMemcpy(obj->token_offset, offsets.data(), offsets.size() * sizeof(int32_t), hipMemcpyHostToDevice);
-    if (e == hipSuccess && !chars.empty()) e = hipMemcpy(obj->token_chars, chars.data(), chars.size(), hipMemcpyHostToDevice);
-    if (e != hipSuccess) return fail_with(e);
+    token_offsets[i + 1] = static_cast<int32_t>(token_chars.size());
   }
+  hipError_t e = hipGetDevice(&obj->device);
+  if (e != hipSuccess) return fail_with(e);
+  bool ok = obj->store.allocate(&obj->ascii, 128) && obj->store.allocate(&obj->bmp, bmp.size()) &&
+            obj->store.allocate(&obj->entries, entries.size()) && obj->store.allocate(&obj->second, second.size());
+  if (ok && !tokens.empty())
+    ok = obj->store.allocate(&obj->token_offset, token_offsets.size()) && obj->store.allocate(&obj->token_chars, std::max<size_t>(token_chars.size(), 1));
+  if (!ok) return fail_with(hipErrorOutOfMemory);
+  e = hipMemcpyAsync(obj->ascii, ascii, sizeof(ascii), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(obj->bmp, bmp.data(), bmp.size() * sizeof(uint4), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(obj->entries, entries.data(), entries.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(obj->second, second.data(), second.size() * sizeof(uint64_t), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess && !tokens.empty())
+    e = hipMemcpyAsync(obj->token_offset, token_offsets.data(), token_offsets.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess && !token_chars.empty()) e = hipMemcpyAsync(obj->token_chars, token_chars.data(), token_chars.size(), hipMemcpyHostToDevice, stream);
+  hipError_t const synced = hipStreamSynchronize(stream);  // the host copies die at return
+  if (e == hipSuccess) e = synced;
+  if (e != hipSuccess) return fail_with(e);
   *out = obj;
   return NVTEXT_AMD_SUCCESS;
 }
 
 void nvtext_amd_character_normalizer_destroy(nvtext_amd_character_normalizer* normalizer)
 {
-  if (!normalizer) return;
-  (void)hipFree(normalizer->ascii);
-  (void)hipFree(normalizer->bmp);
-  (void)hipFree(normalizer->entries);
-  (void)hipFree(normalizer->second);
-  (void)hipFree(normalizer->token_chars);
-  (void)hipFree(normalizer->token_offset);
-  delete normalizer;
+  delete normalizer;  // the store hands the tables back
 }
 
 nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_column* input, const nvtext_amd_character_normalizer* normalizer,

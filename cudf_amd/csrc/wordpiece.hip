@@ -112,6 +112,7 @@ __host__ __device__ __forceinline__ uint32_t carried_bit(uint32_t h) { return 0x
 
 struct nvtext_amd_wordpiece_vocabulary {
   nvtext_amd::VocabTable table{};
+  nvtext_amd::DeviceStore store;  // the tables, from the allocator given at creation
   void* d_slots     = nullptr;
   void* d_pool      = nullptr;
   void* d_lens      = nullptr;
@@ -1628,7 +1629,6 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
                                                          nvtext_amd_wordpiece_vocabulary** out)
 {
   using namespace nvtext_amd;
-  (void)mr;  // the tables live as long as the object: plain hipMalloc / hipFree
   if (!vocabulary || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nullptr;
   // cpp/src/text/wordpiece_tokenize.cu:217-218
@@ -1737,8 +1737,12 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   if (unk < 0) unk = host_find(slots, mask, blocks, "[unk]");
   v->slot_bytes = capacity * sizeof(HostSlot);
   v->pool_bytes = blocks.size() + 16;
-  if (hipMalloc(&v->d_slots, v->slot_bytes) != hipSuccess || hipMalloc(&v->d_pool, v->pool_bytes) != hipSuccess ||
-      hipMalloc(&v->d_lens, lens.size() * sizeof(uint32_t)) != hipSuccess || hipMalloc(&v->d_short, short_ids.size() * sizeof(int32_t)) != hipSuccess) {
+  v->store.bind(mr, stream);
+  v->d_slots = v->store.allocate(v->slot_bytes);
+  v->d_pool  = v->store.allocate(v->pool_bytes);
+  v->d_lens  = v->store.allocate(lens.size() * sizeof(uint32_t));
+  v->d_short = v->store.allocate(short_ids.size() * sizeof(int32_t));
+  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
@@ -1766,12 +1770,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
 
 void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
 {
-  if (!v) return;
-  if (v->d_slots) (void)hipFree(v->d_slots);
-  if (v->d_pool) (void)hipFree(v->d_pool);
-  if (v->d_lens) (void)hipFree(v->d_lens);
-  if (v->d_short) (void)hipFree(v->d_short);
-  delete v;
+  delete v;  // the store hands the tables back
 }
 
 int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* v) { return v ? v->table.unk_id : -1; }

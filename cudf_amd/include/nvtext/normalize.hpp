@@ -10,18 +10,34 @@ namespace nvtext {
 struct character_normalizer {
   /** Throws std::invalid_argument if special_tokens has nulls. */
   character_normalizer(bool do_lower_case, cudf::strings_column_view const& special_tokens, cuda::stream_ref stream = cudf::get_default_stream(),
-                       rmm::device_async_resource_ref mr = cudf::get_current_device_resource_ref())
-  {
-    nvtext_amd_strings_column const c = special_tokens.c_view();
-    nvtext_amd_allocator storage{};
-    detail::throw_on_error(nvtext_amd_character_normalizer_create(do_lower_case ? 1 : 0, &c, stream.get(), mr.c_allocator(storage), &_impl));
-  }
-  ~character_normalizer() { nvtext_amd_character_normalizer_destroy(_impl); }
-  character_normalizer(character_normalizer const&)            = delete;
-  character_normalizer& operator=(character_normalizer const&) = delete;
+                       rmm::device_async_resource_ref mr = cudf::get_current_device_resource_ref());
+  ~character_normalizer();
 
-  nvtext_amd_character_normalizer* _impl{nullptr};
+  struct character_normalizer_impl;
+  std::unique_ptr<character_normalizer_impl> _impl;
 };
+
+/** Owns the handle of the C ABI and, with it, the allocator struct that the handle's tables go back to. */
+struct character_normalizer::character_normalizer_impl {
+  nvtext_amd_allocator storage{};
+  nvtext_amd_character_normalizer* handle{nullptr};
+  character_normalizer_impl()                                            = default;
+  character_normalizer_impl(character_normalizer_impl const&)            = delete;
+  character_normalizer_impl& operator=(character_normalizer_impl const&) = delete;
+  ~character_normalizer_impl() { nvtext_amd_character_normalizer_destroy(handle); }
+};
+
+inline character_normalizer::character_normalizer(bool do_lower_case, cudf::strings_column_view const& special_tokens, cuda::stream_ref stream,
+                                                  rmm::device_async_resource_ref mr)
+  : _impl(std::make_unique<character_normalizer_impl>())
+{
+  nvtext_amd_strings_column const c = special_tokens.c_view();
+  detail::throw_on_error(
+    nvtext_amd_character_normalizer_create(do_lower_case ? 1 : 0, &c, stream.get(), mr.c_allocator(_impl->storage), &_impl->handle));
+}
+
+// defined where character_normalizer_impl is complete, as the owner of a unique_ptr to it must be
+inline character_normalizer::~character_normalizer() = default;
 
 namespace detail {
 // an empty STRING column view, the default of create_character_normalizer's special_tokens
@@ -64,7 +80,7 @@ inline std::unique_ptr<cudf::column> normalize_characters(cudf::strings_column_v
   nvtext_amd_strings_column const c = input.c_view();
   nvtext_amd_allocator storage{};
   nvtext_amd_strings_result out{};
-  detail::throw_on_error(nvtext_amd_normalize_characters(&c, normalizer._impl, stream.get(), mr.c_allocator(storage), &out));
+  detail::throw_on_error(nvtext_amd_normalize_characters(&c, normalizer._impl->handle, stream.get(), mr.c_allocator(storage), &out));
   return detail::make_strings_result(out, stream, mr);
 }
 

@@ -10,18 +10,33 @@ namespace nvtext {
 struct wordpiece_vocabulary {
   /** Throws std::invalid_argument if `input` is empty or has nulls. */
   wordpiece_vocabulary(cudf::strings_column_view const& input, cuda::stream_ref stream = cudf::get_default_stream(),
-                       rmm::device_async_resource_ref mr = cudf::get_current_device_resource_ref())
-  {
-    nvtext_amd_strings_column const c = input.c_view();
-    nvtext_amd_allocator storage{};
-    detail::throw_on_error(nvtext_amd_wordpiece_vocabulary_create(&c, stream.get(), mr.c_allocator(storage), &_impl));
-  }
-  ~wordpiece_vocabulary() { nvtext_amd_wordpiece_vocabulary_destroy(_impl); }
-  wordpiece_vocabulary(wordpiece_vocabulary const&)            = delete;
-  wordpiece_vocabulary& operator=(wordpiece_vocabulary const&) = delete;
+                       rmm::device_async_resource_ref mr = cudf::get_current_device_resource_ref());
+  ~wordpiece_vocabulary();
 
-  nvtext_amd_wordpiece_vocabulary* _impl{nullptr};
+  struct wordpiece_vocabulary_impl;
+  std::unique_ptr<wordpiece_vocabulary_impl> _impl;
 };
+
+/** Owns the handle of the C ABI and, with it, the allocator struct that the handle's tables go back to. */
+struct wordpiece_vocabulary::wordpiece_vocabulary_impl {
+  nvtext_amd_allocator storage{};
+  nvtext_amd_wordpiece_vocabulary* handle{nullptr};
+  wordpiece_vocabulary_impl()                                            = default;
+  wordpiece_vocabulary_impl(wordpiece_vocabulary_impl const&)            = delete;
+  wordpiece_vocabulary_impl& operator=(wordpiece_vocabulary_impl const&) = delete;
+  ~wordpiece_vocabulary_impl() { nvtext_amd_wordpiece_vocabulary_destroy(handle); }
+};
+
+inline wordpiece_vocabulary::wordpiece_vocabulary(cudf::strings_column_view const& input, cuda::stream_ref stream,
+                                                  rmm::device_async_resource_ref mr)
+  : _impl(std::make_unique<wordpiece_vocabulary_impl>())
+{
+  nvtext_amd_strings_column const c = input.c_view();
+  detail::throw_on_error(nvtext_amd_wordpiece_vocabulary_create(&c, stream.get(), mr.c_allocator(_impl->storage), &_impl->handle));
+}
+
+// defined where wordpiece_vocabulary_impl is complete, as the owner of a unique_ptr to it must be
+inline wordpiece_vocabulary::~wordpiece_vocabulary() = default;
 
 inline std::unique_ptr<wordpiece_vocabulary> load_wordpiece_vocabulary(
   cudf::strings_column_view const& input, cuda::stream_ref stream = cudf::get_default_stream(),
@@ -43,7 +58,7 @@ inline std::unique_ptr<cudf::column> wordpiece_tokenize(cudf::strings_column_vie
   nvtext_amd_strings_column const c = input.c_view();
   nvtext_amd_allocator storage{};
   nvtext_amd_list_column out{};
-  detail::throw_on_error(nvtext_amd_wordpiece_tokenize(&c, vocabulary._impl, max_words_per_row, stream.get(), mr.c_allocator(storage), &out));
+  detail::throw_on_error(nvtext_amd_wordpiece_tokenize(&c, vocabulary._impl->handle, max_words_per_row, stream.get(), mr.c_allocator(storage), &out));
   return detail::make_list_result(out, stream, mr);
 }
 

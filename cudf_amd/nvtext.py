@@ -12,6 +12,7 @@ every computation happens in libnvtext_amd.so.
 from __future__ import annotations
 
 import ctypes as C
+import sys
 from dataclasses import dataclass
 from typing import Dict, Optional
 
@@ -345,13 +346,13 @@ class CharacterNormalizer:
         self.do_lower_case = bool(do_lower_case)
 
     def __del__(self):
-        h = getattr(self, "_h", None)
-        if h:
+        # the tables go back through the allocator's callback into Python: not while the interpreter is shutting down
+        h, self._h = getattr(self, "_h", None), None
+        if h and not sys.is_finalizing():
             try:
                 _capi.load().nvtext_amd_character_normalizer_destroy(h)
             except Exception:
                 pass
-            self._h = None
 
 
 def normalize_characters(input: DeviceStringsColumn, normalizer: CharacterNormalizer) -> DeviceStringsColumn:
@@ -393,13 +394,13 @@ class WordPieceVocabulary:
         self.unk_id = int(L.nvtext_amd_wordpiece_vocabulary_unk_id(h))
 
     def __del__(self):
-        h = getattr(self, "_h", None)
-        if h:
+        # the tables go back through the allocator's callback into Python: not while the interpreter is shutting down
+        h, self._h = getattr(self, "_h", None), None
+        if h and not sys.is_finalizing():
             try:
                 _capi.load().nvtext_amd_wordpiece_vocabulary_destroy(h)
             except Exception:
                 pass
-            self._h = None
 
 
 def wordpiece_tokenize(input: DeviceStringsColumn, vocabulary: WordPieceVocabulary, max_words_per_row: int = 0) -> DeviceListColumn:

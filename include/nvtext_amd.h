@@ -235,8 +235,10 @@ void nvtext_amd_fixed_column_free(nvtext_amd_fixed_column* col, void* stream, co
 /* Replaces nvtext::load_wordpiece_vocabulary / wordpiece_vocabulary::wordpiece_vocabulary
  * (cpp/include/nvtext/wordpiece_tokenize.hpp:26-66; cpp/src/text/wordpiece_tokenize.cu:213-293).
  * Token id = row index.  Fails with INVALID_ARGUMENT for an empty vocabulary or one with nulls.
- * The object owns a device copy of the entries and its lookup tables; it is immutable and
- * may be shared by concurrent calls. */
+ * The object owns a device copy of the entries and its lookup tables, allocated through `mr` on `stream`
+ * (NULL: hipMalloc) and handed back the same way by _destroy, so the allocator's ctx and the stream must
+ * outlive the object, as a memory resource must outlive what it allocated.  It is immutable and may be
+ * shared by concurrent calls. */
 nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_strings_column* vocabulary,
                                                          void* stream,
                                                          const nvtext_amd_allocator* mr,
@@ -265,8 +267,9 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
  * removed (control and format characters; accents when lower-casing), replaced by a space (whitespace) or
  * replaced by its lower-cased, accent-stripped form of one to three code points.  special_tokens (NULL or
  * empty for none) are bracketed tokens such as "[PAD]" that keep their case and their brackets unpadded;
- * nulls among them give INVALID_ARGUMENT.  Belongs to the device that is current at creation; immutable and
- * shareable between concurrent calls. */
+ * nulls among them give INVALID_ARGUMENT.  The tables (14.4 MB) come from `mr` on `stream` (NULL: hipMalloc)
+ * and go back the same way in _destroy: the allocator's ctx and the stream must outlive the object.  Belongs to
+ * the device that is current at creation; immutable and shareable between concurrent calls. */
 nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case,
                                                          const nvtext_amd_strings_column* special_tokens,
                                                          void* stream,
@@ -290,16 +293,6 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
 
 /* Returns the buffers of a strings result to the allocator they came from. */
 void nvtext_amd_strings_result_free(nvtext_amd_strings_result* col, void* stream, const nvtext_amd_allocator* mr);
-
-/* Kernel timing for benchmarks.  The reference marks these entry points with NVTX ranges
- * (CUDF_FUNC_RANGE, cpp/src/text/minhash.cu:699, cpp/src/text/wordpiece_tokenize.cu:897) and is
- * timed from outside with Nsight; here the library itself brackets each of its kernels with HIP
- * events on the caller's stream while profiling is on.  nvtext_amd_profile_read synchronises the
- * recorded events, returns up to `capacity` (name, milliseconds) pairs in launch order and clears
- * the record; the names are static strings.  Off by default; not thread-safe against concurrent
- * entry-point calls. */
-void    nvtext_amd_profile_enable(int32_t on);
-int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t capacity);
 
 /* Releases the buffers of a result through the allocator that produced them. */
 void nvtext_amd_list_column_free(nvtext_amd_list_column* col, void* stream, const nvtext_amd_allocator* mr);

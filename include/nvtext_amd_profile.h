@@ -1,0 +1,28 @@
+/*
+ * nvtext_amd_profile.h -- kernel timing hooks of libnvtext_amd.so for benchmarks and profiling scripts.
+ * Not part of the product interface in nvtext_amd.h: the record behind these calls is one global list,
+ * not safe against entry-point calls on other threads.
+ */
+#ifndef NVTEXT_AMD_PROFILE_H
+#define NVTEXT_AMD_PROFILE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Kernel timing for benchmarks.  The reference marks these entry points with NVTX ranges
+ * (CUDF_FUNC_RANGE, cpp/src/text/minhash.cu:699, cpp/src/text/wordpiece_tokenize.cu:897) and is
+ * timed from outside with Nsight; here the library itself brackets each of its kernels with HIP
+ * events on the caller's stream while profiling is on.  nvtext_amd_profile_read synchronises the
+ * recorded events, returns up to `capacity` (name, milliseconds) pairs in launch order and clears
+ * the record; the names are static strings.  Off by default; not thread-safe against concurrent
+ * entry-point calls. */
+void    nvtext_amd_profile_enable(int32_t on);
+int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NVTEXT_AMD_PROFILE_H */

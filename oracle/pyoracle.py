@@ -213,9 +213,13 @@ class Vocabulary:
         self.unk_id = int(lib().oracle_vocab_unk_id(h))
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().oracle_vocab_destroy(self._h)
-            self._h = None
+        # at interpreter exit the module's globals may be gone already: then the process ends with the memory anyway
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib is not None:
+            try:
+                _lib.oracle_vocab_destroy(h)
+            except Exception:
+                pass
 
 
 def wordpiece_tokenize(col, vocab: Vocabulary, max_words_per_row: int = 0, nthreads: int = 1):

@@ -482,6 +482,58 @@ void test_wordpiece_edges()
   EXPECT_THROW(nvtext::load_wordpiece_vocabulary(cudf::strings_column_view(nulls.view)), std::invalid_argument);
 }
 
+// A memory resource that counts what is out: the vocabulary and the normalizer must take their tables from the
+// resource given to them and give every byte back when they die, as results and temporaries do.
+struct CountingResource final : rmm::mr::device_memory_resource {
+  long live_buffers = 0, live_bytes = 0, requests = 0;
+  void* allocate_async(std::size_t bytes, cuda::stream_ref) override
+  {
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) return nullptr;
+    ++live_buffers, ++requests, live_bytes += static_cast<long>(bytes);
+    return p;
+  }
+  void deallocate_async(void* p, std::size_t bytes, cuda::stream_ref) noexcept override
+  {
+    (void)hipDeviceSynchronize();
+    (void)hipFree(p);
+    --live_buffers, live_bytes -= static_cast<long>(bytes);
+  }
+};
+
+void test_objects_use_the_callers_resource()
+{
+  std::printf("objects take their tables from the caller's memory resource\n");
+  CountingResource mr;
+  {
+    auto vocabulary = make_strings({"ate", "brown", "cheese", "dog", "fox", "jumped", "lazy", "quick", "over", "the", "[UNK]"});
+    auto vocab      = nvtext::load_wordpiece_vocabulary(cudf::strings_column_view(vocabulary.view), cudf::get_default_stream(), mr);
+    CHECK(mr.live_buffers >= 1 && mr.live_bytes > 0);
+    long const held = mr.live_bytes;
+    auto input      = make_strings({"the quick brown fox jumped over the lazy dog", "the quick brown fox quacked"});
+    {
+      auto result = nvtext::wordpiece_tokenize(cudf::strings_column_view(input.view), *vocab, 0, cudf::get_default_stream(), mr);
+      L<int32_t> expected{{{9, 7, 1, 4, 5, 8, 9, 6, 3}}, {{9, 7, 1, 4, 10}}};
+      CHECK(same(download<int32_t>(*result), expected));
+      CHECK(mr.live_bytes > held);
+    }
+    CHECK(mr.live_bytes == held);  // the result and the temporaries are back, the tables are not
+  }
+  CHECK(mr.live_buffers == 0 && mr.live_bytes == 0);
+  {
+    auto normalizer = nvtext::create_character_normalizer(true, nvtext::detail::no_special_tokens(), cudf::get_default_stream(), mr);
+    CHECK(mr.live_bytes > 14000000);  // the code point tables
+    long const held = mr.live_bytes;
+    auto input      = make_strings({"Hello, World"});
+    {
+      auto result = nvtext::normalize_characters(cudf::strings_column_view(input.view), *normalizer, cudf::get_default_stream(), mr);
+      CHECK(download_strings(*result) == std::vector<Text>{Text{"hello ,  world"}});
+    }
+    CHECK(mr.live_bytes == held);
+  }
+  CHECK(mr.live_buffers == 0 && mr.live_bytes == 0);
+}
+
 int main()
 {
   int devices = 0;
@@ -498,6 +550,7 @@ int main()
   test_wordpiece();
   test_wordpiece_subwords();
   test_wordpiece_edges();
+  test_objects_use_the_callers_resource();
   HIP_OK(hipDeviceSynchronize());
   for (void* p : g_allocs) (void)hipFree(p);
   std::printf(g_failures ? "FAILED (%d checks)\n" : "ALL PASSED\n", g_failures);
