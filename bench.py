@@ -27,25 +27,27 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 4963c5f)"
 MEASURED_TRAFFIC_C2 = {
-    "wordpiece_word_kernel": (0, 0),
-    "wordpiece_oov_kernel": (0, 0),
-    "wordpiece_emit_kernel": (0, 0),
+    "range_first_row_kernel": (11875278, 123200),
+    "wordpiece_word_kernel": (1754914329, 1734655787),
+    "wordpiece_oov_kernel": (889721092, 1082239081),
+    "wordpiece_emit_kernel": (1391823477, 893789876),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (0, 0),
-    "normalize_write_kernel": (0, 0),
+    "normalize_count_kernel": (4575874773, 63532924),
+    "normalize_tile_rows_kernel": (73449477, 7941632),
+    "normalize_write_kernel": (5470172390, 4746099715),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
 # moves issue in fewer than 4 cycles).  The floor is the instruction sequence of the inner loop: uint32, one
-# v_mad_u64_u32 per product and one v_min3_u32 per two; uint64, three v_mad_u64_u32, and / shift / 64-bit add (2) of the
-# fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products.
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md"
+# v_mad_u64_u32 per product and one v_min3_u32 per two (1.5); uint64, three v_mad_u64_u32 and an add for the product,
+# and / shift / 64-bit add (2) of the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products (9.5).
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 4963c5f)"
 MINHASH_VALU = {
-    "C3": {"floor": 1.5, "measured": 2.0, "issue": 1.00},
-    "C4": {"floor": 8.5, "measured": 13.5, "issue": 1.00},
+    "C3": {"floor": 1.5, "measured": 2.02, "issue": 1.00},
+    "C4": {"floor": 9.5, "measured": 13.53, "issue": 1.11},
 }
 
 
@@ -189,6 +191,8 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="row-count multiplier of the headline workload (1.0 = 4M rows)")
     ap.add_argument("--minhash-scale", type=float, default=1.0, help="row-count multiplier of the C3/C4/C5 legs (0 = skip)")
     ap.add_argument("--reference-shapes", type=int, default=1, help="run the reference's own benchmark shapes (0 = skip)")
+    ap.add_argument("--legs", default="c2,c3,c4,ngrams,jaccard,c5,ref",
+                    help="which workloads to run (profiling runs take them one group at a time); without c2 the line has no value")
     ap.add_argument("--cpu-sample-rows", type=int, default=4_000_000, help="rows of the workload given to the host oracle")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -210,53 +214,79 @@ def main():
         threads, src = host_threads(orc)
         log(f"[bench] host oracle: {threads} threads ({src}); hardware_concurrency() = {orc.hardware_threads()}")
     side_steps = max(3, args.steps // 2)
+    legs = set(args.legs.split(","))
+    unknown = legs - {"c2", "c3", "c4", "ngrams", "jaccard", "c5", "ref"}
+    if unknown:
+        sys.exit(f"bench.py: unknown legs {sorted(unknown)}")
+    if args.minhash_scale <= 0:
+        legs -= {"c3", "c4", "ngrams", "jaccard", "c5"}
+    if not args.reference_shapes:
+        legs.discard("ref")
 
     # ------------------------------------------------------------------ headline: wordpiece_tokenize on C2
-    t0 = time.time()
-    wl = datagen.config2(args.scale)
-    host = wl.rows
-    log(f"[bench] C2 generated: rows={host.size} chars={host.chars_bytes / 1e9:.3f} GB in {time.time() - t0:.1f}s")
-    dcol = nvtext.DeviceStringsColumn.from_host(host)
-    dvoc = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(wl.vocab))
-    mw = wl.params["max_words_per_row"]
-    keep = {}
+    line = None
+    if "c2" in legs:
+        t0 = time.time()
+        wl = datagen.config2(args.scale)
+        host = wl.rows
+        log(f"[bench] C2 generated: rows={host.size} chars={host.chars_bytes / 1e9:.3f} GB in {time.time() - t0:.1f}s")
+        dcol = nvtext.DeviceStringsColumn.from_host(host)
+        dvoc = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(wl.vocab))
+        mw = wl.params["max_words_per_row"]
+        keep = {}
 
-    def step():
-        keep["o"] = nvtext.wordpiece_tokenize(dcol, dvoc, mw)
-        return keep["o"]
+        def step():
+            keep["o"] = nvtext.wordpiece_tokenize(dcol, dvoc, mw)
+            return keep["o"]
 
-    sec, head, kt = measure(step, args.steps, args.warmup, _capi, torch)
-    tokens = keep["o"].child_size
-    in_b = input_bytes(host)
-    out_b = 4 * tokens + 4 * (host.size + 1) + ((host.size + 7) // 8 if host.mask is not None else 0)
-    log(f"[bench] tokenize: {head}, tokens={tokens}")
-    roofline = hbm_roofline(in_b + out_b, sec, kt, MEASURED_TRAFFIC_C2 if args.scale == 1.0 else None)
-    roofline["all_kernels_ms"] = head["kernels_ms"]
-    roofline["peak_bytes_per_input_byte"] = round(head["peak_device_bytes"] / in_b, 3)
+        sec, head, kt = measure(step, args.steps, args.warmup, _capi, torch)
+        tokens = keep["o"].child_size
+        in_b = input_bytes(host)
+        out_b = 4 * tokens + 4 * (host.size + 1) + ((host.size + 7) // 8 if host.mask is not None else 0)
+        log(f"[bench] tokenize: {head}, tokens={tokens}")
+        roofline = hbm_roofline(in_b + out_b, sec, kt, MEASURED_TRAFFIC_C2 if args.scale == 1.0 else None)
+        roofline["all_kernels_ms"] = head["kernels_ms"]
+        # what a call holds beyond its result at its peak, per input byte
+        roofline["temporaries_bytes"] = head["peak_device_bytes"] - out_b
+        roofline["temporaries_per_input_byte"] = round((head["peak_device_bytes"] - out_b) / in_b, 3)
 
-    # ------------------------------------------------------------------ host oracle on a bounded sample (also the parity check)
-    cpu = None
-    parity = "skipped"
-    if orc:
-        n = min(args.cpu_sample_rows, host.size)
-        sample = host.slice(0, n)
-        ovoc = orc.Vocabulary(wl.vocab)
-        t0 = time.perf_counter()
-        exp = orc.wordpiece_tokenize(sample, ovoc, mw, nthreads=threads)
-        cpu_s = time.perf_counter() - t0
-        cpu = cpu_leg(orc, round(input_bytes(sample) / cpu_s / 1e9, 4), cpu_s,
-                      f"first {n} rows of the same workload ({sample.chars_bytes / 1e6:.0f} MB)")
-        cpu["mrows_per_s"] = round(n / cpu_s / 1e6, 3)
-        got = nvtext.wordpiece_tokenize(dcol.slice(0, n, 0), dvoc, mw).to_host()
-        parity = "PASS" if got.equals(exp) else "FAIL"
-        log(f"[bench] oracle: {cpu_s:.2f}s on {threads} threads; parity {parity}")
-        del exp, got
-    del dcol, keep
+        # ------------------------------------------------------------------ host oracle on a bounded sample (also the parity check)
+        cpu = None
+        parity = "skipped"
+        if orc:
+            n = min(args.cpu_sample_rows, host.size)
+            sample = host.slice(0, n)
+            ovoc = orc.Vocabulary(wl.vocab)
+            t0 = time.perf_counter()
+            exp = orc.wordpiece_tokenize(sample, ovoc, mw, nthreads=threads)
+            cpu_s = time.perf_counter() - t0
+            cpu = cpu_leg(orc, round(input_bytes(sample) / cpu_s / 1e9, 4), cpu_s,
+                          f"first {n} rows of the same workload ({sample.chars_bytes / 1e6:.0f} MB)")
+            cpu["mrows_per_s"] = round(n / cpu_s / 1e6, 3)
+            got = nvtext.wordpiece_tokenize(dcol.slice(0, n, 0), dvoc, mw).to_host()
+            parity = "PASS" if got.equals(exp) else "FAIL"
+            log(f"[bench] oracle: {cpu_s:.2f}s on {threads} threads; parity {parity}")
+            del exp, got
+        del dcol, keep
+
+        line = {
+            "metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline",
+            "value": round(in_b / sec / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(sec * 1e3, 4), "median_ms": head["median_ms"], "peak_device_bytes": head["peak_device_bytes"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "u8/int32", "data": "synthetic",
+            "config": {"workload": f"C2 wordpiece_tokenize x{args.scale}", "rows": host.size, "chars_bytes": host.chars_bytes,
+                       "vocab_entries": wl.vocab.size, "max_words_per_row": mw, "tokens_out": tokens, "offsets": "int32"},
+            "mrows_per_s": round(host.size / sec / 1e6, 3),
+            "roofline": roofline, "cpu_baseline": cpu, "parity_vs_oracle": parity,
+        }
 
     # ------------------------------------------------------------------ minhash legs (C3 uint32, C4 uint64)
     extra = {}
-    if args.minhash_scale > 0:
+    if legs & {"c3", "c4"}:
         for name, fn in (("C3", nvtext.minhash), ("C4", nvtext.minhash64)):
+            if name.lower() not in legs:
+                continue
             torch.cuda.empty_cache()
             t0 = time.time()
             w = datagen.CONFIGS[name](args.minhash_scale)
@@ -297,7 +327,7 @@ def main():
             del dc, keep
 
     # ------------------------------------------------------------------ minhash_ngrams over the words of C3 (a quarter of its rows)
-    if args.minhash_scale > 0:
+    if "ngrams" in legs:
         torch.cuda.empty_cache()
         t0 = time.time()
         w = datagen.config3(0.25 * args.minhash_scale)
@@ -335,7 +365,7 @@ def main():
         del dl, keep
 
     # ------------------------------------------------------------------ jaccard_index of neighbouring rows of C3 (a quarter of its rows)
-    if args.minhash_scale > 0:
+    if "jaccard" in legs:
         torch.cuda.empty_cache()
         w = datagen.config3(0.25 * args.minhash_scale)
         n = w.rows.size - 1
@@ -366,7 +396,7 @@ def main():
         del dc, d1, d2, keep
 
     # ------------------------------------------------------------------ C5: UTF-8 rows, int64 offsets, 250k vocabulary
-    if args.minhash_scale > 0:
+    if "c5" in legs:
         torch.cuda.empty_cache()
         t0 = time.time()
         w = datagen.config5(args.minhash_scale)
@@ -385,7 +415,9 @@ def main():
         ntok = keep["o"].child_size
         talg = ib + 4 * ntok + 4 * (w.rows.size + 1) + ((w.rows.size + 7) // 8 if w.rows.mask is not None else 0)
         tleg.update({"input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": ntok,
-                     "peak_bytes_per_input_byte": round(tleg["peak_device_bytes"] / ib, 3), "roofline": hbm_roofline(talg, tsec, tk)})
+                     "temporaries_bytes": tleg["peak_device_bytes"] - (talg - ib),
+                     "temporaries_per_input_byte": round((tleg["peak_device_bytes"] - (talg - ib)) / ib, 3),
+                     "roofline": hbm_roofline(talg, tsec, tk)})
         leg = {"workload": f"C5 x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes, "offsets": "int64",
                "vocab_entries": w.vocab.size, "tokenize": tleg}
         keep.clear()
@@ -442,20 +474,12 @@ def main():
         del dc, dv5, keep
 
     # ------------------------------------------------------------------ the reference's own benchmark shapes
-    if args.reference_shapes:
+    if "ref" in legs:
         extra["reference_shapes"] = reference_shapes(args, orc, _capi, datagen, nvtext, HostStringsColumn, np, torch)
 
-    line = {
-        "metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline",
-        "value": round(in_b / sec / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(sec * 1e3, 4), "median_ms": head["median_ms"], "peak_device_bytes": head["peak_device_bytes"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8/int32", "data": "synthetic",
-        "config": {"workload": f"C2 wordpiece_tokenize x{args.scale}", "rows": host.size, "chars_bytes": host.chars_bytes,
-                   "vocab_entries": wl.vocab.size, "max_words_per_row": mw, "tokens_out": tokens, "offsets": "int32"},
-        "mrows_per_s": round(host.size / sec / 1e6, 3),
-        "roofline": roofline, "cpu_baseline": cpu, "parity_vs_oracle": parity,
-    }
+    if line is None:
+        line = {"metric": "input GB/s + Mrows/s, wordpiece_tokenize & minhash, 1 MI355X, % of roofline", "value": None, "unit": "GB/s",
+                "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "legs": sorted(legs)}
     line.update(extra)
     print(json.dumps(line), flush=True)
 
