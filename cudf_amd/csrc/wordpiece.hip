@@ -12,23 +12,22 @@
 //     are also what gets hashed; the table for a 30k-entry vocabulary is 2 MiB and stays in L2.
 //     A hashed length filter (which key lengths exist for a given first three bytes) lets the
 //     longest-match search skip the lengths that cannot match.
-//   * probe pass: a wavefront is four groups of 16 lanes; a group owns a run of consecutive rows holding an
-//     equal share of the column's work and walks one row at a time in 256-byte chunks, 16 bytes per lane.
-//     Spaces become a 16-bit mask per lane with four SWAR operations per dword; word starts and ends are bit
-//     operations on that mask; DPP scans place the words of the chunk in an LDS list.  Then lanes <-> words,
-//     the four groups pooled: ONE probe per word.  A hit stores the token in the row's word arena (one slot
-//     per word, floor(bytes/2)+1 slots per row); a miss stores a marker and queues the word with its first
-//     16 bytes.
-//   * out-of-vocabulary pass: one lane per queued word, all lanes busy.  Words of up to 16 bytes are tokenized
-//     in registers, the greedy longest-match rule reduced to bit operations on a mask of candidate lengths,
-//     one table probe per trip; longer words go through a general state machine in a second kernel.  (Inside
-//     the probe pass this chain of dependent probes would idle 90 % of the lanes.)
-//   * a device-wide scan of the per-row token counts makes the int32 list offsets; the emit pass expands the
-//     word arena into the tokens, a block of rows with an even number of tokens per wavefront; the few words
-//     with more pieces than a result record keeps are tokenized again, into place, by a kernel of their own.
-//     No chars-sized temporary is written.
-//   * without a word limit, rows beyond 32 KiB are cut at spaces into pieces that go through all of this as
-//     rows of their own (a row is walked by 16 lanes: a row of megabytes would keep the device waiting).
+//   * the column's bytes are cut into tiles of 2048 bytes from the 16-byte aligned address below its first byte,
+//     without regard to rows; 16 tiles form a range, and every pass hands out ranges to wavefronts.
+//   * word pass: a wavefront takes a range and walks its tiles: bytes staged in LDS (the next tile's loads in
+//     flight), row starts marked as extra separators, spaces found with four SWAR operations per dword (16 bytes per
+//     lane), word starts and ends paired through scans, the words past a row's limit dropped; then lanes <->
+//     words: ONE lookup per word in straight-line code.  Every word gets one 4-byte slot, densely per range: its
+//     token, or the index of its 32-byte record (first 16 bytes, length, place) in the queue of words that are
+//     not in the vocabulary as they stand.  Rows get the number of words of their range before them.
+//   * out-of-vocabulary pass: one lane per queued word, lanes refilled from LDS as words finish.  Words of up to
+//     16 bytes are tokenized in registers, the greedy longest-match rule reduced to bit operations on a mask of
+//     candidate lengths, one table lookup per trip; the result (up to seven tokens and their number) takes the
+//     place of the queue record.  Longer words go through a general state machine in a second kernel.
+//   * a device-wide scan of the ranges' token counts gives every range its place in the result; the emit pass
+//     (a wavefront per range) expands the word slots into the tokens and turns the rows' word counts into list
+//     offsets.  The few words with more pieces than a record keeps are tokenized again, into place, by a kernel
+//     of their own.  No chars-sized temporary is written: 2.4 bytes of temporaries per input byte.
 #include "common.cuh"
 
 #include <algorithm>

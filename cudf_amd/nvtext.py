@@ -345,10 +345,11 @@ class CharacterNormalizer:
         self._h = h
         self.do_lower_case = bool(do_lower_case)
 
-    def __del__(self):
+    def __del__(self, _finalizing=sys.is_finalizing):
         # the tables go back through the allocator's callback into Python: not while the interpreter is shutting down
+        # (when this module's globals may be gone already, hence the default argument)
         h, self._h = getattr(self, "_h", None), None
-        if h and not sys.is_finalizing():
+        if h and not _finalizing():
             try:
                 _capi.load().nvtext_amd_character_normalizer_destroy(h)
             except Exception:
@@ -393,10 +394,11 @@ class WordPieceVocabulary:
         self._h = h
         self.unk_id = int(L.nvtext_amd_wordpiece_vocabulary_unk_id(h))
 
-    def __del__(self):
+    def __del__(self, _finalizing=sys.is_finalizing):
         # the tables go back through the allocator's callback into Python: not while the interpreter is shutting down
+        # (when this module's globals may be gone already, hence the default argument)
         h, self._h = getattr(self, "_h", None), None
-        if h and not sys.is_finalizing():
+        if h and not _finalizing():
             try:
                 _capi.load().nvtext_amd_wordpiece_vocabulary_destroy(h)
             except Exception:
