@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libnvtext_amd.so")
+# NVTEXT_AMD_LIB names another build of the library (experiments; the default is the in-tree build)
+LIB_PATH = os.environ.get("NVTEXT_AMD_LIB") or os.path.join(_HERE, "libnvtext_amd.so")
 
 SUCCESS, INVALID_ARGUMENT, OVERFLOW, LOGIC_ERROR, DEVICE_ERROR, ALLOC_FAILED = range(6)
 TYPE_INT32, TYPE_UINT32, TYPE_UINT64, TYPE_FLOAT32 = 3, 7, 8, 9

@@ -124,6 +124,9 @@ __host__ __device__ __forceinline__ void slots_of(uint32_t cp, NormTables const&
   }
 }
 
+constexpr int kWaveLeads = 256;  // first bytes of longer characters per wavefront (512 input bytes) that the counting pass lists
+
+template <bool SLOTS>
 struct NormLds {
   alignas(16) uint32_t raw[kRawWords];  // the input bytes of the tile and its surroundings, zero outside the column
   uint32_t ascii[128];                 // code points below 0x80: slot 0 | slot 1 << 8 | slot 2 << 16 | bytes << 24
@@ -131,9 +134,12 @@ struct NormLds {
     // first byte of slot k of tile position i - kSlotBase; only filled where special tokens can be.  A first byte
     // tells '[', ']', a space and a-z from everything else, which is all the special tokens look at or change.
     alignas(8) uint8_t slot[3][kSlots];
-    uint32_t staged[(kStageBytes + 8) / 4];  // afterwards: the tile's output bytes
+    uint32_t staged[(kStageBytes + 8) / 4 + 4];  // afterwards: the tile's output bytes (and room for the dwords of a string that starts at the last one)
   };
-  alignas(16) uint16_t prefix[kNormTile + 8];  // bytes the tile writes before each position; [tile] = all of them
+  union {
+    alignas(16) uint16_t prefix[kNormTile + 8];  // bytes the tile writes before each position; [tile] = all of them
+    uint16_t lead_pos[kNormThreads / kWave][kWaveLeads];  // (before that: the tile positions of the first bytes of a wavefront's longer characters)
+  };
   uint32_t scan[kNormThreads / kWave + 1];
   uint32_t bracket;  // some lane of the tile saw what can open a special token
 };
@@ -144,11 +150,13 @@ struct Owned {
 };
 
 // Slot `at` of the flat slot sequence (three per position).
-__device__ __forceinline__ uint8_t& flat_slot(NormLds& lds, int at) { return lds.slot[at % 3][at / 3]; }
+template <bool S>
+__device__ __forceinline__ uint8_t& flat_slot(NormLds<S>& lds, int at) { return lds.slot[at % 3][at / 3]; }
 
 // Compares the candidate in flat slots [from, to] (spaces and empty slots skipped, one byte per character) with
 // special token `i`: < 0, 0, > 0 as the candidate sorts before, equal to or after it.
-__device__ int compare_candidate(NormLds& lds, int from, int to, NormTables const& t, int32_t i)
+template <bool S>
+__device__ int compare_candidate(NormLds<S>& lds, int from, int to, NormTables const& t, int32_t i)
 {
   const uint8_t* tok = t.token_chars + t.token_offset[i];
   int32_t const tl   = t.token_offset[i + 1] - t.token_offset[i];
@@ -171,7 +179,8 @@ __device__ __forceinline__ bool has_byte(uint32_t v, uint32_t byte)
 
 // Whether a special token opens at slot index i (its slot 1 holds '['): the flat slot of its ']' if so, else -1.
 // special_tokens_kernel, cpp/src/text/normalize.cu:283-301.
-__device__ int token_opens_at(NormLds& lds, NormTables const& t, int i)
+template <bool S>
+__device__ int token_opens_at(NormLds<S>& lds, NormTables const& t, int i)
 {
   if (lds.slot[1][i] != '[') return -1;
   int const from = 3 * i + 1;
@@ -200,7 +209,8 @@ __device__ int token_opens_at(NormLds& lds, NormTables const& t, int i)
 // special_tokens_kernel (normalize.cu:270-316) over lds.slot, in two steps so that every decision reads unchanged
 // slots.  A lane looks at its own positions; the first kBefore lanes also at the positions before the tile (a '['
 // in the positions after the tile belongs to the next tile).
-__device__ void apply_special_tokens(NormLds& lds, NormTables const& t)
+template <bool S>
+__device__ void apply_special_tokens(NormLds<S>& lds, NormTables const& t)
 {
   int const tid = threadIdx.x;
   int found_to[kNormItems + 1];
@@ -272,7 +282,8 @@ __device__ __forceinline__ uint32_t wide_size(uint32_t w, NormTables const& t)
 }
 
 // The slots (and sizes) of the eight positions whose bytes are lo64; hi64 = bytes 4..11.  Returns the bytes they produce.
-__device__ __forceinline__ uint32_t owned_slots(NormLds const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t, Owned& mine,
+template <bool S>
+__device__ __forceinline__ uint32_t owned_slots(NormLds<S> const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t, Owned& mine,
                                                 uint32_t (&size)[kNormItems])
 {
   uint32_t sum = 0;
@@ -311,21 +322,114 @@ __device__ __forceinline__ uint32_t owned_slots(NormLds const& lds, uint64_t lo6
   return sum;
 }
 
-// The same count without the slots, for the pass that only sizes the output.
-__device__ __forceinline__ uint32_t owned_size(NormLds const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t)
+// The bytes of up to three slots side by side, first slot first: (lo, hi) = bytes 0..7 and 8..11.
+__device__ __forceinline__ void slots_to_string(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t& d0, uint32_t& d1, uint32_t& d2)
+{
+  uint32_t const b0  = bytes_of(s0);
+  uint32_t const b01 = b0 + bytes_of(s1);  // <= 8
+  uint64_t lo        = s0 | (static_cast<uint64_t>(s1) << (8u * b0));
+  uint64_t const t   = s2;
+  uint32_t const sh  = 8u * b01;
+  lo |= b01 < 8u ? t << (sh & 63u) : 0ull;
+  d2 = b01 >= 8u ? s2 : b01 > 4u ? static_cast<uint32_t>(t >> ((64u - sh) & 63u)) : 0u;
+  d0 = static_cast<uint32_t>(lo);
+  d1 = static_cast<uint32_t>(lo >> 32);
+}
+
+// owned_slots for the pass that writes: what each position turns into as a string of bytes (mine.s[j][0..2] = bytes
+// 0..11, zero padded) instead of slots, ready to be placed.
+template <bool S>
+__device__ __forceinline__ uint32_t owned_strings(NormLds<S> const& lds, uint64_t lo64, uint64_t hi64, NormTables const& t, Owned& mine,
+                                                  uint32_t (&size)[kNormItems])
 {
   uint32_t sum = 0;
 #pragma unroll
   for (int j = 0; j < kNormItems; ++j) {
     uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
-    uint32_t const e = lds.ascii[b & 0x7Fu];
-    sum += b < 0x80u ? e >> 24 : 0u;
+    uint32_t const e = lds.ascii[b & 0x7Fu];  // read in any case: no branch
+    uint32_t const d = b < 0x80u ? e : 0u;
+    mine.s[j][0]     = d & 0xFFFFFFu;  // one byte per slot, empty slots last: the slots side by side are the string
+    mine.s[j][1]     = 0u;
+    mine.s[j][2]     = 0u;
+    size[j]          = d >> 24;
+    sum += size[j];
   }
-  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;
+  uint64_t leads = lo64 & (lo64 << 1) & 0x8080808080808080ull;  // bit 7 of the bytes >= 0xC0
   while (leads) {
     int const at = (__ffsll(static_cast<long long>(leads)) - 1) >> 3;
     leads &= leads - 1ull;
-    sum += wide_size(static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3))), t);
+    uint32_t const w = static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3)));
+    uint32_t s0, s1, s2, d0, d1, d2;
+    uint32_t const bytes = wide_slots(w, t, s0, s1, s2);
+    slots_to_string(s0, s1, s2, d0, d1, d2);
+    sum += bytes;
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+      uint32_t const here = static_cast<uint32_t>((static_cast<int32_t>(j ^ at) - 1) >> 31);  // all ones where j == at
+      mine.s[j][0] = (mine.s[j][0] & ~here) | (d0 & here);
+      mine.s[j][1] = (mine.s[j][1] & ~here) | (d1 & here);
+      mine.s[j][2] = (mine.s[j][2] & ~here) | (d2 & here);
+      size[j]      = (size[j] & ~here) | (bytes & here);
+    }
+  }
+  return sum;
+}
+
+__device__ __forceinline__ void wave_lds_sync()
+{
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The bytes that the wavefront's 512 positions produce, for the pass that only sizes the output (a lane's return value
+// holds the sizes of characters that are not its own: only the sum over the wavefront means something).
+// One-byte characters go through the table in LDS, lanes <-> bytes.  The first bytes of longer characters are few
+// and unevenly spread (none in English text, every other byte in Cyrillic or Greek), and each needs a read of the
+// code point tables: the wavefront lists them and goes through the list lanes <-> characters, every lane at work.
+// `byte0` = the byte offset in lds.raw of the tile's first byte.
+template <bool SLOTS>
+__device__ __forceinline__ uint32_t owned_dense(NormLds<SLOTS>& lds, uint64_t lo64, uint64_t hi64, uint32_t byte0, NormTables const& t)
+{
+  uint32_t sum = 0;
+#pragma unroll
+  for (int j = 0; j < kNormItems; ++j) {
+    uint32_t const b = static_cast<uint32_t>(lo64 >> (8 * j)) & 0xFFu;
+    uint32_t const e = lds.ascii[b & 0x7Fu];  // read in any case: no branch
+    sum += b < 0x80u ? e >> 24 : 0u;
+  }
+  uint64_t const leads  = lo64 & (lo64 << 1) & 0x8080808080808080ull;  // bit 7 of the bytes >= 0xC0
+  uint32_t const mine_n = static_cast<uint32_t>(__builtin_popcountll(leads));
+  uint32_t const incl   = wave_inclusive_scan(mine_n);
+  uint32_t const first  = incl - mine_n;
+  uint32_t const all    = wave_bcast(incl, kWave - 1);
+  if (all == 0) return sum;
+  if (all > static_cast<uint32_t>(kWaveLeads)) {
+    // more than every other byte begins a character: not text; every lane walks its own
+    uint64_t l = leads;
+    while (l) {
+      int const at = (__ffsll(static_cast<long long>(l)) - 1) >> 3;
+      l &= l - 1ull;
+      sum += wide_size(static_cast<uint32_t>((at < 4 ? lo64 : hi64) >> (8 * (at & 3))), t);
+    }
+    return sum;
+  }
+  int const lane       = lane_id();
+  uint16_t* const list = lds.lead_pos[threadIdx.x / kWave];
+  {
+    uint32_t i = first;
+#pragma unroll
+    for (int j = 0; j < kNormItems; ++j) {
+      bool const is = ((leads >> (8 * j + 7)) & 1ull) != 0;
+      if (is) list[i] = static_cast<uint16_t>(kNormItems * threadIdx.x + j);
+      i += is ? 1u : 0u;
+    }
+  }
+  wave_lds_sync();
+  for (uint32_t r = lane; r < all; r += kWave) {
+    uint32_t const off = byte0 + list[r];
+    uint32_t const w   = __builtin_amdgcn_alignbit(lds.raw[(off >> 2) + 1], lds.raw[off >> 2], 8u * (off & 3u));
+    sum += wide_size(w, t);
   }
   return sum;
 }
@@ -333,7 +437,7 @@ __device__ __forceinline__ uint32_t owned_size(NormLds const& lds, uint64_t lo64
 // One tile: the slots of the lane's positions, special tokens applied.  Returns the bytes they produce.  Without
 // SLOTS only that number is wanted: the slots are then built only in tiles that may hold a special token.
 template <bool SLOTS>
-__device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t, Owned& mine,
+__device__ __forceinline__ uint32_t tile_slots(NormLds<SLOTS>& lds, const uint8_t* chars, int64_t t0, int64_t n, NormTables const& t, Owned& mine,
                                                uint32_t (&size)[kNormItems])
 {
   int const tid = threadIdx.x;
@@ -374,7 +478,12 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
   uint32_t const next = __builtin_amdgcn_alignbit(r3, r2, shift);
   uint64_t const lo64 = (static_cast<uint64_t>(own1) << 32) | own0;
   uint64_t const hi64 = (static_cast<uint64_t>(next) << 32) | own1;
-  uint32_t sum        = SLOTS ? owned_slots(lds, lo64, hi64, t, mine, size) : owned_size(lds, lo64, hi64, t);
+  // (the pass that wants the slots keeps them in registers all the way: listing the longer characters for it as well
+  // saves it 4 % of its instructions and costs it two of its seven wavefronts per SIMD, 8.6 -> 10.7 ms on the
+  // multilingual workload; the pass that only counts gains 13 % from the list)
+  uint32_t sum;
+  if constexpr (SLOTS) sum = owned_strings(lds, lo64, hi64, t, mine, size);
+  else sum = owned_dense(lds, lo64, hi64, mis + kRawBefore, t);
 
   if (t.tokens > 0) {
     // A special token starts at a position whose slot 1 is '['.  Tiles without one skip the exchange through LDS.
@@ -383,8 +492,9 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
     // needed) and, when the slots have not been built, for the lane's own bytes (a superset, which is harmless).
     bool bracket = false;
     if (SLOTS) {
+      // (strings: a '[' is padded like all punctuation, so it is the middle byte of " [ ")
 #pragma unroll
-      for (int j = 0; j < kNormItems; ++j) bracket |= mine.s[j][1] == '[';
+      for (int j = 0; j < kNormItems; ++j) bracket |= ((mine.s[j][0] >> 8) & 0xFFu) == '[';
     } else {
       bracket = has_byte(own0, '[') || has_byte(own1, '[');
       if ((lo64 & (lo64 << 1) & 0x8080808080808080ull) != 0)
@@ -399,7 +509,7 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
     if (ballot64(bracket) != 0 && lane_id() == 0) lds.bracket = 1u;
     lds_barrier();
     if (lds.bracket != 0u) {
-      if (!SLOTS) owned_slots(lds, lo64, hi64, t, mine, size);
+      owned_slots(lds, lo64, hi64, t, mine, size);  // (the slots themselves, whatever mine held)
 #pragma unroll
       for (int k = 0; k < 3; ++k) {
         uint32_t a = 0, b = 0;
@@ -454,6 +564,7 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
         }
         size[j] = bytes_of(mine.s[j][0]) + bytes_of(mine.s[j][1]) + bytes_of(mine.s[j][2]);
         sum += size[j];
+        if (SLOTS) slots_to_string(mine.s[j][0], mine.s[j][1], mine.s[j][2], mine.s[j][0], mine.s[j][1], mine.s[j][2]);
       }
     }
   }
@@ -464,7 +575,7 @@ __device__ __forceinline__ uint32_t tile_slots(NormLds& lds, const uint8_t* char
 __global__ void __launch_bounds__(kNormThreads, 8) normalize_count_kernel(const uint8_t* __restrict__ chars, int64_t n, NormTables t,
                                                                        uint32_t* __restrict__ tile_bytes)
 {
-  __shared__ NormLds lds;
+  __shared__ NormLds<false> lds;
   int64_t const t0 = static_cast<int64_t>(blockIdx.x) * kNormTile;
   Owned mine;
   uint32_t size[kNormItems];
@@ -496,15 +607,16 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
                                                                        const int32_t* __restrict__ tile_row, uint8_t* __restrict__ out_chars,
                                                                        void* __restrict__ out_offsets, int offsets_are_int64)
 {
-  __shared__ NormLds lds;
+  __shared__ NormLds<true> lds;
   int const tid        = threadIdx.x;
   int64_t const t0     = static_cast<int64_t>(blockIdx.x) * kNormTile;
-  int64_t const t1     = min(t0 + kNormTile, n);
   uint64_t const base  = tile_offset[blockIdx.x];
   // the rows that start in this tile are looked up now; the barriers below do not wait for global loads, so this
   // one is back when the tile is done
   int64_t const rows     = col.size;
   int64_t const my_row   = static_cast<int64_t>(tile_row[blockIdx.x]) + tid;
+  // the rows that start in this tile end where the next tile's begin (the last tile also takes the end of the last row)
+  int64_t const row_end  = blockIdx.x + 1 == gridDim.x ? rows + 1 : static_cast<int64_t>(tile_row[blockIdx.x + 1]);
   uint32_t start_lo = 0, start_hi = 0;  // the raw offset entry; not touched before the end
   if (my_row <= rows) {
     if (col.is64) {
@@ -518,6 +630,12 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
   Owned mine;
   uint32_t size[kNormItems];
   uint32_t const sum = tile_slots<true>(lds, col.chars + first, t0, n, t, mine, size);
+  // the buffer that the output bytes are assembled in starts out as zeros (the scan's barriers stand between this
+  // and the first byte placed); in a tile that went through the special tokens it lies where the slots' first bytes
+  // were, which the other wavefronts may still be reading
+  if (t.tokens > 0 && lds.bracket != 0u) lds_barrier();
+  for (int i = tid; i < static_cast<int>(sizeof(lds.staged) / 16); i += kNormThreads) reinterpret_cast<uint4*>(lds.staged)[i] = make_uint4(0u, 0u, 0u, 0u);
+  if (tid < static_cast<int>(sizeof(lds.staged) % 16) / 4) lds.staged[sizeof(lds.staged) / 16 * 4 + tid] = 0u;
   uint32_t total;
   uint32_t const before = block_exclusive_scan_lds<kNormThreads>(sum, lds.scan, &total);
   {
@@ -542,17 +660,18 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
     uint8_t* const sb   = reinterpret_cast<uint8_t*>(lds.staged);
     uint32_t o          = lead + before;
     uint32_t const mine_end = o + sum;
-    uint32_t all = 0;
+    uint32_t big = 0;
 #pragma unroll
-    for (int j = 0; j < kNormItems; ++j) all |= mine.s[j][0] | mine.s[j][1] | mine.s[j][2];
-    if (ballot64(all > 0xFFu) == 0) {
-      // every character of the wavefront's output is one byte: a position's (up to three) bytes travel together.
-      // A position that starts in the lane's last three bytes is skipped; those bytes are kept in `last` (the
-      // four bytes written last, newest on top) and stored one by one at the end.
+    for (int j = 0; j < kNormItems; ++j) big |= (mine.s[j][0] >> 24) | mine.s[j][1] | mine.s[j][2];
+    if (ballot64(big != 0u) == 0) {
+      // no position of the wavefront turns into more than three bytes: a position's bytes travel together, as one
+      // (unaligned) dword whose spare bytes the next positions overwrite.  A position that starts in the lane's last
+      // three bytes is skipped; those bytes are kept in `last` (the four bytes written last, newest on top) and
+      // stored one by one at the end.
       uint32_t last = 0;
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
-        uint32_t const three = mine.s[j][0] | (mine.s[j][1] << 8) | (mine.s[j][2] << 16);
+        uint32_t const three = mine.s[j][0];
         if (size[j] != 0u && o + 4u <= mine_end) __builtin_memcpy(sb + o, &three, 4);
         last = __builtin_amdgcn_alignbit(three, last, 8u * size[j]);
         o += size[j];
@@ -561,23 +680,25 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
       if (sum >= 2u) sb[mine_end - 2u] = static_cast<uint8_t>(last >> 16);
       if (sum >= 3u) sb[mine_end - 3u] = static_cast<uint8_t>(last >> 8);
     } else {
+      // longer strings: every position's bytes (zero padded) are or-ed into the aligned dwords they fall into;
+      // the buffer was cleared, and what the neighbours put into a shared dword is theirs
+      bool const past8 = ballot64(mine.s[0][2] | mine.s[1][2] | mine.s[2][2] | mine.s[3][2] | mine.s[4][2] | mine.s[5][2] | mine.s[6][2] |
+                                  mine.s[7][2]) != 0;
 #pragma unroll
       for (int j = 0; j < kNormItems; ++j) {
-#pragma unroll
-        for (int k = 0; k < 3; ++k) {
-          uint32_t v = mine.s[j][k];
-          if (v) {
-            if (o + 4u <= mine_end) {
-              __builtin_memcpy(sb + o, &v, 4);
-              o += bytes_of(v);
-            } else {
-              do {
-                sb[o++] = static_cast<uint8_t>(v);
-                v >>= 8;
-              } while (v);
-            }
-          }
+        uint32_t const sh   = 8u * (o & 3u);
+        uint32_t* const at  = lds.staged + (o >> 2);
+        uint64_t const a    = static_cast<uint64_t>(mine.s[j][0]) << sh;
+        uint64_t const b    = static_cast<uint64_t>(mine.s[j][1]) << sh;
+        atomicOr(at, static_cast<uint32_t>(a));
+        atomicOr(at + 1, static_cast<uint32_t>(a >> 32) | static_cast<uint32_t>(b));
+        atomicOr(at + 2, static_cast<uint32_t>(b >> 32));
+        if (past8) {  // (a character that turns into three characters of three bytes, or into characters beyond U+FFFF)
+          uint64_t const c = static_cast<uint64_t>(mine.s[j][2]) << sh;
+          atomicOr(at + 2, static_cast<uint32_t>(c));
+          atomicOr(at + 3, static_cast<uint32_t>(c >> 32));
         }
+        o += size[j];
       }
     }
     lds_barrier();
@@ -599,26 +720,16 @@ __global__ void __launch_bounds__(kNormThreads) normalize_write_kernel(ColView c
     // more than four output bytes per input byte (only input that is not UTF-8 gets there): byte by byte
     uint8_t* o = dst + before;
 #pragma unroll
-    for (int j = 0; j < kNormItems; ++j) {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        uint32_t v = mine.s[j][k];
-        while (v) {
-          *o++ = static_cast<uint8_t>(v);
-          v >>= 8;
-        }
-      }
-    }
+    for (int j = 0; j < kNormItems; ++j)
+      for (uint32_t k = 0; k < size[j]; ++k) *o++ = static_cast<uint8_t>((k < 4 ? mine.s[j][0] : k < 8 ? mine.s[j][1] : mine.s[j][2]) >> (8u * (k & 3u)));
     lds_barrier();  // lds.prefix is complete for the rows below
   }
 
   // rows whose first byte lies in [t0, t1) -- in [t0, n] for the last tile -- start at base + prefix
-  bool const last_tile   = blockIdx.x == gridDim.x - 1;
   int64_t const my_start = (col.is64 ? static_cast<int64_t>((static_cast<uint64_t>(start_hi) << 32) | start_lo)
                                      : static_cast<int64_t>(static_cast<int32_t>(start_lo))) - first;
-  for (int64_t r = my_row; r <= rows; r += kNormThreads) {
+  for (int64_t r = my_row; r < row_end; r += kNormThreads) {  // (more than one trip only in a tile of very short rows)
     int64_t const p = r == my_row ? my_start : col.off(r) - first;
-    if (p > t1 || (p == t1 && !last_tile)) break;
     uint64_t const at = base + lds.prefix[p - t0];
     if (offsets_are_int64) static_cast<int64_t*>(out_offsets)[r] = static_cast<int64_t>(at);
     else static_cast<int32_t*>(out_offsets)[r] = static_cast<int32_t>(at);
