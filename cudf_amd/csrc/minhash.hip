@@ -219,11 +219,23 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       uint32_t count = 0;  // compacted hashes so far (wave-uniform)
+      // In a tile of one-byte characters of a row of at least `width` bytes every window is `width` bytes long: the
+      // hash then runs with a length that the compiler knows to be the same in every lane (its loops over the
+      // blocks and the tail become scalar branches instead of masked ones).
+      bool const plain         = all_ascii && n >= static_cast<int64_t>(width);
+      uint32_t const width_all = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(width));
       for (uint32_t q = 0; q < cnt; q += kWave) {
         uint32_t const p = q + lane;
         bool valid       = false;
         T hv             = 0;
-        if (p < cnt) {
+        if (plain) {
+          valid = p < cnt && n - (base + p) >= static_cast<int64_t>(width_all);
+          if (valid) {
+            WordSrc const src{lds.bytes, mis + p};
+            hv = H::hash(src, width_all, seed);
+            hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
+          }
+        } else if (p < cnt) {
           int64_t const gpos = base + p;
           WordSrc const src{lds.bytes, mis + p};
           uint32_t hlen;
