@@ -1449,7 +1449,7 @@ __global__ void __launch_bounds__(kTokThreads, 8) wordpiece_emit_kernel(uint32_t
     uint32_t row_k = r_win + lane < r_end ? static_cast<uint32_t>(offsets[r_win + lane]) : 0xFFFFFFFFu;
     // three stages in flight: the slot two rounds ahead, the queue record of a word from the queue one round ahead, the
     // round being written (the pass is bound by the latency of its reads)
-    auto load_slot = [&](uint32_t k) -> uint32_t { return k < nwords ? slots[k] : 0u; };
+    auto load_slot = [&](uint32_t k) -> uint32_t { return k < nwords ? load_stream(slots + k) : 0u; };
     auto load_record = [&](uint32_t k, uint32_t v, uint4& ra, uint4& rb) {
       if (k < nwords && (v & kOovMark) != 0 && v != 0xFFFFFFFFu) {
         const uint4* const src = reinterpret_cast<const uint4*>(queue + (v & ~kOovMark));
