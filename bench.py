@@ -27,27 +27,27 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 4963c5f)"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 75be55d)"
 MEASURED_TRAFFIC_C2 = {
-    "range_first_row_kernel": (11875278, 123200),
-    "wordpiece_word_kernel": (1754914329, 1734655787),
-    "wordpiece_oov_kernel": (889721092, 1082239081),
-    "wordpiece_emit_kernel": (1391823477, 893789876),
+    "range_first_row_kernel": (11875775, 123200),
+    "wordpiece_word_kernel": (1756246204, 1735976310),
+    "wordpiece_oov_kernel": (889776598, 1082622472),
+    "wordpiece_emit_kernel": (1391750247, 874985493),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (4575874773, 63532924),
-    "normalize_tile_rows_kernel": (73449477, 7941632),
-    "normalize_write_kernel": (5470172390, 4746099715),
+    "normalize_count_kernel": (4575177542, 63532923),
+    "normalize_tile_rows_kernel": (73449996, 7941631),
+    "normalize_write_kernel": (5469626416, 4672540030),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
 # moves issue in fewer than 4 cycles).  The floor is the instruction sequence of the inner loop: uint32, one
 # v_mad_u64_u32 per product and one v_min3_u32 per two (1.5); uint64, three v_mad_u64_u32 and an add for the product,
 # and / shift / 64-bit add (2) of the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products (9.5).
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 4963c5f)"
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 75be55d)"
 MINHASH_VALU = {
-    "C3": {"floor": 1.5, "measured": 2.02, "issue": 1.00},
-    "C4": {"floor": 9.5, "measured": 13.53, "issue": 1.11},
+    "C3": {"floor": 1.5, "measured": 1.98, "issue": 1.00},
+    "C4": {"floor": 9.5, "measured": 13.39, "issue": 1.11},
 }
 
 
