@@ -84,8 +84,14 @@ struct VocabTable {
   // Direct tables for keys of one and two bytes: short_ids[kind * 65536 + (byte0 | byte1 << 8)] for two bytes,
   // short_ids[131072 + kind * 256 + byte0] for one; the token id, or INT32_MIN when there is no such key.
   const int32_t* short_ids;
+  // The length filter once more, exact, for the keys of the second key space (the "##" entries) that begin with three
+  // lower-case ASCII letters c0 c1 c2: letters3[((c0 - 'a') * 26 + (c1 - 'a')) * 26 + (c2 - 'a')] has bit i set when
+  // some such key is i + 3 bytes long (3..18).  Small enough for LDS.
+  const uint16_t* letters3;
 };
 constexpr uint32_t kShortIds = 2 * 65536 + 2 * 256;
+constexpr uint32_t kLetters3 = 26 * 26 * 26;
+constexpr uint32_t kLetters2 = 26 * 26;
 
 __host__ __device__ __forceinline__ uint32_t length_filter_index(uint32_t kind, uint32_t first3)
 {
@@ -116,6 +122,7 @@ struct nvtext_amd_wordpiece_vocabulary {
   void* d_pool      = nullptr;
   void* d_lens      = nullptr;
   void* d_short     = nullptr;
+  void* d_letters   = nullptr;
   size_t slot_bytes = 0;
   size_t pool_bytes = 0;
   int32_t entries   = 0;
@@ -578,6 +585,33 @@ struct ShortWord {
     return o;
   }
 
+  // The opening of the next piece of the word (second key space), when the piece before it has been dropped.  Pieces
+  // that begin with lower-case ASCII letters, as nearly all do in text of that alphabet, get it from tables in LDS
+  // (l3: the exact length filter by three letters; pair: the ids of the two-letter keys; both of the second key
+  // space); the others from the tables in memory, as request() does.
+  __device__ __forceinline__ Opening request_next(VocabTable const& t, const int32_t* first_ids, const uint16_t* l3, const int32_t* pair) const
+  {
+    uint32_t const b   = r[0];
+    uint32_t const x   = b & 0x00FFFFFFu;
+    uint32_t const low = x & 0x007F7F7Fu;
+    // bit 7 of each of the three bytes that is no lower-case letter (bytes past the word are zeros: none of them is)
+    uint32_t const bad = (~(low + 0x001F1F1Fu) | (low + 0x00050505u) | x) & 0x00808080u;
+    bool const ok3     = bad == 0u;
+    bool const ok2     = (bad & 0x00008080u) == 0u;
+    uint32_t const c0 = x & 0xFFu, c1 = (x >> 8) & 0xFFu, c2 = x >> 16;
+    uint32_t const i2 = c0 * 26u + c1 - 97u * 27u;
+    uint32_t const i3 = i2 * 26u + c2 - 97u;
+    Opening o;
+    o.id1               = first_ids[256 + c0];
+    uint32_t const len3 = l3[ok3 ? i3 : 0u];
+    int32_t const two   = pair[ok2 ? i2 : 0u];
+    o.lens              = ok3 ? (len3 | 0xFFFF0000u) : 0xFFFFFFFFu;
+    o.id2               = ok2 ? two : kNone;
+    if (!ok3 && rem >= 3) o.lens = t.lens[length_filter_index(1u, x) & t.lens_mask];
+    if (!ok2 && rem >= 2) o.id2 = t.short_ids[65536 + (b & 0xFFFFu)];
+    return o;
+  }
+
   // The piece at start begins: its candidate lengths are those on a character boundary, no longer than the rest of
   // the word or the longest key, and not ruled out by the length filter of its first three bytes.
   // (What the opening holds is not looked at here but when the next trip begins: by then its reads have arrived.)
@@ -646,13 +680,13 @@ struct ShortWord {
   // One trip: looks up the longest remaining candidate of three bytes and more; when none of those is left, the
   // candidates of two bytes and of one byte are settled from the ids the opening gave, without hashing or further
   // reads.  (The length filter leaves few candidates: a piece that has any has 1.4 on average, so a second lookup in
-  // the same trip would mostly be wasted work; and requesting, in the same breath, the openings of the pieces that
-  // could come next costs more in scattered reads than the waits it saves: measured, 18 % slower.)
+  // the same trip would mostly be wasted work.)
   // (Measured and left out: requesting, in the same breath, the openings of the pieces that could come next, so that no
   // trip waits twice: 18 % slower, the scattered reads cost more than the waits they save; settling pieces that need
-  // no lookup several to a trip: fewer trips, each slower by more.)
+  // no lookup several to a trip, also with their openings coming from LDS: fewer trips, each slower by more, and the
+  // registers it takes cost wavefronts per SIMD, which this loop needs: 1.03 ms with 8 of them, 1.07 with 6, 1.28 with 4.)
   template <typename Emit>
-  __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, Emit&& emit)
+  __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, const uint16_t* l3, const int32_t* pair, Emit&& emit)
   {
     uint32_t const kind = count ? 1u : 0u;
     cand &= (lens << 2) | 3u;
@@ -700,7 +734,7 @@ struct ShortWord {
     cand  = longer_left | (cand & 3u);
     if (hit && !done) {
       advance(len);  // next piece: the rest of the word (381-395)
-      open_piece(t, 1, request(t, first_ids, 1u, 0u));
+      open_piece(t, 1, request_next(t, first_ids, l3, pair));
     }
   }
 };
@@ -715,7 +749,7 @@ struct ShortWord {
 //   * out-of-vocabulary pass: one lane per queued word; the result takes the place of the queue entry.
 //   * emit pass: a wavefront per range expands the word slots into the tokens and gives every row that starts in the
 //     range its list offset.
-constexpr int kRangeTiles    = 16;
+constexpr int kRangeTiles    = 8;
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueChunk = 512;  // queue entries a wavefront of the word pass reserves at a time
 // A word slot: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or kOovMark | index of the word's queue entry
@@ -773,18 +807,35 @@ struct TileArgs {
   uint32_t* overflow;      // set when a range has more words than range_cap
 };
 
-// The next unit of work for a wavefront of a persistent kernel: its first one is its own number in the grid (the counter
-// starts at the number of wavefronts), the following ones come from the counter.  Atomics on one address run at about
-// 150 M/s: eight thousand wavefronts that all begin by asking the counter wait 55 microseconds between them, which was
-// a tenth of a call on two million short rows.  (Looking at the counter with a coherent load before asking, to spare the
-// one request too many that every wavefront ends with, made the three passes two to four times slower.)
-__device__ __forceinline__ uint32_t next_unit(uint32_t* counter, bool first, uint32_t my_number, int lane)
+// The flag words of a tokenize call (indices of 32-bit words; what is asked for with atomics has a 128-byte line of its own):
+constexpr uint32_t kCounterGroups = 8;
+constexpr uint32_t kFlagLine      = 32;
+constexpr uint32_t kFlagOverflow  = 1;                                          // a range had more words than slots
+constexpr uint32_t kFlagQueueSize = 2;                                          // queue entries reserved
+constexpr uint32_t kFlagLonger    = 1 * kFlagLine;                              // words of more than 16 bytes
+constexpr uint32_t kFlagAgain     = 2 * kFlagLine;                              // words of more tokens than a queue record keeps
+constexpr uint32_t kFlagWordUnits = 3 * kFlagLine;                              // kCounterGroups work counters of the word pass, a line each
+constexpr uint32_t kFlagOovUnits  = kFlagWordUnits + kCounterGroups * kFlagLine;  // and of the out-of-vocabulary pass
+constexpr uint32_t kFlagWords     = kFlagOovUnits + kCounterGroups * kFlagLine;
+
+// The next unit of work for a wavefront of a persistent kernel: its first one is its own number in the grid, the
+// following ones come from a counter.  Atomics on one address run at about 150 M/s: eight thousand wavefronts that all
+// begin by asking one counter wait 55 microseconds between them, which was a tenth of a call on two million short
+// rows; and with units small enough to even out the end of the kernel (ranges of 16 KB: a hundred thousand requests
+// and more per GB of text), one counter made the word pass 16 % slower than it is with kCounterGroups of them, each in
+// a line of its own: counter g serves the wavefronts g, g + kCounterGroups, .. and hands out the units g,
+// g + kCounterGroups, .. (it starts at the number of those wavefronts).  (Looking at the counter with a coherent load
+// before asking, to spare the one request too many that every wavefront ends with, made the passes two to four times
+// slower.)
+__device__ __forceinline__ uint32_t next_unit(uint32_t* counters, bool first, uint32_t my_number, int lane)
 {
   // (my_number is the same in every lane, which the compiler cannot know: as a scalar, so that what depends on it stays scalar)
-  if (first) return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(my_number)));
-  uint32_t unit = 0xFFFFFFFFu;
-  if (lane == 0) unit = atomicAdd(counter, 1u);
-  return wave_bcast(unit, 0);
+  uint32_t const me = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(my_number)));
+  if (first) return me;
+  uint32_t const g = me % kCounterGroups;
+  uint32_t n       = 0xFFFFFFFFu / kCounterGroups - 1u;
+  if (lane == 0) n = atomicAdd(counters + g * kFlagLine, 1u);
+  return wave_bcast(n, 0) * kCounterGroups + g;
 }
 
 __device__ __forceinline__ void wave_lds_sync()
@@ -1245,8 +1296,9 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
 // lane each, by the general state machine over the chars in memory, 64 and more at a time or at the end.
 constexpr uint32_t kOovBlock = 512;
 constexpr int kRefillAt      = 32;
-constexpr int kOovWaves      = 4;
+constexpr int kOovWaves      = 16;  // (two workgroups to a CU, 73 KB of LDS each, 8 wavefronts per SIMD)
 constexpr int kOovThreads    = kOovWaves * kWave;
+constexpr int kRareThreads   = 256;  // the kernels for the few words that this one leaves
 struct OovLds {
   alignas(16) uint4 staged[kWave][2];  // 64 queue entries
 };
@@ -1258,7 +1310,12 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTabl
 {
   __shared__ OovLds lds_all[kOovWaves];
   __shared__ int32_t first_ids[512];  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
+  __shared__ int32_t pair_ids[kLetters2];  // the ids of the keys of two lower-case letters, second key space
+  __shared__ uint16_t letters3[kLetters3];
   for (int i = threadIdx.x; i < 512; i += kOovThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
+  for (uint32_t i = threadIdx.x; i < kLetters2; i += kOovThreads) pair_ids[i] = table.short_ids[65536 + ((i / 26u + 'a') | ((i % 26u + 'a') << 8))];
+  for (uint32_t i = threadIdx.x; i < kLetters3 / 2; i += kOovThreads)
+    reinterpret_cast<uint32_t*>(letters3)[i] = reinterpret_cast<const uint32_t*>(table.letters3)[i];
   __syncthreads();
   if (*queue_size > queue_cap) return;  // the queue was too small: the host repeats the passes with a larger one
   uint32_t const total = *queue_size;
@@ -1412,21 +1469,21 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTabl
       if (drained && ballot64(busy) == 0) break;
       continue;
     }
-    if (busy && !sw.done) sw.step(table, first_ids, keep_token);
+    if (busy && !sw.done) sw.step(table, first_ids, letters3, pair_ids, keep_token);
   }
   add_together(acc_count != 0);
 }
 
 // The queued words of more than 16 bytes, which the kernel above has listed: one lane per word, the general state
 // machine over the chars in memory.
-__global__ void __launch_bounds__(kOovThreads) wordpiece_oov_long_kernel(VocabTable table, const uint4* abase, OovEntry* __restrict__ queue,
+__global__ void __launch_bounds__(kRareThreads) wordpiece_oov_long_kernel(VocabTable table, const uint4* abase, OovEntry* __restrict__ queue,
                                                                          const uint32_t* __restrict__ queue_size, uint32_t queue_cap,
                                                                          const uint32_t* __restrict__ longer, const uint32_t* __restrict__ longer_count,
                                                                          uint32_t* __restrict__ range_tokens)
 {
   if (*queue_size > queue_cap) return;  // (see wordpiece_oov_kernel)
   uint32_t const n = *longer_count;
-  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
+  for (uint32_t i = blockIdx.x * kRareThreads + threadIdx.x; i < n; i += gridDim.x * kRareThreads) {
     uint32_t const q   = longer[i];
     OovEntry const e   = queue[q];
     uint32_t const wl  = e.len_flags & 0xFFu;
@@ -1551,12 +1608,12 @@ __global__ void __launch_bounds__(kTokThreads, 8) wordpiece_emit_kernel(uint32_t
 // and left the index of each one's first token in the child in its record, beside where and how long the word is):
 // tokenized again, straight into place.  One lane per word; kept apart from the emit pass so that that is compiled for
 // its common case.
-__global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(VocabTable table, const uint4* abase, const OovEntry* __restrict__ queue,
+__global__ void __launch_bounds__(kRareThreads) wordpiece_retokenize_kernel(VocabTable table, const uint4* abase, const OovEntry* __restrict__ queue,
                                                                            const uint32_t* __restrict__ again, const uint32_t* __restrict__ again_count,
                                                                            int32_t* __restrict__ child)
 {
   uint32_t const n = *again_count;
-  for (uint32_t i = blockIdx.x * kOovThreads + threadIdx.x; i < n; i += gridDim.x * kOovThreads) {
+  for (uint32_t i = blockIdx.x * kRareThreads + threadIdx.x; i < n; i += gridDim.x * kRareThreads) {
     OovEntry const e   = queue[again[i]];  // head[0] = place in the child, head[3] = coord[1], len_flags, range, coord[0] as they were; coord[1] = the count
     uint32_t const cnt = e.coord[1];
     int64_t const at   = static_cast<int64_t>((static_cast<uint64_t>(e.head[3]) << 32) | e.coord[0]);
@@ -1567,11 +1624,19 @@ __global__ void __launch_bounds__(kOovThreads) wordpiece_retokenize_kernel(Vocab
   }
 }
 
-// flags[0..63] of a tokenize call: zeros, but for the work counters of the word pass [0] and the out-of-vocabulary pass [3]
+// The flag words of a tokenize call: zeros, but for the work counters, which start past the units that the wavefronts
+// take by their place in the grid (counter g serves the wavefronts g, g + kCounterGroups, .. and hands out the units
+// g, g + kCounterGroups, ..).
 __global__ void tokenize_flags_kernel(uint32_t* flags, uint32_t word_waves, uint32_t oov_waves)
 {
-  uint32_t const i = threadIdx.x;
-  flags[i]         = i == 0 ? word_waves : i == 3 ? oov_waves : 0u;
+  for (uint32_t i = threadIdx.x; i < kFlagWords; i += blockDim.x) {
+    uint32_t v = 0;
+    if (i >= kFlagWordUnits && i % kFlagLine == 0) {
+      uint32_t const g = (i - kFlagWordUnits) / kFlagLine;
+      v = ((g < kCounterGroups ? word_waves : oov_waves) + kCounterGroups - 1u - g % kCounterGroups) / kCounterGroups;
+    }
+    flags[i] = v;
+  }
 }
 
 struct RangeTokensOf {
@@ -1741,10 +1806,14 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   size_t lens_size = 1024;
   while (lens_size < 4 * keys) lens_size <<= 1;
   std::vector<uint32_t> lens(lens_size, 0u);
+  std::vector<uint16_t> letters3(kLetters3, uint16_t{0});
+  auto letter = [](uint8_t c) { return c >= 'a' && c <= 'z'; };
   auto note_length = [&](uint32_t kind, const uint8_t* key, uint32_t len) {
     if (len < 3) return;
     uint32_t const first3 = key[0] | (uint32_t{key[1]} << 8) | (uint32_t{key[2]} << 16);
     lens[length_filter_index(kind, first3) & (lens_size - 1)] |= 1u << length_filter_bit(len);
+    if (kind == 1 && len <= 18 && letter(key[0]) && letter(key[1]) && letter(key[2]))
+      letters3[((key[0] - 'a') * 26u + (key[1] - 'a')) * 26u + (key[2] - 'a')] |= static_cast<uint16_t>(1u << (len - 3));
   };
   for (int32_t i = 0; i < V; ++i) {
     int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
@@ -1779,7 +1848,8 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->d_pool  = v->store.allocate(v->pool_bytes);
   v->d_lens  = v->store.allocate(lens.size() * sizeof(uint32_t));
   v->d_short = v->store.allocate(short_ids.size() * sizeof(int32_t));
-  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short) {
+  v->d_letters = v->store.allocate(letters3.size() * sizeof(uint16_t));
+  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
@@ -1787,8 +1857,9 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   hipError_t e2 = blocks.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, blocks.data(), blocks.size(), hipMemcpyHostToDevice, stream);
   hipError_t e4 = hipMemcpyAsync(v->d_lens, lens.data(), lens.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
   hipError_t e5 = hipMemcpyAsync(v->d_short, short_ids.data(), short_ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
+  hipError_t e6 = hipMemcpyAsync(v->d_letters, letters3.data(), letters3.size() * sizeof(uint16_t), hipMemcpyHostToDevice, stream);
   hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
-  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess) {
+  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess || e6 != hipSuccess) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_DEVICE_ERROR, "vocabulary upload failed");
   }
@@ -1801,6 +1872,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.lens        = static_cast<const uint32_t*>(v->d_lens);
   v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
   v->table.short_ids   = static_cast<const int32_t*>(v->d_short);
+  v->table.letters3    = static_cast<const uint16_t*>(v->d_letters);
   *out            = v;
   return NVTEXT_AMD_SUCCESS;
 }
@@ -1949,7 +2021,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
                                   static_cast<size_t>(nranges) * sizeof(uint32_t),
                                   (static_cast<size_t>(nranges) + 1) * sizeof(int64_t),
                                   scan_temp_bytes(nranges),
-                                  256,
+                                  kFlagWords * sizeof(uint32_t),
                                   static_cast<size_t>(qcap) * sizeof(OovEntry),
                                   static_cast<size_t>(qcap) * sizeof(uint32_t)};
     TempParts<9> const temps(mr, temp_bytes);
@@ -1960,7 +2032,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     uint32_t* const tokens    = temps.part<uint32_t>(3);
     int64_t* const bases      = temps.part<int64_t>(4);
     uint64_t* const scan_tmp  = temps.part<uint64_t>(5);
-    uint32_t* const flags     = temps.part<uint32_t>(6);  // [0] ranges handed out by the word pass, [1] a range had more words than slots, [2] queue entries, [3] blocks handed out by the out-of-vocabulary pass, [4] ranges handed out by the emit pass, [5] words of more than 16 bytes, [6] words of more tokens than a queue record keeps
+    uint32_t* const flags     = temps.part<uint32_t>(6);
     OovEntry* const queue     = temps.part<OovEntry>(7);
     uint32_t* const longer    = temps.part<uint32_t>(8);  // queue indices of the words of more than 16 bytes
     args.range_cap       = range_cap;
@@ -1971,11 +2043,11 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     args.offsets_out     = out->offsets;
     args.queue           = queue;
     args.queue_cap       = qcap;
-    args.queue_size      = flags + 2;
-    args.counter         = flags;
-    args.overflow        = flags + 1;
+    args.queue_size      = flags + kFlagQueueSize;
+    args.counter         = flags + kFlagWordUnits;
+    args.overflow        = flags + kFlagOverflow;
     // the two work counters start past the units that the wavefronts take by their place in the grid
-    hipLaunchKernelGGL(tokenize_flags_kernel, dim3(1), dim3(64), 0, stream, flags, word_grid * kTokWaves, oov_grid * kOovWaves);
+    hipLaunchKernelGGL(tokenize_flags_kernel, dim3(1), dim3(256), 0, stream, flags, word_grid * kTokWaves, oov_grid * kOovWaves);
     hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 1 + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
     {
       ProfileScope ps("wordpiece_word_kernel", stream);
@@ -1983,13 +2055,13 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     }
     {
       ProfileScope ps("wordpiece_oov_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(oov_grid), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue, flags + 2, qcap, tokens,
-                         flags + 3, longer, flags + 5);
+      hipLaunchKernelGGL(wordpiece_oov_kernel, dim3(oov_grid), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue, flags + kFlagQueueSize, qcap, tokens,
+                         flags + kFlagOovUnits, longer, flags + kFlagLonger);
     }
     {
       ProfileScope ps("wordpiece_oov_long_kernel", stream);
-      hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue,
-                         flags + 2, qcap, longer, flags + 5, tokens);
+      hipLaunchKernelGGL(wordpiece_oov_long_kernel, dim3(static_cast<unsigned>(cus)), dim3(kRareThreads), 0, stream, vocabulary->table, args.abase, queue,
+                         flags + kFlagQueueSize, qcap, longer, flags + kFlagLonger, tokens);
     }
     // where the tokens of each range go; the total decides the child size
     // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
@@ -2027,11 +2099,11 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     {
       ProfileScope ps("wordpiece_emit_kernel", stream);
       hipLaunchKernelGGL(wordpiece_emit_kernel, dim3(emit_grid), dim3(kTokThreads), 0, stream, nranges, arena, range_cap, words, bases, first_row, queue,
-                         out->offsets, static_cast<int32_t*>(out->child), longer, flags + 6);
+                         out->offsets, static_cast<int32_t*>(out->child), longer, flags + kFlagAgain);
       // (the list of longer words has served its purpose by now: its memory takes the list of words to do again, at most
       // one entry per queued word)
-      hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kOovThreads), 0, stream, vocabulary->table, args.abase, queue,
-                         longer, flags + 6, static_cast<int32_t*>(out->child));
+      hipLaunchKernelGGL(wordpiece_retokenize_kernel, dim3(static_cast<unsigned>(cus)), dim3(kRareThreads), 0, stream, vocabulary->table, args.abase, queue,
+                         longer, flags + kFlagAgain, static_cast<int32_t*>(out->child));
     }
     break;
   }

@@ -634,6 +634,53 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
     assert exp.child.size > 5000
 
 
+def test_wordpiece_pieces_of_letters_and_of_their_neighbours(nv, orc):
+    """Later pieces of a word ("##" keys) over an alphabet of lower-case letters and the bytes next to them in ASCII
+    ('`' before 'a', '{' after 'z', capitals, digits): the library serves the pieces that begin with two or three
+    lower-case letters from small tables of their own and the others from the general ones, and both have to say the
+    same as the oracle; keys of every length from 1 to 20 bytes, so that the tables' longest lengths (18) and the
+    keys beyond them are met."""
+    rng = np.random.default_rng(77)
+    letters = list("azmb")
+    others = list("`{AZ09")
+    alphabet = letters * 3 + others
+    vocab = ["[UNK]"]
+    seen = set(vocab)
+    for c in letters + others[:3]:
+        for v in (c, "##" + c):
+            seen.add(v)
+            vocab.append(v)
+    while len(vocab) < 2500:
+        n = int(rng.choice([2, 2, 3, 3, 3, 4, 5, 6, 8, 9, 12, 15, 16, 17, 18, 19, 20]))
+        k = "".join(rng.choice(alphabet if rng.random() < 0.6 else letters, n))
+        v = "##" + k if rng.random() < 0.7 else k
+        if v not in seen:
+            seen.add(v)
+            vocab.append(v)
+    keys = [v[2:] if v.startswith("##") else v for v in vocab[1:]]
+    rows = []
+    for _ in range(3000):
+        ws = []
+        for _ in range(int(rng.integers(1, 20))):
+            t = rng.random()
+            if t < 0.6:  # keys glued together, cut to the 16 bytes and fewer that the short-word path takes, or longer
+                w = "".join(keys[int(rng.integers(0, len(keys)))] for _ in range(int(rng.integers(1, 4))))
+                ws.append(w[: int(rng.integers(1, 17))] if rng.random() < 0.7 else w)
+            else:
+                ws.append("".join(rng.choice(alphabet, int(rng.integers(1, 17)))))
+        rows.append(" ".join(ws))
+    host = strings(rows, np.int32)
+    hv = strings(vocab)
+    for mw in (0, 7):
+        got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
+        exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4)
+        assert_same(got, exp, f"letters and neighbours mw={mw}")
+    assert exp.child.size > 30000
+    # the test means to meet known and unknown words alike
+    unk = int((exp.child == 0).sum())
+    assert 0 < unk < exp.child.size
+
+
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype):
     """Rows of hundreds of kilobytes (which the library tokenizes in pieces cut at spaces when there is no word limit)
