@@ -1507,24 +1507,38 @@ __global__ void __launch_bounds__(kRareThreads) wordpiece_oov_long_kernel(VocabT
 }
 
 // ------------------------------------------------------------------ emit pass
-// A wavefront takes a range: walks its word slots 64 at a time, in order; a word from the queue has its tokens (or
-// their number) in its queue record; a wave scan of the token counts places the tokens, and every lane writes its own
-// word's.  The rows that start in the range (the word pass left each the number of the range's words before it) are
-// walked alongside: a row that begins at one of the 64 words gets that word's place as its list offset.
+// A wavefront takes a range: walks its word slots 128 at a time, in order, two neighbouring words per lane; a word
+// from the queue has its tokens (or their number) in its queue record; a wave scan of the lanes' token counts places
+// the tokens, and every lane writes its own words'.  The rows that start in the range (the word pass left each the
+// number of the range's words before it) are walked alongside: a row that begins at one of the 128 words gets that
+// word's place as its list offset.
+// Two things decide the pass' speed.  The counter a wavefront waits on counts reads and writes alike, out of order
+// between the two, so every wait for a read is a wait for everything, and what a wavefront has in flight is what one
+// round asks for: hence two words per lane (0.21 -> 0.16 ms on two million short rows of known words).  And a vector
+// memory instruction takes the address unit about as long for a few lanes as for sixty-four: written word by word, the
+// second to seventh tokens of the words that have them were an instruction each for a handful of lanes; put side by
+// side in LDS first and written 64 at a time, the same tokens take a third of the instructions (0.69 -> 0.55 ms on
+// 3.2 GB of text with one word in seven from the queue).
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 __global__ void __launch_bounds__(kTokThreads, 8) wordpiece_emit_kernel(uint32_t nranges, const uint32_t* __restrict__ arena, uint32_t range_cap,
                                                                      const uint32_t* __restrict__ range_words, const int64_t* __restrict__ range_base,
                                                                      const uint32_t* __restrict__ range_first_row, OovEntry* __restrict__ queue,
                                                                      int32_t* __restrict__ offsets, int32_t* __restrict__ child,
                                                                      uint32_t* __restrict__ again, uint32_t* __restrict__ again_count)
 {
-  int const lane           = lane_id();
-  uint32_t const my_number = blockIdx.x * kTokWaves + threadIdx.x / kWave;
+  constexpr uint32_t kRound = 2 * kWave;
+  constexpr uint32_t kStage = 768;  // tokens of a round that are put in order in LDS before they are written
+  __shared__ uint32_t stage_all[kTokWaves][kStage];
+  uint32_t* const stage     = stage_all[threadIdx.x / kWave];
+  int const lane            = lane_id();
+  uint32_t const my_number  = blockIdx.x * kTokWaves + threadIdx.x / kWave;
   // The ranges cost this pass about the same, so every wavefront takes every W-th one (W wavefronts in the grid):
   // faster here than taking them from a counter as they go, as the other two passes do (0.71 against 0.77 ms on
   // 3.2 GB of text, 0.21 against 0.26 ms on two million short rows).
   uint32_t const stride_units = gridDim.x * kTokWaves;
   for (uint32_t range = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(my_number))); range < nranges;
        range += stride_units) {
+    // (a range's slots begin at an even index, and so does a lane's pair)
     const uint32_t* const slots = arena + static_cast<int64_t>(range) * range_cap;
     uint32_t const nwords       = range_words[range];
     int64_t const base          = range_base[range];
@@ -1535,58 +1549,110 @@ __global__ void __launch_bounds__(kTokThreads, 8) wordpiece_emit_kernel(uint32_t
     uint32_t done               = 0;  // tokens of the range so far
     // the words of the range before my row
     uint32_t row_k = r_win + lane < r_end ? static_cast<uint32_t>(offsets[r_win + lane]) : 0xFFFFFFFFu;
-    // three stages in flight: the slot two rounds ahead, the queue record of a word from the queue one round ahead, the
-    // round being written (the pass is bound by the latency of its reads)
-    auto load_slot = [&](uint32_t k) -> uint32_t { return k < nwords ? load_stream(slots + k) : 0u; };
+    // in flight: the slots two rounds ahead, the queue records of the next round's words from the queue, this round's writes
+    auto load_slots = [&](uint32_t k) -> uint2 {  // slots k, k + 1 (k even; the second may lie past the range's words: not looked at then)
+      if (k >= nwords) return make_uint2(0u, 0u);
+      u32x2_t const v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(slots + k));
+      return make_uint2(v.x, v.y);
+    };
+    auto from_queue = [&](uint32_t k, uint32_t v) { return k < nwords && (v & kOovMark) != 0 && v != 0xFFFFFFFFu; };
     auto load_record = [&](uint32_t k, uint32_t v, uint4& ra, uint4& rb) {
-      if (k < nwords && (v & kOovMark) != 0 && v != 0xFFFFFFFFu) {
+      if (from_queue(k, v)) {
         const uint4* const src = reinterpret_cast<const uint4*>(queue + (v & ~kOovMark));
         ra = src[0];
         rb = src[1];
       }
     };
-    uint32_t v_nxt = load_slot(lane), v_far = load_slot(kWave + lane);
-    uint4 a_nxt = make_uint4(0u, 0u, 0u, 0u), b_nxt = a_nxt;
-    load_record(lane, v_nxt, a_nxt, b_nxt);
-    for (uint32_t j0 = 0; j0 < nwords; j0 += kWave) {
-      uint32_t const k  = j0 + lane;
-      bool const active = k < nwords;
-      uint32_t const v  = v_nxt;
-      uint4 const ra = a_nxt, rb = b_nxt;
+    uint2 v_nxt = load_slots(2u * lane), v_far = load_slots(kRound + 2u * lane);
+    uint4 a0_nxt = make_uint4(0u, 0u, 0u, 0u), b0_nxt = a0_nxt, a1_nxt = a0_nxt, b1_nxt = a0_nxt;
+    load_record(2u * lane, v_nxt.x, a0_nxt, b0_nxt);
+    load_record(2u * lane + 1u, v_nxt.y, a1_nxt, b1_nxt);
+    for (uint32_t j0 = 0; j0 < nwords; j0 += kRound) {
+      uint32_t const k  = j0 + 2u * lane;
+      uint2 const v     = v_nxt;
+      uint4 const ra0 = a0_nxt, rb0 = b0_nxt, ra1 = a1_nxt, rb1 = b1_nxt;
       v_nxt = v_far;
-      load_record(k + kWave, v_nxt, a_nxt, b_nxt);
-      v_far = load_slot(k + 2 * kWave);
-      bool const marked   = active && (v & kOovMark) != 0 && v != 0xFFFFFFFFu;
-      uint32_t const cnt  = !active ? 0u : marked ? rb.w : 1u;
-      uint32_t const incl = wave_inclusive_scan(cnt);
-      uint32_t const ex   = incl - cnt;
+      load_record(k + kRound, v_nxt.x, a0_nxt, b0_nxt);
+      load_record(k + kRound + 1u, v_nxt.y, a1_nxt, b1_nxt);
+      v_far = load_slots(k + 2u * kRound);
+      bool const act0 = k < nwords, act1 = k + 1u < nwords;
+      bool const q0 = from_queue(k, v.x), q1 = from_queue(k + 1u, v.y);
+      uint32_t const c0   = !act0 ? 0u : q0 ? rb0.w : 1u;
+      uint32_t const c1   = !act1 ? 0u : q1 ? rb1.w : 1u;
+      uint32_t const incl = wave_inclusive_scan(c0 + c1);
+      uint32_t const ex   = incl - (c0 + c1);  // tokens of the round before my first word
       uint32_t const tot  = wave_bcast(incl, kWave - 1);
       int32_t* const dst  = dst0 + done + ex;
-      bool const more     = marked && cnt > kOovKeep;
-      if (more) {
-        // more tokens than a record keeps (seldom): noted for wordpiece_retokenize_kernel, with the place of the word's
-        // first token in the child left in its record
-        uint32_t const q                 = v & ~kOovMark;
-        again[atomicAdd(again_count, 1u)] = q;
-        queue[q].head[0]                 = static_cast<uint32_t>(base + done + ex);
-      } else if (active) {
-        dst[0] = static_cast<int32_t>(marked ? ra.x : v);
-        if (ballot64(marked && cnt > 1u) != 0) {
-          if (marked && cnt > 1u) dst[1] = static_cast<int32_t>(ra.y);
-          if (marked && cnt > 2u) dst[2] = static_cast<int32_t>(ra.z);
-          if (ballot64(marked && cnt > 3u) != 0) {
-            if (marked && cnt > 3u) dst[3] = static_cast<int32_t>(ra.w);
-            if (marked && cnt > 4u) dst[4] = static_cast<int32_t>(rb.x);
-            if (marked && cnt > 5u) dst[5] = static_cast<int32_t>(rb.y);
-            if (marked && cnt > 6u) dst[6] = static_cast<int32_t>(rb.z);
-          }
+      if (ballot64(q0 || q1) == 0) {
+        // no word of the round comes from the queue: a token each, the pair side by side
+        if (act1) {
+          uint32_t const w[2] = {v.x, v.y};
+          __builtin_memcpy(dst, w, 8);  // (one 8-byte store; dst is 4-byte aligned)
+        } else if (act0) {
+          dst[0] = static_cast<int32_t>(v.x);
         }
+      } else if (tot <= kStage) {
+        // the tokens of the round side by side in LDS, then written 64 at a time
+        auto stage_word = [&](bool active, bool queued, uint32_t slot, uint32_t cnt, uint4 const& ra, uint4 const& rb, uint32_t at) {
+          if (queued && cnt > kOovKeep) {
+            // more tokens than a record keeps (seldom): noted for wordpiece_retokenize_kernel, with the place of the
+            // word's first token in the child left in its record (what is written there now is overwritten then)
+            uint32_t const q                  = slot & ~kOovMark;
+            again[atomicAdd(again_count, 1u)] = q;
+            queue[q].head[0]                  = static_cast<uint32_t>(base + done + at);
+          } else if (active) {
+            stage[at] = queued ? ra.x : slot;
+            if (ballot64(queued && cnt > 1u) != 0) {
+              if (queued && cnt > 1u) stage[at + 1] = ra.y;
+              if (queued && cnt > 2u) stage[at + 2] = ra.z;
+              if (ballot64(queued && cnt > 3u) != 0) {
+                if (queued && cnt > 3u) stage[at + 3] = ra.w;
+                if (queued && cnt > 4u) stage[at + 4] = rb.x;
+                if (queued && cnt > 5u) stage[at + 5] = rb.y;
+                if (queued && cnt > 6u) stage[at + 6] = rb.z;
+              }
+            }
+          }
+        };
+        wave_lds_sync();  // (the writes of the round before have read their tokens)
+        stage_word(act0, q0, v.x, c0, ra0, rb0, ex);
+        stage_word(act1, q1, v.y, c1, ra1, rb1, ex + c0);
+        wave_lds_sync();
+        int32_t* const out = dst0 + done;
+        for (uint32_t i = lane; i < tot; i += kWave) out[i] = static_cast<int32_t>(stage[i]);
+      } else {
+        auto write_word = [&](bool active, bool queued, uint32_t slot, uint32_t cnt, uint4 const& ra, uint4 const& rb, int32_t* d) {
+          if (queued && cnt > kOovKeep) {
+            // more tokens than a record keeps (seldom): noted for wordpiece_retokenize_kernel, with the place of the
+            // word's first token in the child left in its record
+            uint32_t const q                  = slot & ~kOovMark;
+            again[atomicAdd(again_count, 1u)] = q;
+            queue[q].head[0]                  = static_cast<uint32_t>(d - child);
+          } else if (active) {
+            d[0] = static_cast<int32_t>(queued ? ra.x : slot);
+            if (ballot64(queued && cnt > 1u) != 0) {
+              if (queued && cnt > 1u) d[1] = static_cast<int32_t>(ra.y);
+              if (queued && cnt > 2u) d[2] = static_cast<int32_t>(ra.z);
+              if (ballot64(queued && cnt > 3u) != 0) {
+                if (queued && cnt > 3u) d[3] = static_cast<int32_t>(ra.w);
+                if (queued && cnt > 4u) d[4] = static_cast<int32_t>(rb.x);
+                if (queued && cnt > 5u) d[5] = static_cast<int32_t>(rb.y);
+                if (queued && cnt > 6u) d[6] = static_cast<int32_t>(rb.z);
+              }
+            }
+          }
+        };
+        write_word(act0, q0, v.x, c0, ra0, rb0, dst);
+        write_word(act1, q1, v.y, c1, ra1, rb1, dst + c0);
       }
-      // rows that begin at one of these words (or, in the last round, after the last word: the lanes past it
+      // rows that begin at one of these words (or, in the last round, after the last word: the positions past it
       // hold the round's total)
+      uint32_t const places = ex | (c0 << 16);  // (a round has fewer than 2^16 tokens: 128 words of fewer than 200 each)
       for (;;) {
-        bool const mine  = lane >= static_cast<int>(row_used) && row_k < j0 + kWave;  // (row_k >= j0: the rows are in order)
-        uint32_t const e = static_cast<uint32_t>(__shfl(static_cast<int>(ex), static_cast<int>((row_k - j0) & 63u)));
+        bool const mine   = lane >= static_cast<int>(row_used) && row_k < j0 + kRound;  // (row_k >= j0: the rows are in order)
+        uint32_t const at = row_k - j0;
+        uint32_t const pl = static_cast<uint32_t>(__shfl(static_cast<int>(places), static_cast<int>((at >> 1) & 63u)));
+        uint32_t const e  = (pl & 0xFFFFu) + ((at & 1u) != 0 ? pl >> 16 : 0u);
         if (mine) offsets[r_win + lane] = static_cast<int32_t>(base + done + e);
         row_used += static_cast<uint32_t>(__builtin_popcountll(ballot64(mine)));
         if (row_used < kWave) break;
