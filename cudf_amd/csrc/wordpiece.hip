@@ -782,6 +782,8 @@ struct TileLds {
   static constexpr uint32_t kWordCap = TILE / 4;
   uint32_t word_guard[1];                     // (takes the end of the word that ran into the tile)
   uint32_t word[kWordCap];                    // per word: start | end << 16
+  static constexpr uint32_t kQueueStage = 16;
+  alignas(16) uint4 queued[kQueueStage][2];   // the queue records of a round of 64 words (when there are no more than these), to be written side by side
 };
 
 struct TileArgs {
@@ -1246,16 +1248,30 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
               if (lane == 0) fresh = atomicAdd(a.queue_size, kQueueChunk);
               fresh = wave_bcast(fresh, 0);
             }
+            // (a vector memory instruction costs the address unit about the same for ten lanes as for sixty-four: the
+            // records of a round, ten of them on average, go side by side through LDS and out with one instruction)
+            bool const staged = nm <= TileLds<TILE>::kQueueStage;
             if (defer != 0) {
               uint32_t const rank = lanes_below(mm);
               uint32_t const q    = rank < room ? q_pos + rank : fresh + (rank - room);
-              if (q < a.queue_cap) {
-                int64_t const at = tb + s;
+              int64_t const at    = tb + s;
+              uint4 const first   = make_uint4(head[0], head[1], head[2], head[3]);
+              uint4 const second  = make_uint4(wl | (defer == 2u ? kUnprobed : 0u), range, static_cast<uint32_t>(at), static_cast<uint32_t>(static_cast<uint64_t>(at) >> 32));
+              if (staged) {
+                lds.queued[rank][0] = first;
+                lds.queued[rank][1] = second;
+              } else if (q < a.queue_cap) {
                 uint4* const dst = reinterpret_cast<uint4*>(a.queue + q);
-                store_stream(dst, make_uint4(head[0], head[1], head[2], head[3]));
-                store_stream(dst + 1, make_uint4(wl | (defer == 2u ? kUnprobed : 0u), range, static_cast<uint32_t>(at), static_cast<uint32_t>(static_cast<uint64_t>(at) >> 32)));
+                store_stream(dst, first);
+                store_stream(dst + 1, second);
               }
               value = kOovMark | q;
+            }
+            if (staged) {
+              wave_lds_sync();
+              uint32_t const e = static_cast<uint32_t>(lane) >> 1;
+              uint32_t const q = e < room ? q_pos + e : fresh + (e - room);
+              if (e < nm && q < a.queue_cap) store_stream(reinterpret_cast<uint4*>(a.queue + q) + (lane & 1), lds.queued[e][lane & 1]);
             }
             if (nm > room) {
               q_pos = fresh + (nm - room);
