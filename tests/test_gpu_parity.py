@@ -634,6 +634,29 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
     assert exp.child.size > 5000
 
 
+@pytest.mark.parametrize("letters", [5, 7, 8, 12])
+def test_wordpiece_every_word_splits_into_as_many_pieces_as_it_has_letters(nv, orc, letters):
+    """A vocabulary of single letters only, so that a word of k letters is k tokens: rounds of the library's last pass
+    in which every word brings five tokens (its usual way of writing them), seven (more tokens in a round than it puts in
+    order before writing: each word's are then written by themselves), eight and twelve (more than a word's record
+    keeps: tokenized again into place)."""
+    rng = np.random.default_rng(100 + letters)
+    alphabet = list("abcdefgh")
+    vocab = ["[UNK]"] + alphabet + ["##" + c for c in alphabet]
+    rows = []
+    for _ in range(400):
+        n = int(rng.integers(0, 60))
+        rows.append(" ".join("".join(rng.choice(alphabet, letters)) for _ in range(n)))
+    rows[7] = ""
+    host = strings(rows, np.int32)
+    hv = strings(vocab)
+    for mw in (0, 11):
+        got = nv.wordpiece_tokenize(dev(nv, host), nv.WordPieceVocabulary(dev(nv, hv)), mw).to_host()
+        exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4)
+        assert_same(got, exp, f"{letters} letters mw={mw}")
+    assert exp.child.size > 400 * 5 * letters
+
+
 def test_wordpiece_pieces_of_letters_and_of_their_neighbours(nv, orc):
     """Later pieces of a word ("##" keys) over an alphabet of lower-case letters and the bytes next to them in ASCII
     ('`' before 'a', '{' after 'z', capitals, digits): the library serves the pieces that begin with two or three
