@@ -145,6 +145,21 @@ __device__ __forceinline__ void trim_key8(uint32_t len, uint32_t& lo, uint32_t& 
   hi &= nhi >= 4 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << (8 * nhi));
 }
 
+// trim[len] (len 0..16): the masks that keep bytes [0, len) of sixteen, as four dwords; what trim_key8 computes, read
+// from LDS where a kernel trims a key for every word.
+__device__ __forceinline__ void fill_trim_table(uint4* trim)
+{
+  if (threadIdx.x <= 16) {
+    uint32_t m[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      int const n = min(max(static_cast<int>(threadIdx.x) - 4 * d, 0), 4);
+      m[d]        = n >= 4 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << (8 * n));
+    }
+    trim[threadIdx.x] = make_uint4(m[0], m[1], m[2], m[3]);
+  }
+}
+
 // A word inside the bytes a wavefront has staged in LDS: `bytes` points at the staged dwords, `start` is the
 // byte index of the word's first byte in them.  Everything a word of fewer than kMaxWord bytes can touch is staged.
 struct TileWord {
@@ -642,15 +657,14 @@ struct ShortWord {
     if (probed) cand &= ~(1u << (len - 1));
   }
 
-  __device__ __forceinline__ Probe probe_of(VocabTable const& t, uint32_t kind, uint32_t l) const
+  __device__ __forceinline__ Probe probe_of(VocabTable const& t, const uint4* trim, uint32_t kind, uint32_t l) const
   {
     Probe pr;
-    pr.k0 = r[0];
-    pr.k1 = r[1];
-    trim_key8(min(l, 8u), pr.k0, pr.k1);
-    uint32_t h  = key_hash_block(key_hash_init(l), pr.k0, pr.k1);
-    uint32_t k2 = r[2], k3 = r[3];
-    trim_key8(l > 8 ? l - 8u : 0u, k2, k3);
+    uint4 const keep = trim[l];  // (l <= 16)
+    pr.k0            = r[0] & keep.x;
+    pr.k1            = r[1] & keep.y;
+    uint32_t h       = key_hash_block(key_hash_init(l), pr.k0, pr.k1);
+    uint32_t const k2 = r[2] & keep.z, k3 = r[3] & keep.w;
     uint32_t const h2 = key_hash_block(h, k2, k3);
     h                 = l > 8 ? h2 : h;
     uint32_t b;
@@ -686,7 +700,8 @@ struct ShortWord {
   // no lookup several to a trip, also with their openings coming from LDS: fewer trips, each slower by more, and the
   // registers it takes cost wavefronts per SIMD, which this loop needs: 1.03 ms with 8 of them, 1.07 with 6, 1.28 with 4.)
   template <typename Emit>
-  __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, const uint16_t* l3, const int32_t* pair, Emit&& emit)
+  __device__ __forceinline__ void step(VocabTable const& t, const int32_t* first_ids, const uint16_t* l3, const int32_t* pair, const uint4* trim,
+                                       Emit&& emit)
   {
     uint32_t const kind = count ? 1u : 0u;
     cand &= (lens << 2) | 3u;
@@ -697,7 +712,7 @@ struct ShortWord {
     Probe pa;
     uint4 a0 = make_uint4(0u, 0u, 0u, 0u), a1 = a0;
     if (has_a) {
-      pa = probe_of(t, kind, la);
+      pa = probe_of(t, trim, kind, la);
       a0 = t.slots[2 * pa.bucket];
       a1 = t.slots[2 * pa.bucket + 1];
     }
@@ -930,6 +945,9 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
   constexpr uint32_t kWordCap = TileLds<TILE>::kWordCap;
   static_assert(kBlocks % kWave == 0, "whole wavefronts of blocks");
   __shared__ TileLds<TILE> lds_all[kTokWaves];
+  __shared__ uint4 trim[17];
+  fill_trim_table(trim);
+  __syncthreads();
   TileLds<TILE>& lds  = lds_all[threadIdx.x / kWave];
   int const lane      = lane_id();
   uint32_t const rows = static_cast<uint32_t>(a.col.size);
@@ -1217,8 +1235,11 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
           uint32_t head[4];
           tw.head16(head);
           uint32_t const wl16 = min(wl, 16u);
-          trim_key8(wl16, head[0], head[1]);
-          trim_key8(wl16 > 8 ? wl16 - 8u : 0u, head[2], head[3]);
+          uint4 const keep    = trim[wl16];
+          head[0] &= keep.x;
+          head[1] &= keep.y;
+          head[2] &= keep.z;
+          head[3] &= keep.w;
           Probe pr;
           pr.k0             = head[0];
           pr.k1             = head[1];
@@ -1328,6 +1349,8 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTabl
   __shared__ int32_t first_ids[512];  // the ids of the one-byte keys of both key spaces: looked at whenever a piece of a word begins
   __shared__ int32_t pair_ids[kLetters2];  // the ids of the keys of two lower-case letters, second key space
   __shared__ uint16_t letters3[kLetters3];
+  __shared__ uint4 trim[17];
+  fill_trim_table(trim);
   for (int i = threadIdx.x; i < 512; i += kOovThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
   for (uint32_t i = threadIdx.x; i < kLetters2; i += kOovThreads) pair_ids[i] = table.short_ids[65536 + ((i / 26u + 'a') | ((i % 26u + 'a') << 8))];
   for (uint32_t i = threadIdx.x; i < kLetters3 / 2; i += kOovThreads)
@@ -1485,7 +1508,7 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTabl
       if (drained && ballot64(busy) == 0) break;
       continue;
     }
-    if (busy && !sw.done) sw.step(table, first_ids, letters3, pair_ids, keep_token);
+    if (busy && !sw.done) sw.step(table, first_ids, letters3, pair_ids, trim, keep_token);
   }
   add_together(acc_count != 0);
 }
