@@ -31,6 +31,7 @@
 #include "common.cuh"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <limits>
@@ -898,10 +899,24 @@ __device__ __forceinline__ uint32_t count_word_starts(const uint4* abase, int64_
   return total;
 }
 
-// range_first_row[g] = the first row (0..rows) that starts at or after the first byte of range g; [nranges] = rows
+// range_first_row[g] = the first row (0..rows) that starts at or after the first byte of range g; [nranges] = rows.
+// The first workgroup also sets the flag words of the call: zeros, but for the work counters, which start past the
+// units that the wavefronts take by their place in the grid (counter g serves the wavefronts g, g + kCounterGroups, ..
+// and hands out the units g, g + kCounterGroups, ..).
 __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32_t cbeg, int64_t range_bytes, uint32_t nranges,
-                                       uint32_t* __restrict__ range_first_row)
+                                       uint32_t* __restrict__ range_first_row, uint32_t* __restrict__ flags, uint32_t word_waves,
+                                       uint32_t oov_waves)
 {
+  if (blockIdx.x == 0) {
+    for (uint32_t i = threadIdx.x; i < kFlagWords; i += blockDim.x) {
+      uint32_t v = 0;
+      if (i >= kFlagWordUnits && i % kFlagLine == 0) {
+        uint32_t const c = (i - kFlagWordUnits) / kFlagLine;
+        v = ((c < kCounterGroups ? word_waves : oov_waves) + kCounterGroups - 1u - c % kCounterGroups) / kCounterGroups;
+      }
+      flags[i] = v;
+    }
+  }
   uint32_t const g = blockIdx.x * blockDim.x + threadIdx.x;
   if (g > nranges) return;
   int64_t const target = static_cast<int64_t>(g) * range_bytes;
@@ -1729,21 +1744,6 @@ __global__ void __launch_bounds__(kRareThreads) wordpiece_retokenize_kernel(Voca
   }
 }
 
-// The flag words of a tokenize call: zeros, but for the work counters, which start past the units that the wavefronts
-// take by their place in the grid (counter g serves the wavefronts g, g + kCounterGroups, .. and hands out the units
-// g, g + kCounterGroups, ..).
-__global__ void tokenize_flags_kernel(uint32_t* flags, uint32_t word_waves, uint32_t oov_waves)
-{
-  for (uint32_t i = threadIdx.x; i < kFlagWords; i += blockDim.x) {
-    uint32_t v = 0;
-    if (i >= kFlagWordUnits && i % kFlagLine == 0) {
-      uint32_t const g = (i - kFlagWordUnits) / kFlagLine;
-      v = ((g < kCounterGroups ? word_waves : oov_waves) + kCounterGroups - 1u - g % kCounterGroups) / kCounterGroups;
-    }
-    flags[i] = v;
-  }
-}
-
 struct RangeTokensOf {
   const uint32_t* counts;
   __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
@@ -2083,9 +2083,15 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   (void)hipGetDevice(&device);
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
   // persistent kernels: as many workgroups as can be resident at once
-  auto resident = [&](const void* kernel, int threads) -> int64_t {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 2;
+  // (asked of the runtime once per kernel and device: the answer does not change, and a call on a small column is
+  // short enough for three such questions to show)
+  auto resident = [&](const void* kernel, int threads, int which) -> int64_t {
+    static std::atomic<int> known[16][6];
+    int per_cu = device >= 0 && device < 16 ? known[device][which].load(std::memory_order_relaxed) : 0;
+    if (per_cu == 0) {
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 2;
+      if (device >= 0 && device < 16) known[device][which].store(per_cu, std::memory_order_relaxed);
+    }
     return static_cast<int64_t>(per_cu) * cus;
   };
   bool const is64  = input->offsets_is_int64 != 0;
@@ -2093,10 +2099,10 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   void (*const word_kernel)(TileArgs) = is64 ? (limit ? wordpiece_word_kernel<kTile, true, true> : wordpiece_word_kernel<kTile, true, false>)
                                              : (limit ? wordpiece_word_kernel<kTile, false, true> : wordpiece_word_kernel<kTile, false, false>);
   unsigned const word_grid = static_cast<unsigned>(
-    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(word_kernel), kTokThreads)));
-  unsigned const oov_grid  = static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads));
+    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(word_kernel), kTokThreads, (is64 ? 2 : 0) + (limit ? 1 : 0))));
+  unsigned const oov_grid  = static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads, 4));
   unsigned const emit_grid = static_cast<unsigned>(
-    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads)));
+    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads, 5)));
 
   TileArgs args{};
   args.col          = v;
@@ -2151,9 +2157,8 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     args.queue_size      = flags + kFlagQueueSize;
     args.counter         = flags + kFlagWordUnits;
     args.overflow        = flags + kFlagOverflow;
-    // the two work counters start past the units that the wavefronts take by their place in the grid
-    hipLaunchKernelGGL(tokenize_flags_kernel, dim3(1), dim3(256), 0, stream, flags, word_grid * kTokWaves, oov_grid * kOovWaves);
-    hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 1 + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row);
+    hipLaunchKernelGGL(range_first_row_kernel, dim3((nranges + 1 + 255) / 256), dim3(256), 0, stream, v, first_offset, cbeg, kRange, nranges, first_row,
+                       flags, word_grid * kTokWaves, oov_grid * kOovWaves);
     {
       ProfileScope ps("wordpiece_word_kernel", stream);
       hipLaunchKernelGGL(word_kernel, dim3(word_grid), dim3(kTokThreads), 0, stream, args);
@@ -2171,11 +2176,19 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     // where the tokens of each range go; the total decides the child size
     // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(RangeTokensOf{tokens}, static_cast<int64_t>(nranges), bases, scan_tmp, stream);
+    // the total (the last word of the scan's temporaries) and the first flag words (the part after it) in one copy
     uint32_t state[3] = {0, 0, 0};
-    hipError_t e      = hipMemcpyAsync(&total, scan_tmp + scan_tiles(nranges), sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(state, flags, sizeof(state), hipMemcpyDeviceToHost, stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+    {
+      const char* const from = reinterpret_cast<const char*>(scan_tmp + scan_tiles(nranges));
+      size_t const span      = static_cast<size_t>(reinterpret_cast<const char*>(flags + 3) - from);
+      alignas(8) char both[256 + 8 + sizeof(state)];
+      if (span > sizeof(both)) return give_up(NVTEXT_AMD_LOGIC_ERROR, "unexpected layout of the temporaries");
+      hipError_t e = hipMemcpyAsync(both, from, span, hipMemcpyDeviceToHost, stream);
+      if (e == hipSuccess) e = hipStreamSynchronize(stream);
+      if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+      std::memcpy(&total, both, sizeof(total));
+      std::memcpy(state, both + span - sizeof(state), sizeof(state));
+    }
 #ifdef WP_PHASE_TIMING
     {
       unsigned long long ph[10];
