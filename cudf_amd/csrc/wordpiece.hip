@@ -33,6 +33,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -765,7 +766,7 @@ struct ShortWord {
 //   * out-of-vocabulary pass: one lane per queued word; the result takes the place of the queue entry.
 //   * emit pass: a wavefront per range expands the word slots into the tokens and gives every row that starts in the
 //     range its list offset.
-constexpr int kRangeTiles    = 8;
+constexpr int kRangeTiles    = 8;     // tiles per range at most (a large column); a small column has fewer, so that every wavefront gets several ranges
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueChunk = 512;  // queue entries a wavefront of the word pass reserves at a time
 // A word slot: the token id (0 .. 2^31-1, or -1 for an absent [UNK]), or kOovMark | index of the word's queue entry
@@ -812,6 +813,7 @@ struct TileArgs {
   uint32_t cbeg;           // coordinate of the view's first byte (0..15)
   uint32_t nranges;
   int32_t max_words;
+  int32_t range_tiles;     // tiles of a range
   uint32_t range_cap;      // word slots of a range
   const uint32_t* range_first_row;
   uint32_t* arena;         // the word slots of range g from arena[g * range_cap], densely, in order
@@ -986,8 +988,8 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
   for (bool first = true;; first = false) {
     uint32_t const range = next_unit(a.counter, first, my_number, lane);
     if (range >= a.nranges) break;
-    int64_t t           = static_cast<int64_t>(range) * kRangeTiles;
-    int64_t const t_end = min(t + kRangeTiles, a.ntiles);
+    int64_t t           = static_cast<int64_t>(range) * a.range_tiles;
+    int64_t const t_end = min(t + a.range_tiles, a.ntiles);
     uint32_t r_cur      = a.range_first_row[range];
     uint32_t cursor     = 0;  // words of this range so far
     uint32_t known      = 0;  // of them, in the vocabulary (or too long: one unknown token each)
@@ -2070,14 +2072,10 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   }
 
   constexpr int kTile         = 2048;
-  constexpr int64_t kRange    = static_cast<int64_t>(kTile) * kRangeTiles;
   const uint8_t* const first_byte = v.chars + first_offset;
   uint32_t const cbeg             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(first_byte) & 15u);
   int64_t const cend              = cbeg + (last_offset - first_offset);
   int64_t const ntiles            = (cend + kTile - 1) / kTile;
-  int64_t const nranges64         = (ntiles + kRangeTiles - 1) / kRangeTiles;
-  if (nranges64 > 0x7FFFFFF0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
-  uint32_t const nranges = static_cast<uint32_t>(nranges64);
 
   int device = 0, cus = 256;
   (void)hipGetDevice(&device);
@@ -2098,8 +2096,23 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   bool const limit = max_words_per_row > 0;
   void (*const word_kernel)(TileArgs) = is64 ? (limit ? wordpiece_word_kernel<kTile, true, true> : wordpiece_word_kernel<kTile, true, false>)
                                              : (limit ? wordpiece_word_kernel<kTile, false, true> : wordpiece_word_kernel<kTile, false, false>);
+  int64_t const word_resident = resident(reinterpret_cast<const void*>(word_kernel), kTokThreads, (is64 ? 2 : 0) + (limit ? 1 : 0));
+  // A range is what a wavefront works through by itself, one tile after the other: kRangeTiles tiles when that still
+  // leaves every wavefront of the word pass eight ranges or more (the last ones then end close together), fewer in a
+  // smaller column (2M rows of 120 bytes: 0.34 -> 0.30 ms for the word pass).
+  int range_tiles = kRangeTiles;
+  while (range_tiles > 1 && ntiles / range_tiles < 8 * word_resident * kTokWaves) range_tiles >>= 1;
+  // (for tests, which have no column of a gigabyte to give: NVTEXT_AMD_RANGE_TILES=1|2|4|8 sets the size whatever the column's)
+  if (const char* const forced = std::getenv("NVTEXT_AMD_RANGE_TILES")) {
+    int const want = std::atoi(forced);
+    if (want == 1 || want == 2 || want == 4 || want == 8) range_tiles = want;
+  }
+  int64_t const kRange    = static_cast<int64_t>(kTile) * range_tiles;
+  int64_t const nranges64 = (ntiles + range_tiles - 1) / range_tiles;
+  if (nranges64 > 0x7FFFFFF0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
+  uint32_t const nranges = static_cast<uint32_t>(nranges64);
   unsigned const word_grid = static_cast<unsigned>(
-    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(word_kernel), kTokThreads, (is64 ? 2 : 0) + (limit ? 1 : 0))));
+    std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, word_resident));
   unsigned const oov_grid  = static_cast<unsigned>(resident(reinterpret_cast<const void*>(wordpiece_oov_kernel), kOovThreads, 4));
   unsigned const emit_grid = static_cast<unsigned>(
     std::min<int64_t>((static_cast<int64_t>(nranges) + kTokWaves - 1) / kTokWaves, resident(reinterpret_cast<const void*>(wordpiece_emit_kernel), kTokThreads, 5)));
@@ -2113,6 +2126,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   args.ntiles       = ntiles;
   args.cbeg         = cbeg;
   args.nranges      = nranges;
+  args.range_tiles  = range_tiles;
   args.max_words    = max_words_per_row;
 
   // Word slots per range and queue entries.  A range of ordinary text has a word per five or six bytes, and about a

@@ -425,9 +425,19 @@ def make_vocab(rng, n, letters, with_unk=True):
     return vocab
 
 
+@pytest.fixture(params=["column", "8"], ids=["ranges_by_column_size", "ranges_of_8_tiles"])
+def range_tiles(request, monkeypatch):
+    """The tokenizer gives a wavefront ranges of 1 to 8 tiles, the fewer the smaller the column; the columns of these
+    tests are all small, so the tests that take this fixture run a second time with the size that a column of a
+    gigabyte gets (the library reads NVTEXT_AMD_RANGE_TILES at every call)."""
+    if request.param != "column":
+        monkeypatch.setenv("NVTEXT_AMD_RANGE_TILES", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("max_words", [0, 7, 1000])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
-def test_wordpiece_random_vs_oracle(nv, orc, max_words, dtype):
+def test_wordpiece_random_vs_oracle(nv, orc, max_words, dtype, range_tiles):
     rng = np.random.default_rng(77 + max_words)
     letters = "abcdefghijkl"
     vocab = make_vocab(rng, 3000, letters)
@@ -485,7 +495,7 @@ def _tile_kernel_launches(nv, fn):
 @pytest.mark.parametrize("max_words", [0, 5, 100000])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 @pytest.mark.parametrize("shape", ["few rows", "many rows"])
-def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shape, dtype, max_words):
+def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shape, dtype, max_words, range_tiles):
     """Text whose ranges give more than three tokens per eight bytes (here two-letter words that are not in the
     vocabulary and fall apart into letters: two tokens per three bytes) does not fit the arena of the first
     attempt: the call has to notice, run the tile pass again with room for a token per byte, and give the same
@@ -516,7 +526,7 @@ def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shap
     assert_same(got.to_host(), orc.wordpiece_tokenize(plain, orc.Vocabulary(hv), max_words, nthreads=8), "plain text afterwards")
 
 
-def test_wordpiece_rows_of_one_byte_and_tiles_of_more_words_than_a_unit(nv, orc):
+def test_wordpiece_rows_of_one_byte_and_tiles_of_more_words_than_a_unit(nv, orc, range_tiles):
     """Every byte a row of its own (row starts separate words as spaces do: cpp/src/text/wordpiece_tokenize.cu:515-523), so a
     tile of 2048 bytes holds 2048 words, four times what is looked up at a time, and a token per byte; then the
     same bytes as words of one letter between spaces (1024 words per tile).  With a word limit a one-byte row has
@@ -538,7 +548,7 @@ def test_wordpiece_rows_of_one_byte_and_tiles_of_more_words_than_a_unit(nv, orc)
     assert orc.wordpiece_tokenize(one_byte_rows, ovoc, 0, nthreads=8).child.size == n
 
 
-def test_wordpiece_utf8_vs_oracle(nv, orc):
+def test_wordpiece_utf8_vs_oracle(nv, orc, range_tiles):
     rng = np.random.default_rng(99)
     base = list("abcdeé漢字ñ語😀")
     vocab = ["[unk]"] + base + ["##" + c for c in base[:8]]
@@ -559,7 +569,7 @@ def test_wordpiece_utf8_vs_oracle(nv, orc):
         assert_same(got, orc.wordpiece_tokenize(host, orc.Vocabulary(hv), mw, nthreads=4), f"utf8 mw={mw}")
 
 
-def test_wordpiece_sliced_nulls_vs_oracle(nv, orc):
+def test_wordpiece_sliced_nulls_vs_oracle(nv, orc, range_tiles):
     rng = np.random.default_rng(123)
     vocab = make_vocab(rng, 500, "abcdef")
     rows = []
@@ -579,7 +589,7 @@ def test_wordpiece_sliced_nulls_vs_oracle(nv, orc):
             assert_same(nv.wordpiece_tokenize(ds, dv, mw).to_host(), orc.wordpiece_tokenize(hs, ov, mw), f"slice {lo}:{hi} mw={mw}")
 
 
-def test_wordpiece_row_longer_than_chunks(nv, orc):
+def test_wordpiece_row_longer_than_chunks(nv, orc, range_tiles):
     """One row spanning many 256-byte chunks, with words straddling chunk boundaries."""
     rng = np.random.default_rng(321)
     vocab = make_vocab(rng, 2000, "abcdefgh")
@@ -635,7 +645,7 @@ def test_wordpiece_long_keys_and_many_pieces(nv, orc):
 
 
 @pytest.mark.parametrize("letters", [5, 7, 8, 12])
-def test_wordpiece_every_word_splits_into_as_many_pieces_as_it_has_letters(nv, orc, letters):
+def test_wordpiece_every_word_splits_into_as_many_pieces_as_it_has_letters(nv, orc, letters, range_tiles):
     """A vocabulary of single letters only, so that a word of k letters is k tokens: rounds of the library's last pass
     in which every word brings five tokens (its usual way of writing them), seven (more tokens in a round than it puts in
     order before writing: each word's are then written by themselves), eight and twelve (more than a word's record
@@ -705,7 +715,7 @@ def test_wordpiece_pieces_of_letters_and_of_their_neighbours(nv, orc):
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
-def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype):
+def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype, range_tiles):
     """Rows of hundreds of kilobytes (which the library tokenizes in pieces cut at spaces when there is no word limit)
     among short ones: with words of every length at the places where the cuts fall, a row that is one long word, a
     row that is mostly spaces, null rows, and the same column sliced."""
@@ -733,7 +743,7 @@ def test_wordpiece_very_long_rows_are_cut_at_spaces(nv, orc, dtype):
 
 
 @pytest.mark.parametrize("max_words", [0, 4])
-def test_wordpiece_long_runs_of_rows_without_bytes(nv, orc, max_words):
+def test_wordpiece_long_runs_of_rows_without_bytes(nv, orc, max_words, range_tiles):
     """Hundreds of thousands of empty and null rows in a row, before, between and after rows with text: the rows are
     shared out by work, and rows without bytes must neither be lost nor all fall to one group of lanes."""
     vocab = strings(["[UNK]", "hello", "world", "##s", "a", "b"])
