@@ -27,24 +27,24 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit e4d5e05)"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit d582704)"
 MEASURED_TRAFFIC_C2 = {
-    "range_first_row_kernel": (15959288, 246368),
-    "wordpiece_word_kernel": (1744831551, 1525719505),
-    "wordpiece_oov_kernel": (915428588, 844072134),
-    "wordpiece_emit_kernel": (1394081413, 905196941),
+    "range_first_row_kernel": (15970454, 248800),
+    "wordpiece_word_kernel": (1746710404, 1523748637),
+    "wordpiece_oov_kernel": (915002311, 846801296),
+    "wordpiece_emit_kernel": (1394015035, 905182598),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (4575180756, 63532928),
-    "normalize_tile_rows_kernel": (73449619, 7941632),
-    "normalize_write_kernel": (5469612756, 4672381653),
+    "normalize_count_kernel": (4575176291, 63532922),
+    "normalize_tile_rows_kernel": (73449676, 7941631),
+    "normalize_write_kernel": (5469595334, 4672364160),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
 # moves issue in fewer than 4 cycles).  The floor is the instruction sequence of the inner loop: uint32, one
 # v_mad_u64_u32 per product and one v_min3_u32 per two (1.5); uint64, three v_mad_u64_u32 and an add for the product,
 # and / shift / 64-bit add (2) of the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products (9.5).
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit e4d5e05)"
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit d582704)"
 MINHASH_VALU = {
     "C3": {"floor": 1.5, "measured": 1.98, "issue": 1.00},
     "C4": {"floor": 9.5, "measured": 13.39, "issue": 1.11},
