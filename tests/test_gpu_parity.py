@@ -425,7 +425,7 @@ def make_vocab(rng, n, letters, with_unk=True):
     return vocab
 
 
-@pytest.fixture(params=["column", "8"], ids=["ranges_by_column_size", "ranges_of_8_tiles"])
+@pytest.fixture(params=["column", "2", "8"], ids=["ranges_by_column_size", "ranges_of_2_tiles", "ranges_of_8_tiles"])
 def range_tiles(request, monkeypatch):
     """The tokenizer gives a wavefront ranges of 1 to 8 tiles, the fewer the smaller the column; the columns of these
     tests are all small, so the tests that take this fixture run a second time with the size that a column of a
