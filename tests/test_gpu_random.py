@@ -1,0 +1,129 @@
+"""GPU parity on randomly drawn columns: every operation of the library against the host oracle, over columns whose
+shape, alphabet, vocabulary, offsets type, nulls and slicing are drawn from a seed.  Bit-exact.  The tokenizer runs
+with its unit of work sized by the column and, a second time, as a column of a gigabyte would have it."""
+import numpy as np
+import pytest
+
+from cudf_amd.arrow_host import HostStringsColumn
+
+pytestmark = pytest.mark.gpu
+
+LETTERS = list("abcdefghijklmnopqrstuvwxyz")
+OTHERS = list("éüñ漢字😀")
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from cudf_amd import nvtext
+    from cudf_amd import _capi
+    _capi.load()  # fails loudly if the HIP library is missing
+    return nvtext
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import pyoracle
+    return pyoracle
+
+
+def draw_column(rng):
+    """(rows as a HostStringsColumn, vocabulary entries, the rows as Python strings or None)"""
+    utf8 = rng.random() < 0.4
+    alphabet = LETTERS[: int(rng.integers(2, 27))] + (OTHERS if utf8 else [])
+    entries = int(rng.choice([5, 50, 500, 5000]))
+    vocab = ["[UNK]"] if rng.random() < 0.9 else ["x0"]
+    seen = set(vocab)
+    longest = int(rng.choice([3, 6, 12, 24, 40]))
+    tries = 0
+    while len(vocab) < entries and tries < 20 * entries:
+        tries += 1
+        s = "".join(rng.choice(alphabet, int(rng.integers(1, longest + 1))))
+        if rng.random() < 0.4:
+            s = "##" + s
+        if s not in seen:
+            seen.add(s)
+            vocab.append(s)
+    stems = [v for v in vocab if not v.startswith("##") and v != "[UNK]"] or ["a"]
+    n = int(rng.choice([1, 3, 70, 1000, 8000]))
+    p_null = float(rng.choice([0, 0.1]))
+    long_at = int(rng.integers(0, n)) if rng.random() < 0.3 else -1
+    rows = []
+    for i in range(n):
+        u = rng.random()
+        if u < p_null:
+            rows.append(None)
+            continue
+        if u < p_null + 0.05:
+            rows.append("")
+            continue
+        words = int(rng.integers(1, 60)) if i != long_at else int(rng.integers(8000, 30000))
+        ws = []
+        for _ in range(words):
+            t = rng.random()
+            if t < 0.6:
+                ws.append(stems[int(rng.integers(0, len(stems)))])
+            elif t < 0.9:
+                ws.append("".join(rng.choice(alphabet, int(rng.integers(1, 20)))))
+            else:
+                ws.append("".join(rng.choice(alphabet, int(rng.integers(20, 260)))))
+        rows.append((" " if rng.random() < 0.8 else "  ").join(ws))
+    host = HostStringsColumn.from_pylist(rows)
+    if rng.random() < 0.3:
+        host = HostStringsColumn(host.chars, host.offsets.astype(np.int64), host.mask, host.size, host.offset, host.null_count)
+    if n > 4 and rng.random() < 0.4:
+        lo = int(rng.integers(0, n // 2))
+        hi = int(rng.integers(lo + 1, n + 1))
+        host = host.slice(lo, hi)
+    return host, vocab, rows
+
+
+@pytest.mark.parametrize("seed", range(4100, 4140))
+def test_random_column_every_operation_vs_oracle(nv, orc, seed, monkeypatch):
+    from oracle import normalize_py
+    rng = np.random.default_rng(seed)
+    host, vocab, rows = draw_column(rng)
+    what = f"seed {seed}: {host.size} rows, {len(vocab)} entries, offsets {host.offsets.dtype}, first row {host.offset}"
+    d = nv.DeviceStringsColumn.from_host(host)
+    hv = HostStringsColumn.from_pylist(vocab)
+    dv = nv.WordPieceVocabulary(nv.DeviceStringsColumn.from_host(hv))
+    ov = orc.Vocabulary(hv)
+    for max_words in (0, int(rng.choice([1, 5, 100]))):
+        if max_words > 0 and any(r is not None and r.endswith("  ") for r in rows):
+            continue  # (trailing double spaces with a word limit: the reference reads past the row there)
+        exp = orc.wordpiece_tokenize(host, ov, max_words, nthreads=8)
+        for tiles in (None, "8"):
+            if tiles is None:
+                monkeypatch.delenv("NVTEXT_AMD_RANGE_TILES", raising=False)
+            else:
+                monkeypatch.setenv("NVTEXT_AMD_RANGE_TILES", tiles)
+            got = nv.wordpiece_tokenize(d, dv, max_words).to_host()
+            assert got.equals(exp), f"wordpiece_tokenize max_words={max_words} range tiles {tiles}, {what}"
+    monkeypatch.delenv("NVTEXT_AMD_RANGE_TILES", raising=False)
+
+    P = int(rng.choice([1, 7, 64, 256]))
+    width = int(rng.choice([2, 4, 5, 9, 20]))
+    if host.size * P < 2**31 - 1:
+        a = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        b = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        assert nv.minhash(d, 7, a, b, width).to_host().equals(orc.minhash(host, 7, a, b, width, nthreads=8)), f"minhash P={P} width={width}, {what}"
+        a64 = rng.integers(1, 2**63, P, dtype=np.uint64)
+        b64 = rng.integers(0, 2**63, P, dtype=np.uint64)
+        assert nv.minhash64(d, 11, a64, b64, width).to_host().equals(orc.minhash64(host, 11, a64, b64, width, nthreads=8)), \
+            f"minhash64 P={P} width={width}, {what}"
+
+    lower = bool(rng.random() < 0.5)
+    tokens = [b"[CLS]", b"[SEP]"] if rng.random() < 0.5 else []
+    special = nv.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist([t.decode() for t in tokens])) if tokens else None
+    got = nv.normalize_characters(d, nv.CharacterNormalizer(lower, special)).to_host()
+    exp = normalize_py.normalize_characters_native(host, lower, tokens, nthreads=8)
+    assert np.array_equal(got.chars, exp.chars) and np.array_equal(got.offsets, exp.offsets), f"normalize_characters lower={lower}, {what}"
+
+    if host.size >= 2:
+        h1, h2 = host.slice(0, host.size - 1), host.slice(1, host.size)
+        got = nv.jaccard_index(nv.DeviceStringsColumn.from_host(h1), nv.DeviceStringsColumn.from_host(h2), width).to_host()
+        exp = orc.jaccard_index(h1, h2, width, nthreads=8)
+        valid = exp.validity()
+        assert got.size == exp.size and got.null_count == exp.null_count and np.array_equal(got.validity(), valid), f"jaccard_index, {what}"
+        assert np.array_equal(got.values.view(np.uint32)[valid], exp.values.view(np.uint32)[valid]), f"jaccard_index width={width}, {what}"
