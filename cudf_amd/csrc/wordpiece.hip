@@ -81,7 +81,8 @@ struct VocabTable {
   // Length filter: lens[length_filter_index(kind, first three key bytes) & lens_mask] has bit i (i < 31) set
   // when some key of that key space with those first bytes is i + 3 bytes long, bit 31 for 34 bytes and more.
   // Entries are shared by hashing, so a set bit promises nothing, a clear bit rules the length out.
-  const uint32_t* lens;
+  // (stored as 16-bit words: bits 0..14 for 3..17 bytes, bit 15 for 18 bytes and more; filter_word() spreads it out)
+  const uint16_t* lens;
   uint32_t lens_mask;
   // Direct tables for keys of one and two bytes: short_ids[kind * 65536 + (byte0 | byte1 << 8)] for two bytes,
   // short_ids[131072 + kind * 256 + byte0] for one; the token id, or INT32_MIN when there is no such key.
@@ -103,6 +104,9 @@ __host__ __device__ __forceinline__ uint32_t length_filter_index(uint32_t kind, 
   return x ^ (x >> 13);
 }
 __host__ __device__ __forceinline__ uint32_t length_filter_bit(uint32_t len) { return len >= 34 ? 31u : len - 3u; }
+// The stored form of a filter word and back: the lengths of 18 bytes and more share one bit.
+__host__ __device__ __forceinline__ uint16_t packed_filter_word(uint32_t w) { return static_cast<uint16_t>((w & 0x7FFFu) | ((w >> 15) ? 0x8000u : 0u)); }
+__host__ __device__ __forceinline__ uint32_t filter_word(uint32_t stored) { return (stored & 0x7FFFu) | ((stored & 0x8000u) ? 0xFFFF8000u : 0u); }
 
 __host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t h, uint32_t kind, uint32_t len, uint32_t* bucket)
 {
@@ -450,7 +454,7 @@ struct OovStepper {
 
   __device__ __forceinline__ void load_filter(VocabTable const& t, uint32_t kind)
   {
-    lens = len - start >= 3 ? t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask] : 0xFFFFFFFFu;
+    lens = len - start >= 3 ? filter_word(t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask]) : 0xFFFFFFFFu;
   }
 
   // probed: the whole word has been looked up and is known to be absent
@@ -594,7 +598,7 @@ struct ShortWord {
     uint32_t const b    = dword_at(p);
     uint32_t const left = rem - min(p, rem);
     Opening o;
-    uint32_t const lens = t.lens[length_filter_index(kind, b & 0x00FFFFFFu) & t.lens_mask];
+    uint32_t const lens = filter_word(t.lens[length_filter_index(kind, b & 0x00FFFFFFu) & t.lens_mask]);
     int32_t const two   = t.short_ids[kind * 65536 + (b & 0xFFFFu)];
     o.id1               = first_ids[kind * 256 + (b & 0xFFu)];
     o.lens              = left >= 3 ? lens : 0xFFFFFFFFu;
@@ -624,7 +628,7 @@ struct ShortWord {
     int32_t const two   = pair[ok2 ? i2 : 0u];
     o.lens              = ok3 ? (len3 | 0xFFFF0000u) : 0xFFFFFFFFu;
     o.id2               = ok2 ? two : kNone;
-    if (!ok3 && rem >= 3) o.lens = t.lens[length_filter_index(1u, x) & t.lens_mask];
+    if (!ok3 && rem >= 3) o.lens = filter_word(t.lens[length_filter_index(1u, x) & t.lens_mask]);
     if (!ok2 && rem >= 2) o.id2 = t.short_ids[65536 + (b & 0xFFFFu)];
     return o;
   }
@@ -1953,7 +1957,9 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->store.bind(mr, stream);
   v->d_slots = v->store.allocate(v->slot_bytes);
   v->d_pool  = v->store.allocate(v->pool_bytes);
-  v->d_lens  = v->store.allocate(lens.size() * sizeof(uint32_t));
+  std::vector<uint16_t> lens16(lens.size());
+  for (size_t i = 0; i < lens.size(); ++i) lens16[i] = packed_filter_word(lens[i]);
+  v->d_lens  = v->store.allocate(lens16.size() * sizeof(uint16_t));
   v->d_short = v->store.allocate(short_ids.size() * sizeof(int32_t));
   v->d_letters = v->store.allocate(letters3.size() * sizeof(uint16_t));
   if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters) {
@@ -1962,7 +1968,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   }
   hipError_t e1 = hipMemcpyAsync(v->d_slots, slots.data(), v->slot_bytes, hipMemcpyHostToDevice, stream);
   hipError_t e2 = blocks.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, blocks.data(), blocks.size(), hipMemcpyHostToDevice, stream);
-  hipError_t e4 = hipMemcpyAsync(v->d_lens, lens.data(), lens.size() * sizeof(uint32_t), hipMemcpyHostToDevice, stream);
+  hipError_t e4 = hipMemcpyAsync(v->d_lens, lens16.data(), lens16.size() * sizeof(uint16_t), hipMemcpyHostToDevice, stream);
   hipError_t e5 = hipMemcpyAsync(v->d_short, short_ids.data(), short_ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
   hipError_t e6 = hipMemcpyAsync(v->d_letters, letters3.data(), letters3.size() * sizeof(uint16_t), hipMemcpyHostToDevice, stream);
   hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
@@ -1976,7 +1982,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.unk_id      = unk;
   v->table.max_len[0]  = max_len[0];
   v->table.max_len[1]  = max_len[1];
-  v->table.lens        = static_cast<const uint32_t*>(v->d_lens);
+  v->table.lens        = static_cast<const uint16_t*>(v->d_lens);
   v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
   v->table.short_ids   = static_cast<const int32_t*>(v->d_short);
   v->table.letters3    = static_cast<const uint16_t*>(v->d_letters);
