@@ -37,6 +37,7 @@ EXPORTS = [
     "nvtext_amd_list_column_free",
     "nvtext_amd_profile_enable",
     "nvtext_amd_profile_read",
+    "nvtext_amd_profile_set_range_tiles",
 ]
 
 
@@ -224,12 +225,19 @@ def load():
     L.nvtext_amd_profile_enable.argtypes = [C.c_int32]
     L.nvtext_amd_profile_read.restype = C.c_int32
     L.nvtext_amd_profile_read.argtypes = [C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.c_int32]
+    L.nvtext_amd_profile_set_range_tiles.restype = None
+    L.nvtext_amd_profile_set_range_tiles.argtypes = [C.c_int32]
     _lib = L
     return L
 
 
 def profile_enable(on: bool) -> None:
     load().nvtext_amd_profile_enable(1 if on else 0)
+
+
+def set_range_tiles(tiles: int) -> None:
+    """Test knob: ranges of `tiles` (1, 2, 4, 8) tiles in every later wordpiece_tokenize call; 0 = sized by the column."""
+    load().nvtext_amd_profile_set_range_tiles(int(tiles))
 
 
 def profile_read(capacity: int = 4096):

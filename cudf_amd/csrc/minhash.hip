@@ -786,9 +786,9 @@ nvtext_amd_status nvtext_amd_minhash_preallocated(const nvtext_amd_strings_colum
   if (width < 2) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameter width should be an integer value of 2 or greater");
   if (a_count <= 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B cannot be empty");
   if (a_count != b_count) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B should have the same number of elements");
+  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
   if (static_cast<uint64_t>(input->size) * static_cast<uint64_t>(a_count) >= static_cast<uint64_t>(std::numeric_limits<int32_t>::max()))
     return fail(NVTEXT_AMD_OVERFLOW, "The number of parameters times the number of input rows exceeds the column size limit");
-  if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");
   if (input->null_count > 0 && !input->null_mask) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null_count > 0 requires a null mask");
   if (input->size > kPreallocatedMaxRows)
     return fail(NVTEXT_AMD_INVALID_ARGUMENT, "more rows than nvtext_amd_minhash_preallocated takes (NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS)");

@@ -770,6 +770,8 @@ struct ShortWord {
 //   * out-of-vocabulary pass: one lane per queued word; the result takes the place of the queue entry.
 //   * emit pass: a wavefront per range expands the word slots into the tokens and gives every row that starts in the
 //     range its list offset.
+// Tiles per range that nvtext_amd_profile_set_range_tiles asked for (0: sized by the column).
+std::atomic<int> g_forced_range_tiles{0};
 constexpr int kRangeTiles    = 8;     // tiles per range at most (a large column); a small column has fewer, so that every wavefront gets several ranges
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueChunk = 512;  // queue entries a wavefront of the word pass reserves at a time
@@ -936,19 +938,6 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
   range_first_row[g] = lo;
 }
 
-#ifdef WP_PHASE_TIMING
-#define WP_PHASE(i)                                         \
-  {                                                         \
-    uint64_t const now_ = __builtin_amdgcn_s_memtime();     \
-    phase_t[i] += now_ - phase_last;                        \
-    phase_last = now_;                                      \
-  }
-#elif defined(WP_MARK)
-#define WP_PHASE(i) asm volatile("; WPMARK " #i);
-#else
-#define WP_PHASE(i)
-#endif
-
 // One tile at a time per wavefront: stage its bytes (and the 256 after it) in LDS; mark the row starts in it; find
 // word starts and ends (lanes <-> 16-byte blocks: spaces by SWAR, row starts as extra separators); with a word limit,
 // drop the words past each row's limit; list the words (word k pairs start k with end k); look all of them up (lanes
@@ -957,10 +946,6 @@ __global__ void range_first_row_kernel(ColView col, int64_t first_offset, uint32
 template <int TILE, bool IS64, bool LIMIT>
 __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs a)
 {
-#ifdef WP_PHASE_TIMING
-  uint64_t phase_t[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  uint64_t phase_last  = __builtin_amdgcn_s_memtime();
-#endif
   constexpr int kBlocks       = TILE / 16;
   constexpr int kSubs         = kBlocks / kWave;
   constexpr uint32_t kWordCap = TileLds<TILE>::kWordCap;
@@ -1035,7 +1020,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
       if (t + 1 < t_end) request_tile(t + 1);
       for (int i = lane; i < kBlocks + kOverBlocks + 1; i += kWave) lds.bound[i] = 0;
       wave_lds_sync();
-      WP_PHASE(0)
 
       // ---- the rows that start in the tile: [r_first, r_end)
       uint32_t const r_first = r_cur;
@@ -1053,7 +1037,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
       }
       uint32_t const r_end = r_cur;
       wave_lds_sync();
-      WP_PHASE(1)
 
       // ---- word starts and ends
       uint32_t nw = 0, ne = 0, inside0 = 0;  // words that start in the tile, words that end in it, the tile begins inside a word
@@ -1088,7 +1071,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
         ne = base >> 16;
       }
       wave_lds_sync();
-      WP_PHASE(2)
 
       // word starts at positions below x (0 <= x)
       auto words_before = [&](uint32_t x) -> uint32_t {
@@ -1189,7 +1171,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
           a.offsets_out[r] = static_cast<int32_t>(cursor + words_before(p < TILE ? static_cast<uint32_t>(p) : static_cast<uint32_t>(TILE)));
         }
       }
-      WP_PHASE(3)
 
       // ---- the words, at most kWordCap at a time (only a tile of one- and two-byte rows or words has more)
       for (uint32_t w_lo = 0;; w_lo += kWordCap) {
@@ -1239,7 +1220,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
           if (lane == 0) word16[2 * (nwc - 1) + 1] = static_cast<uint16_t>(endpos);
         }
         wave_lds_sync();
-        WP_PHASE(4)
 
         // ---- look the words up; the ones that are not in the vocabulary, or not decided here, go to the queue
         if (cursor + nwc > a.range_cap) spill = true;
@@ -1327,7 +1307,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
         }
         cursor += nwc;
         wave_lds_sync();
-        WP_PHASE(5)
         if (w_hi == nw) break;
       }
     }
@@ -1340,10 +1319,6 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
   // the reserved entries that no word took
   for (uint32_t q = q_pos + lane; q < q_lim; q += kWave)
     if (q < a.queue_cap) a.queue[q].len_flags = 0;
-#ifdef WP_PHASE_TIMING
-  if (lane == 0)
-    for (int i = 0; i < 10; ++i) atomicAdd(reinterpret_cast<unsigned long long*>(a.overflow + 7) + i, static_cast<unsigned long long>(phase_t[i]));
-#endif
 }
 
 // ------------------------------------------------------------------ out-of-vocabulary pass
@@ -1995,6 +1970,11 @@ void nvtext_amd_wordpiece_vocabulary_destroy(nvtext_amd_wordpiece_vocabulary* v)
   delete v;  // the store hands the tables back
 }
 
+void nvtext_amd_profile_set_range_tiles(int32_t tiles)
+{
+  nvtext_amd::g_forced_range_tiles.store(tiles == 1 || tiles == 2 || tiles == 4 || tiles == 8 ? tiles : 0, std::memory_order_relaxed);
+}
+
 int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* v) { return v ? v->table.unk_id : -1; }
 
 nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
@@ -2108,11 +2088,8 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   // smaller column (2M rows of 120 bytes: 0.34 -> 0.30 ms for the word pass).
   int range_tiles = kRangeTiles;
   while (range_tiles > 1 && ntiles / range_tiles < 8 * word_resident * kTokWaves) range_tiles >>= 1;
-  // (for tests, which have no column of a gigabyte to give: NVTEXT_AMD_RANGE_TILES=1|2|4|8 sets the size whatever the column's)
-  if (const char* const forced = std::getenv("NVTEXT_AMD_RANGE_TILES")) {
-    int const want = std::atoi(forced);
-    if (want == 1 || want == 2 || want == 4 || want == 8) range_tiles = want;
-  }
+  // (tests, which have no column of a gigabyte to give, set the size through nvtext_amd_profile_set_range_tiles)
+  if (int const want = g_forced_range_tiles.load(std::memory_order_relaxed)) range_tiles = want;
   int64_t const kRange    = static_cast<int64_t>(kTile) * range_tiles;
   int64_t const nranges64 = (ntiles + range_tiles - 1) / range_tiles;
   if (nranges64 > 0x7FFFFFF0) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
@@ -2209,22 +2186,14 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
       std::memcpy(&total, both, sizeof(total));
       std::memcpy(state, both + span - sizeof(state), sizeof(state));
     }
-#ifdef WP_PHASE_TIMING
-    {
-      unsigned long long ph[10];
-      (void)hipMemcpy(ph, flags + 8, sizeof(ph), hipMemcpyDeviceToHost);
-      unsigned long long sum = 0;
-      for (auto x : ph) sum += x;
-      static const char* const names[10] = {"stage", "rows", "detect", "cap", "lists", "probe", "-", "-", "-", "-"};
-      for (int i = 0; i < 6; ++i) fprintf(stderr, "%s %.1f%%  ", names[i], 100.0 * ph[i] / (sum ? sum : 1));
-      fprintf(stderr, "\n");
-    }
-#endif
     bool const words_over = state[1] != 0, queue_over = state[2] > qcap;
     if (words_over || queue_over) {
       if (attempt > 0 || state[2] > 0x7FFFFFF0u) return give_up(NVTEXT_AMD_LOGIC_ERROR, "words exceed internal limit");
       if (words_over) range_cap = static_cast<uint32_t>(kRange + 8);
-      queue_capacity = std::max<uint64_t>(queue_capacity, state[2]);
+      // state[2] counts the chunks of kQueueChunk entries that the wavefronts reserved, the unused rest of each
+      // wavefront's last chunk included; which ranges a wavefront gets differs from one attempt to the next, and with it
+      // that rest: a chunk per wavefront on top of what this attempt reserved covers every assignment.
+      queue_capacity = std::max<uint64_t>(queue_capacity, static_cast<uint64_t>(state[2]) + static_cast<uint64_t>(word_grid) * kTokWaves * kQueueChunk);
       continue;
     }
     if (total > static_cast<uint64_t>(std::numeric_limits<int32_t>::max())) return give_up(NVTEXT_AMD_OVERFLOW, "Size of output exceeds the column size limit");

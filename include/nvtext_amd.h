@@ -171,7 +171,9 @@ nvtext_amd_status nvtext_amd_minhash64(const nvtext_amd_strings_column* input,
  * Temporaries live in an array inside the library, one copy per device, so the call makes no allocation and
  * releases nothing; in exchange it takes at most NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS rows (more is
  * NVTEXT_AMD_INVALID_ARGUMENT), and two calls that overlap in time on one device race on that array: keep the
- * calls of a device on one stream, or order them otherwise. */
+ * calls of a device on one stream, or order them otherwise.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress, under a lock): make one call on every device outside of any stream capture before the calls
+ * that are captured. */
 #define NVTEXT_AMD_MINHASH_PREALLOCATED_MAX_ROWS 1048576
 nvtext_amd_status nvtext_amd_minhash_preallocated(const nvtext_amd_strings_column* input,
                                                   uint32_t seed,

@@ -22,6 +22,12 @@ extern "C" {
 void    nvtext_amd_profile_enable(int32_t on);
 int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t capacity);
 
+/* Test knob.  nvtext_amd_wordpiece_tokenize hands its wavefronts ranges of 1, 2, 4 or 8 tiles of 2048 bytes, the
+ * fewer the smaller the column, so only a column of hundreds of megabytes runs with the largest.  tiles = 1, 2, 4 or 8
+ * makes every later call of the process use that size whatever the column's, so that small test columns cover the code
+ * as a large column runs it; any other value gives the choice back to the library.  Results do not depend on it. */
+void    nvtext_amd_profile_set_range_tiles(int32_t tiles);
+
 #ifdef __cplusplus
 }
 #endif

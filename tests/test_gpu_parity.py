@@ -426,13 +426,14 @@ def make_vocab(rng, n, letters, with_unk=True):
 
 
 @pytest.fixture(params=["column", "2", "8"], ids=["ranges_by_column_size", "ranges_of_2_tiles", "ranges_of_8_tiles"])
-def range_tiles(request, monkeypatch):
+def range_tiles(request):
     """The tokenizer gives a wavefront ranges of 1 to 8 tiles, the fewer the smaller the column; the columns of these
     tests are all small, so the tests that take this fixture run a second time with the size that a column of a
-    gigabyte gets (the library reads NVTEXT_AMD_RANGE_TILES at every call)."""
-    if request.param != "column":
-        monkeypatch.setenv("NVTEXT_AMD_RANGE_TILES", request.param)
-    return request.param
+    gigabyte gets (set through the library's test knob, nvtext_amd_profile_set_range_tiles)."""
+    from cudf_amd import _capi
+    _capi.set_range_tiles(0 if request.param == "column" else int(request.param))
+    yield request.param
+    _capi.set_range_tiles(0)
 
 
 @pytest.mark.parametrize("max_words", [0, 7, 1000])

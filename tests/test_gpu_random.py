@@ -4,6 +4,7 @@ with its unit of work sized by the column and, a second time, as a column of a g
 import numpy as np
 import pytest
 
+from cudf_amd import _capi
 from cudf_amd.arrow_host import HostStringsColumn
 
 pytestmark = pytest.mark.gpu
@@ -80,7 +81,7 @@ def draw_column(rng):
 
 
 @pytest.mark.parametrize("seed", range(4100, 4140))
-def test_random_column_every_operation_vs_oracle(nv, orc, seed, monkeypatch):
+def test_random_column_every_operation_vs_oracle(nv, orc, seed):
     from oracle import normalize_py
     rng = np.random.default_rng(seed)
     host, vocab, rows = draw_column(rng)
@@ -94,13 +95,12 @@ def test_random_column_every_operation_vs_oracle(nv, orc, seed, monkeypatch):
             continue  # (trailing double spaces with a word limit: the reference reads past the row there)
         exp = orc.wordpiece_tokenize(host, ov, max_words, nthreads=8)
         for tiles in (None, "8"):
-            if tiles is None:
-                monkeypatch.delenv("NVTEXT_AMD_RANGE_TILES", raising=False)
-            else:
-                monkeypatch.setenv("NVTEXT_AMD_RANGE_TILES", tiles)
-            got = nv.wordpiece_tokenize(d, dv, max_words).to_host()
+            _capi.set_range_tiles(0 if tiles is None else int(tiles))
+            try:
+                got = nv.wordpiece_tokenize(d, dv, max_words).to_host()
+            finally:
+                _capi.set_range_tiles(0)
             assert got.equals(exp), f"wordpiece_tokenize max_words={max_words} range tiles {tiles}, {what}"
-    monkeypatch.delenv("NVTEXT_AMD_RANGE_TILES", raising=False)
 
     P = int(rng.choice([1, 7, 64, 256]))
     width = int(rng.choice([2, 4, 5, 9, 20]))

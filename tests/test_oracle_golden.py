@@ -323,3 +323,35 @@ def test_copy_bitmask_shift():
     m = orc.copy_bitmask(sl)
     from cudf_amd.arrow_host import unpack_validity
     assert np.array_equal(unpack_validity(m, sl.size), col.validity()[7:101])
+
+
+# ----------------------------------------------------------------------------- null rows that keep their bytes
+def test_null_rows_that_keep_bytes_reduce_to_covered_cases():
+    """Non-empty nulls are legal libcudf input (cpp/include/cudf/copying.hpp:946-962) and no reference vector holds one.
+    What the code says of them reduces each operation to a case the vectors do cover: without a word limit the tokenizer
+    never reads the validity (cpp/src/text/wordpiece_tokenize.cu:503-568), so the tokens are those of the same buffers
+    without a mask; with a limit a null row has no words (:778), as if it were empty; minhash drops the slots of null
+    rows (cpp/src/text/minhash.cu:626-628), as if the rows had been emptied first."""
+    from cudf_amd.arrow_host import HostStringsColumn, pack_validity
+    texts = ["abc de abc", "de f", "", "gab c abc", "f", "c c c c"]
+    valid = np.array([False, True, True, False, False, True])
+    for dtype in (np.int32, np.int64):
+        base = strings(texts, dtype)
+        kept = HostStringsColumn(base.chars, base.offsets, pack_validity(valid), len(texts), 0, int((~valid).sum()))
+        emptied = strings([t if v else None for t, v in zip(texts, valid)], dtype)
+        vocab = orc.Vocabulary(strings(["[UNK]", "abc", "de", "f", "gab", "c"]))
+        all_tokens = orc.wordpiece_tokenize(base, vocab, 0)
+        got = orc.wordpiece_tokenize(kept, vocab, 0)
+        assert np.array_equal(got.child, all_tokens.child) and np.array_equal(got.offsets, all_tokens.offsets)
+        assert got.null_count == 3 and np.array_equal(got.validity(), valid)
+        assert got.to_pylist()[1] == [2, 3] and got.child.tolist()[:3] == [1, 2, 1]   # the null row 0 has its three tokens
+        for max_words in (1, 2, 50):
+            assert orc.wordpiece_tokenize(kept, vocab, max_words).equals(orc.wordpiece_tokenize(emptied, vocab, max_words))
+        a = np.array([3, 11, 7], np.uint32)
+        b = np.array([1, 2, 5], np.uint32)
+        assert orc.minhash(kept, 0, a, b, 4).equals(orc.minhash(emptied, 0, a, b, 4))
+        assert orc.minhash64(kept, 7, a.astype(np.uint64), b.astype(np.uint64), 4).equals(
+            orc.minhash64(emptied, 7, a.astype(np.uint64), b.astype(np.uint64), 4))
+        other = strings(["abc de", "de f", "x", "gab c", "f f", "c c"], dtype)
+        j1, j2 = orc.jaccard_index(kept, other, 2), orc.jaccard_index(emptied, other, 2)
+        assert j1.equals(j2)

@@ -31,11 +31,17 @@ def _both(nv, torch, host, P, width, seed):
     offsets = torch.full((host.size + 1,), -1, dtype=torch.int32, device="cuda")
     child = torch.full(((host.size - host.null_count) * P + 5,), -1, dtype=torch.int32, device="cuda")
     mask = torch.zeros(((host.size + 31) // 32,), dtype=torch.int32, device="cuda") if host.mask is not None else None
+    # a call of a few rows first: the one-time lookup of the scratch array's address on this device is not what is checked
+    warm = nv.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(["warm up", "the symbol lookup"]))
+    nv.minhash_preallocated(warm, seed, a, b, width, torch.zeros(3, dtype=torch.int32, device="cuda"),
+                            torch.zeros(2 * P, dtype=torch.int32, device="cuda"), None)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]   # hipMemGetInfo: sees a plain hipMalloc, which torch's own count does not
     nv.minhash_preallocated(col, seed, a, b, width, offsets, child, mask)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call took device memory"
     assert np.array_equal(offsets.cpu().numpy(), exp.offsets)
     got = child.cpu().numpy().view(np.uint32)
     assert np.array_equal(got[:exp.child.size], exp.child)
