@@ -56,18 +56,25 @@ struct HashTraits<uint64_t> {
   // Permutation (minhash.cu:350-351): ((hv*a + b) mod 2^64) % (2^61-1), see Fold<uint64_t>.
 };
 
-// (h * a + b) mod 2^64 in three full-rate multiply-adds and one add: lo64 = h.lo*a.lo + b; the two cross
-// products are summed separately (their high halves fall off the end) and added to the high dword.
-__device__ __forceinline__ uint64_t mul_add_u64(uint64_t h, uint64_t a, uint64_t b)
+// ((h * a + b) mod 2^64) folded once mod 2^61 - 1, that is (x & p) + (x >> 61) for the 64-bit x: at most p + 7.
+// x = h.lo * a.lo + b as one 64-bit multiply-add, the low halves of the two cross products added to its high dword
+// where it stands; the fold is a shift and a mask of that dword and one more multiply-add (q * 1 + x) for the carry.
+// Eight instructions, and none that only moves a value: the register pair that one multiply-add writes is the one
+// the next reads (written out with 64-bit adds, the compiler copies halves of pairs about for every product).
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint64_t permute_fold_u64(uint64_t h, uint64_t a, uint64_t b)
 {
   uint32_t const hl = static_cast<uint32_t>(h), hh = static_cast<uint32_t>(h >> 32);
   uint32_t const al = static_cast<uint32_t>(a), ah = static_cast<uint32_t>(a >> 32);
-  uint64_t x, t;
+  uint64_t x;
   asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(x) : "v"(hl), "v"(al), "v"(b) : "vcc");
-  asm("v_mad_u64_u32 %0, vcc, %1, %2, 0" : "=v"(t) : "v"(hl), "v"(ah) : "vcc");
-  asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(t) : "v"(hh), "v"(al), "v"(t) : "vcc");
-  uint32_t const hi = static_cast<uint32_t>(x >> 32) + static_cast<uint32_t>(t);
-  return (static_cast<uint64_t>(hi) << 32) | static_cast<uint32_t>(x);
+  u32x2_t xp = __builtin_bit_cast(u32x2_t, x);
+  xp.y += hl * ah + hh * al;
+  uint32_t const q = xp.y >> 29;
+  xp.y &= 0x1FFFFFFFu;
+  uint64_t y;
+  asm("v_mad_u64_u32 %0, vcc, %1, 1, %2" : "=v"(y) : "v"(q), "v"(__builtin_bit_cast(uint64_t, xp)) : "vcc");
+  return y;
 }
 
 // min of two values below 2^62 in one instruction: such bit patterns are non-negative finite doubles
@@ -143,7 +150,8 @@ struct Fold<uint64_t, K> {
   // x mod p for x < 2^64: x = q*2^61 + r with q <= 7, so y = r + q <= p + 7.
   static __device__ __forceinline__ uint64_t fold_once(uint64_t x) { return (x & p) + (x >> 61); }
 
-  static constexpr uint32_t kPerTrip = 2;
+  // hashes per trip: with one parameter per lane, four (the loop's own instructions weigh twice as much there)
+  static constexpr uint32_t kPerTrip = K == 1 ? 4 : 2;
   static __device__ __forceinline__ void run(const uint64_t* hashes, uint32_t padded, uint32_t first, uint32_t stride,
                                              const uint64_t (&a)[K], const uint64_t (&b)[K], uint64_t (&m)[K])
   {
@@ -153,13 +161,18 @@ struct Fold<uint64_t, K> {
     // reduced value, so they can never displace a correct minimum.
     uint32_t top = 0;
     for (uint32_t i = first; i < padded; i += stride) {
-      uint64_t const h0 = hashes[i], h1 = hashes[i + 1];
+      uint64_t h[kPerTrip];
+#pragma unroll
+      for (uint32_t j = 0; j < kPerTrip; ++j) h[j] = hashes[i + j];
 #pragma unroll
       for (int k = 0; k < K; ++k) {
-        uint64_t const y0 = fold_once(mul_add_u64(h0, a[k], b[k]));
-        uint64_t const y1 = fold_once(mul_add_u64(h1, a[k], b[k]));
-        top               = max(max(top, static_cast<uint32_t>(y0 >> 32)), static_cast<uint32_t>(y1 >> 32));
-        m[k]              = min_below_2_62(min_below_2_62(m[k], y0), y1);
+#pragma unroll
+        for (uint32_t j = 0; j < kPerTrip; j += 2) {
+          uint64_t const y0 = permute_fold_u64(h[j], a[k], b[k]);
+          uint64_t const y1 = permute_fold_u64(h[j + 1], a[k], b[k]);
+          top               = max(max(top, static_cast<uint32_t>(y0 >> 32)), static_cast<uint32_t>(y1 >> 32));
+          m[k]              = min_below_2_62(min_below_2_62(m[k], y0), y1);
+        }
       }
     }
     if (ballot64(top >= 0x1FFFFFFFu) != 0) {
@@ -224,30 +237,51 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       // blocks and the tail become scalar branches instead of masked ones).
       bool const plain         = all_ascii && n >= static_cast<int64_t>(width);
       uint32_t const width_all = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(width));
-      for (uint32_t q = 0; q < cnt; q += kWave) {
-        uint32_t const p = q + lane;
-        bool valid       = false;
-        T hv             = 0;
-        if (plain) {
-          valid = p < cnt && n - (base + p) >= static_cast<int64_t>(width_all);
+      if (plain) {
+        for (uint32_t q = 0; q < cnt; q += kWave) {
+          uint32_t const p = q + lane;
+          bool const valid = p < cnt && n - (base + p) >= static_cast<int64_t>(width_all);
+          T hv             = 0;
           if (valid) {
             WordSrc const src{lds.bytes, mis + p};
             hv = H::hash(src, width_all, seed);
             hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
           }
-        } else if (p < cnt) {
-          int64_t const gpos = base + p;
-          WordSrc const src{lds.bytes, mis + p};
-          uint32_t hlen;
-          valid = window_at(src, row + gpos, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen);
-          if (valid) {
-            hv = H::hash(src, hlen, seed);
-            hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
-          }
+          uint64_t const vm = ballot64(valid);
+          if (valid) lds.hashes[count + lanes_below(vm)] = hv;
+          count += static_cast<uint32_t>(__builtin_popcountll(vm));
         }
-        uint64_t const vm = ballot64(valid);
-        if (valid) lds.hashes[count + lanes_below(vm)] = hv;
-        count += static_cast<uint32_t>(__builtin_popcountll(vm));
+      } else {
+        // A tile with longer characters: all of them are found at once, and where they follow one another without a gap
+        // a lane takes a character, not a byte, and reads its window's length from the list of characters instead of
+        // walking.  (A row shorter than `width` comes here too, whatever its bytes.)
+        CharMap map;
+        map.exact = false;
+        if (!all_ascii) map.build(lds.bytes, mis, len, cnt, base + len == n, lds.chars, lane);
+        uint32_t const items = map.exact ? map.windows : cnt;  // characters, or byte positions
+        for (uint32_t q = 0; q < items; q += kWave) {
+          uint32_t const item = q + lane;
+          bool valid          = false;
+          T hv                = 0;
+          if (item < items) {
+            uint32_t p = item, hlen;
+            if (map.exact) {
+              valid = map.window(item, len, base == 0, width, lds.chars, &p, &hlen);
+            } else {
+              int64_t const gpos = base + p;
+              WordSrc const at{lds.bytes, mis + p};
+              valid = window_at(at, row + gpos, n - gpos, len - p, gpos == 0, all_ascii, width, &hlen);
+            }
+            if (valid) {
+              WordSrc const src{lds.bytes, mis + p};
+              hv = H::hash(src, hlen, seed);
+              hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
+            }
+          }
+          uint64_t const vm = ballot64(valid);
+          if (valid) lds.hashes[count + lanes_below(vm)] = hv;
+          count += static_cast<uint32_t>(__builtin_popcountll(vm));
+        }
       }
       fold_hashes<T, K>(lds, count, a, b, m, lane, pk);
     }
@@ -287,8 +321,13 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
   }
 }
 
-// One workgroup per (row, parameter chunk): the first kSpan bytes of the row.  The rows lie along x and, beyond
-// kMaxRowBlocks of them, along z (a grid holds 2^32 threads at most in one dimension).
+// One workgroup per (four consecutive rows, parameter chunk).  A row of up to kSoloBytes is done by one wavefront alone
+// (wavefront w takes row w of the four: nothing to combine, the minima go from the registers to the result); a longer
+// row is shared by the four wavefronts, which split its first kSpan bytes and combine through LDS, one such row after the
+// other.  The groups lie along x and, beyond kMaxRowBlocks of them, along z.
+constexpr int64_t kSoloBytes = 1024;
+constexpr int kGroupRows      = kWaves;
+
 template <typename T, int K>
 __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
                                                                 int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out)
@@ -296,39 +335,60 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][K * kWave];
 
-  int64_t const r = static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x;
-  if (r >= col.size || !col.valid(r)) return;
+  int64_t const r0 = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * kGroupRows;
+  if (r0 >= col.size) return;
+  int const lane           = lane_id();
+  int const wave           = threadIdx.x / kWave;
   int32_t const chunk_base = blockIdx.y * (K * kWave);
-  int64_t const o          = col.off(r);
-  int64_t const n          = col.off(r + 1) - o;
-  T* dst                   = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
   int32_t const in_chunk   = min(K * kWave, P - chunk_base);
-  if (n == 0) {
-    for (int j = threadIdx.x; j < in_chunk; j += kThreads) dst[j] = T{0};
-    return;
-  }
-  int const lane   = lane_id();
-  int const wave   = threadIdx.x / kWave;
-  Packing const pk = K == 1 ? packing_for(P) : Packing{kWave, 1};
+  Packing const pk         = K == 1 ? packing_for(P) : Packing{kWave, 1};
   T a[K], b[K], m[K];
   load_params<T, K>(pa, pb, P, chunk_base, pk.param_lane(lane), a, b, m);
 
-  int64_t const span = min(n, static_cast<int64_t>(kSpan));
-  int64_t sec        = (span + kWaves - 1) / kWaves;
-  sec                = (sec + kWave - 1) / kWave * kWave;
-  int64_t const sb   = min(span, wave * sec);
-  int64_t const se   = min(span, sb + sec);
-  if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
+  int const rows_here = static_cast<int>(min(static_cast<int64_t>(kGroupRows), col.size - r0));
+  int const wave_s    = __builtin_amdgcn_readfirstlane(wave);  // (the same in every lane: what depends on it stays scalar)
 
-  if (K == 1) m[0] = pk.combine(m[0]);
+  // step -1: the short row of this wavefront (row `wave` of the four); steps 0..3: this wavefront's part of the rows
+  // that are too long for that, one after the other
+  for (int step = -1; step < rows_here; ++step) {
+    bool const solo = step < 0;
+    int const i     = solo ? wave_s : step;
+    if (i >= rows_here || !col.valid(r0 + i)) continue;
+    int64_t const o = col.off(r0 + i);
+    int64_t const n = col.off(r0 + i + 1) - o;
+    if (solo != (n <= kSoloBytes)) continue;
 #pragma unroll
-  for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
-  __syncthreads();
-  for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
-    T v = red[0][j];
+    for (int k = 0; k < K; ++k) m[k] = std::numeric_limits<T>::max();
+    int64_t sb = 0, se = n;
+    if (!solo) {
+      int64_t const span = min(n, static_cast<int64_t>(kSpan));
+      int64_t sec        = (span + kWaves - 1) / kWaves;
+      sec                = (sec + kWave - 1) / kWave * kWave;
+      sb                 = min(span, wave * sec);
+      se                 = min(span, sb + sec);
+    }
+    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
+    if (K == 1) m[0] = pk.combine(m[0]);
+    T* const dst = out + static_cast<int64_t>(out_offsets[r0 + i]) + chunk_base;
+    if (solo) {
+      // nothing to combine: the minima go from the registers to the result; an empty row is zeros (minhash.cu:318)
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
-    dst[j] = v;
+      for (int k = 0; k < K; ++k) {
+        int32_t const j = lane + kWave * k;  // (with fewer than 64 parameters the first lanes hold one each, in order)
+        if (j < in_chunk) dst[j] = n > 0 ? m[k] : T{0};
+      }
+    } else {
+      __syncthreads();  // (the row before has been read out of red)
+#pragma unroll
+      for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+      __syncthreads();
+      for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
+        T v = red[0][j];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
+        dst[j] = v;
+      }
+    }
   }
 }
 
@@ -403,15 +463,16 @@ __global__ void uniform_offsets_kernel(int32_t* out, int32_t rows, int32_t P)
   if (i <= rows) out[i] = static_cast<int32_t>(i * P);
 }
 
-constexpr int32_t kMaxRowBlocks = 1 << 22;
+constexpr int32_t kMaxRowBlocks = 1 << 20;
 
 template <typename T, int K>
 void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, const int32_t* offsets,
                     const uint32_t* extra_prefix, T* child, hipStream_t stream)
 {
   int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
-  dim3 grid(static_cast<unsigned>(std::min(v.size, kMaxRowBlocks)), static_cast<unsigned>(chunks),
-            static_cast<unsigned>((v.size + kMaxRowBlocks - 1) / kMaxRowBlocks));
+  int32_t const groups = (v.size + kGroupRows - 1) / kGroupRows;  // four rows to a workgroup
+  dim3 grid(static_cast<unsigned>(std::min(groups, kMaxRowBlocks)), static_cast<unsigned>(chunks),
+            static_cast<unsigned>((groups + kMaxRowBlocks - 1) / kMaxRowBlocks));
   {
     ProfileScope ps("minhash_rows_kernel", stream);
     hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);

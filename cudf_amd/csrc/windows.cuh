@@ -20,6 +20,7 @@ template <typename T>
 struct WaveLds {
   uint32_t bytes[kTileWords];
   alignas(16) T hashes[kTile + 4];
+  uint32_t chars[kTile + kHalo];  // the characters that start in the staged bytes, in order: start | end << 16 (see CharMap)
 };
 
 // Stage row bytes [base, base+len) into dst; returns the byte offset of `base` inside it.
@@ -44,6 +45,73 @@ __device__ __forceinline__ uint32_t stage_bytes(const uint8_t* row, int64_t base
   *all_ascii = ballot64(hibits != 0) == 0;
   return mis;
 }
+
+// The characters of the staged bytes of a tile, found by the whole wavefront at once, for tiles that hold bytes beyond
+// ASCII.  The reference walks from every window start byte by byte, adding up what each first byte of a character
+// says of its length until `width` characters are counted (cpp/include/cudf/strings/string_view.cuh:67-80).  Where
+// every character of the staged bytes ends exactly where the next one starts, that sum is the distance from the start
+// of character k to the end of character k + width - 1: the characters are listed in LDS (start | end << 16, in
+// order), a lane takes a character instead of a byte position, and a window costs two reads of the list.  Other tiles
+// (stray continuation bytes, first bytes that promise more than follows) keep the walk.
+struct CharMap {
+  uint32_t count;    // characters that start in the staged bytes
+  uint32_t windows;  // of them, in the tile's window starts (the first `cnt` staged bytes)
+  bool exact;        // the list gives every window of the tile its length
+  bool at_row_end;   // the staged bytes reach the end of the row
+
+  // staged: the tile's bytes in LDS, its first byte at byte offset `mis`; len of them are the row's, the first cnt are
+  // window starts; chars: the list (room for a character per staged byte).
+  __device__ __forceinline__ void build(const uint32_t* staged, uint32_t mis, uint32_t len, uint32_t cnt, bool reaches_row_end, uint32_t* chars,
+                                        int lane)
+  {
+    const uint8_t* const sb = reinterpret_cast<const uint8_t*>(staged) + mis;
+    at_row_end              = reaches_row_end;
+    count                   = 0;
+    windows                 = 0;
+    for (uint32_t base = 0; base < len; base += kWave) {
+      uint32_t const pos   = base + static_cast<uint32_t>(lane);
+      uint32_t const b     = pos < len ? sb[pos] : 0x80u;
+      bool const start     = !is_utf8_continuation(b);
+      uint64_t const found = ballot64(start);
+      if (start) chars[count + lanes_below(found)] = pos | ((pos + static_cast<uint32_t>(bytes_in_utf8_byte(b))) << 16);
+      count += static_cast<uint32_t>(__builtin_popcountll(found));
+      if (base < cnt) windows += static_cast<uint32_t>(__builtin_popcountll(ballot64(start && pos < cnt)));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // every character but the first begins where the one before it ends
+    bool broken = false;
+    for (uint32_t k0 = 0; k0 < count; k0 += kWave) {
+      uint32_t const k = k0 + static_cast<uint32_t>(lane);
+      if (k >= 1 && k < count) broken = broken || (chars[k - 1] >> 16) != (chars[k] & 0xFFFFu);
+    }
+    // the last one: ends with the row, or, when the row goes on, begins in the last four staged bytes (then every window
+    // start of the tile, at least 4 * width bytes before the end of the staged bytes, has its `width` characters listed)
+    bool tail = false;
+    if (count > 0) {
+      uint32_t const last = chars[count - 1];
+      tail                = reaches_row_end ? (last >> 16) == len : len - (last & 0xFFFFu) <= 4u;
+    }
+    exact = tail && ballot64(broken) == 0;
+  }
+
+  // The window that begins with character k (k < windows): whether it counts, where it starts and its bytes.
+  // row_start: staged byte 0 is the row's first byte.
+  __device__ __forceinline__ bool window(uint32_t k, uint32_t len, bool row_start, int32_t width, const uint32_t* chars, uint32_t* pos,
+                                         uint32_t* hlen) const
+  {
+    uint32_t const first = chars[k] & 0xFFFFu;
+    *pos                 = first;
+    if (k + static_cast<uint32_t>(width) <= count) {
+      *hlen = (chars[k + static_cast<uint32_t>(width) - 1u] >> 16) - first;
+      return true;
+    }
+    // fewer than `width` characters are left (the staged bytes reach the end of the row): only the row's first position counts
+    *hlen = len - first;
+    return row_start && first == 0;
+  }
+};
 
 // Decides whether a window starts at this position and how many bytes it hashes
 // (cpp/src/text/minhash.cu:120-133 with cpp/include/cudf/strings/string_view.cuh:67-80).

@@ -135,7 +135,7 @@ def test_minhash_few_parameters_share_the_lanes_of_a_wavefront(nv, orc):
 
 
 def test_minhash_more_rows_than_a_grid_has_workgroups(nv, orc):
-    """More rows than the launch has workgroups (the cap is 2^22, a grid holds 2^32 threads): rows share workgroups."""
+    """More rows than a launch has workgroups along x (2^20 of them, four rows each): the rest lie along z."""
     rows = (1 << 22) + 12345
     rng = np.random.default_rng(17)
     lengths = rng.integers(0, 6, rows)
