@@ -183,6 +183,19 @@ def valu_object(name):
             "valu_issue": v["issue"], "frac": round(v["floor"] / v["measured"] * min(1.0, v["issue"]), 3), "source": VALU_SOURCE}
 
 
+# Peak of the VALUs: 1024 SIMDs x 2.4 GHz / 4 cycles per wave64 instruction = 614.4 G wave-instructions/s
+# (profiles/valu_instruction_rates.md: multiply-adds issue in 4.7 cycles, which this figure does not discount).
+VALU_WAVE_INST_PER_S = 1024 * 2.4e9 / 4
+
+
+def valu_from_rate(perm_per_s, bits):
+    """For a leg without a counter run of its own: the share of the VALUs' peak issue rate that the floor sequence of the
+    inner loop alone accounts for at the measured permutation rate (64 permutations per wave-instruction)."""
+    floor = 1.5 if bits == 32 else 8.5
+    return {"bound": "valu issue", "floor_inst_per_perm": floor,
+            "frac": round(perm_per_s / 64 * floor / VALU_WAVE_INST_PER_S, 3), "source": "measured rate x floor / peak issue rate"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -485,82 +498,86 @@ def main():
 
 
 def reference_shapes(args, orc, _capi, datagen, nvtext, HostStringsColumn, np, torch):
-    """The shapes of the reference's own benchmarks, largest row counts: minhash over 60,000 rows whose lengths are normal
-    between 0 and 28,000 bytes, hash_width 12 / 24, 26 / 260 parameters, both hash widths
-    (cpp/benchmarks/text/minhash.cpp:16-62), and wordpiece_tokenize over 2,097,152 copies of a 32-word row with a
-    six-entry vocabulary, max_words 0 / 20 / 40 (cpp/benchmarks/text/subword.cpp:18-52).  Random printable ASCII stands in
-    for the reference's random strings; parity against the host oracle on the first rows of each shape."""
+    """The shapes of the reference's own benchmarks.  minhash over rows whose lengths are normal between 0 and
+    row_width bytes: 60,000 x 28,000 with hash_width 12 / 24, 26 / 260 parameters and both hash widths, and the corners
+    15,000 x 6,000 and 30,000 x 50,000 at hash_width 12 (cpp/benchmarks/text/minhash.cpp:16-62); wordpiece_tokenize
+    over 32,768 / 262,144 / 2,097,152 copies of a 32-word row with a six-entry vocabulary, max_words 0 / 20 / 40
+    (cpp/benchmarks/text/subword.cpp:18-52).  Random printable ASCII stands in for the reference's random strings;
+    parity against the host oracle on the first rows of each shape."""
     legs = {"minhash": [], "wordpiece_tokenize": []}
     steps = max(3, args.steps // 2)
     threads = host_threads(orc)[0] if orc else 0
 
-    rows, row_width = 60_000, 28_000
-    rng = np.random.default_rng(20231)
-    lengths = np.clip(rng.normal(row_width / 2, row_width / 6, rows), 0, row_width).astype(np.int64)
-    offsets = np.zeros(rows + 1, np.int32)
-    np.cumsum(lengths, out=offsets[1:])
-    chars = rng.integers(32, 127, int(offsets[-1]), dtype=np.uint8)
-    col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
-    dc = nvtext.DeviceStringsColumn.from_host(col)
-    ib = input_bytes(col)
-    log(f"[bench] reference minhash shape: rows={rows} chars={col.chars_bytes / 1e9:.3f} GB")
-    for bits, fn in ((32, nvtext.minhash), (64, nvtext.minhash64)):
-        signed = np.int32 if bits == 32 else np.int64
-        for nparams in (26, 260):
-            a, b = datagen.make_params(nparams, bits, 7)
-            da = torch.from_numpy(a.view(signed)).cuda()
-            db = torch.from_numpy(b.view(signed)).cuda()
-            for width in (12, 24):
-                keep = {}
+    for rows, row_width, widths, param_counts in ((60_000, 28_000, (12, 24), (26, 260)), (15_000, 6_000, (12,), (26, 260)),
+                                                  (30_000, 50_000, (12,), (26, 260))):
+        rng = np.random.default_rng(20231)
+        lengths = np.clip(rng.normal(row_width / 2, row_width / 6, rows), 0, row_width).astype(np.int64)
+        offsets = np.zeros(rows + 1, np.int32)
+        np.cumsum(lengths, out=offsets[1:])
+        chars = rng.integers(32, 127, int(offsets[-1]), dtype=np.uint8)
+        col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
+        dc = nvtext.DeviceStringsColumn.from_host(col)
+        ib = input_bytes(col)
+        log(f"[bench] reference minhash shape: rows={rows} row_width={row_width} chars={col.chars_bytes / 1e9:.3f} GB")
+        for bits, fn in ((32, nvtext.minhash), (64, nvtext.minhash64)):
+            signed = np.int32 if bits == 32 else np.int64
+            for nparams in param_counts:
+                a, b = datagen.make_params(nparams, bits, 7)
+                da = torch.from_numpy(a.view(signed)).cuda()
+                db = torch.from_numpy(b.view(signed)).cuda()
+                for width in widths:
+                    keep = {}
 
-                def mstep():
-                    keep["o"] = fn(dc, 0, da, db, width)
-                    return keep["o"]
+                    def mstep():
+                        keep["o"] = fn(dc, 0, da, db, width)
+                        return keep["o"]
 
-                msec, leg, _ = measure(mstep, steps, 1, _capi, torch)
-                windows = int(np.maximum(lengths - (width - 1), (lengths > 0).astype(np.int64)).sum())
-                leg.update({"num_rows": rows, "row_width": row_width, "hash_width": width, "parameters": nparams, "hash_type": bits,
-                            "input_GBps": round(ib / msec / 1e9, 2), "gperm_per_s": round(windows * nparams / msec / 1e9, 1)})
-                if orc:
-                    n = 400 if bits == 32 else 100
-                    smp = col.slice(0, n)
-                    exp = (orc.minhash if bits == 32 else orc.minhash64)(smp, 0, a, b, width, nthreads=threads)
-                    got = fn(dc.slice(0, n, 0), 0, da, db, width).to_host()
-                    leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
-                log(f"[bench] reference minhash: {leg}")
-                legs["minhash"].append(leg)
-                del keep
-    del dc, col, chars
+                    msec, leg, _ = measure(mstep, steps, 1, _capi, torch)
+                    windows = int(np.maximum(lengths - (width - 1), (lengths > 0).astype(np.int64)).sum())
+                    leg.update({"num_rows": rows, "row_width": row_width, "hash_width": width, "parameters": nparams, "hash_type": bits,
+                                "input_GBps": round(ib / msec / 1e9, 2), "gperm_per_s": round(windows * nparams / msec / 1e9, 1),
+                                "valu": valu_from_rate(windows * nparams / msec, bits)})
+                    if orc:
+                        n = (400 if bits == 32 else 100) * 28_000 // row_width
+                        smp = col.slice(0, n)
+                        exp = (orc.minhash if bits == 32 else orc.minhash64)(smp, 0, a, b, width, nthreads=threads)
+                        got = fn(dc.slice(0, n, 0), 0, da, db, width).to_host()
+                        leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
+                    log(f"[bench] reference minhash: {leg}")
+                    legs["minhash"].append(leg)
+                    del keep
+        del dc, col, chars
 
-    rows = 2_097_152
     text = b"This is a test " * 8
-    chars = np.frombuffer(text * rows, dtype=np.uint8)
-    offsets = (np.arange(rows + 1, dtype=np.int64) * len(text)).astype(np.int32)
-    col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
     vocab = HostStringsColumn.from_pylist(["", "[UNK]", "This", "is", "a", "test"])
-    dc = nvtext.DeviceStringsColumn.from_host(col)
     dv = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(vocab))
-    ib = input_bytes(col)
-    for max_words in (0, 20, 40):
-        keep = {}
+    for rows in (32_768, 262_144, 2_097_152):
+        chars = np.frombuffer(text * rows, dtype=np.uint8)
+        offsets = (np.arange(rows + 1, dtype=np.int64) * len(text)).astype(np.int32)
+        col = HostStringsColumn(chars, offsets, None, rows, 0, 0)
+        dc = nvtext.DeviceStringsColumn.from_host(col)
+        ib = input_bytes(col)
+        for max_words in (0, 20, 40):
+            keep = {}
 
-        def tstep():
-            keep["o"] = nvtext.wordpiece_tokenize(dc, dv, max_words)
-            return keep["o"]
+            def tstep():
+                keep["o"] = nvtext.wordpiece_tokenize(dc, dv, max_words)
+                return keep["o"]
 
-        tsec, leg, tk = measure(tstep, steps, 1, _capi, torch)
-        ntok = keep["o"].child_size
-        leg.update({"num_rows": rows, "max_words": max_words, "chars_bytes": col.chars_bytes, "tokens_out": ntok,
-                    "input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(rows / tsec / 1e6, 2),
-                    "roofline": hbm_roofline(ib + 4 * ntok + 4 * (rows + 1), tsec, tk)})
-        if orc:
-            n = 100_000
-            exp = orc.wordpiece_tokenize(col.slice(0, n), orc.Vocabulary(vocab), max_words, nthreads=threads)
-            got = nvtext.wordpiece_tokenize(dc.slice(0, n, 0), dv, max_words).to_host()
-            leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
-        log(f"[bench] reference wordpiece_tokenize: {leg}")
-        legs["wordpiece_tokenize"].append(leg)
-        del keep
+            tsec, leg, tk = measure(tstep, steps if rows > 300_000 else 4 * steps, 1, _capi, torch)
+            ntok = keep["o"].child_size
+            leg.update({"num_rows": rows, "max_words": max_words, "chars_bytes": col.chars_bytes, "tokens_out": ntok,
+                        "input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(rows / tsec / 1e6, 2),
+                        "launches": len(tk), "roofline": hbm_roofline(ib + 4 * ntok + 4 * (rows + 1), tsec, tk)})
+            if orc:
+                n = min(rows, 100_000)
+                exp = orc.wordpiece_tokenize(col.slice(0, n), orc.Vocabulary(vocab), max_words, nthreads=threads)
+                got = nvtext.wordpiece_tokenize(dc.slice(0, n, 0), dv, max_words).to_host()
+                leg["parity"] = ("PASS" if got.equals(exp) else "FAIL") + f" (first {n} rows)"
+            log(f"[bench] reference wordpiece_tokenize: {leg}")
+            legs["wordpiece_tokenize"].append(leg)
+            del keep
+        del dc, col
     return legs
 
 

@@ -367,7 +367,7 @@ __device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t v, uint64_t*
 
 // ------------------------------------------------------------------ device-wide exclusive scan
 // out[i] = sum_{j<i} f(j) for i in [0, n]  (n+1 entries; out[n] is the total).
-// Three launches: per-tile sums, scan of the tile sums (one workgroup), rescan + add.
+// Three launches: per-tile sums, scan of the tile sums (one workgroup), rescan + add; one launch for a few thousand values.
 constexpr int kScanThreads = 256;
 constexpr int kScanItems   = 8;
 constexpr int kScanTile    = kScanThreads * kScanItems;
@@ -415,6 +415,40 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n
   }
 }
 
+// The whole scan by one workgroup, for the few thousand values of a small call: one launch instead of three.
+// tile_sums[tiles] receives the grand total, as scan_tile_offsets_kernel leaves it.
+constexpr int64_t kScanSmallTiles = 4;
+template <typename F, typename OutT>
+__global__ void __launch_bounds__(kScanThreads) scan_small_kernel(F f, int64_t n, uint64_t* total_out, OutT* out)
+{
+  __shared__ uint64_t lds[kScanThreads / kWave + 1];
+  uint64_t carry = 0;
+  for (int64_t tile = 0; tile * kScanTile < n; ++tile) {
+    int64_t const base = tile * kScanTile + static_cast<int64_t>(threadIdx.x) * kScanItems;
+    uint64_t vals[kScanItems];
+    uint64_t s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      int64_t const i = base + k;
+      vals[k]         = (i < n) ? static_cast<uint64_t>(f(i)) : 0;
+      s += vals[k];
+    }
+    uint64_t total;
+    uint64_t run = block_exclusive_scan64<kScanThreads>(s, lds, &total) + carry;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      int64_t const i = base + k;
+      if (i < n) out[i] = static_cast<OutT>(run);
+      run += vals[k];
+    }
+    carry += total;
+  }
+  if (threadIdx.x == 0) {
+    out[n]     = static_cast<OutT>(carry);
+    *total_out = carry;
+  }
+}
+
 inline int64_t scan_tiles(int64_t n) { return (n + kScanTile - 1) / kScanTile; }
 inline size_t scan_temp_bytes(int64_t n) { return static_cast<size_t>(scan_tiles(n) + 1) * sizeof(uint64_t); }
 
@@ -424,10 +458,23 @@ template <typename F, typename OutT>
 void device_exclusive_scan(F f, int64_t n, OutT* out, uint64_t* temp, hipStream_t stream)
 {
   int64_t const tiles = scan_tiles(n);
+  if (tiles <= kScanSmallTiles) {
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(scan_small_kernel<F, OutT>), dim3(1), dim3(kScanThreads), 0, stream, f, n, temp + tiles, out);
+    return;
+  }
   hipLaunchKernelGGL(HIP_KERNEL_NAME(scan_tile_sums_kernel<F>), dim3(static_cast<unsigned>(tiles)), dim3(kScanThreads), 0, stream, f, n, temp);
   hipLaunchKernelGGL(scan_tile_offsets_kernel, dim3(1), dim3(kScanThreads), 0, stream, temp, tiles);
   hipLaunchKernelGGL(HIP_KERNEL_NAME(scan_apply_kernel<F, OutT>), dim3(static_cast<unsigned>(tiles)), dim3(kScanThreads), 0, stream, f, n, temp, out);
 }
+
+// ------------------------------------------------------------------ scalars for the host
+// Eight 64-bit words of pinned host memory that kernels write and the host reads once the stream is synchronised (a
+// copy of a few bytes into ordinary host memory goes through a staging buffer and costs ten microseconds and more).
+// One buffer per host thread, allocated at the thread's first call and kept until the process ends; nullptr when the
+// allocation failed (the callers then copy).
+uint64_t* host_scalars();
+// dst[0] = offsets[first_index], dst[1] = offsets[last_index] (offsets of 32 or 64 bits)
+void launch_read_two_offsets(const void* offsets, int is64, int64_t first_index, int64_t last_index, uint64_t* dst, hipStream_t stream);
 
 // ------------------------------------------------------------------ bitmask copy
 // dst bit i = src bit (i + begin_bit); bits past `bits` are cleared

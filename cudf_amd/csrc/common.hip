@@ -109,6 +109,36 @@ __global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, int64_t count)
 }
 }  // namespace
 
+namespace {
+__global__ void read_two_offsets_kernel(const void* offsets, int is64, int64_t first_index, int64_t last_index, uint64_t* dst)
+{
+  int64_t const i = threadIdx.x == 0 ? first_index : last_index;
+  dst[threadIdx.x] = static_cast<uint64_t>(is64 ? static_cast<const int64_t*>(offsets)[i] : static_cast<int64_t>(static_cast<const int32_t*>(offsets)[i]));
+}
+}  // namespace
+
+uint64_t* host_scalars()
+{
+  struct Slot {
+    uint64_t* p = nullptr;
+    bool tried  = false;
+  };
+  thread_local Slot slot;
+  if (!slot.tried) {
+    slot.tried = true;
+    void* p    = nullptr;
+    // portable: usable whichever device the thread has current at a later call
+    if (hipHostMalloc(&p, 8 * sizeof(uint64_t), hipHostMallocPortable) == hipSuccess) slot.p = static_cast<uint64_t*>(p);
+    else (void)hipGetLastError();
+  }
+  return slot.p;
+}
+
+void launch_read_two_offsets(const void* offsets, int is64, int64_t first_index, int64_t last_index, uint64_t* dst, hipStream_t stream)
+{
+  hipLaunchKernelGGL(read_two_offsets_kernel, dim3(1), dim3(2), 0, stream, offsets, is64, first_index, last_index, dst);
+}
+
 void launch_copy_bitmask(uint32_t* dst, const uint32_t* src, int32_t begin_bit, int32_t bits, hipStream_t stream)
 {
   int32_t const words = (bits + 31) / 32;

@@ -805,8 +805,6 @@ struct TileLds {
   static constexpr uint32_t kWordCap = TILE / 4;
   uint32_t word_guard[1];                     // (takes the end of the word that ran into the tile)
   uint32_t word[kWordCap];                    // per word: start | end << 16
-  static constexpr uint32_t kQueueStage = 16;
-  alignas(16) uint4 queued[kQueueStage][2];   // the queue records of a round of 64 words (when there are no more than these), to be written side by side
 };
 
 struct TileArgs {
@@ -1221,8 +1219,17 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
         }
         wave_lds_sync();
 
-        // ---- look the words up; the ones that are not in the vocabulary, or not decided here, go to the queue
+        // ---- look the words up; the ones that are not in the vocabulary, or not decided here, go to the queue.
+        // A round of 64 words has ten such words on average, too few for the work of building and storing their
+        // records: a round only gives each its place in the queue (which its slot names) and lists it, at the front
+        // of the list of words itself (entry c of the listed words never lies behind the word it came from); the
+        // records of all of them are built and stored afterwards, lanes <-> listed words.
         if (cursor + nwc > a.range_cap) spill = true;
+        uint32_t const room = q_lim - q_pos;  // left of the reserved entries: used up before the next ones are begun
+        uint32_t fresh      = 0;              // where the next ones begin, once they are needed
+        bool have_fresh     = false;
+        uint32_t listed     = 0;
+        auto queue_place = [&](uint32_t c) { return c < room ? q_pos + c : fresh + (c - room); };
         for (uint32_t k0 = 0; k0 < nwc; k0 += kWave) {
           uint32_t const k   = k0 + lane;
           bool const active  = k < nwc;
@@ -1262,48 +1269,49 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
           uint32_t const defer = !active || too_long || found ? 0u : (wl > 16 || (vd == 2u && wl <= table.max_len[0])) ? 2u : 1u;
           uint32_t value       = too_long ? static_cast<uint32_t>(table.unk_id) : static_cast<uint32_t>(id);
           uint64_t const mm    = ballot64(defer != 0);
-          if (mm != 0) {
-            uint32_t const nm   = static_cast<uint32_t>(__builtin_popcountll(mm));
-            uint32_t const room = q_lim - q_pos;  // left of the reserved entries: used up before the next ones are begun
-            uint32_t fresh      = 0;
-            if (nm > room) {
-              if (lane == 0) fresh = atomicAdd(a.queue_size, kQueueChunk);
-              fresh = wave_bcast(fresh, 0);
-            }
-            // (a vector memory instruction costs the address unit about the same for ten lanes as for sixty-four: the
-            // records of a round, ten of them on average, go side by side through LDS and out with one instruction)
-            bool const staged = nm <= TileLds<TILE>::kQueueStage;
-            if (defer != 0) {
-              uint32_t const rank = lanes_below(mm);
-              uint32_t const q    = rank < room ? q_pos + rank : fresh + (rank - room);
-              int64_t const at    = tb + s;
-              uint4 const first   = make_uint4(head[0], head[1], head[2], head[3]);
-              uint4 const second  = make_uint4(wl | (defer == 2u ? kUnprobed : 0u), range, static_cast<uint32_t>(at), static_cast<uint32_t>(static_cast<uint64_t>(at) >> 32));
-              if (staged) {
-                lds.queued[rank][0] = first;
-                lds.queued[rank][1] = second;
-              } else if (q < a.queue_cap) {
-                uint4* const dst = reinterpret_cast<uint4*>(a.queue + q);
-                store_stream(dst, first);
-                store_stream(dst + 1, second);
-              }
-              value = kOovMark | q;
-            }
-            if (staged) {
-              wave_lds_sync();
-              uint32_t const e = static_cast<uint32_t>(lane) >> 1;
-              uint32_t const q = e < room ? q_pos + e : fresh + (e - room);
-              if (e < nm && q < a.queue_cap) store_stream(reinterpret_cast<uint4*>(a.queue + q) + (lane & 1), lds.queued[e][lane & 1]);
-            }
-            if (nm > room) {
-              q_pos = fresh + (nm - room);
-              q_lim = fresh + kQueueChunk;
-            } else {
-              q_pos += nm;
-            }
+          uint32_t const nm    = static_cast<uint32_t>(__builtin_popcountll(mm));
+          if (listed + nm > room && !have_fresh) {
+            if (lane == 0) fresh = atomicAdd(a.queue_size, kQueueChunk);
+            fresh      = wave_bcast(fresh, 0);
+            have_fresh = true;
           }
+          if (defer != 0) {
+            uint32_t const c = listed + lanes_below(mm);
+            lds.word[c]      = rec | (defer << 12);  // (a word starts below 2048: bits 12 and 13 of its entry are free)
+            value            = kOovMark | queue_place(c);
+          }
+          listed += nm;
           known += static_cast<uint32_t>(__builtin_popcountll(ballot64(active && defer == 0)));
           if (active && !spill) region[cursor + k] = value;
+        }
+        wave_lds_sync();
+        // the records of the listed words: the word's first 16 bytes, its length, its range and where it begins
+        for (uint32_t c0 = 0; c0 < listed; c0 += kWave) {
+          uint32_t const c = c0 + lane;
+          if (c < listed) {
+            uint32_t const entry = lds.word[c];
+            uint32_t const s     = entry & 0xFFFu;
+            uint32_t const wl    = (entry >> 16) - s + 1u;
+            uint32_t const defer = (entry >> 12) & 3u;
+            TileWord const tw{lds.bytes, 16u + s};
+            uint32_t head[4];
+            tw.head16(head);
+            uint4 const keep = trim[min(wl, 16u)];
+            int64_t const at = tb + s;
+            uint32_t const q = queue_place(c);
+            if (q < a.queue_cap) {
+              uint4* const dst = reinterpret_cast<uint4*>(a.queue + q);
+              store_stream(dst, make_uint4(head[0] & keep.x, head[1] & keep.y, head[2] & keep.z, head[3] & keep.w));
+              store_stream(dst + 1, make_uint4(wl | (defer == 2u ? kUnprobed : 0u), range, static_cast<uint32_t>(at),
+                                               static_cast<uint32_t>(static_cast<uint64_t>(at) >> 32)));
+            }
+          }
+        }
+        if (listed > room) {
+          q_pos = fresh + (listed - room);
+          q_lim = fresh + kQueueChunk;
+        } else {
+          q_pos += listed;
         }
         cursor += nwc;
         wave_lds_sync();
@@ -1346,13 +1354,15 @@ __global__ void __launch_bounds__(kOovThreads, 8) wordpiece_oov_kernel(VocabTabl
   __shared__ int32_t pair_ids[kLetters2];  // the ids of the keys of two lower-case letters, second key space
   __shared__ uint16_t letters3[kLetters3];
   __shared__ uint4 trim[17];
+  // an empty queue (a small call, text that is all in the vocabulary), or one that was too small (the host repeats the
+  // passes with a larger one): nothing to do, and the tables need not be fetched
+  if (*queue_size == 0 || *queue_size > queue_cap) return;
   fill_trim_table(trim);
   for (int i = threadIdx.x; i < 512; i += kOovThreads) first_ids[i] = table.short_ids[2 * 65536 + i];
   for (uint32_t i = threadIdx.x; i < kLetters2; i += kOovThreads) pair_ids[i] = table.short_ids[65536 + ((i / 26u + 'a') | ((i % 26u + 'a') << 8))];
   for (uint32_t i = threadIdx.x; i < kLetters3 / 2; i += kOovThreads)
     reinterpret_cast<uint32_t*>(letters3)[i] = reinterpret_cast<const uint32_t*>(table.letters3)[i];
   __syncthreads();
-  if (*queue_size > queue_cap) return;  // the queue was too small: the host repeats the passes with a larger one
   uint32_t const total = *queue_size;
   OovLds& lds          = lds_all[threadIdx.x / kWave];
   int const lane       = lane_id();
@@ -1725,6 +1735,15 @@ __global__ void __launch_bounds__(kRareThreads) wordpiece_retokenize_kernel(Voca
   }
 }
 
+// What the host needs to know before the emit pass: the number of tokens, whether a range ran out of word slots, the
+// queue entries reserved.
+__global__ void publish_state_kernel(const uint64_t* __restrict__ total, const uint32_t* __restrict__ flags, uint64_t* __restrict__ dst)
+{
+  if (threadIdx.x == 0) dst[0] = *total;
+  if (threadIdx.x == 1) dst[1] = flags[kFlagOverflow];
+  if (threadIdx.x == 2) dst[2] = flags[kFlagQueueSize];
+}
+
 struct RangeTokensOf {
   const uint32_t* counts;
   __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
@@ -2032,7 +2051,15 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   // the bytes between them are what is tokenized
   size_t const ow = input->offsets_is_int64 ? 8 : 4;
   int64_t first_offset = 0, last_offset = 0;
-  {
+  uint64_t* const scalars = host_scalars();  // pinned words that kernels write for the host (nullptr: copy instead)
+  if (scalars) {
+    launch_read_two_offsets(input->offsets, input->offsets_is_int64 != 0, input->offset, static_cast<int64_t>(input->offset) + rows, scalars, stream);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+    first_offset = static_cast<int64_t>(scalars[0]);
+    last_offset  = static_cast<int64_t>(scalars[1]);
+  } else {
     unsigned char buf[16] = {0};
     const uint8_t* d_off  = static_cast<const uint8_t*>(input->offsets) + static_cast<size_t>(input->offset) * ow;
     hipError_t e          = hipMemcpyAsync(buf, d_off, ow, hipMemcpyDeviceToHost, stream);
@@ -2173,9 +2200,18 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
     // where the tokens of each range go; the total decides the child size
     // (cpp/include/cudf/detail/sizes_to_offsets_iterator.cuh:302-339)
     device_exclusive_scan(RangeTokensOf{tokens}, static_cast<int64_t>(nranges), bases, scan_tmp, stream);
-    // the total (the last word of the scan's temporaries) and the first flag words (the part after it) in one copy
+    // the total (the last word of the scan's temporaries) and the first flag words: written to the pinned words by a
+    // kernel of one wavefront, or, without those, fetched in one copy (the flags lie right behind the scan's temporaries)
     uint32_t state[3] = {0, 0, 0};
-    {
+    if (scalars) {
+      hipLaunchKernelGGL(publish_state_kernel, dim3(1), dim3(kWave), 0, stream, scan_tmp + scan_tiles(nranges), flags, scalars + 2);
+      hipError_t e = hipGetLastError();
+      if (e == hipSuccess) e = hipStreamSynchronize(stream);
+      if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+      total    = scalars[2];
+      state[1] = static_cast<uint32_t>(scalars[3]);
+      state[2] = static_cast<uint32_t>(scalars[4]);
+    } else {
       const char* const from = reinterpret_cast<const char*>(scan_tmp + scan_tiles(nranges));
       size_t const span      = static_cast<size_t>(reinterpret_cast<const char*>(flags + 3) - from);
       alignas(8) char both[256 + 8 + sizeof(state)];
