@@ -38,6 +38,7 @@ EXPORTS = [
     "nvtext_amd_profile_enable",
     "nvtext_amd_profile_read",
     "nvtext_amd_profile_set_range_tiles",
+    "nvtext_amd_profile_set_sizing_sample",
 ]
 
 
@@ -227,6 +228,8 @@ def load():
     L.nvtext_amd_profile_read.argtypes = [C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.c_int32]
     L.nvtext_amd_profile_set_range_tiles.restype = None
     L.nvtext_amd_profile_set_range_tiles.argtypes = [C.c_int32]
+    L.nvtext_amd_profile_set_sizing_sample.restype = None
+    L.nvtext_amd_profile_set_sizing_sample.argtypes = [C.c_int32]
     _lib = L
     return L
 
@@ -238,6 +241,11 @@ def profile_enable(on: bool) -> None:
 def set_range_tiles(tiles: int) -> None:
     """Test knob: ranges of `tiles` (1, 2, 4, 8) tiles in every later wordpiece_tokenize call; 0 = sized by the column."""
     load().nvtext_amd_profile_set_range_tiles(int(tiles))
+
+
+def set_sizing_sample(on: bool) -> None:
+    """Test knob: whether wordpiece_tokenize sizes its first attempt from a sample of the column (the default)."""
+    load().nvtext_amd_profile_set_sizing_sample(1 if on else 0)
 
 
 def profile_read(capacity: int = 4096):

@@ -468,10 +468,12 @@ void device_exclusive_scan(F f, int64_t n, OutT* out, uint64_t* temp, hipStream_
 }
 
 // ------------------------------------------------------------------ scalars for the host
-// Eight 64-bit words of pinned host memory that kernels write and the host reads once the stream is synchronised (a
-// copy of a few bytes into ordinary host memory goes through a staging buffer and costs ten microseconds and more).
-// One buffer per host thread, allocated at the thread's first call and kept until the process ends; nullptr when the
-// allocation failed (the callers then copy).
+// A few KB of pinned host memory that kernels write and the host reads once the stream is synchronised (a copy of a
+// few bytes into ordinary host memory goes through a staging buffer and costs ten microseconds and more): eight 64-bit
+// words, and behind them room for kHostSampleWords 32-bit words.  One buffer per host thread, allocated at the thread's
+// first call and kept until the process ends; nullptr when the allocation failed (the callers then copy).
+constexpr size_t kHostSampleWords = 3 * 512;
+constexpr size_t kHostScalarBytes = 8 * sizeof(uint64_t) + kHostSampleWords * sizeof(uint32_t);
 uint64_t* host_scalars();
 // dst[0] = offsets[first_index], dst[1] = offsets[last_index] (offsets of 32 or 64 bits)
 void launch_read_two_offsets(const void* offsets, int is64, int64_t first_index, int64_t last_index, uint64_t* dst, hipStream_t stream);

@@ -128,7 +128,7 @@ uint64_t* host_scalars()
     slot.tried = true;
     void* p    = nullptr;
     // portable: usable whichever device the thread has current at a later call
-    if (hipHostMalloc(&p, 8 * sizeof(uint64_t), hipHostMallocPortable) == hipSuccess) slot.p = static_cast<uint64_t*>(p);
+    if (hipHostMalloc(&p, kHostScalarBytes, hipHostMallocPortable) == hipSuccess) slot.p = static_cast<uint64_t*>(p);
     else (void)hipGetLastError();
   }
   return slot.p;

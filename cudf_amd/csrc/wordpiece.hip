@@ -772,6 +772,8 @@ struct ShortWord {
 //     range its list offset.
 // Tiles per range that nvtext_amd_profile_set_range_tiles asked for (0: sized by the column).
 std::atomic<int> g_forced_range_tiles{0};
+// Whether a call sizes its first attempt from a sample of the column (nvtext_amd_profile_set_sizing_sample).
+std::atomic<int> g_sizing_sample{1};
 constexpr int kRangeTiles    = 8;     // tiles per range at most (a large column); a small column has fewer, so that every wavefront gets several ranges
 constexpr int kOverBlocks    = 16;   // 16-byte blocks staged past the tile: a word that starts in the tile ends in them, or is kMaxWord bytes or more
 constexpr uint32_t kQueueChunk = 512;  // queue entries a wavefront of the word pass reserves at a time
@@ -1735,6 +1737,61 @@ __global__ void __launch_bounds__(kRareThreads) wordpiece_retokenize_kernel(Voca
   }
 }
 
+// ------------------------------------------------------------------ a sample of the column, for sizing
+// How many words a byte of this column has, and how many of them will be queued, decides the sizes of the word slots
+// and of the queue; text in another language than the vocabulary's, or of very short words, needs several times what
+// ordinary text does, and finding that out by running out of room costs the word pass a second time.  So the call
+// first looks at kSampleWindows windows of kSampleBytes spread evenly over the column's bytes, one wavefront each:
+// words as maximal runs of bytes that are not spaces (rows and the word limit are left aside: an estimate), each
+// looked up whole.  It runs on the offsets alone, before the host knows where the bytes begin, and leaves the view's
+// first and last offset for the host as well: the call synchronises once for both.
+constexpr int kSampleWindows = 512;
+constexpr int kSampleBytes   = 512;
+constexpr int kSampleTail    = 208;  // bytes staged past a window: a word that starts in it ends there, or is kMaxWord bytes or more
+static_assert(3 * kSampleWindows <= kHostSampleWords, "a window's three counts fit the pinned words");
+
+__global__ void __launch_bounds__(kWave) wordpiece_sample_kernel(ColView col, VocabTable table, uint64_t* __restrict__ first_last,
+                                                               uint32_t* __restrict__ counts)
+{
+  __shared__ uint32_t staged[(kSampleBytes + kSampleTail + 8) / 4 + 4];  // byte 4 + x of it: byte x of the window; byte 3: the one before
+  int const lane      = lane_id();
+  int64_t const first = col.off(0), last = col.off(col.size);
+  if (blockIdx.x == 0 && lane == 0) {
+    first_last[0] = static_cast<uint64_t>(first);
+    first_last[1] = static_cast<uint64_t>(last);
+  }
+  int64_t const span    = last - first;
+  int64_t const windows = min(static_cast<int64_t>(kSampleWindows), (span + kSampleBytes - 1) / kSampleBytes);
+  uint32_t words = 0, queued = 0, bytes = 0;
+  if (static_cast<int64_t>(blockIdx.x) < windows) {
+    int64_t const begin = first + span / windows * blockIdx.x;
+    int64_t const end   = min(last, begin + kSampleBytes);
+    bytes               = static_cast<uint32_t>(end - begin);
+    uint8_t* const sb   = reinterpret_cast<uint8_t*>(staged);
+    for (int i = lane; i < 4 + kSampleBytes + kSampleTail + 8; i += kWave) {
+      int64_t const g = begin + i - 4;
+      sb[i]           = (g >= first && g < last) ? col.chars[g] : uint8_t{0x20};  // outside the view: a space
+    }
+    wave_lds_sync();
+    // a lane takes eight byte positions and the words that start there
+    constexpr uint32_t kMine = kSampleBytes / kWave;
+    for (uint32_t p = kMine * lane; p < kMine * lane + kMine && p < bytes; ++p) {
+      if (sb[4 + p] == 0x20u || sb[3 + p] != 0x20u) continue;
+      uint32_t len = 1;
+      while (len < kMaxWord && sb[4 + p + len] != 0x20u) ++len;
+      ++words;
+      if (len >= kMaxWord) continue;  // one unknown token, never queued
+      if (len > 16 || lookup_slow(table, 0u, TileWord{staged, 4u + p}, 0u, len) == kNone) ++queued;
+    }
+  }
+  uint32_t const w = wave_bcast(wave_inclusive_scan(words), kWave - 1), q = wave_bcast(wave_inclusive_scan(queued), kWave - 1);
+  if (lane == 0) {
+    counts[3 * blockIdx.x]     = w;
+    counts[3 * blockIdx.x + 1] = q;
+    counts[3 * blockIdx.x + 2] = bytes;
+  }
+}
+
 // What the host needs to know before the emit pass: the number of tokens, whether a range ran out of word slots, the
 // queue entries reserved.
 __global__ void publish_state_kernel(const uint64_t* __restrict__ total, const uint32_t* __restrict__ flags, uint64_t* __restrict__ dst)
@@ -1994,6 +2051,8 @@ void nvtext_amd_profile_set_range_tiles(int32_t tiles)
   nvtext_amd::g_forced_range_tiles.store(tiles == 1 || tiles == 2 || tiles == 4 || tiles == 8 ? tiles : 0, std::memory_order_relaxed);
 }
 
+void nvtext_amd_profile_set_sizing_sample(int32_t on) { nvtext_amd::g_sizing_sample.store(on != 0 ? 1 : 0, std::memory_order_relaxed); }
+
 int32_t nvtext_amd_wordpiece_vocabulary_unk_id(const nvtext_amd_wordpiece_vocabulary* v) { return v ? v->table.unk_id : -1; }
 
 nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column* input, const nvtext_amd_wordpiece_vocabulary* vocabulary,
@@ -2052,13 +2111,24 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   size_t const ow = input->offsets_is_int64 ? 8 : 4;
   int64_t first_offset = 0, last_offset = 0;
   uint64_t* const scalars = host_scalars();  // pinned words that kernels write for the host (nullptr: copy instead)
+  bool const sampling     = g_sizing_sample.load(std::memory_order_relaxed) != 0;
+  double sample_words = 0, sample_queued = 0, sample_bytes = 0;  // what the sample found (nothing without the pinned words)
   if (scalars) {
-    launch_read_two_offsets(input->offsets, input->offsets_is_int64 != 0, input->offset, static_cast<int64_t>(input->offset) + rows, scalars, stream);
+    uint32_t* const counts = reinterpret_cast<uint32_t*>(scalars + 8);
+    if (sampling)
+      hipLaunchKernelGGL(wordpiece_sample_kernel, dim3(kSampleWindows), dim3(kWave), 0, stream, v, vocabulary->table, scalars, counts);
+    else
+      launch_read_two_offsets(input->offsets, input->offsets_is_int64 != 0, input->offset, static_cast<int64_t>(input->offset) + rows, scalars, stream);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(stream);
     if (e != hipSuccess) return give_up(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
     first_offset = static_cast<int64_t>(scalars[0]);
     last_offset  = static_cast<int64_t>(scalars[1]);
+    for (int i = 0; sampling && i < kSampleWindows; ++i) {
+      sample_words += counts[3 * i];
+      sample_queued += counts[3 * i + 1];
+      sample_bytes += counts[3 * i + 2];
+    }
   } else {
     unsigned char buf[16] = {0};
     const uint8_t* d_off  = static_cast<const uint8_t*>(input->offsets) + static_cast<size_t>(input->offset) * ow;
@@ -2146,6 +2216,16 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
   // room for a word per byte, the exact number of queue entries.
   uint32_t range_cap      = static_cast<uint32_t>(kRange * 5 / 16);
   uint64_t queue_capacity = static_cast<uint64_t>((last_offset - first_offset) >> 5) + static_cast<uint64_t>(word_grid) * kTokWaves * kQueueChunk + 4096;
+  if (sample_bytes > 0) {
+    // what the sample calls for, with half as much again for the ranges that are denser than the column as a whole
+    // (never less than the sizes above: a sample can miss; the second attempt remains)
+    double const per_byte_words  = std::max(sample_words / sample_bytes, static_cast<double>(rows) / static_cast<double>(last_offset - first_offset));
+    double const per_byte_queued = sample_queued / sample_bytes;
+    range_cap = static_cast<uint32_t>(std::min<double>(static_cast<double>(kRange + 8), std::max<double>(range_cap, per_byte_words * 1.5 * static_cast<double>(kRange) + 256)));
+    range_cap = (range_cap + 1u) & ~1u;  // (a range's slots begin at an even index)
+    queue_capacity = std::max<uint64_t>(queue_capacity, static_cast<uint64_t>(per_byte_queued * 1.25 * static_cast<double>(last_offset - first_offset)) +
+                                                          static_cast<uint64_t>(word_grid) * kTokWaves * kQueueChunk + 4096);
+  }
   uint64_t total = 0;
   for (int attempt = 0;; ++attempt) {
     if (queue_capacity > 0x7FFFFFF0ull) queue_capacity = 0x7FFFFFF0ull;

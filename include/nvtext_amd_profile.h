@@ -28,6 +28,12 @@ int32_t nvtext_amd_profile_read(const char** names, float* milliseconds, int32_t
  * as a large column runs it; any other value gives the choice back to the library.  Results do not depend on it. */
 void    nvtext_amd_profile_set_range_tiles(int32_t tiles);
 
+/* Test knob.  nvtext_amd_wordpiece_tokenize sizes the temporaries of its first attempt from a sample of the column and
+ * repeats its passes with larger ones when a range or the queue runs out of room all the same.  on = 0 makes every later
+ * call of the process skip the sample, so that columns which the sample sizes correctly still reach the second attempt;
+ * any other value switches it back on (the default).  Results do not depend on it. */
+void    nvtext_amd_profile_set_sizing_sample(int32_t on);
+
 #ifdef __cplusplus
 }
 #endif

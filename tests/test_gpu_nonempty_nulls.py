@@ -147,9 +147,24 @@ def test_wordpiece_retry_on_a_column_of_many_more_ranges_than_wavefronts(nv, orc
     exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), 0, nthreads=8)
     assert exp.child.size == 2 * words
     _capi.set_range_tiles(1)
+    _capi.set_sizing_sample(False)   # (the sample of the column would size the first attempt right: no second one)
     try:
         for attempt in range(3):
-            got = nv.wordpiece_tokenize(dcol, dv, 0).to_host()
-            assert got.equals(exp), f"call {attempt}"
+            _capi.profile_enable(True)
+            _capi.profile_read()
+            got = nv.wordpiece_tokenize(dcol, dv, 0)
+            launches = sum(1 for name, _ in _capi.profile_read() if name == "wordpiece_word_kernel")
+            _capi.profile_enable(False)
+            assert launches == 2, launches
+            assert got.to_host().equals(exp), f"call {attempt}"
+        _capi.set_sizing_sample(True)
+        _capi.profile_enable(True)
+        _capi.profile_read()
+        got = nv.wordpiece_tokenize(dcol, dv, 0)
+        launches = sum(1 for name, _ in _capi.profile_read() if name == "wordpiece_word_kernel")
+        assert launches == 1, launches
+        assert got.to_host().equals(exp), "sized by the sample"
     finally:
+        _capi.profile_enable(False)
         _capi.set_range_tiles(0)
+        _capi.set_sizing_sample(True)

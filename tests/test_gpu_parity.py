@@ -493,15 +493,26 @@ def _tile_kernel_launches(nv, fn):
     return out, sum(1 for n in names if n == "wordpiece_word_kernel")
 
 
+@pytest.fixture(params=[False, True], ids=["sized_by_default", "sized_by_sample"])
+def sizing_sample(request):
+    """wordpiece_tokenize sizes its first attempt from a sample of the column; without the sample (the library's test
+    knob) a column that needs more than the default sizes reaches the second attempt."""
+    from cudf_amd import _capi
+    _capi.set_sizing_sample(request.param)
+    yield request.param
+    _capi.set_sizing_sample(True)
+
+
 @pytest.mark.parametrize("max_words", [0, 5, 100000])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 @pytest.mark.parametrize("shape", ["few rows", "many rows"])
-def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shape, dtype, max_words, range_tiles):
+def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shape, dtype, max_words, range_tiles, sizing_sample):
     """Text whose ranges give more than three tokens per eight bytes (here two-letter words that are not in the
-    vocabulary and fall apart into letters: two tokens per three bytes) does not fit the arena of the first
-    attempt: the call has to notice, run the tile pass again with room for a token per byte, and give the same
-    result as the oracle (greedy rule: cpp/src/text/wordpiece_tokenize.cu:349-407).  A million such words, in
-    a few long rows and in many short ones; the two launches are read off the library's kernel timing."""
+    vocabulary and fall apart into letters: two tokens per three bytes) does not fit the arena of an attempt with
+    the default sizes: the call has to notice, run the tile pass again with room for a token per byte, and give the
+    same result as the oracle (greedy rule: cpp/src/text/wordpiece_tokenize.cu:349-407).  A million such words, in
+    a few long rows and in many short ones; the launches are read off the library's kernel timing: two without the
+    sample of the column that sizes the first attempt, one with it."""
     rng = np.random.default_rng(5)
     letters = "abcdefgh"
     vocab = ["[UNK]"] + list(letters) + ["##" + c for c in letters] + ["abcdefgh"]
@@ -518,7 +529,8 @@ def test_wordpiece_more_tokens_than_the_first_attempt_has_room_for(nv, orc, shap
     exp = orc.wordpiece_tokenize(host, orc.Vocabulary(hv), max_words, nthreads=8)
     assert_same(got.to_host(), exp, f"{shape}, max_words={max_words}")
     if max_words != 5 or shape == "many rows":
-        assert launches == 2, launches  # (five words of a long row are too few tokens to fill anything)
+        # (five words of a long row are too few tokens to fill anything; the sample looks at the text, not at the limit)
+        assert launches == (1 if sizing_sample else 2), launches
         assert exp.child.size > 1_000_000
     # ordinary text right afterwards: one launch, nothing left over from the call before
     plain = strings(["abcdefgh " * 2000] * 50, dtype)
