@@ -44,27 +44,28 @@ namespace {
 
 constexpr uint32_t kMaxWord = 200;  // wordpiece_tokenize.cu:300: words this long become one [UNK]
 
-__host__ __device__ __forceinline__ uint32_t mix32(uint32_t h)
+// Key hash, 64 bits: the key is consumed in 8-byte blocks (two little-endian dwords, zero padded), every dword times an
+// odd constant of its own, summed: for a key of up to 16 bytes four multiply-adds of 32 x 32 + 64 bits, the unit the
+// vector ALUs have, and nothing that waits for the step before it beyond the running sum.  (A bucket needs the key's
+// home and fifteen bits to tell keys apart, not an avalanche: the home comes from the low bits of the sum's upper half,
+// which every bit of the key reaches, the tag from the top of its lower half.)  The two key spaces multiply the first
+// dword by different constants; the length is not hashed (the slot holds it).  Blocks from the third on (keys of more
+// than 16 bytes) rotate the sum first, so that the constants can be used again.
+constexpr uint32_t kMulFirst[2] = {0x9E3779B1u, 0xD2B74407u};
+constexpr uint32_t kMulSecond = 0x85EBCA77u, kMulThird = 0xC2B2AE3Du, kMulFourth = 0x27D4EB2Fu;
+__host__ __device__ __forceinline__ uint64_t key_hash_first(uint32_t kind, uint32_t lo, uint32_t hi)
 {
-  h ^= h >> 16;
-  h *= 0x85ebca6bu;
-  h ^= h >> 13;
-  h *= 0xc2b2ae35u;
-  h ^= h >> 16;
-  return h;
+  return static_cast<uint64_t>(lo) * (kind ? kMulFirst[1] : kMulFirst[0]) + static_cast<uint64_t>(hi) * kMulSecond;
 }
-
-// Key hash: the key is consumed in 8-byte blocks (two little-endian dwords, zero padded).
-__host__ __device__ __forceinline__ uint32_t key_hash_init(uint32_t len) { return len * 0xC2B2AE3Du; }
-__host__ __device__ __forceinline__ uint32_t key_hash_block(uint32_t h, uint32_t lo, uint32_t hi)
+// block: 1 for key bytes [8, 16), 2 for [16, 24), ..
+__host__ __device__ __forceinline__ uint64_t key_hash_next(uint64_t h, uint32_t lo, uint32_t hi, uint32_t block)
 {
-  h = (h ^ lo) * 0x9E3779B1u;
-  h = (h ^ hi) * 0x85EBCA77u;
-  return h ^ (h >> 15);
+  if (block > 1) h = (h << 25) | (h >> 39);
+  return h + static_cast<uint64_t>(lo) * kMulThird + static_cast<uint64_t>(hi) * kMulFourth;
 }
 
 // slot.x = (tag15 << 17) | (carried8 << 9) | (kind << 8) | len   (0 = empty; len in 1..199).  carried8, in slot 0 of a bucket only:
-//          one of eight bits per key that has been carried past this bucket (which bit: carried_bit() of the key's hash)
+//          one of eight bits per key that has been carried past this bucket (which bit: HashParts::fp of the key)
 // slot.y = token id; in slot 0 of a bucket, bit 31 says that some key has been carried past this bucket
 //          (kSearchOn: a key that is not in a bucket without the bit is not in the table)
 // slot.z, slot.w = the key itself when len <= 8 (zero padded), else (byte offset of the key in the pool, 0);
@@ -76,6 +77,7 @@ struct VocabTable {
   const uint4* slots;
   const uint8_t* pool;
   uint32_t bucket_mask;  // buckets - 1
+  uint32_t bucket_bits;  // log2(buckets)
   int32_t unk_id;
   uint32_t max_len[2];   // longest key of each key space (longer candidates cannot match)
   // Length filter: lens[length_filter_index(kind, first three key bytes) & lens_mask] has bit i (i < 31) set
@@ -108,15 +110,25 @@ __host__ __device__ __forceinline__ uint32_t length_filter_bit(uint32_t len) { r
 __host__ __device__ __forceinline__ uint16_t packed_filter_word(uint32_t w) { return static_cast<uint16_t>((w & 0x7FFFu) | ((w >> 15) ? 0x8000u : 0u)); }
 __host__ __device__ __forceinline__ uint32_t filter_word(uint32_t stored) { return (stored & 0x7FFFu) | ((stored & 0x8000u) ? 0xFFFF8000u : 0u); }
 
-__host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t h, uint32_t kind, uint32_t len, uint32_t* bucket)
+// What a lookup takes from a key's hash: the two halves folded and multiplied once more (the top bits of such a product
+// depend on every bit of both halves), the key's home bucket from the top `bucket_bits` bits, the tag and the carried
+// bit (see above) from the bits below them.
+struct HashParts {
+  uint32_t bucket;  // home bucket
+  uint32_t tag;     // slot.x of a matching slot without kind and length: bits 17..31
+  uint32_t fp;      // the bit that the key sets in the carried8 field of the buckets it is carried past
+};
+__host__ __device__ __forceinline__ HashParts hash_parts(uint64_t h, uint32_t bucket_bits)
 {
-  uint32_t const x = mix32(h + kind * 0x7F4A7C15u);
-  *bucket          = x;
-  return (x & 0xFFFE0000u) | (kind << 8) | len;
+  uint32_t const x    = (static_cast<uint32_t>(h) ^ static_cast<uint32_t>(h >> 32)) * 0x9E3779B1u;
+  uint32_t const rest = x << bucket_bits;  // (bucket_bits: 5 .. 30)
+  HashParts p;
+  p.bucket = x >> (32u - bucket_bits);
+  p.tag    = rest & 0xFFFE0000u;
+  p.fp     = 0x200u << (rest >> 29);
+  return p;
 }
-// The bit that a key with hash h sets in the carried8 field of the buckets it is carried past: a key that is not in
-// its home bucket and does not find its bit there is not in the table.
-__host__ __device__ __forceinline__ uint32_t carried_bit(uint32_t h) { return 0x200u << ((h * 0x9E3779B1u) >> 29); }
+__host__ __device__ __forceinline__ uint32_t slot_word0(uint32_t tag, uint32_t kind, uint32_t len) { return tag | (kind << 8) | len; }
 
 }  // namespace
 }  // namespace nvtext_amd
@@ -222,18 +234,18 @@ struct GlobalWord {
 struct Probe {
   uint32_t k0, k1;  // key bytes [0, 8), zero padded
   uint32_t want;    // slot.x of a matching slot (without the carried8 field)
-  uint32_t fp;      // carried_bit() of the key
+  uint32_t fp;      // HashParts::fp of the key
   uint32_t bucket;  // home bucket (already masked)
 };
 
 // Hash contribution of key bytes [8, len) (keys that do not fit the slot; kept out of line).
 template <typename W>
-__device__ __forceinline__ uint32_t hash_long_key(W const& w, uint32_t p, uint32_t len, uint32_t h)
+__device__ __forceinline__ uint64_t hash_long_key(W const& w, uint32_t p, uint32_t len, uint64_t h)
 {
   for (uint32_t done = 8; done < len; done += 8) {
     uint32_t b0, b1;
     w.key8(p + done, len - done, &b0, &b1);
-    h = key_hash_block(h, b0, b1);
+    h = key_hash_next(h, b0, b1, done >> 3);
   }
   return h;
 }
@@ -246,12 +258,12 @@ __device__ __forceinline__ Probe make_probe(VocabTable const& t, uint32_t kind, 
   pr.k0 = raw0;
   pr.k1 = raw1;
   trim_key8(len, pr.k0, pr.k1);
-  uint32_t h = key_hash_block(key_hash_init(len), pr.k0, pr.k1);
+  uint64_t h = key_hash_first(kind, pr.k0, pr.k1);
   if (len > 8) h = hash_long_key(w, p, len, h);
-  uint32_t b;
-  pr.want   = slot_word0(h, kind, len, &b);
-  pr.fp     = carried_bit(h);
-  pr.bucket = b & t.bucket_mask;
+  HashParts const hp = hash_parts(h, t.bucket_bits);
+  pr.want            = slot_word0(hp.tag, kind, len);
+  pr.fp              = hp.fp;
+  pr.bucket          = hp.bucket;
   return pr;
 }
 
@@ -669,14 +681,12 @@ struct ShortWord {
     uint4 const keep = trim[l];  // (l <= 16)
     pr.k0            = r[0] & keep.x;
     pr.k1            = r[1] & keep.y;
-    uint32_t h       = key_hash_block(key_hash_init(l), pr.k0, pr.k1);
-    uint32_t const k2 = r[2] & keep.z, k3 = r[3] & keep.w;
-    uint32_t const h2 = key_hash_block(h, k2, k3);
-    h                 = l > 8 ? h2 : h;
-    uint32_t b;
-    pr.want   = slot_word0(h, kind, l, &b);
-    pr.fp     = carried_bit(h);
-    pr.bucket = b & t.bucket_mask;
+    // (the third and fourth dword of a key of up to 8 bytes are zeros after the trim: they add nothing)
+    uint64_t const h = key_hash_next(key_hash_first(kind, pr.k0, pr.k1), r[2] & keep.z, r[3] & keep.w, 1u);
+    HashParts const hp = hash_parts(h, t.bucket_bits);
+    pr.want            = slot_word0(hp.tag, kind, l);
+    pr.fp              = hp.fp;
+    pr.bucket          = hp.bucket;
     return pr;
   }
 
@@ -1253,13 +1263,12 @@ __global__ void __launch_bounds__(kTokThreads, 6) wordpiece_word_kernel(TileArgs
           Probe pr;
           pr.k0             = head[0];
           pr.k1             = head[1];
-          uint32_t const h1 = key_hash_block(key_hash_init(wl16), pr.k0, pr.k1);
-          uint32_t const h2 = key_hash_block(h1, head[2], head[3]);
-          uint32_t const h  = wl16 > 8 ? h2 : h1;
-          uint32_t bk;
-          pr.want   = slot_word0(h, 0, wl16, &bk);
-          pr.fp     = carried_bit(h);
-          pr.bucket = bk & table.bucket_mask;
+          // (the third and fourth dword of a word of up to 8 bytes are zeros after the trim: they add nothing)
+          uint64_t const h = key_hash_next(key_hash_first(0u, pr.k0, pr.k1), head[2], head[3], 1u);
+          HashParts const hp = hash_parts(h, table.bucket_bits);
+          pr.want            = slot_word0(hp.tag, 0u, wl16);
+          pr.fp              = hp.fp;
+          pr.bucket          = hp.bucket;
           uint4 const s0 = table.slots[2 * pr.bucket];
           uint4 const s1 = table.slots[2 * pr.bucket + 1];
           int32_t id  = kNone;
@@ -1781,7 +1790,22 @@ __global__ void __launch_bounds__(kWave) wordpiece_sample_kernel(ColView col, Vo
       while (len < kMaxWord && sb[4 + p + len] != 0x20u) ++len;
       ++words;
       if (len >= kMaxWord) continue;  // one unknown token, never queued
-      if (len > 16 || lookup_slow(table, 0u, TileWord{staged, 4u + p}, 0u, len) == kNone) ++queued;
+      if (len > 16) {
+        ++queued;
+        continue;
+      }
+      // queued as the word pass queues: whatever the word's home bucket does not settle
+      TileWord const tw{staged, 4u + p};
+      uint32_t k[4];
+      tw.head16(k);
+      trim_key8(min(len, 8u), k[0], k[1]);
+      trim_key8(len > 8 ? len - 8u : 0u, k[2], k[3]);
+      Probe const pr = make_probe(table, 0u, tw, 0u, len, k[0], k[1]);
+      uint4 const s0 = table.slots[2 * pr.bucket], s1 = table.slots[2 * pr.bucket + 1];
+      int32_t id;
+      uint32_t vd = verdict(pr, s0, s1, len, &id);
+      if (vd == 2u && len > 8) vd = verdict_16(table, pr, s0, s1, k, &id);
+      if (vd != 1u) ++queued;
     }
   }
   uint32_t const w = wave_bcast(wave_inclusive_scan(words), kWave - 1), q = wave_bcast(wave_inclusive_scan(queued), kWave - 1);
@@ -1819,13 +1843,14 @@ void host_key8(const uint8_t* key, uint32_t len, uint32_t* k0, uint32_t* k1)
   std::memcpy(k1, buf + 4, 4);
 }
 
-uint32_t host_hash(const uint8_t* key, uint32_t len)
+uint64_t host_hash(uint32_t kind, const uint8_t* key, uint32_t len)
 {
-  uint32_t h = key_hash_init(len);
-  for (uint32_t done = 0; done < len; done += 8) {
-    uint32_t lo, hi;
+  uint32_t lo, hi;
+  host_key8(key, len, &lo, &hi);
+  uint64_t h = key_hash_first(kind, lo, hi);
+  for (uint32_t done = 8; done < len; done += 8) {
     host_key8(key + done, len - done, &lo, &hi);
-    h = key_hash_block(h, lo, hi);
+    h = key_hash_next(h, lo, hi, done >> 3);
   }
   return h;
 }
@@ -1836,13 +1861,13 @@ bool host_same(HostSlot const& s, uint32_t w0, const std::vector<uint8_t>& pool,
   return len <= 8 ? (s.z == k0 && s.w == k1) : (std::memcmp(pool.data() + s.z, key, len) == 0);
 }
 
-void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::vector<uint8_t>& pool, uint32_t kind, const uint8_t* key,
+void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, uint32_t bucket_bits, const std::vector<uint8_t>& pool, uint32_t kind, const uint8_t* key,
                  uint32_t len, uint32_t pool_off, int32_t id)
 {
-  uint32_t b;
-  uint32_t const hh = host_hash(key, len);
-  uint32_t const w0 = slot_word0(hh, kind, len, &b);
-  uint32_t const fp = carried_bit(hh);
+  HashParts const hp = hash_parts(host_hash(kind, key, len), bucket_bits);
+  uint32_t b         = hp.bucket;
+  uint32_t const w0  = slot_word0(hp.tag, kind, len);
+  uint32_t const fp  = hp.fp;
   uint32_t k0 = 0, k1 = 0;
   if (len <= 8) host_key8(key, len, &k0, &k1);
   for (;;) {
@@ -1865,12 +1890,13 @@ void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::
   }
 }
 
-int32_t host_find(const std::vector<HostSlot>& slots, uint32_t bucket_mask, const std::vector<uint8_t>& pool, const char* text)
+int32_t host_find(const std::vector<HostSlot>& slots, uint32_t bucket_mask, uint32_t bucket_bits, const std::vector<uint8_t>& pool, const char* text)
 {
   uint32_t const len = static_cast<uint32_t>(std::strlen(text));
   const uint8_t* key = reinterpret_cast<const uint8_t*>(text);
-  uint32_t b;
-  uint32_t const w0 = slot_word0(host_hash(key, len), 0, len, &b);
+  HashParts const hp = hash_parts(host_hash(0, key, len), bucket_bits);
+  uint32_t b         = hp.bucket;
+  uint32_t const w0  = slot_word0(hp.tag, 0, len);
   uint32_t k0 = 0, k1 = 0;
   host_key8(key, len, &k0, &k1);
   for (;;) {
@@ -1937,6 +1963,8 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   while (capacity < 2 * keys) capacity <<= 1;
   if (capacity > (size_t{1} << 31)) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
   uint32_t const mask = static_cast<uint32_t>(capacity / 2 - 1);  // buckets of two slots
+  uint32_t bucket_bits = 0;
+  while ((1u << bucket_bits) < capacity / 2) ++bucket_bits;
   std::vector<HostSlot> slots(capacity, HostSlot{0, 0, 0, 0});
   uint32_t max_len[2] = {0, 0};
   // keys of more than 8 bytes, zero padded to whole 8-byte blocks
@@ -1953,12 +1981,12 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
     int64_t const len = e - b;
     // entries of 200 bytes or more can never equal a tokenizable word or piece; empty ones are never looked up
     if (len >= 1 && len < kMaxWord) {
-      host_insert(slots, mask, blocks, 0, pool.data() + b, static_cast<uint32_t>(len), add_blocks(pool.data() + b, static_cast<uint32_t>(len)), i);
+      host_insert(slots, mask, bucket_bits, blocks, 0, pool.data() + b, static_cast<uint32_t>(len), add_blocks(pool.data() + b, static_cast<uint32_t>(len)), i);
       max_len[0] = std::max(max_len[0], static_cast<uint32_t>(len));
     }
     // wordpiece_tokenize.cu:184-192: "##" entries also live, without the prefix, in the second key space
     if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') {
-      host_insert(slots, mask, blocks, 1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), add_blocks(pool.data() + b + 2, static_cast<uint32_t>(len - 2)), i);
+      host_insert(slots, mask, bucket_bits, blocks, 1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), add_blocks(pool.data() + b + 2, static_cast<uint32_t>(len - 2)), i);
       max_len[1] = std::max(max_len[1], static_cast<uint32_t>(len - 2));
     }
   }
@@ -2001,8 +2029,8 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   auto* v = new nvtext_amd_wordpiece_vocabulary;
   v->entries = V;
   // wordpiece_tokenize.cu:199-209, 273-275
-  int32_t unk = host_find(slots, mask, blocks, "[UNK]");
-  if (unk < 0) unk = host_find(slots, mask, blocks, "[unk]");
+  int32_t unk = host_find(slots, mask, bucket_bits, blocks, "[UNK]");
+  if (unk < 0) unk = host_find(slots, mask, bucket_bits, blocks, "[unk]");
   v->slot_bytes = capacity * sizeof(HostSlot);
   v->pool_bytes = blocks.size() + 16;
   v->store.bind(mr, stream);
@@ -2030,6 +2058,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.slots  = static_cast<const uint4*>(v->d_slots);
   v->table.pool   = static_cast<const uint8_t*>(v->d_pool);
   v->table.bucket_mask = mask;
+  v->table.bucket_bits = bucket_bits;
   v->table.unk_id      = unk;
   v->table.max_len[0]  = max_len[0];
   v->table.max_len[1]  = max_len[1];
