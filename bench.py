@@ -434,6 +434,26 @@ def main():
         leg = {"workload": f"C5 x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes, "offsets": "int64",
                "vocab_entries": w.vocab.size, "tokenize": tleg}
         keep.clear()
+        # the same rows with the vocabulary of C2, which knows next to none of their words: four times the queued words per
+        # byte that ordinary text has.  The call sizes its first attempt from a sample of the column; `word_pass_launches`
+        # says whether that held (1) or the passes had to be repeated with larger temporaries (2).
+        dv2 = nvtext.WordPieceVocabulary(nvtext.DeviceStringsColumn.from_host(datagen.config2(0.001).vocab))
+
+        def fstep():
+            keep["o"] = nvtext.wordpiece_tokenize(dc, dv2, p["max_words_per_row"])
+            return keep["o"]
+
+        fsec, fleg, _ = measure(fstep, max(2, side_steps // 2), 1, _capi, torch)
+        _capi.profile_enable(True)
+        _capi.profile_read()
+        fstep()
+        torch.cuda.synchronize()
+        fleg.update({"workload": "C5 rows, the 30,522-entry vocabulary of C2", "input_GBps": round(ib / fsec / 1e9, 2), "tokens_out": keep["o"].child_size,
+                     "word_pass_launches": sum(1 for name, _ in _capi.profile_read() if name == "wordpiece_word_kernel")})
+        _capi.profile_enable(False)
+        leg["tokenize_foreign_vocabulary"] = fleg
+        keep.clear()
+        del dv2
         # normalize_characters, the step that precedes the tokenizer in a BERT pipeline (lower-casing, five special tokens)
         special = nvtext.DeviceStringsColumn.from_host(HostStringsColumn.from_pylist(["[CLS]", "[SEP]", "[PAD]", "[MASK]", "[UNK]"]))
         normalizer = nvtext.CharacterNormalizer(True, special)

@@ -1830,83 +1830,186 @@ struct RangeTokensOf {
   __device__ uint64_t operator()(int64_t i) const { return counts[i]; }
 };
 
-// ------------------------------------------------------------------ vocabulary construction (host)
-struct HostSlot {
-  uint32_t x, y, z, w;
+// ------------------------------------------------------------------ vocabulary construction (device)
+// The reference inserts the entries into its two maps on the device (cpp/src/text/wordpiece_tokenize.cu:213-282); so
+// does this: a kernel that counts the keys and the bytes of the longer ones (the host sizes the tables from that, its
+// one wait), a kernel that enters every key into the table, the length filter and the direct tables with atomics, a
+// kernel that settles entries that occur twice (the first one wins, as when a host enters them in order), one that
+// packs the length filter and looks up the unknown token.  An entry gives up to two keys: itself, and, when it begins
+// with "##", what follows (cpp/src/text/wordpiece_tokenize.cu:184-192).
+struct VocabKey {
+  const uint8_t* bytes;
+  uint32_t len;  // 0: no key
 };
-
-void host_key8(const uint8_t* key, uint32_t len, uint32_t* k0, uint32_t* k1)
+__device__ __forceinline__ VocabKey vocabulary_key(ColView const& v, int64_t entry, uint32_t kind)
 {
-  uint8_t buf[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  std::memcpy(buf, key, len < 8 ? len : 8);
-  std::memcpy(k0, buf, 4);
-  std::memcpy(k1, buf + 4, 4);
+  int64_t const b = v.off(entry), e = v.off(entry + 1);
+  int64_t const n = e - b;
+  VocabKey k{v.chars + b, 0u};
+  // entries of kMaxWord bytes or more can never equal a tokenizable word or piece; empty ones are never looked up
+  if (kind == 0) {
+    if (n >= 1 && n < kMaxWord) k.len = static_cast<uint32_t>(n);
+  } else if (n >= 3 && n - 2 < kMaxWord && v.chars[b] == '#' && v.chars[b + 1] == '#') {
+    k.bytes += 2;
+    k.len = static_cast<uint32_t>(n - 2);
+  }
+  return k;
 }
 
-uint64_t host_hash(uint32_t kind, const uint8_t* key, uint32_t len)
+struct VocabCounts {
+  unsigned long long pool_bytes;  // keys of more than 8 bytes, each padded to whole 8-byte blocks
+  uint32_t keys;
+  uint32_t max_len[2];
+  uint32_t pool_cursor;           // (build kernel) the next free byte of the pool
+  int32_t unk_id;                 // (last kernel)
+};
+
+__global__ void vocabulary_measure_kernel(ColView v, VocabCounts* __restrict__ counts)
+{
+  int64_t const t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= 2 * static_cast<int64_t>(v.size)) return;
+  uint32_t const kind = static_cast<uint32_t>(t & 1);
+  VocabKey const k    = vocabulary_key(v, t >> 1, kind);
+  if (k.len == 0) return;
+  atomicAdd(&counts->keys, 1u);
+  if (k.len > 8) atomicAdd(&counts->pool_bytes, static_cast<unsigned long long>((k.len + 7u) & ~7u));
+  atomicMax(&counts->max_len[kind], k.len);
+}
+
+// A key's bytes [p, p + 8) as two dwords, zero padded past the key.
+__device__ __forceinline__ void vocabulary_key8(VocabKey const& k, uint32_t p, uint32_t* lo, uint32_t* hi)
+{
+  uint32_t w[2] = {0u, 0u};
+  for (uint32_t i = 0; i < 8 && p + i < k.len; ++i) w[i >> 2] |= static_cast<uint32_t>(k.bytes[p + i]) << (8 * (i & 3u));
+  *lo = w[0];
+  *hi = w[1];
+}
+__device__ __forceinline__ uint64_t vocabulary_hash(VocabKey const& k, uint32_t kind)
 {
   uint32_t lo, hi;
-  host_key8(key, len, &lo, &hi);
+  vocabulary_key8(k, 0, &lo, &hi);
   uint64_t h = key_hash_first(kind, lo, hi);
-  for (uint32_t done = 8; done < len; done += 8) {
-    host_key8(key + done, len - done, &lo, &hi);
+  for (uint32_t done = 8; done < k.len; done += 8) {
+    vocabulary_key8(k, done, &lo, &hi);
     h = key_hash_next(h, lo, hi, done >> 3);
   }
   return h;
 }
 
-bool host_same(HostSlot const& s, uint32_t w0, const std::vector<uint8_t>& pool, const uint8_t* key, uint32_t len, uint32_t k0, uint32_t k1)
-{
-  if ((s.x & ~kCarried) != w0) return false;
-  return len <= 8 ? (s.z == k0 && s.w == k1) : (std::memcmp(pool.data() + s.z, key, len) == 0);
-}
+struct VocabBuild {
+  uint32_t* slots;      // the table as dwords: slot s at [4 s, 4 s + 4)
+  uint8_t* pool;
+  uint32_t* lens32;     // the length filter, a 32-bit word per entry (packed afterwards)
+  uint32_t* short_ids;  // as VocabTable::short_ids, "no such key" = 0x80000000 (above every id)
+  uint32_t* letters3;   // as VocabTable::letters3, two entries to a word
+  uint32_t bucket_mask, bucket_bits, lens_mask;
+};
 
-void host_insert(std::vector<HostSlot>& slots, uint32_t bucket_mask, uint32_t bucket_bits, const std::vector<uint8_t>& pool, uint32_t kind, const uint8_t* key,
-                 uint32_t len, uint32_t pool_off, int32_t id)
+__global__ void vocabulary_insert_kernel(ColView v, VocabBuild t, VocabCounts* __restrict__ counts)
 {
-  HashParts const hp = hash_parts(host_hash(kind, key, len), bucket_bits);
-  uint32_t b         = hp.bucket;
-  uint32_t const w0  = slot_word0(hp.tag, kind, len);
-  uint32_t const fp  = hp.fp;
-  uint32_t k0 = 0, k1 = 0;
-  if (len <= 8) host_key8(key, len, &k0, &k1);
-  for (;;) {
-    b &= bucket_mask;
-    for (int j = 0; j < 2; ++j) {
-      HostSlot& s = slots[2 * static_cast<size_t>(b) + j];
-      if (s.x == 0) {
-        s.x = w0;
-        s.y = static_cast<uint32_t>(id);
-        s.z = len <= 8 ? k0 : pool_off;
-        s.w = len <= 8 ? k1 : 0u;
+  int64_t const th = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (th >= 2 * static_cast<int64_t>(v.size)) return;
+  uint32_t const kind = static_cast<uint32_t>(th & 1);
+  uint32_t const id   = static_cast<uint32_t>(th >> 1);
+  VocabKey const k    = vocabulary_key(v, th >> 1, kind);
+  if (k.len == 0) return;
+  uint32_t k0, k1;
+  vocabulary_key8(k, 0, &k0, &k1);
+  // the length filter over the first three bytes, and its exact twin for pieces of lower-case letters
+  if (k.len >= 3) {
+    atomicOr(&t.lens32[length_filter_index(kind, k0 & 0x00FFFFFFu) & t.lens_mask], 1u << length_filter_bit(k.len));
+    uint32_t const c0 = k0 & 0xFFu, c1 = (k0 >> 8) & 0xFFu, c2 = (k0 >> 16) & 0xFFu;
+    auto letter = [](uint32_t c) { return c >= 'a' && c <= 'z'; };
+    if (kind == 1 && k.len <= 18 && letter(c0) && letter(c1) && letter(c2)) {
+      uint32_t const at = ((c0 - 'a') * 26u + (c1 - 'a')) * 26u + (c2 - 'a');
+      atomicOr(&t.letters3[at >> 1], (1u << (k.len - 3)) << (16u * (at & 1u)));
+    }
+  }
+  // the direct tables of the keys of one and two bytes: the first entry with a key wins
+  if (k.len <= 2) {
+    uint32_t const at = k.len == 2 ? kind * 65536u + (k0 & 0xFFFFu) : 2u * 65536u + kind * 256u + (k0 & 0xFFu);
+    atomicMin(&t.short_ids[at], id);
+  }
+  // the table: the first empty slot from the key's home bucket on is taken with a compare-and-swap of its first word; an
+  // entry that occurs twice takes two slots here (whether a full slot holds the same key cannot be told while its owner
+  // may still be writing it) and is settled by the next kernel
+  uint32_t pool_off = 0;
+  if (k.len > 8) {
+    pool_off = atomicAdd(&counts->pool_cursor, (k.len + 7u) & ~7u);
+    for (uint32_t i = 0; i < k.len; ++i) t.pool[pool_off + i] = k.bytes[i];  // (the pool starts as zeros: the padding)
+  }
+  HashParts const hp = hash_parts(vocabulary_hash(k, kind), t.bucket_bits);
+  uint32_t const w0  = slot_word0(hp.tag, kind, k.len);
+  for (uint32_t b = hp.bucket;; b = (b + 1) & t.bucket_mask) {
+    for (uint32_t j = 0; j < 2; ++j) {
+      uint32_t* const slot = t.slots + 4 * (2 * static_cast<size_t>(b) + j);
+      if (atomicCAS(slot, 0u, w0) == 0u) {
+        atomicOr(slot + 1, id);  // (others may be setting kSearchOn in this word at this moment)
+        slot[2] = k.len <= 8 ? k0 : pool_off;
+        slot[3] = k.len <= 8 ? k1 : 0u;
         return;
       }
-      // the same key again: the first entry wins (duplicates are undefined in the reference)
-      if (host_same(s, w0, pool, key, len, k0, k1)) return;
     }
-    slots[2 * static_cast<size_t>(b)].y |= kSearchOn;  // the key is carried past this bucket
-    slots[2 * static_cast<size_t>(b)].x |= fp;
-    ++b;
+    atomicOr(t.slots + 8 * static_cast<size_t>(b) + 1, kSearchOn);  // the key is carried past this bucket
+    atomicOr(t.slots + 8 * static_cast<size_t>(b), hp.fp);
   }
 }
 
-int32_t host_find(const std::vector<HostSlot>& slots, uint32_t bucket_mask, uint32_t bucket_bits, const std::vector<uint8_t>& pool, const char* text)
+// Entries that occur twice: every one of them looks for the first slot on its way that holds its key and leaves the
+// smaller id there (lookups stop at that slot; the other slots with the key are never reached).
+__global__ void vocabulary_settle_kernel(ColView v, VocabBuild t)
 {
-  uint32_t const len = static_cast<uint32_t>(std::strlen(text));
-  const uint8_t* key = reinterpret_cast<const uint8_t*>(text);
-  HashParts const hp = hash_parts(host_hash(0, key, len), bucket_bits);
-  uint32_t b         = hp.bucket;
-  uint32_t const w0  = slot_word0(hp.tag, 0, len);
-  uint32_t k0 = 0, k1 = 0;
-  host_key8(key, len, &k0, &k1);
-  for (;;) {
-    b &= bucket_mask;
-    for (int j = 0; j < 2; ++j) {
-      HostSlot const& s = slots[2 * static_cast<size_t>(b) + j];
-      if (s.x == 0) return -1;
-      if (host_same(s, w0, pool, key, len, k0, k1)) return static_cast<int32_t>(s.y & ~kSearchOn);
+  int64_t const th = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (th >= 2 * static_cast<int64_t>(v.size)) return;
+  uint32_t const kind = static_cast<uint32_t>(th & 1);
+  uint32_t const id   = static_cast<uint32_t>(th >> 1);
+  VocabKey const k    = vocabulary_key(v, th >> 1, kind);
+  if (k.len == 0) return;
+  uint32_t k0, k1;
+  vocabulary_key8(k, 0, &k0, &k1);
+  HashParts const hp = hash_parts(vocabulary_hash(k, kind), t.bucket_bits);
+  uint32_t const w0  = slot_word0(hp.tag, kind, k.len);
+  for (uint32_t b = hp.bucket;; b = (b + 1) & t.bucket_mask) {
+    for (uint32_t j = 0; j < 2; ++j) {
+      uint32_t* const slot = t.slots + 4 * (2 * static_cast<size_t>(b) + j);
+      uint32_t const x     = slot[0];
+      if (x == 0) return;  // (cannot happen: the key is in the table)
+      if ((x & ~kCarried) != w0) continue;
+      bool same = slot[2] == k0 && slot[3] == k1;
+      if (k.len > 8) {
+        same = true;
+        for (uint32_t i = 0; same && i < k.len; ++i) same = t.pool[slot[2] + i] == k.bytes[i];
+      }
+      if (!same) continue;
+      for (uint32_t seen = slot[1];;) {
+        uint32_t const want = (seen & kSearchOn) | min(seen & ~kSearchOn, id);
+        uint32_t const was  = atomicCAS(slot + 1, seen, want);
+        if (was == seen) break;
+        seen = was;
+      }
+      return;
     }
-    ++b;
+  }
+}
+
+// The length filter in its stored form, "no such key" of the direct tables as the lookups expect it, and the id of
+// the unknown token (cpp/src/text/wordpiece_tokenize.cu:199-209, 273-275: "[UNK]", else "[unk]", else -1).
+__global__ void vocabulary_finish_kernel(VocabTable table, const uint32_t* __restrict__ lens32, uint16_t* __restrict__ lens16, uint32_t lens_size,
+                                         int32_t* __restrict__ short_ids, VocabCounts* __restrict__ counts)
+{
+  uint32_t const stride = gridDim.x * blockDim.x;
+  uint32_t const t      = blockIdx.x * blockDim.x + threadIdx.x;
+  for (uint32_t i = t; i < lens_size; i += stride) lens16[i] = packed_filter_word(lens32[i]);
+  for (uint32_t i = t; i < kShortIds; i += stride)
+    if (static_cast<uint32_t>(short_ids[i]) == 0x80000000u) short_ids[i] = kNone;  // (the same bits: kNone is INT32_MIN)
+  if (t == 0) {
+    int32_t unk = kNone;
+    for (int which = 0; which < 2 && unk == kNone; ++which) {
+      // "[UNK]" / "[unk]" as two dwords
+      RegWord const w{{which == 0 ? 0x4B4E555Bu : 0x6B6E755Bu, 0x0000005Du, 0u, 0u}};
+      unk = lookup(table, 0u, w, 0u, 5u, w.r[0], w.r[1]);
+    }
+    counts->unk_id = unk == kNone ? -1 : unk;
   }
 }
 
@@ -1925,147 +2028,88 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   if (vocabulary->size == 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary must not be empty");
   if (vocabulary->null_count > 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary must not have nulls");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Mr const temp_mr{mr, stream};
+  int32_t const V = vocabulary->size;
+  ColView const entries = make_view(*vocabulary);
+  unsigned const key_grid = static_cast<unsigned>((2 * static_cast<int64_t>(V) + 255) / 256);
 
-  // bring the entries to the host (one-time, a few MB at most)
-  int32_t const V      = vocabulary->size;
-  size_t const ow      = vocabulary->offsets_is_int64 ? 8 : 4;
-  std::vector<uint8_t> h_off((static_cast<size_t>(V) + 1) * ow);
-  const uint8_t* d_off = static_cast<const uint8_t*>(vocabulary->offsets) + static_cast<size_t>(vocabulary->offset) * ow;
-  NVTEXT_HIP_TRY(hipMemcpyAsync(h_off.data(), d_off, h_off.size(), hipMemcpyDeviceToHost, stream));
+  // how many keys, how many bytes of keys that do not fit a slot: the host's one wait before the tables exist
+  Temp counts_mem(temp_mr, sizeof(VocabCounts));
+  if (!counts_mem.ok()) return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
+  VocabCounts* const d_counts = counts_mem.as<VocabCounts>();
+  launch_fill_u32(reinterpret_cast<uint32_t*>(d_counts), 0u, sizeof(VocabCounts) / sizeof(uint32_t), stream);
+  hipLaunchKernelGGL(vocabulary_measure_kernel, dim3(key_grid), dim3(256), 0, stream, entries, d_counts);
+  VocabCounts counts{};
+  NVTEXT_HIP_TRY(hipGetLastError());
+  NVTEXT_HIP_TRY(hipMemcpyAsync(&counts, d_counts, sizeof(counts), hipMemcpyDeviceToHost, stream));
   NVTEXT_HIP_TRY(hipStreamSynchronize(stream));
-  auto off_at = [&](int32_t i) -> int64_t {
-    if (ow == 8) {
-      int64_t v;
-      std::memcpy(&v, h_off.data() + static_cast<size_t>(i) * 8, 8);
-      return v;
-    }
-    int32_t v;
-    std::memcpy(&v, h_off.data() + static_cast<size_t>(i) * 4, 4);
-    return v;
-  };
-  int64_t const first = off_at(0), last = off_at(V);
-  if (last < first) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary offsets are not monotone");
-  std::vector<uint8_t> pool(static_cast<size_t>(last - first));
-  if (!pool.empty()) {
-    NVTEXT_HIP_TRY(hipMemcpyAsync(pool.data(), vocabulary->chars + first, pool.size(), hipMemcpyDeviceToHost, stream));
-    NVTEXT_HIP_TRY(hipStreamSynchronize(stream));
-  }
+  if (counts.pool_bytes > 0xFFFFFFF0ull) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
 
   // both key spaces share one table (wordpiece_tokenize.cu:224-263 builds two maps of capacity 2x each)
-  size_t keys = 0;
-  for (int32_t i = 0; i < V; ++i) {
-    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
-    int64_t const len = e - b;
-    if (len >= 1 && len < kMaxWord) ++keys;
-    if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') ++keys;
-  }
-  size_t capacity = 64;
+  size_t const keys = counts.keys;
+  size_t capacity   = 64;
   while (capacity < 2 * keys) capacity <<= 1;
   if (capacity > (size_t{1} << 31)) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
   uint32_t const mask = static_cast<uint32_t>(capacity / 2 - 1);  // buckets of two slots
   uint32_t bucket_bits = 0;
   while ((1u << bucket_bits) < capacity / 2) ++bucket_bits;
-  std::vector<HostSlot> slots(capacity, HostSlot{0, 0, 0, 0});
-  uint32_t max_len[2] = {0, 0};
-  // keys of more than 8 bytes, zero padded to whole 8-byte blocks
-  std::vector<uint8_t> blocks;
-  auto add_blocks = [&](const uint8_t* key, uint32_t len) -> uint32_t {
-    if (len <= 8) return 0u;
-    size_t const at = blocks.size();
-    blocks.resize(at + ((static_cast<size_t>(len) + 7) & ~size_t{7}), 0);
-    std::memcpy(blocks.data() + at, key, len);
-    return static_cast<uint32_t>(at);
-  };
-  for (int32_t i = 0; i < V; ++i) {
-    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
-    int64_t const len = e - b;
-    // entries of 200 bytes or more can never equal a tokenizable word or piece; empty ones are never looked up
-    if (len >= 1 && len < kMaxWord) {
-      host_insert(slots, mask, bucket_bits, blocks, 0, pool.data() + b, static_cast<uint32_t>(len), add_blocks(pool.data() + b, static_cast<uint32_t>(len)), i);
-      max_len[0] = std::max(max_len[0], static_cast<uint32_t>(len));
-    }
-    // wordpiece_tokenize.cu:184-192: "##" entries also live, without the prefix, in the second key space
-    if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') {
-      host_insert(slots, mask, bucket_bits, blocks, 1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), add_blocks(pool.data() + b + 2, static_cast<uint32_t>(len - 2)), i);
-      max_len[1] = std::max(max_len[1], static_cast<uint32_t>(len - 2));
-    }
-  }
-  if (blocks.size() > 0xFFFFFFF0ull) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "vocabulary too large");
-
-  // length filter over the first three bytes of every key of three bytes and more
   size_t lens_size = 1024;
   while (lens_size < 4 * keys) lens_size <<= 1;
-  std::vector<uint32_t> lens(lens_size, 0u);
-  std::vector<uint16_t> letters3(kLetters3, uint16_t{0});
-  auto letter = [](uint8_t c) { return c >= 'a' && c <= 'z'; };
-  auto note_length = [&](uint32_t kind, const uint8_t* key, uint32_t len) {
-    if (len < 3) return;
-    uint32_t const first3 = key[0] | (uint32_t{key[1]} << 8) | (uint32_t{key[2]} << 16);
-    lens[length_filter_index(kind, first3) & (lens_size - 1)] |= 1u << length_filter_bit(len);
-    if (kind == 1 && len <= 18 && letter(key[0]) && letter(key[1]) && letter(key[2]))
-      letters3[((key[0] - 'a') * 26u + (key[1] - 'a')) * 26u + (key[2] - 'a')] |= static_cast<uint16_t>(1u << (len - 3));
-  };
-  for (int32_t i = 0; i < V; ++i) {
-    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
-    int64_t const len = e - b;
-    if (len >= 1 && len < kMaxWord) note_length(0, pool.data() + b, static_cast<uint32_t>(len));
-    if (len >= 3 && len - 2 < kMaxWord && pool[b] == '#' && pool[b + 1] == '#') note_length(1, pool.data() + b + 2, static_cast<uint32_t>(len - 2));
-  }
-
-  // direct tables for the keys of one and two bytes (the first entry with a key wins, as in the table)
-  std::vector<int32_t> short_ids(kShortIds, kNone);
-  auto note_short = [&](uint32_t kind, const uint8_t* key, uint32_t len, int32_t id) {
-    if (len > 2) return;
-    size_t const at = len == 2 ? kind * 65536u + (key[0] | (uint32_t{key[1]} << 8)) : 2 * 65536u + kind * 256u + key[0];
-    if (short_ids[at] == kNone) short_ids[at] = id;
-  };
-  for (int32_t i = 0; i < V; ++i) {
-    int64_t const b = off_at(i) - first, e = off_at(i + 1) - first;
-    int64_t const len = e - b;
-    if (len >= 1 && len <= 2) note_short(0, pool.data() + b, static_cast<uint32_t>(len), i);
-    if (len >= 3 && len <= 4 && pool[b] == '#' && pool[b + 1] == '#') note_short(1, pool.data() + b + 2, static_cast<uint32_t>(len - 2), i);
-  }
 
   auto* v = new nvtext_amd_wordpiece_vocabulary;
-  v->entries = V;
-  // wordpiece_tokenize.cu:199-209, 273-275
-  int32_t unk = host_find(slots, mask, bucket_bits, blocks, "[UNK]");
-  if (unk < 0) unk = host_find(slots, mask, bucket_bits, blocks, "[unk]");
-  v->slot_bytes = capacity * sizeof(HostSlot);
-  v->pool_bytes = blocks.size() + 16;
+  v->entries    = V;
+  v->slot_bytes = capacity * sizeof(uint4);
+  v->pool_bytes = static_cast<size_t>(counts.pool_bytes) + 16;
   v->store.bind(mr, stream);
-  v->d_slots = v->store.allocate(v->slot_bytes);
-  v->d_pool  = v->store.allocate(v->pool_bytes);
-  std::vector<uint16_t> lens16(lens.size());
-  for (size_t i = 0; i < lens.size(); ++i) lens16[i] = packed_filter_word(lens[i]);
-  v->d_lens  = v->store.allocate(lens16.size() * sizeof(uint16_t));
-  v->d_short = v->store.allocate(short_ids.size() * sizeof(int32_t));
-  v->d_letters = v->store.allocate(letters3.size() * sizeof(uint16_t));
-  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters) {
+  v->d_slots   = v->store.allocate(v->slot_bytes);
+  v->d_pool    = v->store.allocate(v->pool_bytes);
+  v->d_lens    = v->store.allocate(lens_size * sizeof(uint16_t));
+  v->d_short   = v->store.allocate(kShortIds * sizeof(int32_t));
+  v->d_letters = v->store.allocate(kLetters3 * sizeof(uint16_t));
+  Temp lens32(temp_mr, lens_size * sizeof(uint32_t));
+  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters || !lens32.ok()) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
-  hipError_t e1 = hipMemcpyAsync(v->d_slots, slots.data(), v->slot_bytes, hipMemcpyHostToDevice, stream);
-  hipError_t e2 = blocks.empty() ? hipSuccess : hipMemcpyAsync(v->d_pool, blocks.data(), blocks.size(), hipMemcpyHostToDevice, stream);
-  hipError_t e4 = hipMemcpyAsync(v->d_lens, lens16.data(), lens16.size() * sizeof(uint16_t), hipMemcpyHostToDevice, stream);
-  hipError_t e5 = hipMemcpyAsync(v->d_short, short_ids.data(), short_ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
-  hipError_t e6 = hipMemcpyAsync(v->d_letters, letters3.data(), letters3.size() * sizeof(uint16_t), hipMemcpyHostToDevice, stream);
-  hipError_t e3 = hipStreamSynchronize(stream);  // host vectors die at return
-  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess || e6 != hipSuccess) {
-    nvtext_amd_wordpiece_vocabulary_destroy(v);
-    return fail(NVTEXT_AMD_DEVICE_ERROR, "vocabulary upload failed");
-  }
-  v->table.slots  = static_cast<const uint4*>(v->d_slots);
-  v->table.pool   = static_cast<const uint8_t*>(v->d_pool);
+  launch_fill_u32(static_cast<uint32_t*>(v->d_slots), 0u, static_cast<int64_t>(capacity) * 4, stream);
+  launch_fill_u32(static_cast<uint32_t*>(v->d_pool), 0u, static_cast<int64_t>(v->pool_bytes / 4), stream);  // (the sizes are multiples of 8)
+  launch_fill_u32(lens32.as<uint32_t>(), 0u, static_cast<int64_t>(lens_size), stream);
+  launch_fill_u32(static_cast<uint32_t*>(v->d_short), 0x80000000u, kShortIds, stream);
+  launch_fill_u32(static_cast<uint32_t*>(v->d_letters), 0u, kLetters3 / 2, stream);
+
+  v->table.slots       = static_cast<const uint4*>(v->d_slots);
+  v->table.pool        = static_cast<const uint8_t*>(v->d_pool);
   v->table.bucket_mask = mask;
   v->table.bucket_bits = bucket_bits;
-  v->table.unk_id      = unk;
-  v->table.max_len[0]  = max_len[0];
-  v->table.max_len[1]  = max_len[1];
+  v->table.unk_id      = -1;
+  v->table.max_len[0]  = counts.max_len[0];
+  v->table.max_len[1]  = counts.max_len[1];
   v->table.lens        = static_cast<const uint16_t*>(v->d_lens);
   v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
   v->table.short_ids   = static_cast<const int32_t*>(v->d_short);
   v->table.letters3    = static_cast<const uint16_t*>(v->d_letters);
+
+  VocabBuild build{};
+  build.slots       = static_cast<uint32_t*>(v->d_slots);
+  build.pool        = static_cast<uint8_t*>(v->d_pool);
+  build.lens32      = lens32.as<uint32_t>();
+  build.short_ids   = static_cast<uint32_t*>(v->d_short);
+  build.letters3    = static_cast<uint32_t*>(v->d_letters);
+  build.bucket_mask = mask;
+  build.bucket_bits = bucket_bits;
+  build.lens_mask   = static_cast<uint32_t>(lens_size - 1);
+  hipLaunchKernelGGL(vocabulary_insert_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, d_counts);
+  hipLaunchKernelGGL(vocabulary_settle_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build);
+  hipLaunchKernelGGL(vocabulary_finish_kernel, dim3(256), dim3(256), 0, stream, v->table, lens32.as<uint32_t>(), static_cast<uint16_t*>(v->d_lens),
+                     static_cast<uint32_t>(lens_size), static_cast<int32_t*>(v->d_short), d_counts);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpyAsync(&counts, d_counts, sizeof(counts), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);  // (the id of the unknown token; the temporaries are still in use until here)
+  if (e != hipSuccess) {
+    nvtext_amd_wordpiece_vocabulary_destroy(v);
+    return fail(NVTEXT_AMD_DEVICE_ERROR, hipGetErrorString(e));
+  }
+  v->table.unk_id = counts.unk_id;
   *out            = v;
   return NVTEXT_AMD_SUCCESS;
 }
