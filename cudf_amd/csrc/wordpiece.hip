@@ -1905,16 +1905,56 @@ struct VocabBuild {
   uint32_t bucket_mask, bucket_bits, lens_mask;
 };
 
-__global__ void vocabulary_insert_kernel(ColView v, VocabBuild t, VocabCounts* __restrict__ counts)
+// The table is filled in three steps so that, among the keys with one home bucket, the two that come first in the
+// vocabulary get its two slots (vocabulary files list their most frequent entries first, and a word that is not in its
+// home bucket costs the tokenizer a second look): every key bids for slot 0 of its home with an atomic minimum of its
+// number (step 1); the winners write their slots, the others bid for slot 1 (step 2); those winners write theirs,
+// and what is left, the keys that are carried past their home, takes the first slot from the next bucket on that nobody
+// has won or taken (step 3, compare-and-swap).
+constexpr uint32_t kNoBid = 0xFFFFFFFFu;
+
+struct VocabKeyParts {
+  VocabKey key;
+  uint32_t k0, k1;   // key bytes [0, 8)
+  HashParts hp;
+  uint32_t w0;       // slot.x of the key
+  uint32_t number;   // 2 * entry + key space: the order of the vocabulary
+};
+__device__ __forceinline__ bool vocabulary_key_parts(ColView const& v, VocabBuild const& t, VocabKeyParts* p)
 {
   int64_t const th = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (th >= 2 * static_cast<int64_t>(v.size)) return;
+  if (th >= 2 * static_cast<int64_t>(v.size)) return false;
   uint32_t const kind = static_cast<uint32_t>(th & 1);
-  uint32_t const id   = static_cast<uint32_t>(th >> 1);
-  VocabKey const k    = vocabulary_key(v, th >> 1, kind);
-  if (k.len == 0) return;
-  uint32_t k0, k1;
-  vocabulary_key8(k, 0, &k0, &k1);
+  p->number           = static_cast<uint32_t>(th);
+  p->key              = vocabulary_key(v, th >> 1, kind);
+  if (p->key.len == 0) return false;
+  vocabulary_key8(p->key, 0, &p->k0, &p->k1);
+  p->hp = hash_parts(vocabulary_hash(p->key, kind), t.bucket_bits);
+  p->w0 = slot_word0(p->hp.tag, kind, p->key.len);
+  return true;
+}
+// Writes the key into a slot that is its alone.  (Slot 0 of a bucket may be getting its flags at this moment: its first
+// two words are or-ed in; the slots start as zeros.)
+__device__ __forceinline__ void vocabulary_write_slot(VocabBuild const& t, VocabCounts* counts, VocabKeyParts const& p, uint32_t* slot, bool claimed)
+{
+  uint32_t pool_off = 0;
+  if (p.key.len > 8) {
+    pool_off = atomicAdd(&counts->pool_cursor, (p.key.len + 7u) & ~7u);
+    for (uint32_t i = 0; i < p.key.len; ++i) t.pool[pool_off + i] = p.key.bytes[i];  // (the pool starts as zeros: the padding)
+  }
+  if (!claimed) atomicOr(slot, p.w0);
+  atomicOr(slot + 1, p.number >> 1);
+  slot[2] = p.key.len <= 8 ? p.k0 : pool_off;
+  slot[3] = p.key.len <= 8 ? p.k1 : 0u;
+}
+
+// step 1; also the length filter and the direct tables
+__global__ void vocabulary_bid_kernel(ColView v, VocabBuild t, uint32_t* __restrict__ bid0)
+{
+  VocabKeyParts p;
+  if (!vocabulary_key_parts(v, t, &p)) return;
+  uint32_t const kind = p.number & 1u, id = p.number >> 1, k0 = p.k0;
+  VocabKey const& k = p.key;
   // the length filter over the first three bytes, and its exact twin for pieces of lower-case letters
   if (k.len >= 3) {
     atomicOr(&t.lens32[length_filter_index(kind, k0 & 0x00FFFFFFu) & t.lens_mask], 1u << length_filter_bit(k.len));
@@ -1930,28 +1970,48 @@ __global__ void vocabulary_insert_kernel(ColView v, VocabBuild t, VocabCounts* _
     uint32_t const at = k.len == 2 ? kind * 65536u + (k0 & 0xFFFFu) : 2u * 65536u + kind * 256u + (k0 & 0xFFu);
     atomicMin(&t.short_ids[at], id);
   }
-  // the table: the first empty slot from the key's home bucket on is taken with a compare-and-swap of its first word; an
-  // entry that occurs twice takes two slots here (whether a full slot holds the same key cannot be told while its owner
-  // may still be writing it) and is settled by the next kernel
-  uint32_t pool_off = 0;
-  if (k.len > 8) {
-    pool_off = atomicAdd(&counts->pool_cursor, (k.len + 7u) & ~7u);
-    for (uint32_t i = 0; i < k.len; ++i) t.pool[pool_off + i] = k.bytes[i];  // (the pool starts as zeros: the padding)
+  atomicMin(&bid0[p.hp.bucket], p.number);
+}
+
+// step 2
+__global__ void vocabulary_first_slot_kernel(ColView v, VocabBuild t, VocabCounts* __restrict__ counts, const uint32_t* __restrict__ bid0,
+                                             uint32_t* __restrict__ bid1)
+{
+  VocabKeyParts p;
+  if (!vocabulary_key_parts(v, t, &p)) return;
+  if (bid0[p.hp.bucket] == p.number)
+    vocabulary_write_slot(t, counts, p, t.slots + 8 * static_cast<size_t>(p.hp.bucket), false);
+  else
+    atomicMin(&bid1[p.hp.bucket], p.number);
+}
+
+// step 3
+__global__ void vocabulary_other_slots_kernel(ColView v, VocabBuild t, VocabCounts* __restrict__ counts, const uint32_t* __restrict__ bid0,
+                                              const uint32_t* __restrict__ bid1)
+{
+  VocabKeyParts p;
+  if (!vocabulary_key_parts(v, t, &p)) return;
+  uint32_t const home = p.hp.bucket;
+  if (bid0[home] == p.number) return;
+  if (bid1[home] == p.number) {
+    vocabulary_write_slot(t, counts, p, t.slots + 8 * static_cast<size_t>(home) + 4, false);
+    return;
   }
-  HashParts const hp = hash_parts(vocabulary_hash(k, kind), t.bucket_bits);
-  uint32_t const w0  = slot_word0(hp.tag, kind, k.len);
-  for (uint32_t b = hp.bucket;; b = (b + 1) & t.bucket_mask) {
-    for (uint32_t j = 0; j < 2; ++j) {
-      uint32_t* const slot = t.slots + 4 * (2 * static_cast<size_t>(b) + j);
-      if (atomicCAS(slot, 0u, w0) == 0u) {
-        atomicOr(slot + 1, id);  // (others may be setting kSearchOn in this word at this moment)
-        slot[2] = k.len <= 8 ? k0 : pool_off;
-        slot[3] = k.len <= 8 ? k1 : 0u;
-        return;
-      }
-    }
+  // both slots of the home bucket went to keys that come earlier in the vocabulary: carried on
+  for (uint32_t b = home;;) {
     atomicOr(t.slots + 8 * static_cast<size_t>(b) + 1, kSearchOn);  // the key is carried past this bucket
-    atomicOr(t.slots + 8 * static_cast<size_t>(b), hp.fp);
+    atomicOr(t.slots + 8 * static_cast<size_t>(b), p.hp.fp);
+    b = (b + 1) & t.bucket_mask;
+    // a slot that some key has won is (or will be) full; the first of the others that is empty is taken
+    uint32_t* const slot0 = t.slots + 8 * static_cast<size_t>(b);
+    if (bid0[b] == kNoBid && atomicCAS(slot0, 0u, p.w0) == 0u) {
+      vocabulary_write_slot(t, counts, p, slot0, true);
+      return;
+    }
+    if (bid1[b] == kNoBid && atomicCAS(slot0 + 4, 0u, p.w0) == 0u) {
+      vocabulary_write_slot(t, counts, p, slot0 + 4, true);
+      return;
+    }
   }
 }
 
@@ -2067,13 +2127,15 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->d_short   = v->store.allocate(kShortIds * sizeof(int32_t));
   v->d_letters = v->store.allocate(kLetters3 * sizeof(uint16_t));
   Temp lens32(temp_mr, lens_size * sizeof(uint32_t));
-  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters || !lens32.ok()) {
+  Temp bids(temp_mr, capacity * sizeof(uint32_t));  // per bucket: who gets slot 0, who gets slot 1
+  if (!v->d_slots || !v->d_pool || !v->d_lens || !v->d_short || !v->d_letters || !lens32.ok() || !bids.ok()) {
     nvtext_amd_wordpiece_vocabulary_destroy(v);
     return fail(NVTEXT_AMD_ALLOC_FAILED, "vocabulary allocation failed");
   }
   launch_fill_u32(static_cast<uint32_t*>(v->d_slots), 0u, static_cast<int64_t>(capacity) * 4, stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_pool), 0u, static_cast<int64_t>(v->pool_bytes / 4), stream);  // (the sizes are multiples of 8)
   launch_fill_u32(lens32.as<uint32_t>(), 0u, static_cast<int64_t>(lens_size), stream);
+  launch_fill_u32(bids.as<uint32_t>(), kNoBid, static_cast<int64_t>(capacity), stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_short), 0x80000000u, kShortIds, stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_letters), 0u, kLetters3 / 2, stream);
 
@@ -2098,7 +2160,11 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   build.bucket_mask = mask;
   build.bucket_bits = bucket_bits;
   build.lens_mask   = static_cast<uint32_t>(lens_size - 1);
-  hipLaunchKernelGGL(vocabulary_insert_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, d_counts);
+  hipLaunchKernelGGL(vocabulary_bid_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, bids.as<uint32_t>());
+  hipLaunchKernelGGL(vocabulary_first_slot_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, d_counts, bids.as<uint32_t>(),
+                     bids.as<uint32_t>() + capacity / 2);
+  hipLaunchKernelGGL(vocabulary_other_slots_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, d_counts, bids.as<uint32_t>(),
+                     bids.as<uint32_t>() + capacity / 2);
   hipLaunchKernelGGL(vocabulary_settle_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build);
   hipLaunchKernelGGL(vocabulary_finish_kernel, dim3(256), dim3(256), 0, stream, v->table, lens32.as<uint32_t>(), static_cast<uint16_t*>(v->d_lens),
                      static_cast<uint32_t>(lens_size), static_cast<int32_t*>(v->d_short), d_counts);
