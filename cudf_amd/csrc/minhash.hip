@@ -213,6 +213,21 @@ __device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, con
   __builtin_amdgcn_wave_barrier();
 }
 
+// Whether the wavefront has met this hash lately (it is noted either way).  Called by the lanes that have a hash.
+template <typename T>
+__device__ __forceinline__ bool seen_lately(WaveLds<T>& lds, T hv)
+{
+  T* const at  = &lds.recent[static_cast<uint32_t>(hv) & (recent_entries<T>() - 1)];
+  T const was  = *at;
+  *at          = hv;
+  return was == hv;
+}
+template <typename T>
+__device__ __forceinline__ void forget_hashes(WaveLds<T>& lds, int lane)
+{
+  for (int i = lane; i < recent_entries<T>(); i += kWave) lds.recent[i] = T{0};
+}
+
 // Processes the window starts [s_begin, s_end) of one row with one wavefront and folds the
 // permuted hashes into m[K].  Lane l owns parameters chunk_base + l + 64*k.
 template <typename T, int K>
@@ -223,6 +238,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
   if (static_cast<int64_t>(width) * 4 <= kHalo) {
     // usual case: a window (<= 4*width bytes) fits the halo staged behind every tile
     uint32_t const halo = static_cast<uint32_t>(width) * 4u;
+    forget_hashes(lds, lane);  // (the wave barrier after the first tile's staging comes before the first look)
     for (int64_t base = s_begin; base < s_end; base += kTile) {
       uint32_t const cnt = static_cast<uint32_t>(min(static_cast<int64_t>(kTile), s_end - base));
       uint32_t const len = static_cast<uint32_t>(min(n - base, static_cast<int64_t>(cnt + halo)));
@@ -240,13 +256,14 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       if (plain) {
         for (uint32_t q = 0; q < cnt; q += kWave) {
           uint32_t const p = q + lane;
-          bool const valid = p < cnt && n - (base + p) >= static_cast<int64_t>(width_all);
-          T hv             = 0;
+          bool valid = p < cnt && n - (base + p) >= static_cast<int64_t>(width_all);
+          T hv       = 0;
           if (valid) {
             WordSrc const src{lds.bytes, mis + p};
             hv = H::hash(src, width_all, seed);
             hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
           }
+          valid             = valid && !seen_lately(lds, hv);
           uint64_t const vm = ballot64(valid);
           if (valid) lds.hashes[count + lanes_below(vm)] = hv;
           count += static_cast<uint32_t>(__builtin_popcountll(vm));
@@ -278,6 +295,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
               hv = hv < 1 ? T{1} : hv;  // minhash.cu:141
             }
           }
+          valid             = valid && !seen_lately(lds, hv);
           uint64_t const vm = ballot64(valid);
           if (valid) lds.hashes[count + lanes_below(vm)] = hv;
           count += static_cast<uint32_t>(__builtin_popcountll(vm));

@@ -16,10 +16,18 @@ constexpr int kHalo      = 128;                // bytes staged past the tile (wi
 constexpr int kTileWords = (kTile + kHalo + 4 + 24) / 4;  // +4 misalignment, +24 over-read of the hash tail
 constexpr int kSpan      = 16384;              // bytes of a row handled by one workgroup
 
+// Windows repeat (text repeats its words: a tenth of the windows of a tile, a third within 4 KB of ordinary text), and a
+// hash that has been folded once changes no minimum when it is folded again.  Every wavefront keeps the hashes it
+// saw last in a small direct-mapped table and drops a hash that it finds there; what the table has forgotten is folded
+// again, which costs time and nothing else.  Cleared (hashes are never 0) whenever the wavefront begins a row.
+template <typename T>
+constexpr int recent_entries() { return 256; }  // (512 costs the kernels a workgroup per CU: slower but for the longest rows)
+
 template <typename T>
 struct WaveLds {
   uint32_t bytes[kTileWords];
   alignas(16) T hashes[kTile + 4];
+  alignas(16) T recent[recent_entries<T>()];
   uint32_t chars[kTile + kHalo];  // the characters that start in the staged bytes, in order: start | end << 16 (see CharMap)
 };
 
