@@ -56,25 +56,37 @@ struct HashTraits<uint64_t> {
   // Permutation (minhash.cu:350-351): ((hv*a + b) mod 2^64) % (2^61-1), see Fold<uint64_t>.
 };
 
-// ((h * a + b) mod 2^64) folded once mod 2^61 - 1, that is (x & p) + (x >> 61) for the 64-bit x: at most p + 7.
-// x = h.lo * a.lo + b as one 64-bit multiply-add, the low halves of the two cross products added to its high dword
-// where it stands; the fold is a shift and a mask of that dword and one more multiply-add (q * 1 + x) for the carry.
-// Eight instructions, and none that only moves a value: the register pair that one multiply-add writes is the one
-// the next reads (written out with 64-bit adds, the compiler copies halves of pairs about for every product).
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint64_t permute_fold_u64(uint64_t h, uint64_t a, uint64_t b)
+// ((h * a + b) mod 2^64) folded once mod 2^61 - 1, that is (x & p) + (x >> 61) for the 64-bit x: at most p + 7; for two
+// hashes and one (a, b).  x = h.lo * a.lo + b is one 64-bit multiply-add; the two cross products, of which only the low
+// dwords count, are two more, chained (h.lo * a.hi, then h.hi * a.lo added to it), and their sum goes to the high dword
+// of x with a plain 32-bit add, which issues in half the cycles of a multiply or of a three-operand add (left to itself
+// the compiler makes them two multiplies and a three-operand add).  The fold is a shift and a mask of that dword and
+// one more multiply-add (q * 1 + x) for the carry.  Eight instructions per hash, none that only moves a value.  The
+// chained pairs of the two hashes stand interleaved in one block of assembly, so that neither waits for its own first
+// half; everything else is left to the compiler, which puts an idle cycle between instructions it cannot see into.
+__device__ __forceinline__ void permute_fold_u64_pair(uint64_t h0, uint64_t h1, uint64_t a, uint64_t b, uint32_t one, uint64_t* y0,
+                                                      uint64_t* y1)
 {
-  uint32_t const hl = static_cast<uint32_t>(h), hh = static_cast<uint32_t>(h >> 32);
   uint32_t const al = static_cast<uint32_t>(a), ah = static_cast<uint32_t>(a >> 32);
-  uint64_t x;
-  asm("v_mad_u64_u32 %0, vcc, %1, %2, %3" : "=v"(x) : "v"(hl), "v"(al), "v"(b) : "vcc");
-  u32x2_t xp = __builtin_bit_cast(u32x2_t, x);
-  xp.y += hl * ah + hh * al;
-  uint32_t const q = xp.y >> 29;
-  xp.y &= 0x1FFFFFFFu;
-  uint64_t y;
-  asm("v_mad_u64_u32 %0, vcc, %1, 1, %2" : "=v"(y) : "v"(q), "v"(__builtin_bit_cast(uint64_t, xp)) : "vcc");
-  return y;
+  uint32_t const l0 = static_cast<uint32_t>(h0), u0 = static_cast<uint32_t>(h0 >> 32);
+  uint32_t const l1 = static_cast<uint32_t>(h1), u1 = static_cast<uint32_t>(h1 >> 32);
+  uint64_t c0, c1;
+  asm("v_mad_u64_u32 %0, vcc, %2, %6, 0\n\t"
+      "v_mad_u64_u32 %1, vcc, %4, %6, 0\n\t"
+      "v_mad_u64_u32 %0, vcc, %3, %7, %0\n\t"
+      "v_mad_u64_u32 %1, vcc, %5, %7, %1"
+      : "=&v"(c0), "=&v"(c1)
+      : "v"(l0), "v"(u0), "v"(l1), "v"(u1), "v"(ah), "v"(al)
+      : "vcc");
+  uint64_t const x0 = static_cast<uint64_t>(l0) * al + b;
+  uint64_t const x1 = static_cast<uint64_t>(l1) * al + b;
+  uint32_t xh0      = static_cast<uint32_t>(x0 >> 32) + static_cast<uint32_t>(c0);
+  uint32_t xh1      = static_cast<uint32_t>(x1 >> 32) + static_cast<uint32_t>(c1);
+  uint32_t const q0 = xh0 >> 29, q1 = xh1 >> 29;
+  xh0 &= 0x1FFFFFFFu;
+  xh1 &= 0x1FFFFFFFu;
+  *y0 = static_cast<uint64_t>(q0) * one + ((static_cast<uint64_t>(xh0) << 32) | static_cast<uint32_t>(x0));
+  *y1 = static_cast<uint64_t>(q1) * one + ((static_cast<uint64_t>(xh1) << 32) | static_cast<uint32_t>(x1));
 }
 
 // min of two values below 2^62 in one instruction: such bit patterns are non-negative finite doubles
@@ -160,6 +172,8 @@ struct Fold<uint64_t, K> {
     // if it ever happens the tile is folded again exactly.  Unreduced values are >= p, above every
     // reduced value, so they can never displace a correct minimum.
     uint32_t top = 0;
+    uint32_t one;  // the number 1 where the compiler does not see it: q * one + x stays one multiply-add
+    asm("s_mov_b32 %0, 1" : "=s"(one));
     for (uint32_t i = first; i < padded; i += stride) {
       uint64_t h[kPerTrip];
 #pragma unroll
@@ -168,8 +182,8 @@ struct Fold<uint64_t, K> {
       for (int k = 0; k < K; ++k) {
 #pragma unroll
         for (uint32_t j = 0; j < kPerTrip; j += 2) {
-          uint64_t const y0 = permute_fold_u64(h[j], a[k], b[k]);
-          uint64_t const y1 = permute_fold_u64(h[j + 1], a[k], b[k]);
+          uint64_t y0, y1;
+          permute_fold_u64_pair(h[j], h[j + 1], a[k], b[k], one, &y0, &y1);
           top               = max(max(top, static_cast<uint32_t>(y0 >> 32)), static_cast<uint32_t>(y1 >> 32));
           m[k]              = min_below_2_62(min_below_2_62(m[k], y0), y1);
         }
