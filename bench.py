@@ -34,6 +34,12 @@ MEASURED_TRAFFIC_C2 = {
     "wordpiece_oov_kernel": (915002311, 846801296),
     "wordpiece_emit_kernel": (1394015035, 905182598),
 }
+MEASURED_TRAFFIC_C5_TOKENIZE = {
+    "range_first_row_kernel": (0, 0),
+    "wordpiece_word_kernel": (0, 0),
+    "wordpiece_oov_kernel": (0, 0),
+    "wordpiece_emit_kernel": (0, 0),
+}
 MEASURED_TRAFFIC_C5_NORMALIZE = {
     "normalize_count_kernel": (4575176291, 63532922),
     "normalize_tile_rows_kernel": (73449676, 7941631),
@@ -42,12 +48,14 @@ MEASURED_TRAFFIC_C5_NORMALIZE = {
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
 # moves issue in fewer than 4 cycles).  The floor is the instruction sequence of the inner loop: uint32, one
-# v_mad_u64_u32 per product and one v_min3_u32 per two (1.5); uint64, three v_mad_u64_u32 and an add for the product,
-# and / shift / 64-bit add (2) of the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two products (9.5).
+# v_mad_u64_u32 per product and one v_min3_u32 per two (1.5); uint64, three v_mad_u64_u32 and a 32-bit add for (h * a + b)
+# mod 2^64, a shift, a mask and one more v_mad_u64_u32 for the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two
+# products (8.5).
 VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit d582704)"
 MINHASH_VALU = {
     "C3": {"floor": 1.5, "measured": 1.98, "issue": 1.00},
-    "C4": {"floor": 9.5, "measured": 13.39, "issue": 1.11},
+    "C4": {"floor": 8.5, "measured": 13.39, "issue": 1.11},
+    "C5": {"floor": 8.5, "measured": 13.7, "issue": 0.89},
 }
 
 
@@ -430,7 +438,7 @@ def main():
         tleg.update({"input_GBps": round(ib / tsec / 1e9, 2), "mrows_per_s": round(w.rows.size / tsec / 1e6, 3), "tokens_out": ntok,
                      "temporaries_bytes": tleg["peak_device_bytes"] - (talg - ib),
                      "temporaries_per_input_byte": round((tleg["peak_device_bytes"] - (talg - ib)) / ib, 3),
-                     "roofline": hbm_roofline(talg, tsec, tk)})
+                     "roofline": hbm_roofline(talg, tsec, tk, MEASURED_TRAFFIC_C5_TOKENIZE if args.minhash_scale == 1.0 else None)})
         leg = {"workload": f"C5 x{args.minhash_scale}", "rows": w.rows.size, "chars_bytes": w.rows.chars_bytes, "offsets": "int64",
                "vocab_entries": w.vocab.size, "tokenize": tleg}
         keep.clear()
@@ -491,7 +499,23 @@ def main():
             return keep["o"]
 
         msec, mleg, _ = measure(m5step, side_steps, 1, _capi, torch)
-        mleg.update({"input_GBps": round(ib / msec / 1e9, 2), "mrows_per_s": round(w.rows.size / msec / 1e6, 3)})
+        # windows of a row: its characters less width - 1, one for a shorter row that is not empty, none for a null row
+        firsts = ((w.rows.chars & 0xC0) != 0x80)[: int(w.rows.offsets[-1])]
+        begins = w.rows.offsets[:-1].astype(np.int64)
+        inside = int(np.searchsorted(begins, firsts.size))  # (rows that begin at the end of the bytes are empty)
+        row_chars = np.zeros(w.rows.size, np.int64)
+        if inside:
+            row_chars[:inside] = np.add.reduceat(firsts, begins[:inside], dtype=np.int64)
+        row_chars[np.diff(w.rows.offsets) == 0] = 0
+        if w.rows.mask is not None:
+            from cudf_amd.arrow_host import unpack_validity
+            row_chars[~unpack_validity(w.rows.mask, w.rows.size, w.rows.offset)] = 0
+        windows = int(np.where(row_chars >= p["width"], row_chars - (p["width"] - 1), row_chars > 0).sum())
+        del firsts, row_chars
+        mleg.update({"input_GBps": round(ib / msec / 1e9, 2), "mrows_per_s": round(w.rows.size / msec / 1e6, 3),
+                     "windows": windows, "parameters": p["P"], "gperm_per_s": round(windows * p["P"] / msec / 1e9, 1)})
+        if args.minhash_scale == 1.0:
+            mleg["valu"] = valu_object("C5")
         leg["minhash64"] = mleg
         if orc:
             n = min(w.rows.size, 400_000)
