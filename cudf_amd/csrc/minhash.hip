@@ -204,7 +204,7 @@ struct Fold<uint64_t, K> {
 };
 
 template <typename T, int K>
-__device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane,
+__device__ __forceinline__ void fold_hashes(T* hashes, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane,
                                             Packing pk = Packing{kWave, 1})
 {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -214,15 +214,15 @@ __device__ __forceinline__ void fold_hashes(WaveLds<T>& lds, uint32_t count, con
   // a duplicate never changes a minimum
   uint32_t const stride = K > 1 ? Fold<T, K>::kPerTrip : pk.stride(Fold<T, K>::kPerTrip);  // a power of two, at most 64
   uint32_t const padded = (count + stride - 1u) & ~(stride - 1u);
-  if (lane < static_cast<int>(padded - count)) lds.hashes[count + lane] = lds.hashes[0];
+  if (lane < static_cast<int>(padded - count)) hashes[count + lane] = hashes[0];
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   // the usual case keeps the loop counter out of the vector registers
   if (K > 1 || pk.groups == 1)
-    Fold<T, K>::run(lds.hashes, padded, 0u, Fold<T, K>::kPerTrip, a, b, m);
+    Fold<T, K>::run(hashes, padded, 0u, Fold<T, K>::kPerTrip, a, b, m);
   else
-    Fold<T, K>::run(lds.hashes, padded, pk.first(lane, Fold<T, K>::kPerTrip), stride, a, b, m);
+    Fold<T, K>::run(hashes, padded, pk.first(lane, Fold<T, K>::kPerTrip), stride, a, b, m);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
 }
@@ -315,7 +315,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
           count += static_cast<uint32_t>(__builtin_popcountll(vm));
         }
       }
-      fold_hashes<T, K>(lds, count, a, b, m, lane, pk);
+      fold_hashes<T, K>(lds.hashes, count, a, b, m, lane, pk);
     }
   } else {
     // very wide windows: 64 starts at a time, bytes read straight from global memory
@@ -336,7 +336,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       }
       uint64_t const vm = ballot64(valid);
       if (valid) lds.hashes[lanes_below(vm)] = hv;
-      fold_hashes<T, K>(lds, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane, pk);
+      fold_hashes<T, K>(lds.hashes, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane, pk);
     }
   }
 }
@@ -666,7 +666,7 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
                                                                   T* __restrict__ out)
 {
   using H = HashTraits<T>;
-  __shared__ WaveLds<T> lds[kWaves];
+  __shared__ alignas(16) T hashes[kWaves][2 * kWave];  // 64 hashes a trip, padded to the stride of the fold (at most 64 more)
   __shared__ T red[kWaves][K * kWave];
   // the chars of the elements a wavefront is hashing (32-bit hash only: measured 13 % faster there, 9 % slower for the
   // 64-bit hash, whose 16-byte steps cost more to assemble out of LDS than they save)
@@ -729,8 +729,8 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
     }
     if (valid) hv = hv < 1 ? T{1} : hv;  // 237
     uint64_t const vm = ballot64(valid);
-    if (valid) lds[wave].hashes[lanes_below(vm)] = hv;
-    fold_hashes<T, K>(lds[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
+    if (valid) hashes[wave][lanes_below(vm)] = hv;
+    fold_hashes<T, K>(hashes[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
   }
 
 #pragma unroll
