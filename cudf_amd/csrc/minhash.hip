@@ -22,6 +22,7 @@
 
 #include <limits>
 #include <mutex>
+#include <type_traits>
 
 // Scratch of nvtext_amd_minhash_preallocated, the entry point that allocates nothing: the extra-span counts of the
 // rows (rows + 1 values) and behind them the tile sums of the scans.  Every device holds its own copy of the array
@@ -203,16 +204,27 @@ struct Fold<uint64_t, K> {
   }
 };
 
-template <typename T, int K>
-__device__ __forceinline__ void fold_hashes(T* hashes, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane,
-                                            Packing pk = Packing{kWave, 1})
+// The parameters beyond the last full set of 64, when there are at most 32 of them: one more (a, b) pair per lane,
+// shared out over sets of lanes as Packing describes, so that they cost the fold a share of a full set (4 parameters
+// beyond 256: a sixteenth) instead of a whole one.
+template <typename T>
+struct TailParams {
+  T a[1], b[1], m[1];
+  Packing pk;
+};
+struct NoTail {};
+
+template <typename T, int K, typename Tail = NoTail>
+__device__ __forceinline__ void fold_hashes(T* hashes, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane, Packing pk, Tail& tail)
 {
+  constexpr bool kHasTail = !std::is_same<Tail, NoTail>::value;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (count == 0) return;
   // a duplicate never changes a minimum
-  uint32_t const stride = K > 1 ? Fold<T, K>::kPerTrip : pk.stride(Fold<T, K>::kPerTrip);  // a power of two, at most 64
+  uint32_t stride = K > 1 ? Fold<T, K>::kPerTrip : pk.stride(Fold<T, K>::kPerTrip);  // a power of two, at most 64
+  if constexpr (kHasTail) stride = max(stride, tail.pk.stride(Fold<T, 1>::kPerTrip));
   uint32_t const padded = (count + stride - 1u) & ~(stride - 1u);
   if (lane < static_cast<int>(padded - count)) hashes[count + lane] = hashes[0];
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -222,9 +234,18 @@ __device__ __forceinline__ void fold_hashes(T* hashes, uint32_t count, const T (
   if (K > 1 || pk.groups == 1)
     Fold<T, K>::run(hashes, padded, 0u, Fold<T, K>::kPerTrip, a, b, m);
   else
-    Fold<T, K>::run(hashes, padded, pk.first(lane, Fold<T, K>::kPerTrip), stride, a, b, m);
+    Fold<T, K>::run(hashes, padded, pk.first(lane, Fold<T, K>::kPerTrip), pk.stride(Fold<T, K>::kPerTrip), a, b, m);
+  if constexpr (kHasTail)
+    Fold<T, 1>::run(hashes, padded, tail.pk.first(lane, Fold<T, 1>::kPerTrip), tail.pk.stride(Fold<T, 1>::kPerTrip), tail.a, tail.b, tail.m);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
+}
+template <typename T, int K>
+__device__ __forceinline__ void fold_hashes(T* hashes, uint32_t count, const T (&a)[K], const T (&b)[K], T (&m)[K], int lane,
+                                            Packing pk = Packing{kWave, 1})
+{
+  NoTail none;
+  fold_hashes<T, K, NoTail>(hashes, count, a, b, m, lane, pk, none);
 }
 
 // Whether the wavefront has met this hash lately (it is noted either way).  Called by the lanes that have a hash.
@@ -244,9 +265,9 @@ __device__ __forceinline__ void forget_hashes(WaveLds<T>& lds, int lane)
 
 // Processes the window starts [s_begin, s_end) of one row with one wavefront and folds the
 // permuted hashes into m[K].  Lane l owns parameters chunk_base + l + 64*k.
-template <typename T, int K>
+template <typename T, int K, typename Tail>
 __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, int64_t s_begin, int64_t s_end, T seed, int32_t width,
-                                                const T (&a)[K], const T (&b)[K], T (&m)[K], WaveLds<T>& lds, int lane, Packing pk)
+                                                const T (&a)[K], const T (&b)[K], T (&m)[K], WaveLds<T>& lds, int lane, Packing pk, Tail& tail)
 {
   using H = HashTraits<T>;
   if (static_cast<int64_t>(width) * 4 <= kHalo) {
@@ -315,7 +336,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
           count += static_cast<uint32_t>(__builtin_popcountll(vm));
         }
       }
-      fold_hashes<T, K>(lds.hashes, count, a, b, m, lane, pk);
+      fold_hashes<T, K, Tail>(lds.hashes, count, a, b, m, lane, pk, tail);
     }
   } else {
     // very wide windows: 64 starts at a time, bytes read straight from global memory
@@ -336,7 +357,7 @@ __device__ __forceinline__ void process_section(const uint8_t* row, int64_t n, i
       }
       uint64_t const vm = ballot64(valid);
       if (valid) lds.hashes[lanes_below(vm)] = hv;
-      fold_hashes<T, K>(lds.hashes, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane, pk);
+      fold_hashes<T, K, Tail>(lds.hashes, static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane, pk, tail);
     }
   }
 }
@@ -360,22 +381,51 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
 constexpr int64_t kSoloBytes = 1024;
 constexpr int kGroupRows      = kWaves;
 
+// The tail of a launch with TAIL: the P - 64 K parameters (1..32) beyond the K full sets of the one chunk.
+template <typename T, int K, bool TAIL>
+struct TailOf {
+  using type = NoTail;
+  static __device__ __forceinline__ void load(type&, const T*, const T*, int32_t, int) {}
+  static __device__ __forceinline__ void reset(type&) {}
+  static __device__ __forceinline__ void finish(type&) {}
+  static __device__ __forceinline__ T value(type const&) { return T{0}; }
+};
 template <typename T, int K>
+struct TailOf<T, K, true> {
+  using type = TailParams<T>;
+  static __device__ __forceinline__ void load(type& t, const T* pa, const T* pb, int32_t P, int lane)
+  {
+    t.pk            = packing_for(P - K * kWave);
+    int32_t const j = K * kWave + t.pk.param_lane(lane);
+    t.a[0]          = j < P ? pa[j] : T{0};
+    t.b[0]          = j < P ? pb[j] : T{0};
+    t.m[0]          = std::numeric_limits<T>::max();
+  }
+  static __device__ __forceinline__ void reset(type& t) { t.m[0] = std::numeric_limits<T>::max(); }
+  static __device__ __forceinline__ void finish(type& t) { t.m[0] = t.pk.combine(t.m[0]); }  // every set of lanes then holds the minima
+  static __device__ __forceinline__ T value(type const& t) { return t.m[0]; }
+};
+
+template <typename T, int K, bool TAIL>
 __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
                                                                 int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out)
 {
+  using TailT = TailOf<T, K, TAIL>;
+  constexpr int kSets = K + (TAIL ? 1 : 0);
   __shared__ WaveLds<T> lds[kWaves];
-  __shared__ T red[kWaves][K * kWave];
+  __shared__ T red[kWaves][kSets * kWave];
 
   int64_t const r0 = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * kGroupRows;
   if (r0 >= col.size) return;
   int const lane           = lane_id();
   int const wave           = threadIdx.x / kWave;
-  int32_t const chunk_base = blockIdx.y * (K * kWave);
-  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
+  int32_t const chunk_base = blockIdx.y * (K * kWave);  // (with TAIL there is one chunk)
+  int32_t const in_chunk   = min(kSets * kWave, P - chunk_base);
   Packing const pk         = K == 1 ? packing_for(P) : Packing{kWave, 1};
   T a[K], b[K], m[K];
   load_params<T, K>(pa, pb, P, chunk_base, pk.param_lane(lane), a, b, m);
+  typename TailT::type tail;
+  TailT::load(tail, pa, pb, P, lane);
 
   int const rows_here = static_cast<int>(min(static_cast<int64_t>(kGroupRows), col.size - r0));
   int const wave_s    = __builtin_amdgcn_readfirstlane(wave);  // (the same in every lane: what depends on it stays scalar)
@@ -391,6 +441,7 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
     if (solo != (n <= kSoloBytes)) continue;
 #pragma unroll
     for (int k = 0; k < K; ++k) m[k] = std::numeric_limits<T>::max();
+    TailT::reset(tail);
     int64_t sb = 0, se = n;
     if (!solo) {
       int64_t const span = min(n, static_cast<int64_t>(kSpan));
@@ -399,8 +450,9 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
       sb                 = min(span, wave * sec);
       se                 = min(span, sb + sec);
     }
-    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
+    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk, tail);
     if (K == 1) m[0] = pk.combine(m[0]);
+    TailT::finish(tail);
     T* const dst = out + static_cast<int64_t>(out_offsets[r0 + i]) + chunk_base;
     if (solo) {
       // nothing to combine: the minima go from the registers to the result; an empty row is zeros (minhash.cu:318)
@@ -409,10 +461,12 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
         int32_t const j = lane + kWave * k;  // (with fewer than 64 parameters the first lanes hold one each, in order)
         if (j < in_chunk) dst[j] = n > 0 ? m[k] : T{0};
       }
+      if (TAIL && K * kWave + lane < in_chunk) dst[K * kWave + lane] = n > 0 ? TailT::value(tail) : T{0};
     } else {
       __syncthreads();  // (the row before has been read out of red)
 #pragma unroll
       for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+      if (TAIL) red[wave][K * kWave + lane] = TailT::value(tail);
       __syncthreads();
       for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
         T v = red[0][j];
@@ -426,16 +480,18 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
 
 // Extra parts of rows longer than kSpan: task t covers bytes [part*kSpan, (part+1)*kSpan) of its row.
 // extra_prefix[r] = number of extra parts in rows < r (rows+1 entries).
-template <typename T, int K>
+template <typename T, int K, bool TAIL>
 __global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
                                                                  int32_t width, const int32_t* __restrict__ out_offsets,
                                                                  const uint32_t* __restrict__ extra_prefix, T* __restrict__ out)
 {
+  using TailT = TailOf<T, K, TAIL>;
+  constexpr int kSets = K + (TAIL ? 1 : 0);
   __shared__ WaveLds<T> lds[kWaves];
-  __shared__ T red[kWaves][K * kWave];
+  __shared__ T red[kWaves][kSets * kWave];
   uint32_t const total     = extra_prefix[col.size];
   int32_t const chunk_base = blockIdx.y * (K * kWave);
-  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
+  int32_t const in_chunk   = min(kSets * kWave, P - chunk_base);
   int const lane           = lane_id();
   int const wave           = threadIdx.x / kWave;
   Packing const pk         = K == 1 ? packing_for(P) : Packing{kWave, 1};
@@ -452,16 +508,20 @@ __global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T 
     int64_t const n    = col.off(r + 1) - o;
     T a[K], b[K], m[K];
     load_params<T, K>(pa, pb, P, chunk_base, pk.param_lane(lane), a, b, m);
+    typename TailT::type tail;
+    TailT::load(tail, pa, pb, P, lane);
     int64_t const pb0  = part * kSpan;
     int64_t const pe0  = min(n, pb0 + kSpan);
     int64_t const sec  = kSpan / kWaves;
     int64_t const sb   = min(pe0, pb0 + wave * sec);
     int64_t const se   = min(pe0, sb + sec);
-    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk);
+    if (sb < se) process_section<T, K>(col.chars + o, n, sb, se, seed, width, a, b, m, lds[wave], lane, pk, tail);
     if (K == 1) m[0] = pk.combine(m[0]);
+    TailT::finish(tail);
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+    if (TAIL) red[wave][K * kWave + lane] = TailT::value(tail);
     __syncthreads();
     T* dst = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
     for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
@@ -497,24 +557,47 @@ __global__ void uniform_offsets_kernel(int32_t* out, int32_t rows, int32_t P)
 
 constexpr int32_t kMaxRowBlocks = 1 << 20;
 
-template <typename T, int K>
+template <typename T, int K, bool TAIL>
 void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, const int32_t* offsets,
                     const uint32_t* extra_prefix, T* child, hipStream_t stream)
 {
-  int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
+  int32_t const chunks = TAIL ? 1 : (P + K * kWave - 1) / (K * kWave);
   int32_t const groups = (v.size + kGroupRows - 1) / kGroupRows;  // four rows to a workgroup
   dim3 grid(static_cast<unsigned>(std::min(groups, kMaxRowBlocks)), static_cast<unsigned>(chunks),
             static_cast<unsigned>((groups + kMaxRowBlocks - 1) / kMaxRowBlocks));
   {
     ProfileScope ps("minhash_rows_kernel", stream);
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K, TAIL>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
   }
   dim3 grid2(4096, static_cast<unsigned>(chunks));
   {
     ProfileScope ps("minhash_extra_kernel", stream);
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_extra_kernel<T, K>), grid2, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets,
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_extra_kernel<T, K, TAIL>), grid2, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets,
                        extra_prefix, child);
   }
+}
+
+// How the parameters are shared out: chunks of K sets of 64 (every chunk hashes the windows again, and a lane without
+// a parameter still folds), or, for 65 to 288 parameters of which at most 32 lie beyond the last full set, one chunk of
+// K full sets and a tail that costs the fold the share `lanes of a tail set / 64` of a set.  Costs in 64ths of a set.
+struct Sharing {
+  int k;
+  bool tail;
+};
+inline Sharing sharing_for(int32_t P)
+{
+  Sharing best{1, false};
+  int64_t best_cost = std::numeric_limits<int64_t>::max();
+  for (int k = 1; k <= 5; ++k) {  // the larger K (fewer hashing passes) on a tie
+    int64_t const cost = static_cast<int64_t>((P + k * kWave - 1) / (k * kWave)) * k * kWave;
+    if (cost <= best_cost) { best_cost = cost; best = Sharing{k, false}; }
+  }
+  int const full = P / kWave, rest = P % kWave;
+  if (full >= 1 && full <= 4 && rest >= 1 && rest <= 32) {
+    int64_t const cost = static_cast<int64_t>(full) * kWave + packing_for(rest).ppad;
+    if (cost < best_cost) best = Sharing{full, true};
+  }
+  return best;
 }
 
 // The launches of one minhash call: the row offsets of the result, the number of extra workgroup-spans of every
@@ -532,20 +615,17 @@ void run_minhash(const ColView& v, T seed, const T* a, const T* b, int32_t P, in
   device_exclusive_scan(ExtraParts{v}, static_cast<int64_t>(rows), extra_prefix, scan_tmp, stream);
 
   if (child_size > 0) {
-    // every chunk of 64 K parameters hashes the windows again, and a lane without a parameter still folds:
-    // the K that leaves the fewest idle parameter slots, the larger K (fewer hashing passes) on a tie
-    int best_k = 1;
-    int64_t best_slots = std::numeric_limits<int64_t>::max();
-    for (int k = 1; k <= 5; ++k) {
-      int64_t const slots = static_cast<int64_t>((P + k * kWave - 1) / (k * kWave)) * k;
-      if (slots <= best_slots) { best_slots = slots; best_k = k; }
-    }
-    switch (best_k) {
-      case 5: launch_kernels<T, 5>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
-      case 4: launch_kernels<T, 4>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
-      case 3: launch_kernels<T, 3>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
-      case 2: launch_kernels<T, 2>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
-      default: launch_kernels<T, 1>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+    Sharing const sh = sharing_for(P);
+    switch (sh.k * 2 + (sh.tail ? 1 : 0)) {
+      case 10: launch_kernels<T, 5, false>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 9: launch_kernels<T, 4, true>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 8: launch_kernels<T, 4, false>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 7: launch_kernels<T, 3, true>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 6: launch_kernels<T, 3, false>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 5: launch_kernels<T, 2, true>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 4: launch_kernels<T, 2, false>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      case 3: launch_kernels<T, 1, true>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
+      default: launch_kernels<T, 1, false>(v, seed, a, b, P, width, offsets, extra_prefix, child, stream); break;
     }
   }
 }

@@ -118,6 +118,24 @@ def test_minhash_long_rows_cross_workgroups(nv, orc):
     assert_same(nv.minhash64(col, 7, a64, b64, 5).to_host(), orc.minhash64(host, 7, a64, b64, 5, nthreads=8), "minhash64 long")
 
 
+@pytest.mark.parametrize("P", [65, 68, 72, 80, 96, 129, 150, 200, 224, 260, 273, 288])
+def test_minhash_parameters_beyond_the_last_full_set_of_64(nv, orc, P):
+    """65 to 288 parameters of which at most 32 lie beyond the last full set of 64: those share the lanes of a wavefront in
+    sets (4, 8, 16 or 32 lanes to a set) beside the full sets.  Short rows (a wavefront each), rows shared by a workgroup
+    and rows of several spans (the extra workgroups, merged with atomic minima), empty and null rows."""
+    rng = np.random.default_rng(3000 + P)
+    rows = random_rows(rng, 40, 900, utf8=True) + ["a", "", None, "abcdefg " * 700, "".join(rng.choice(list("abcdefghijk "), 50000)),
+                                                   "é漢x " * 9000, "q" * 16384, "r" * 16385, "ab"]
+    host = strings(rows, np.int64)
+    col = dev(nv, host)
+    a32 = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+    b32 = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+    assert_same(nv.minhash(col, 11, a32, b32, 4).to_host(), orc.minhash(host, 11, a32, b32, 4, nthreads=8), f"minhash P={P}")
+    a64 = rng.integers(1, 2**64, P, dtype=np.uint64)
+    b64 = rng.integers(0, 2**64, P, dtype=np.uint64)
+    assert_same(nv.minhash64(col, 12, a64, b64, 6).to_host(), orc.minhash64(host, 12, a64, b64, 6, nthreads=8), f"minhash64 P={P}")
+
+
 def test_minhash_few_parameters_share_the_lanes_of_a_wavefront(nv, orc):
     """With at most 32 parameters the lanes work in sets that each fold a part of the hashes; long rows (every wavefront
     of a workgroup, the extra workgroups) and rows of fewer windows than sets must still give the minimum over all."""
