@@ -153,6 +153,21 @@ class ExtensionMissing(RuntimeError):
     pass
 
 
+def _share_the_hip_runtime_of_torch():
+    """A process must hold ONE HIP runtime: of two, the one that initialises second finds no device.  torch's wheels
+    bring their own libamdhip64 and load it when torch first touches the GPU; the library names its runtime by soname
+    (libamdhip64.so.7) and would take the system's if none is loaded yet.  The device buffers of this host side are
+    torch's, so torch's runtime is loaded first, and the library's dependency then resolves to it.  (A caller without
+    torch, like tests/cpp/nvtext_api_test.cpp, has the system's runtime alone.)"""
+    try:
+        import torch
+    except ImportError:
+        return
+    bundled = os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so")
+    if os.path.exists(bundled):
+        C.CDLL(bundled, mode=C.RTLD_GLOBAL)
+
+
 def load():
     """Loads the HIP library.  There is no fallback: without it the package cannot compute."""
     global _lib
@@ -161,6 +176,7 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise ExtensionMissing(
             f"{LIB_PATH} is missing: build it with `make -C cudf_amd/csrc` (or __graft_entry__.build())")
+    _share_the_hip_runtime_of_torch()
     L = C.CDLL(LIB_PATH)
     L.nvtext_amd_version.restype = C.c_int32
     L.nvtext_amd_version.argtypes = []

@@ -20,6 +20,10 @@ constexpr int kWave = 64;
 // ------------------------------------------------------------------ status
 void set_last_error(const char* msg);
 nvtext_amd_status fail(nvtext_amd_status st, const char* msg);
+// hipGetLastError keeps the last error of the calling thread until somebody reads it, whoever made the failing call
+// (a device query of another library, long before): an entry point reads it away before its own launches, which it
+// checks with the same call, so that it reports no error but its own.
+inline void forget_earlier_errors() { (void)hipGetLastError(); }
 
 #define NVTEXT_HIP_TRY(expr)                                                          \
   do {                                                                                \
