@@ -80,3 +80,44 @@ def test_minhash_preallocated_refuses_more_rows_than_its_scratch_holds():
     nvtext.minhash_preallocated(col, 0, a, a, 4, offsets, child, None)
     torch.cuda.synchronize()
     assert int(offsets[rows - 1]) == rows - 1 and int(child.abs().sum()) == 0   # empty rows: zeros
+
+
+def test_minhash_preallocated_recorded_into_a_hip_graph_and_replayed():
+    """What the entry point is for: a caller under HIP graph capture.  The call is recorded once (after a call outside of
+    any capture, which looks the scratch array's address up) and replayed on new bytes in the same buffers, with eager work
+    and synchronisations of the program's own between the replays; every replay against nvtext_amd_minhash run eagerly."""
+    import torch
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    from cudf_amd import _capi, nvtext as nv
+    _capi.load()
+    rng = np.random.default_rng(99)
+    host = _column(rng, 20_000, 6, True)
+    P, width, seed = 129, 5, 7
+    a = torch.from_numpy(rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32).view(np.int32)).cuda()
+    b = torch.from_numpy(rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32).view(np.int32)).cuda()
+    col = nv.DeviceStringsColumn.from_host(host)
+    offsets = torch.full((host.size + 1,), -1, dtype=torch.int32, device="cuda")
+    child = torch.full(((host.size - host.null_count) * P,), -1, dtype=torch.int32, device="cuda")
+    mask = torch.zeros(((host.size + 31) // 32,), dtype=torch.int32, device="cuda")
+    nv.minhash_preallocated(col, seed, a, b, width, offsets, child, mask)   # outside of capture: the address lookup
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=side):
+        nv.minhash_preallocated(col, seed, a, b, width, offsets, child, mask)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        # new bytes in the same buffer (the rows keep their lengths); the results cleared, so that a replay that does nothing shows
+        fresh = rng.integers(97, 123, host.chars.size, dtype=np.uint8)
+        fresh[rng.random(fresh.size) < 0.15] = 32
+        col.chars.copy_(torch.from_numpy(fresh).cuda())
+        child.fill_(-1)
+        offsets.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        exp = nv.minhash(col, seed, a, b, width).to_host()   # eager, same device bytes
+        assert np.array_equal(offsets.cpu().numpy(), exp.offsets), replay
+        assert np.array_equal(child.cpu().numpy().view(np.uint32), exp.child), replay
+        assert (torch.rand(1000, device="cuda").sum() > 0).item()   # eager work of the program's own between replays
