@@ -10,9 +10,13 @@
 //   * it then switches to lanes <-> parameters: every lane keeps K (a, b) pairs and
 //     K running minima in registers and streams the tile's hashes through LDS
 //     broadcast reads, so the inner loop is v_mad_u64_u32 + v_min only;
-//   * the 4 wavefronts of a workgroup split the first 16 KiB of a row and combine in
-//     LDS (plain store); the rest of a longer row is covered by extra workgroups that
-//     merge with atomic min, so no output pre-initialisation is needed.
+//   * a workgroup takes four rows: a row of up to 1 KiB belongs to one wavefront alone; the 4
+//     wavefronts split the first 16 KiB of a longer row and combine in LDS (plain store); the
+//     rest of a still longer row is covered by extra workgroups that merge with atomic min, so
+//     no output pre-initialisation is needed;
+//   * in a tile with characters of more than one byte the wavefront lists the characters first,
+//     so that a lane takes a character and reads its window's length instead of walking to it;
+//     hashes that the wavefront has folded lately are dropped (a minimum does not mind).
 //
 // Null rows get no output slot (the reference drops them with purge_nonempty_nulls,
 // minhash.cu:626-628), empty rows are all zeros (minhash.cu:318).

@@ -9,11 +9,14 @@
 //   * one open-addressing table of 2-slot buckets (16-byte slots, load <= 0.5) holds both key
 //     spaces: whole entries (kind 0) and "##" entries without their prefix (kind 1).  Keys of
 //     up to 8 bytes sit inside the slot, so a probe is one 32-byte read and the key's two dwords
-//     are also what gets hashed; the table for a 30k-entry vocabulary is 2 MiB and stays in L2.
+//     are also what gets hashed; the table for a 30k-entry vocabulary is 1 MiB and stays in L2.
 //     A hashed length filter (which key lengths exist for a given first three bytes) lets the
-//     longest-match search skip the lengths that cannot match.
+//     longest-match search skip the lengths that cannot match.  The tables are built by kernels: every key bids
+//     for its home bucket with its number in the vocabulary, so the keys that come first get the home slots.
+//   * a sample of the column (512 windows, each word looked up as the word pass will) sizes the word slots and the
+//     queue of the first attempt; what still overflows repeats the passes once with sizes that cannot fail.
 //   * the column's bytes are cut into tiles of 2048 bytes from the 16-byte aligned address below its first byte,
-//     without regard to rows; 16 tiles form a range, and every pass hands out ranges to wavefronts.
+//     without regard to rows; up to 8 tiles form a range, and every pass hands out ranges to wavefronts.
 //   * word pass: a wavefront takes a range and walks its tiles: bytes staged in LDS (the next tile's loads in
 //     flight), row starts marked as extra separators, spaces found with four SWAR operations per dword (16 bytes per
 //     lane), word starts and ends paired through scans, the words past a row's limit dropped; then lanes <->
