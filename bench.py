@@ -27,25 +27,25 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 3cd89cc)"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 52a62a4)"
 MEASURED_TRAFFIC_C2 = {
-    "range_first_row_kernel": (15970280, 248800),
-    "wordpiece_word_kernel": (1742732617, 1556524656),
-    "wordpiece_oov_kernel": (845292281, 863693078),
-    "wordpiece_emit_kernel": (1393674275, 905110660),
+    "range_first_row_kernel": (15971267, 248800),
+    "wordpiece_word_kernel": (1742902922, 1556470962),
+    "wordpiece_oov_kernel": (845578069, 863071956),
+    "wordpiece_emit_kernel": (1393668380, 905192283),
 }
 # (the fetch counter prices a read that misses L2 at a whole 128-byte line whatever was asked for, and counts the misses
 # that the Infinity Cache serves: most of what the tokenizer fetches on C5 is lines of its 8 MB table)
 MEASURED_TRAFFIC_C5_TOKENIZE = {
-    "range_first_row_kernel": (119805271, 995168),
-    "wordpiece_word_kernel": (24307766072, 5160815061),
-    "wordpiece_oov_kernel": (31977698657, 2111174960),
-    "wordpiece_emit_kernel": (4729699524, 3361207332),
+    "range_first_row_kernel": (120135925, 995168),
+    "wordpiece_word_kernel": (24305761872, 5162475317),
+    "wordpiece_oov_kernel": (31977285964, 2110981083),
+    "wordpiece_emit_kernel": (4729721575, 3361248849),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (4575181347, 63532924),
-    "normalize_tile_rows_kernel": (73449633, 7941632),
-    "normalize_write_kernel": (5469619320, 4672656216),
+    "normalize_count_kernel": (4575178161, 63532924),
+    "normalize_tile_rows_kernel": (73449833, 7941632),
+    "normalize_write_kernel": (5469603014, 4672576593),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
@@ -54,7 +54,7 @@ MEASURED_TRAFFIC_C5_NORMALIZE = {
 # mod 2^64, a shift, a mask and one more v_mad_u64_u32 for the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two
 # products (8.5).  Every window of the input counts as one, also those whose hash the wavefront met lately and does not
 # fold again (windows of a row repeat, most in long rows: that is how C4 comes so near the floor).
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 3cd89cc)"
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 52a62a4)"
 MINHASH_VALU = {
     "C3": {"floor": 1.5, "measured": 1.79, "issue": 0.95},
     "C4": {"floor": 8.5, "measured": 8.92, "issue": 0.85},
