@@ -20,10 +20,19 @@ constexpr int kWave = 64;
 // ------------------------------------------------------------------ status
 void set_last_error(const char* msg);
 nvtext_amd_status fail(nvtext_amd_status st, const char* msg);
-// hipGetLastError keeps the last error of the calling thread until somebody reads it, whoever made the failing call
-// (a device query of another library, long before): an entry point reads it away before its own launches, which it
-// checks with the same call, so that it reports no error but its own.
-inline void forget_earlier_errors() { (void)hipGetLastError(); }
+// What every entry point does first.  (1) hipGetLastError keeps the last error of the calling thread until somebody
+// reads it, whoever made the failing call (a device query of another library, long before): it is read away before the
+// entry point's own launches, which are checked with the same call, so that it reports no error but its own.  (2) A
+// named range around the call, as CUDF_FUNC_RANGE() puts an NVTX range around the reference's entry points
+// (cpp/include/cudf/detail/nvtx/ranges.hpp; wordpiece_tokenize.cu:291,897, minhash.cu:699,724): rocprofv3
+// --marker-trace shows it.  The marker library (rocTX) is looked up at first use and left alone when it is absent;
+// the library does not link it.
+struct EntryScope {
+  explicit EntryScope(const char* name);
+  ~EntryScope();
+  EntryScope(const EntryScope&)            = delete;
+  EntryScope& operator=(const EntryScope&) = delete;
+};
 
 #define NVTEXT_HIP_TRY(expr)                                                          \
   do {                                                                                \

@@ -4,7 +4,10 @@
 #include "common.cuh"
 
 #include <cstring>
+#include <mutex>
 #include <vector>
+
+#include <dlfcn.h>
 
 namespace nvtext_amd {
 
@@ -42,6 +45,41 @@ void profile_mark_end(hipStream_t stream)
   // only the record that the matching begin made: a begin that failed leaves nothing to close
   if (g_profile_open) (void)hipEventRecord(g_profile.back().end, stream);
   g_profile_open = false;
+}
+
+namespace {
+using RangePushFn = int (*)(const char*);
+using RangePopFn  = int (*)();
+RangePushFn g_range_push = nullptr;
+RangePopFn g_range_pop   = nullptr;
+std::once_flag g_range_once;
+void find_marker_library()
+{
+  // rocprofv3 listens to the first; the second is the older tracer's
+  for (const char* lib : {"librocprofiler-sdk-roctx.so.1", "libroctx64.so.4"}) {
+    void* const h = dlopen(lib, RTLD_NOW | RTLD_LOCAL);
+    if (!h) continue;
+    auto const push = reinterpret_cast<RangePushFn>(dlsym(h, "roctxRangePushA"));
+    auto const pop  = reinterpret_cast<RangePopFn>(dlsym(h, "roctxRangePop"));
+    if (push && pop) {
+      g_range_push = push;
+      g_range_pop  = pop;
+      return;
+    }
+  }
+}
+}  // namespace
+
+EntryScope::EntryScope(const char* name)
+{
+  (void)hipGetLastError();
+  std::call_once(g_range_once, find_marker_library);
+  if (g_range_push) (void)g_range_push(name);
+}
+
+EntryScope::~EntryScope()
+{
+  if (g_range_pop) (void)g_range_pop();
 }
 
 void set_last_error(const char* msg) { g_last_error = msg ? msg : ""; }

@@ -334,7 +334,7 @@ nvtext_amd_status nvtext_amd_jaccard_index(const nvtext_amd_strings_column* inpu
                                            void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_fixed_column* out)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_jaccard_index");
   if (!input1 || !input2 || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nvtext_amd_fixed_column{};
   // cpp/src/text/jaccard.cu:441-446, same order and messages

@@ -638,7 +638,7 @@ template <typename T>
 nvtext_amd_status minhash_impl(const nvtext_amd_strings_column* input, T seed, const T* a, const T* b, int64_t a_count, int64_t b_count,
                                int32_t width, void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_list_column* out, int32_t type_id)
 {
-  forget_earlier_errors();
+  EntryScope const entry(sizeof(T) == 4 ? "nvtext_amd_minhash" : "nvtext_amd_minhash64");
   if (!input || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nvtext_amd_list_column{};
   // cpp/src/text/minhash.cu:435-446, same order and messages
@@ -851,7 +851,7 @@ nvtext_amd_status minhash_ngrams_impl(const nvtext_amd_list_strings_column* inpu
                                       int64_t a_count, int64_t b_count, void* stream_, const nvtext_amd_allocator* mr_,
                                       nvtext_amd_list_column* out, int32_t type_id)
 {
-  forget_earlier_errors();
+  EntryScope const entry(sizeof(T) == 4 ? "nvtext_amd_minhash_ngrams" : "nvtext_amd_minhash64_ngrams");
   if (!input || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nvtext_amd_list_column{};
   // cpp/src/text/minhash.cu:524-536, same order and messages
@@ -961,7 +961,7 @@ nvtext_amd_status nvtext_amd_minhash_preallocated(const nvtext_amd_strings_colum
                                                   uint32_t* out_child, int64_t out_child_capacity, uint32_t* out_null_mask)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_minhash_preallocated");
   if (!input || !out_offsets) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   if (width < 2) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameter width should be an integer value of 2 or greater");
   if (a_count <= 0) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "Parameters A and B cannot be empty");

@@ -809,7 +809,7 @@ nvtext_amd_status nvtext_amd_character_normalizer_create(int32_t do_lower_case, 
                                                          const nvtext_amd_allocator* mr, nvtext_amd_character_normalizer** out)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_character_normalizer_create");
   if (!out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out               = nullptr;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -933,7 +933,7 @@ nvtext_amd_status nvtext_amd_normalize_characters(const nvtext_amd_strings_colum
                                                   void* stream_, const nvtext_amd_allocator* mr_, nvtext_amd_strings_result* out)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_normalize_characters");
   if (!input || !normalizer || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nvtext_amd_strings_result{};
   if (input->size < 0 || input->null_count < 0 || input->null_count > input->size) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "invalid column sizes");

@@ -2085,7 +2085,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
                                                          nvtext_amd_wordpiece_vocabulary** out)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_wordpiece_vocabulary_create");
   if (!vocabulary || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nullptr;
   // cpp/src/text/wordpiece_tokenize.cu:217-218
@@ -2203,7 +2203,7 @@ nvtext_amd_status nvtext_amd_wordpiece_tokenize(const nvtext_amd_strings_column*
                                                 nvtext_amd_list_column* out)
 {
   using namespace nvtext_amd;
-  forget_earlier_errors();
+  EntryScope const entry("nvtext_amd_wordpiece_tokenize");
   if (!input || !vocabulary || !out) return fail(NVTEXT_AMD_INVALID_ARGUMENT, "null argument");
   *out = nvtext_amd_list_column{};
   // cpp/src/text/wordpiece_tokenize.cu:845-846
