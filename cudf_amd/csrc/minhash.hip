@@ -378,12 +378,25 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
   }
 }
 
-// One workgroup per (four consecutive rows, parameter chunk).  A row of up to kSoloBytes is done by one wavefront alone
-// (wavefront w takes row w of the four: nothing to combine, the minima go from the registers to the result); a longer
-// row is shared by the four wavefronts, which split its first kSpan bytes and combine through LDS, one such row after the
-// other.  The groups lie along x and, beyond kMaxRowBlocks of them, along z.
-constexpr int64_t kSoloBytes = 1024;
-constexpr int kGroupRows      = kWaves;
+// One workgroup per (group of consecutive rows, parameter chunk).  A row of up to kSoloBytes is done by one wavefront
+// alone (wavefront w takes the rows w, w + 4, .. of the group, `solo_per_wave` of them: nothing to combine, the minima go
+// from the registers to the result); a longer row is shared by the four wavefronts, which split its first kSpan bytes
+// and combine through LDS, one such row after the other.  The groups lie along x and, beyond kMaxRowBlocks of them,
+// along z.
+// Rows differ in length, and a workgroup lasts as long as its slowest wavefront: with one short row per wavefront the
+// others waited for the longest of four (8 M rows of about 500 bytes: 88 ms; four rows per wavefront 80 ms, sixteen
+// 77 ms).  More rows per workgroup mean fewer workgroups, and a column of few rows needs them all to fill the device
+// and to even out its end: the host asks for as many rows per wavefront (a power of two, at most kMaxSoloPerWave) as
+// leave at least kMinRowGroups groups.
+constexpr int64_t kSoloBytes      = 1024;
+constexpr int kMaxSoloPerWave     = 16;
+constexpr int32_t kMinRowGroups   = 16384;  // sixteen times the workgroups that 256 CUs hold at four apiece
+inline int solo_rows_per_wave(int32_t rows)
+{
+  int spw = 1;
+  while (spw < kMaxSoloPerWave && rows / (2 * spw * kWaves) >= kMinRowGroups) spw *= 2;
+  return spw;
+}
 
 // The tail of a launch with TAIL: the P - 64 K parameters (1..32) beyond the K full sets of the one chunk.
 template <typename T, int K, bool TAIL>
@@ -412,14 +425,16 @@ struct TailOf<T, K, true> {
 
 template <typename T, int K, bool TAIL>
 __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
-                                                                int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out)
+                                                                int32_t width, const int32_t* __restrict__ out_offsets, T* __restrict__ out,
+                                                                int solo_per_wave)
 {
   using TailT = TailOf<T, K, TAIL>;
   constexpr int kSets = K + (TAIL ? 1 : 0);
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][kSets * kWave];
 
-  int64_t const r0 = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * kGroupRows;
+  int const group_rows = solo_per_wave * kWaves;
+  int64_t const r0     = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * group_rows;
   if (r0 >= col.size) return;
   int const lane           = lane_id();
   int const wave           = threadIdx.x / kWave;
@@ -431,14 +446,14 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
   typename TailT::type tail;
   TailT::load(tail, pa, pb, P, lane);
 
-  int const rows_here = static_cast<int>(min(static_cast<int64_t>(kGroupRows), col.size - r0));
+  int const rows_here = static_cast<int>(min(static_cast<int64_t>(group_rows), col.size - r0));
   int const wave_s    = __builtin_amdgcn_readfirstlane(wave);  // (the same in every lane: what depends on it stays scalar)
 
-  // step -1: the short row of this wavefront (row `wave` of the four); steps 0..3: this wavefront's part of the rows
-  // that are too long for that, one after the other
-  for (int step = -1; step < rows_here; ++step) {
+  // steps below 0: the short rows of this wavefront (rows wave, wave + 4, .. of the group); steps from 0: this
+  // wavefront's part of the rows that are too long for that, one after the other
+  for (int step = -solo_per_wave; step < rows_here; ++step) {
     bool const solo = step < 0;
-    int const i     = solo ? wave_s : step;
+    int const i     = solo ? (step + solo_per_wave) * kWaves + wave_s : step;
     if (i >= rows_here || !col.valid(r0 + i)) continue;
     int64_t const o = col.off(r0 + i);
     int64_t const n = col.off(r0 + i + 1) - o;
@@ -566,12 +581,14 @@ void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P,
                     const uint32_t* extra_prefix, T* child, hipStream_t stream)
 {
   int32_t const chunks = TAIL ? 1 : (P + K * kWave - 1) / (K * kWave);
-  int32_t const groups = (v.size + kGroupRows - 1) / kGroupRows;  // four rows to a workgroup
+  int const solo_per_wave = solo_rows_per_wave(v.size);
+  int32_t const groups    = (v.size + solo_per_wave * kWaves - 1) / (solo_per_wave * kWaves);
   dim3 grid(static_cast<unsigned>(std::min(groups, kMaxRowBlocks)), static_cast<unsigned>(chunks),
             static_cast<unsigned>((groups + kMaxRowBlocks - 1) / kMaxRowBlocks));
   {
     ProfileScope ps("minhash_rows_kernel", stream);
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K, TAIL>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_rows_kernel<T, K, TAIL>), grid, dim3(kThreads), 0, stream, v, seed, a, b, P, width, offsets, child,
+                       solo_per_wave);
   }
   dim3 grid2(4096, static_cast<unsigned>(chunks));
   {

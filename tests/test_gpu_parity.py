@@ -136,6 +136,38 @@ def test_minhash_parameters_beyond_the_last_full_set_of_64(nv, orc, P):
     assert_same(nv.minhash64(col, 12, a64, b64, 6).to_host(), orc.minhash64(host, 12, a64, b64, 6, nthreads=8), f"minhash64 P={P}")
 
 
+@pytest.mark.parametrize("rows", [140_000, 300_000, 600_000, 1_100_000])
+def test_minhash_many_rows_several_short_rows_to_a_wavefront(nv, orc, rows):
+    """From 131,072 rows on a wavefront takes 2, 4, 8 and, from 1,048,576 rows on, 16 short rows of its workgroup's group
+    instead of one.  Mostly rows of a few bytes, nulls and empty rows among them, rows of the group's last places, rows
+    just below and above the length that a wavefront does alone, and rows of several workgroup spans."""
+    from cudf_amd.arrow_host import HostStringsColumn, pack_validity
+    rng = np.random.default_rng(rows)
+    lengths = rng.integers(0, 24, rows)
+    lengths[rng.integers(0, rows, rows // 200)] = rng.integers(1000, 1050, rows // 200)   # either side of 1024 bytes
+    lengths[rng.integers(0, rows, 40)] = rng.integers(5000, 70000, 40)                     # shared by a workgroup; extra workgroups
+    lengths[-1] = 1500
+    lengths[-2] = 3
+    offsets = np.zeros(rows + 1, np.int64)
+    np.cumsum(lengths, out=offsets[1:])
+    chars = rng.integers(97, 105, int(offsets[-1]), dtype=np.uint8)
+    chars[rng.random(chars.size) < 0.2] = 32
+    valid = rng.random(rows) > 0.05
+    host = HostStringsColumn(chars, offsets.astype(np.int32), pack_validity(valid), rows, 0, int((~valid).sum()))
+    col = dev(nv, host)
+    for P in (3, 70):
+        a32 = rng.integers(1, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        b32 = rng.integers(0, 2**32, P, dtype=np.uint64).astype(np.uint32)
+        assert_same(nv.minhash(col, 5, a32, b32, 4).to_host(), orc.minhash(host, 5, a32, b32, 4, nthreads=8), f"minhash rows={rows} P={P}")
+    a64 = rng.integers(1, 2**64, 5, dtype=np.uint64)
+    b64 = rng.integers(0, 2**64, 5, dtype=np.uint64)
+    assert_same(nv.minhash64(col, 6, a64, b64, 7).to_host(), orc.minhash64(host, 6, a64, b64, 7, nthreads=8), f"minhash64 rows={rows}")
+    # a slice whose first row is not the first of a group
+    lo, hi = 3, rows - 5
+    hs = host.slice(lo, hi)
+    assert_same(nv.minhash(col.slice(lo, hi, hs.null_count), 5, a32, b32, 4).to_host(), orc.minhash(hs, 5, a32, b32, 4, nthreads=8), f"sliced rows={rows}")
+
+
 def test_minhash_few_parameters_share_the_lanes_of_a_wavefront(nv, orc):
     """With at most 32 parameters the lanes work in sets that each fold a part of the hashes; long rows (every wavefront
     of a workgroup, the extra workgroups) and rows of fewer windows than sets must still give the minimum over all."""
