@@ -388,7 +388,8 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
 // 77 ms).  More rows per workgroup mean fewer workgroups, and a column of few rows needs them all to fill the device
 // and to even out its end: the host asks for as many rows per wavefront (a power of two, at most kMaxSoloPerWave) as
 // leave at least kMinRowGroups groups.
-constexpr int64_t kSoloBytes      = 1024;
+constexpr int64_t kSoloBytes      = 1024;   // with one row to a wavefront
+constexpr int64_t kSoloBytesMany  = 4096;   // with several: their sum evens out, and a row done alone needs no barrier (2 M rows of 2 KB: 2 % faster than 1024)
 constexpr int kMaxSoloPerWave     = 16;
 constexpr int32_t kMinRowGroups   = 16384;  // sixteen times the workgroups that 256 CUs hold at four apiece
 inline int solo_rows_per_wave(int32_t rows)
@@ -433,7 +434,8 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][kSets * kWave];
 
-  int const group_rows = solo_per_wave * kWaves;
+  int const group_rows     = solo_per_wave * kWaves;
+  int64_t const solo_bytes = solo_per_wave > 1 ? kSoloBytesMany : kSoloBytes;
   int64_t const r0     = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * group_rows;
   if (r0 >= col.size) return;
   int const lane           = lane_id();
@@ -457,7 +459,7 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
     if (i >= rows_here || !col.valid(r0 + i)) continue;
     int64_t const o = col.off(r0 + i);
     int64_t const n = col.off(r0 + i + 1) - o;
-    if (solo != (n <= kSoloBytes)) continue;
+    if (solo != (n <= solo_bytes)) continue;
 #pragma unroll
     for (int k = 0; k < K; ++k) m[k] = std::numeric_limits<T>::max();
     TailT::reset(tail);

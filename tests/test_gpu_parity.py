@@ -140,11 +140,13 @@ def test_minhash_parameters_beyond_the_last_full_set_of_64(nv, orc, P):
 def test_minhash_many_rows_several_short_rows_to_a_wavefront(nv, orc, rows):
     """From 131,072 rows on a wavefront takes 2, 4, 8 and, from 1,048,576 rows on, 16 short rows of its workgroup's group
     instead of one.  Mostly rows of a few bytes, nulls and empty rows among them, rows of the group's last places, rows
-    just below and above the length that a wavefront does alone, and rows of several workgroup spans."""
+    just below and above the lengths that a wavefront does alone (1024 bytes, 4096 with several rows to a wavefront), and
+    rows of several workgroup spans."""
     from cudf_amd.arrow_host import HostStringsColumn, pack_validity
     rng = np.random.default_rng(rows)
     lengths = rng.integers(0, 24, rows)
     lengths[rng.integers(0, rows, rows // 200)] = rng.integers(1000, 1050, rows // 200)   # either side of 1024 bytes
+    lengths[rng.integers(0, rows, 60)] = rng.integers(4080, 4112, 60)                      # and of 4096 (the limit with several rows to a wavefront)
     lengths[rng.integers(0, rows, 40)] = rng.integers(5000, 70000, 40)                     # shared by a workgroup; extra workgroups
     lengths[-1] = 1500
     lengths[-2] = 3
