@@ -763,11 +763,18 @@ struct AlignedSrc {
 constexpr uint32_t kNgramStageBytes = 4096;                             // longest stretch of chars hashed out of LDS
 constexpr uint32_t kNgramStageWords = (kNgramStageBytes + 4 + 28) / 4;  // + misalignment, + over-read of the hash tail
 
-// One workgroup per (row, parameter chunk); its wavefronts take the positions of the row 64 at a time.
+// One workgroup per (group of consecutive rows, parameter chunk), as in minhash_rows_kernel: a row of up to
+// kNgramSoloPositions positions is done by one wavefront alone, 64 positions a trip (wavefront w takes the rows w, w + 4, .. of the group,
+// `solo_per_wave` of them), and its minima go from the registers to the result; a row of more positions is shared by the
+// four wavefronts, which take its positions 64 at a time in turn and combine through LDS, one such row after the other.
+// A column of fewer than 131,072 rows keeps one row to a workgroup, every row shared by the four wavefronts
+// (solo_per_wave 0): it needs its workgroups to fill the device and to even out its end (20,000 rows of 3,000 elements:
+// four rows to a workgroup were 8 % slower).
+constexpr int64_t kNgramSoloPositions = 2048;
 template <typename T, int K>
 __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, int32_t ngrams, T seed, const T* __restrict__ pa,
                                                                   const T* __restrict__ pb, int32_t P, const int32_t* __restrict__ out_offsets,
-                                                                  T* __restrict__ out)
+                                                                  T* __restrict__ out, int solo_per_wave)
 {
   using H = HashTraits<T>;
   __shared__ alignas(16) T hashes[kWaves][2 * kWave];  // 64 hashes a trip, padded to the stride of the fold (at most 64 more)
@@ -777,74 +784,94 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
   constexpr bool kStageRuns = sizeof(T) == 4;
   __shared__ uint32_t run_bytes[kWaves][kStageRuns ? kNgramStageWords : 1];
 
-  int64_t const r = static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x;  // rows along x, then z
-  if (r >= in.size || !in.valid(r)) return;
-  int32_t const chunk_base = blockIdx.y * (K * kWave);
-  int64_t const first      = in.off(r);
-  int64_t const n          = in.off(r + 1) - first;
-  T* dst                   = out + static_cast<int64_t>(out_offsets[r]) + chunk_base;
-  int32_t const in_chunk   = min(K * kWave, P - chunk_base);
-  if (n == 0) {  // minhash.cu:318
-    for (int j = threadIdx.x; j < in_chunk; j += kThreads) dst[j] = T{0};
-    return;
-  }
-  int const lane = lane_id();
-  int const wave = threadIdx.x / kWave;
+  int const group_rows = solo_per_wave > 0 ? solo_per_wave * kWaves : 1;
+  int64_t const r0     = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * group_rows;  // groups along x, then z
+  if (r0 >= in.size) return;
+  int64_t const solo_positions = solo_per_wave > 0 ? kNgramSoloPositions : -1;
+  int32_t const chunk_base     = blockIdx.y * (K * kWave);
+  int32_t const in_chunk       = min(K * kWave, P - chunk_base);
+  int const lane               = lane_id();
+  int const wave               = threadIdx.x / kWave;
+  int const wave_s             = __builtin_amdgcn_readfirstlane(wave);
   T a[K], b[K], m[K];
   load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
 
-  // minhash.cu:311-314 with width = ngrams: the positions that the permutation looks at
-  int64_t const positions = max(static_cast<int64_t>(1), n - ngrams + 1);
-  for (int64_t base = static_cast<int64_t>(wave) * kWave; base < positions; base += kWaves * kWave) {
-    int64_t const idx = base + lane;
-    bool valid        = false;
-    T hv              = 0;
-    int64_t bo = 0, eo = 0;
-    if (idx < positions && in.child.valid(first + idx)) {  // 213-216: a null element starts no run
-      // 218-222: the run ends at element idx + ngrams, clamped to the row; a clamped run counts only at idx 0
-      int64_t const next = min(idx + ngrams, n - 1);
-      if (idx == 0 || next - idx >= ngrams) {
-        // 224-229: the bytes from the start of element idx to the end of element next
-        bo    = in.child.off(first + idx);
-        eo    = in.child.off(first + next + 1);
-        valid = true;
+  int const rows_here = static_cast<int>(min(static_cast<int64_t>(group_rows), in.size - r0));
+  for (int step = -solo_per_wave; step < rows_here; ++step) {
+    bool const solo = step < 0;
+    int const i     = solo ? (step + solo_per_wave) * kWaves + wave_s : step;
+    if (i >= rows_here || !in.valid(r0 + i)) continue;
+    int64_t const first = in.off(r0 + i);
+    int64_t const n     = in.off(r0 + i + 1) - first;
+    // minhash.cu:311-314 with width = ngrams: the positions that the permutation looks at
+    int64_t const positions = max(static_cast<int64_t>(1), n - ngrams + 1);
+    if (solo != (positions <= solo_positions)) continue;
+#pragma unroll
+    for (int k = 0; k < K; ++k) m[k] = std::numeric_limits<T>::max();
+    if (n > 0) {
+      int64_t const trip = solo ? kWave : kWaves * kWave;
+      for (int64_t base = solo ? 0 : static_cast<int64_t>(wave) * kWave; base < positions; base += trip) {
+        int64_t const idx = base + lane;
+        bool valid        = false;
+        T hv              = 0;
+        int64_t bo = 0, eo = 0;
+        if (idx < positions && in.child.valid(first + idx)) {  // 213-216: a null element starts no run
+          // 218-222: the run ends at element idx + ngrams, clamped to the row; a clamped run counts only at idx 0
+          int64_t const next = min(idx + ngrams, n - 1);
+          if (idx == 0 || next - idx >= ngrams) {
+            // 224-229: the bytes from the start of element idx to the end of element next
+            bo    = in.child.off(first + idx);
+            eo    = in.child.off(first + next + 1);
+            valid = true;
+          }
+        }
+        // The runs of these 64 elements overlap and lie side by side in the chars: fetch that stretch once, with
+        // coalesced loads, and hash out of LDS (the hash walks a run dword by dword, each step a dependent read).
+        // A stretch too long for the buffer is hashed straight from memory.
+        int64_t const span_begin = kStageRuns ? in.child.off(first + base) : 0;
+        int64_t const span_end   = kStageRuns ? in.child.off(first + min(base + kWave + ngrams, n)) : 0;
+        if (kStageRuns && span_end - span_begin <= static_cast<int64_t>(kNgramStageBytes)) {
+          bool ascii;
+          uint32_t const mis = stage_bytes(in.child.chars, span_begin, static_cast<uint32_t>(span_end - span_begin), run_bytes[wave], lane, &ascii);
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          if (valid) {
+            WordSrc const src{run_bytes[wave], mis + static_cast<uint32_t>(bo - span_begin)};
+            hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        } else if (valid) {
+          AlignedSrc const src(in.child.chars + bo, static_cast<uint32_t>(eo - bo));
+          hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+        }
+        if (valid) hv = hv < 1 ? T{1} : hv;  // 237
+        uint64_t const vm = ballot64(valid);
+        if (valid) hashes[wave][lanes_below(vm)] = hv;
+        fold_hashes<T, K>(hashes[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
       }
     }
-    // The runs of these 64 elements overlap and lie side by side in the chars: fetch that stretch once, with
-    // coalesced loads, and hash out of LDS (the hash walks a run dword by dword, each step a dependent read).
-    // A stretch too long for the buffer is hashed straight from memory.
-    int64_t const span_begin = kStageRuns ? in.child.off(first + base) : 0;
-    int64_t const span_end   = kStageRuns ? in.child.off(first + min(base + kWave + ngrams, n)) : 0;
-    if (kStageRuns && span_end - span_begin <= static_cast<int64_t>(kNgramStageBytes)) {
-      bool ascii;
-      uint32_t const mis = stage_bytes(in.child.chars, span_begin, static_cast<uint32_t>(span_end - span_begin), run_bytes[wave], lane, &ascii);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      if (valid) {
-        WordSrc const src{run_bytes[wave], mis + static_cast<uint32_t>(bo - span_begin)};
-        hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+    T* const dst = out + static_cast<int64_t>(out_offsets[r0 + i]) + chunk_base;
+    if (solo) {
+      // an empty row is zeros (minhash.cu:318); a row whose every run was skipped keeps the all-ones start value
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        int32_t const j = lane + kWave * k;
+        if (j < in_chunk) dst[j] = n > 0 ? m[k] : T{0};
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    } else if (valid) {
-      AlignedSrc const src(in.child.chars + bo, static_cast<uint32_t>(eo - bo));
-      hv = H::hash(src, static_cast<uint32_t>(eo - bo), seed);
+    } else {
+      __syncthreads();  // (the row before has been read out of red)
+#pragma unroll
+      for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
+      __syncthreads();
+      for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
+        T v = red[0][j];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
+        dst[j] = n > 0 ? v : T{0};
+      }
     }
-    if (valid) hv = hv < 1 ? T{1} : hv;  // 237
-    uint64_t const vm = ballot64(valid);
-    if (valid) hashes[wave][lanes_below(vm)] = hv;
-    fold_hashes<T, K>(hashes[wave], static_cast<uint32_t>(__builtin_popcountll(vm)), a, b, m, lane);
-  }
-
-#pragma unroll
-  for (int k = 0; k < K; ++k) red[wave][k * kWave + lane] = m[k];
-  __syncthreads();
-  for (int j = threadIdx.x; j < in_chunk; j += kThreads) {
-    T v = red[0][j];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) v = min(v, red[w][j]);
-    dst[j] = v;
   }
 }
 
@@ -858,11 +885,15 @@ template <typename T, int K>
 void launch_ngrams(const ListView& v, int32_t ngrams, T seed, const T* a, const T* b, int32_t P, const int32_t* offsets, T* child,
                    hipStream_t stream)
 {
-  int32_t const chunks = (P + K * kWave - 1) / (K * kWave);
-  dim3 grid(static_cast<unsigned>(std::min(v.size, kMaxRowBlocks)), static_cast<unsigned>(chunks),
-            static_cast<unsigned>((v.size + kMaxRowBlocks - 1) / kMaxRowBlocks));
+  int32_t const chunks    = (P + K * kWave - 1) / (K * kWave);
+  int const solo_per_wave = v.size >= 131072 ? solo_rows_per_wave(v.size) : 0;
+  int32_t const group     = solo_per_wave > 0 ? solo_per_wave * kWaves : 1;
+  int32_t const groups    = (v.size + group - 1) / group;
+  dim3 grid(static_cast<unsigned>(std::min(groups, kMaxRowBlocks)), static_cast<unsigned>(chunks),
+            static_cast<unsigned>((groups + kMaxRowBlocks - 1) / kMaxRowBlocks));
   ProfileScope ps("minhash_ngrams_kernel", stream);
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_ngrams_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, ngrams, seed, a, b, P, offsets, child);
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(minhash_ngrams_kernel<T, K>), grid, dim3(kThreads), 0, stream, v, ngrams, seed, a, b, P, offsets, child,
+                     solo_per_wave);
 }
 
 template <typename T>

@@ -340,6 +340,41 @@ def test_minhash_ngrams_random_vs_oracle(nv, orc, P, ngrams):
                         orc.minhash_ngrams(hs, ngrams, 7, a, b), f"ngrams slice {lo}:{hi}")
 
 
+@pytest.mark.parametrize("rows", [150_000, 1_100_000])
+def test_minhash_ngrams_many_rows_several_short_rows_to_a_wavefront(nv, orc, rows):
+    """From 131,072 rows on a wavefront takes several short rows of its workgroup's group (16 from 1,048,576 rows on) and
+    does a row of up to 2048 positions alone.  Mostly rows of a few elements, empty and null rows and null elements among
+    them, rows either side of 2048 positions, a row of many more."""
+    from cudf_amd.arrow_host import HostListStringsColumn, HostStringsColumn, pack_validity
+    rng = np.random.default_rng(rows + 1)
+    sizes = rng.integers(0, 7, rows)
+    sizes[rng.integers(0, rows, 30)] = rng.integers(2040, 2060, 30)
+    sizes[rng.integers(0, rows, 200)] = rng.integers(60, 400, 200)
+    sizes[rows // 2] = 9000
+    sizes[-1] = 70
+    offsets = np.zeros(rows + 1, np.int32)
+    np.cumsum(sizes, out=offsets[1:])
+    count = int(offsets[-1])
+    lengths = rng.integers(0, 6, count)
+    eoff = np.zeros(count + 1, np.int32)
+    np.cumsum(lengths, out=eoff[1:])
+    chars = rng.integers(97, 103, int(eoff[-1]), dtype=np.uint8)
+    evalid = rng.random(count) > 0.03
+    elements = HostStringsColumn(chars, eoff, pack_validity(evalid), count, 0, int((~evalid).sum()))
+    valid = rng.random(rows) > 0.05
+    host = HostListStringsColumn(offsets, elements, pack_validity(valid), rows, 0, int((~valid).sum()))
+    d = ldev(nv, host)
+    a = rng.integers(1, 2**32, 5, dtype=np.uint64).astype(np.uint32)
+    b = rng.integers(0, 2**32, 5, dtype=np.uint64).astype(np.uint32)
+    assert_same(nv.minhash_ngrams(d, 3, 7, a, b).to_host(), orc.minhash_ngrams(host, 3, 7, a, b, nthreads=8), f"ngrams u32 rows={rows}")
+    a64 = rng.integers(1, 2**64, 70, dtype=np.uint64)
+    b64 = rng.integers(0, 2**64, 70, dtype=np.uint64)
+    assert_same(nv.minhash64_ngrams(d, 2, 9, a64, b64).to_host(), orc.minhash64_ngrams(host, 2, 9, a64, b64, nthreads=8), f"ngrams u64 rows={rows}")
+    lo, hi = 5, rows - 3
+    hs = host.slice(lo, hi)
+    assert_same(nv.minhash_ngrams(d.slice(lo, hi, hs.null_count), 3, 7, a, b).to_host(), orc.minhash_ngrams(hs, 3, 7, a, b, nthreads=8), f"sliced rows={rows}")
+
+
 def test_minhash_ngrams_wide_row_and_errors(nv, orc):
     rng = np.random.default_rng(5)
     words = ["".join(rng.choice(list("abcdef"), int(rng.integers(1, 9)))) for _ in range(300_000)]
