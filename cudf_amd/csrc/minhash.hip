@@ -501,8 +501,10 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
 
 // Extra parts of rows longer than kSpan: task t covers bytes [part*kSpan, (part+1)*kSpan) of its row.
 // extra_prefix[r] = number of extra parts in rows < r (rows+1 entries).
+// (uint32: held to the registers of six wavefronts per SIMD, which left to itself the compiler exceeds with four and
+// five sets of parameters: the reference's 260-parameter shapes 3 to 5 % faster; uint64 gains nothing from it.)
 template <typename T, int K, bool TAIL>
-__global__ void __launch_bounds__(kThreads) minhash_extra_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
+__global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 6 : 1) minhash_extra_kernel(ColView col, T seed, const T* __restrict__ pa, const T* __restrict__ pb, int32_t P,
                                                                  int32_t width, const int32_t* __restrict__ out_offsets,
                                                                  const uint32_t* __restrict__ extra_prefix, T* __restrict__ out)
 {
