@@ -578,7 +578,7 @@ __global__ void uniform_offsets_kernel(int32_t* out, int32_t rows, int32_t P)
   if (i <= rows) out[i] = static_cast<int32_t>(i * P);
 }
 
-constexpr int32_t kMaxRowBlocks = 1 << 20;
+constexpr int32_t kMaxRowBlocks = 1 << 15;  // groups along x (a launch of 4 M rows, 64 to a group, has two layers along z: the tests reach them)
 
 template <typename T, int K, bool TAIL>
 void launch_kernels(const ColView& v, T seed, const T* a, const T* b, int32_t P, int32_t width, const int32_t* offsets,

@@ -187,7 +187,7 @@ def test_minhash_few_parameters_share_the_lanes_of_a_wavefront(nv, orc):
 
 
 def test_minhash_more_rows_than_a_grid_has_workgroups(nv, orc):
-    """More rows than a launch has workgroups along x (2^20 of them, four rows each): the rest lie along z."""
+    """More rows than a launch has workgroups along x (2^15 groups of them, 64 rows each at this size): the rest lie along z."""
     rows = (1 << 22) + 12345
     rng = np.random.default_rng(17)
     lengths = rng.integers(0, 6, rows)
