@@ -378,8 +378,8 @@ __device__ __forceinline__ void load_params(const T* pa, const T* pb, int32_t P,
   }
 }
 
-// One workgroup per (group of consecutive rows, parameter chunk).  A row of up to kSoloBytes is done by one wavefront
-// alone (wavefront w takes the rows w, w + 4, .. of the group, `solo_per_wave` of them: nothing to combine, the minima go
+// One workgroup per (group of consecutive rows, parameter chunk).  A row of up to kSoloBytes (kSoloBytesMany when a
+// wavefront takes several) is done by one wavefront alone (wavefront w takes the rows w, w + 4, .. of the group, `solo_per_wave` of them: nothing to combine, the minima go
 // from the registers to the result); a longer row is shared by the four wavefronts, which split its first kSpan bytes
 // and combine through LDS, one such row after the other.  The groups lie along x and, beyond kMaxRowBlocks of them,
 // along z.
