@@ -27,25 +27,25 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 988b304)"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit befb679)"
 MEASURED_TRAFFIC_C2 = {
-    "range_first_row_kernel": (15959611, 248800),
-    "wordpiece_word_kernel": (1742944468, 1556467514),
-    "wordpiece_oov_kernel": (843584914, 863203220),
-    "wordpiece_emit_kernel": (1393677106, 905107583),
+    "range_first_row_kernel": (15965529, 248800),
+    "wordpiece_word_kernel": (1742902056, 1556477948),
+    "wordpiece_oov_kernel": (845504696, 863273263),
+    "wordpiece_emit_kernel": (1393674584, 905141504),
 }
 # (the fetch counter prices a read that misses L2 at a whole 128-byte line whatever was asked for, and counts the misses
 # that the Infinity Cache serves: most of what the tokenizer fetches on C5 is lines of its 8 MB table)
 MEASURED_TRAFFIC_C5_TOKENIZE = {
-    "range_first_row_kernel": (114439189, 995168),
-    "wordpiece_word_kernel": (24297267452, 5163004939),
-    "wordpiece_oov_kernel": (31978098813, 2111316977),
-    "wordpiece_emit_kernel": (4729697021, 3361286511),
+    "range_first_row_kernel": (119723680, 995168),
+    "wordpiece_word_kernel": (24307200821, 5162128338),
+    "wordpiece_oov_kernel": (31978600897, 2112272245),
+    "wordpiece_emit_kernel": (4729715132, 3361269904),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (4575178950, 63532927),
-    "normalize_tile_rows_kernel": (73449825, 7941632),
-    "normalize_write_kernel": (5469620699, 4672509960),
+    "normalize_count_kernel": (4575176981, 63532928),
+    "normalize_tile_rows_kernel": (73449498, 7941632),
+    "normalize_write_kernel": (5469604166, 4672266167),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
@@ -54,7 +54,7 @@ MEASURED_TRAFFIC_C5_NORMALIZE = {
 # mod 2^64, a shift, a mask and one more v_mad_u64_u32 for the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two
 # products (8.5).  Every window of the input counts as one, also those whose hash the wavefront met lately and does not
 # fold again (windows of a row repeat, most in long rows: that is how C4 comes so near the floor).
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 988b304)"
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit befb679)"
 MINHASH_VALU = {
     "C3": {"floor": 1.5, "measured": 1.72, "issue": 0.94},
     "C4": {"floor": 8.5, "measured": 8.92, "issue": 0.85},
