@@ -433,6 +433,7 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
   constexpr int kSets = K + (TAIL ? 1 : 0);
   __shared__ WaveLds<T> lds[kWaves];
   __shared__ T red[kWaves][kSets * kWave];
+  __shared__ uint32_t next_row;
 
   int const group_rows     = solo_per_wave * kWaves;
   int64_t const solo_bytes = solo_per_wave > 1 ? kSoloBytesMany : kSoloBytes;
@@ -449,14 +450,29 @@ __global__ void __launch_bounds__(kThreads, sizeof(T) == 4 ? 7 : 4) minhash_rows
   TailT::load(tail, pa, pb, P, lane);
 
   int const rows_here = static_cast<int>(min(static_cast<int64_t>(group_rows), col.size - r0));
-  int const wave_s    = __builtin_amdgcn_readfirstlane(wave);  // (the same in every lane: what depends on it stays scalar)
+  if (threadIdx.x == 0) next_row = 0;
+  __syncthreads();
 
-  // steps below 0: the short rows of this wavefront (rows wave, wave + 4, .. of the group); steps from 0: this
-  // wavefront's part of the rows that are too long for that, one after the other
-  for (int step = -solo_per_wave; step < rows_here; ++step) {
-    bool const solo = step < 0;
-    int const i     = solo ? (step + solo_per_wave) * kWaves + wave_s : step;
-    if (i >= rows_here || !col.valid(r0 + i)) continue;
+  // First the short rows of the group: a wavefront takes the next one whenever it is done with one (a counter in LDS),
+  // so that the four are done with their short rows at about the same time whatever the rows' lengths.  Then, from
+  // `together` = 0 on, its part of the rows that are too long for that, one after the other.
+  int together = -1;
+  for (;;) {
+    int i;
+    if (together < 0) {
+      int t = 0;
+      if (lane == 0) t = static_cast<int>(atomicAdd(&next_row, 1u));
+      i = __builtin_amdgcn_readfirstlane(t);  // (the same in every lane: what depends on it stays scalar)
+      if (i >= rows_here) {
+        together = 0;
+        continue;
+      }
+    } else {
+      if (together >= rows_here) break;
+      i = together++;
+    }
+    bool const solo = together < 0;
+    if (!col.valid(r0 + i)) continue;
     int64_t const o = col.off(r0 + i);
     int64_t const n = col.off(r0 + i + 1) - o;
     if (solo != (n <= solo_bytes)) continue;
@@ -785,6 +801,7 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
   // 64-bit hash, whose 16-byte steps cost more to assemble out of LDS than they save)
   constexpr bool kStageRuns = sizeof(T) == 4;
   __shared__ uint32_t run_bytes[kWaves][kStageRuns ? kNgramStageWords : 1];
+  __shared__ uint32_t next_row;
 
   int const group_rows = solo_per_wave > 0 ? solo_per_wave * kWaves : 1;
   int64_t const r0     = (static_cast<int64_t>(blockIdx.z) * gridDim.x + blockIdx.x) * group_rows;  // groups along x, then z
@@ -794,15 +811,31 @@ __global__ void __launch_bounds__(kThreads) minhash_ngrams_kernel(ListView in, i
   int32_t const in_chunk       = min(K * kWave, P - chunk_base);
   int const lane               = lane_id();
   int const wave               = threadIdx.x / kWave;
-  int const wave_s             = __builtin_amdgcn_readfirstlane(wave);
   T a[K], b[K], m[K];
   load_params<T, K>(pa, pb, P, chunk_base, lane, a, b, m);
 
   int const rows_here = static_cast<int>(min(static_cast<int64_t>(group_rows), in.size - r0));
-  for (int step = -solo_per_wave; step < rows_here; ++step) {
-    bool const solo = step < 0;
-    int const i     = solo ? (step + solo_per_wave) * kWaves + wave_s : step;
-    if (i >= rows_here || !in.valid(r0 + i)) continue;
+  if (threadIdx.x == 0) next_row = 0;
+  __syncthreads();
+  // the short rows of the group first, each wavefront taking the next one whenever it is done with one; then, from
+  // `together` = 0 on, the rows that all four do together, one after the other (see minhash_rows_kernel)
+  int together = -1;
+  for (;;) {
+    int i;
+    if (together < 0) {
+      int t = 0;
+      if (lane == 0) t = static_cast<int>(atomicAdd(&next_row, 1u));
+      i = __builtin_amdgcn_readfirstlane(t);
+      if (i >= rows_here) {
+        together = 0;
+        continue;
+      }
+    } else {
+      if (together >= rows_here) break;
+      i = together++;
+    }
+    bool const solo = together < 0;
+    if (!in.valid(r0 + i)) continue;
     int64_t const first = in.off(r0 + i);
     int64_t const n     = in.off(r0 + i + 1) - first;
     // minhash.cu:311-314 with width = ngrams: the positions that the permutation looks at
