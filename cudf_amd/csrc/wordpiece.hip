@@ -93,8 +93,11 @@ struct VocabTable {
   // short_ids[131072 + kind * 256 + byte0] for one; the token id, or INT32_MIN when there is no such key.
   const int32_t* short_ids;
   // The length filter once more, exact, for the keys of the second key space (the "##" entries) that begin with three
-  // lower-case ASCII letters c0 c1 c2: letters3[((c0 - 'a') * 26 + (c1 - 'a')) * 26 + (c2 - 'a')] has bit i set when
-  // some such key is i + 3 bytes long (3..18).  Small enough for LDS.
+  // lower-case ASCII letters c0 c1 c2: letters3[((c0 - 'a') * 26 + (c1 - 'a')) * 26 + (c2 - 'a')] has bit i (i < 7) set
+  // when some such key is i + 3 bytes long (3..9), bit 7 when one is longer; and bit 8 + (c3 & 7) when some such key of
+  // four bytes and more has c3 as its fourth byte: a piece whose fourth byte finds no bit has no candidate of more
+  // than three bytes, whatever the lengths say (text that the vocabulary does not know is mostly turned away here,
+  // before a lookup is spent on it).  Small enough for LDS.
   const uint16_t* letters3;
 };
 constexpr uint32_t kShortIds = 2 * 65536 + 2 * 256;
@@ -639,9 +642,11 @@ struct ShortWord {
     uint32_t const i3 = i2 * 26u + c2 - 97u;
     Opening o;
     o.id1               = first_ids[256 + c0];
-    uint32_t const len3 = l3[ok3 ? i3 : 0u];
+    uint32_t const e3   = l3[ok3 ? i3 : 0u];
     int32_t const two   = pair[ok2 ? i2 : 0u];
-    o.lens              = ok3 ? (len3 | 0xFFFF0000u) : 0xFFFFFFFFu;
+    uint32_t len3       = (e3 & 0x7Fu) | ((e3 & 0x80u) ? 0xFFFFFF80u : 0u);
+    if (((e3 >> (8u + ((b >> 24) & 7u))) & 1u) == 0u) len3 &= 1u;  // no key with this fourth byte: three bytes at most
+    o.lens              = ok3 ? len3 : 0xFFFFFFFFu;
     o.id2               = ok2 ? two : kNone;
     if (!ok3 && rem >= 3) o.lens = filter_word(t.lens[length_filter_index(1u, x) & t.lens_mask]);
     if (!ok2 && rem >= 2) o.id2 = t.short_ids[65536 + (b & 0xFFFFu)];
@@ -1963,9 +1968,10 @@ __global__ void vocabulary_bid_kernel(ColView v, VocabBuild t, uint32_t* __restr
     atomicOr(&t.lens32[length_filter_index(kind, k0 & 0x00FFFFFFu) & t.lens_mask], 1u << length_filter_bit(k.len));
     uint32_t const c0 = k0 & 0xFFu, c1 = (k0 >> 8) & 0xFFu, c2 = (k0 >> 16) & 0xFFu;
     auto letter = [](uint32_t c) { return c >= 'a' && c <= 'z'; };
-    if (kind == 1 && k.len <= 18 && letter(c0) && letter(c1) && letter(c2)) {
-      uint32_t const at = ((c0 - 'a') * 26u + (c1 - 'a')) * 26u + (c2 - 'a');
-      atomicOr(&t.letters3[at >> 1], (1u << (k.len - 3)) << (16u * (at & 1u)));
+    if (kind == 1 && letter(c0) && letter(c1) && letter(c2)) {
+      uint32_t const at   = ((c0 - 'a') * 26u + (c1 - 'a')) * 26u + (c2 - 'a');
+      uint32_t const bits = (k.len <= 9 ? 1u << (k.len - 3) : 0x80u) | (k.len >= 4 ? 0x100u << ((k0 >> 24) & 7u) : 0u);
+      atomicOr(&t.letters3[at >> 1], bits << (16u * (at & 1u)));
     }
   }
   // the direct tables of the keys of one and two bytes: the first entry with a key wins
