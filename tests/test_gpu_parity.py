@@ -772,8 +772,9 @@ def test_wordpiece_pieces_of_letters_and_of_their_neighbours(nv, orc):
     """Later pieces of a word ("##" keys) over an alphabet of lower-case letters and the bytes next to them in ASCII
     ('`' before 'a', '{' after 'z', capitals, digits): the library serves the pieces that begin with two or three
     lower-case letters from small tables of their own and the others from the general ones, and both have to say the
-    same as the oracle; keys of every length from 1 to 20 bytes, so that the tables' longest lengths (18) and the
-    keys beyond them are met."""
+    same as the oracle; keys of every length from 1 to 20 bytes, so that the lengths that the three-letter table names
+    one by one (3 to 9) and those that share its last bit are met, and fourth bytes that share a bit of its fourth-byte
+    mask ('z' and 'b', 'a' and 'A' and '9') with and without a key of their own."""
     rng = np.random.default_rng(77)
     letters = list("azmb")
     others = list("`{AZ09")
