@@ -86,8 +86,11 @@ struct VocabTable {
   // Length filter: lens[length_filter_index(kind, first three key bytes) & lens_mask] has bit i (i < 31) set
   // when some key of that key space with those first bytes is i + 3 bytes long, bit 31 for 34 bytes and more.
   // Entries are shared by hashing, so a set bit promises nothing, a clear bit rules the length out.
-  // (stored as 16-bit words: bits 0..14 for 3..17 bytes, bit 15 for 18 bytes and more; filter_word() spreads it out)
-  const uint16_t* lens;
+  // (stored in the low half of a 32-bit word: bits 0..14 for 3..17 bytes, bit 15 for 18 bytes and more; filter_word()
+  // spreads it out.)  The high half says which fourth bytes the keys of four bytes and more of the entry have, bit
+  // 16 + (byte & 15): a piece whose fourth byte finds no bit has no candidate of more than three bytes
+  // (piece_filter_word()).
+  const uint32_t* lens;
   uint32_t lens_mask;
   // Direct tables for keys of one and two bytes: short_ids[kind * 65536 + (byte0 | byte1 << 8)] for two bytes,
   // short_ids[131072 + kind * 256 + byte0] for one; the token id, or INT32_MIN when there is no such key.
@@ -115,6 +118,13 @@ __host__ __device__ __forceinline__ uint32_t length_filter_bit(uint32_t len) { r
 // The stored form of a filter word and back: the lengths of 18 bytes and more share one bit.
 __host__ __device__ __forceinline__ uint16_t packed_filter_word(uint32_t w) { return static_cast<uint16_t>((w & 0x7FFFu) | ((w >> 15) ? 0x8000u : 0u)); }
 __host__ __device__ __forceinline__ uint32_t filter_word(uint32_t stored) { return (stored & 0x7FFFu) | ((stored & 0x8000u) ? 0xFFFF8000u : 0u); }
+// The candidate lengths (bit i: i + 3 bytes) that a filter entry leaves a piece whose first four bytes are first4
+// (bytes past the piece may hold anything: candidates that long do not exist).
+__host__ __device__ __forceinline__ uint32_t piece_filter_word(uint32_t stored, uint32_t first4)
+{
+  uint32_t const w = filter_word(stored & 0xFFFFu);
+  return ((stored >> (16u + ((first4 >> 24) & 15u))) & 1u) ? w : (w & 1u);
+}
 
 // What a lookup takes from a key's hash: the two halves folded and multiplied once more (the top bits of such a product
 // depend on every bit of both halves), the key's home bucket from the top `bucket_bits` bits, the tag and the carried
@@ -472,7 +482,7 @@ struct OovStepper {
 
   __device__ __forceinline__ void load_filter(VocabTable const& t, uint32_t kind)
   {
-    lens = len - start >= 3 ? filter_word(t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask]) : 0xFFFFFFFFu;
+    lens = len - start >= 3 ? piece_filter_word(t.lens[length_filter_index(kind, raw0 & 0x00FFFFFFu) & t.lens_mask], raw0) : 0xFFFFFFFFu;
   }
 
   // probed: the whole word has been looked up and is known to be absent
@@ -616,7 +626,7 @@ struct ShortWord {
     uint32_t const b    = dword_at(p);
     uint32_t const left = rem - min(p, rem);
     Opening o;
-    uint32_t const lens = filter_word(t.lens[length_filter_index(kind, b & 0x00FFFFFFu) & t.lens_mask]);
+    uint32_t const lens = piece_filter_word(t.lens[length_filter_index(kind, b & 0x00FFFFFFu) & t.lens_mask], b);
     int32_t const two   = t.short_ids[kind * 65536 + (b & 0xFFFFu)];
     o.id1               = first_ids[kind * 256 + (b & 0xFFu)];
     o.lens              = left >= 3 ? lens : 0xFFFFFFFFu;
@@ -648,7 +658,7 @@ struct ShortWord {
     if (((e3 >> (8u + ((b >> 24) & 7u))) & 1u) == 0u) len3 &= 1u;  // no key with this fourth byte: three bytes at most
     o.lens              = ok3 ? len3 : 0xFFFFFFFFu;
     o.id2               = ok2 ? two : kNone;
-    if (!ok3 && rem >= 3) o.lens = filter_word(t.lens[length_filter_index(1u, x) & t.lens_mask]);
+    if (!ok3 && rem >= 3) o.lens = piece_filter_word(t.lens[length_filter_index(1u, x) & t.lens_mask], b);
     if (!ok2 && rem >= 2) o.id2 = t.short_ids[65536 + (b & 0xFFFFu)];
     return o;
   }
@@ -1908,6 +1918,7 @@ struct VocabBuild {
   uint32_t* slots;      // the table as dwords: slot s at [4 s, 4 s + 4)
   uint8_t* pool;
   uint32_t* lens32;     // the length filter, a 32-bit word per entry (packed afterwards)
+  uint32_t* lens_final; // the filter as the lookups read it: the fourth-byte bits are set here, the packed lengths join them at the end
   uint32_t* short_ids;  // as VocabTable::short_ids, "no such key" = 0x80000000 (above every id)
   uint32_t* letters3;   // as VocabTable::letters3, two entries to a word
   uint32_t bucket_mask, bucket_bits, lens_mask;
@@ -1965,7 +1976,9 @@ __global__ void vocabulary_bid_kernel(ColView v, VocabBuild t, uint32_t* __restr
   VocabKey const& k = p.key;
   // the length filter over the first three bytes, and its exact twin for pieces of lower-case letters
   if (k.len >= 3) {
-    atomicOr(&t.lens32[length_filter_index(kind, k0 & 0x00FFFFFFu) & t.lens_mask], 1u << length_filter_bit(k.len));
+    uint32_t const entry = length_filter_index(kind, k0 & 0x00FFFFFFu) & t.lens_mask;
+    atomicOr(&t.lens32[entry], 1u << length_filter_bit(k.len));
+    if (k.len >= 4) atomicOr(&t.lens_final[entry], 0x10000u << ((k0 >> 24) & 15u));
     uint32_t const c0 = k0 & 0xFFu, c1 = (k0 >> 8) & 0xFFu, c2 = (k0 >> 16) & 0xFFu;
     auto letter = [](uint32_t c) { return c >= 'a' && c <= 'z'; };
     if (kind == 1 && letter(c0) && letter(c1) && letter(c2)) {
@@ -2063,12 +2076,12 @@ __global__ void vocabulary_settle_kernel(ColView v, VocabBuild t)
 
 // The length filter in its stored form, "no such key" of the direct tables as the lookups expect it, and the id of
 // the unknown token (cpp/src/text/wordpiece_tokenize.cu:199-209, 273-275: "[UNK]", else "[unk]", else -1).
-__global__ void vocabulary_finish_kernel(VocabTable table, const uint32_t* __restrict__ lens32, uint16_t* __restrict__ lens16, uint32_t lens_size,
+__global__ void vocabulary_finish_kernel(VocabTable table, const uint32_t* __restrict__ lens32, uint32_t* __restrict__ lens_final, uint32_t lens_size,
                                          int32_t* __restrict__ short_ids, VocabCounts* __restrict__ counts)
 {
   uint32_t const stride = gridDim.x * blockDim.x;
   uint32_t const t      = blockIdx.x * blockDim.x + threadIdx.x;
-  for (uint32_t i = t; i < lens_size; i += stride) lens16[i] = packed_filter_word(lens32[i]);
+  for (uint32_t i = t; i < lens_size; i += stride) lens_final[i] |= packed_filter_word(lens32[i]);
   for (uint32_t i = t; i < kShortIds; i += stride)
     if (static_cast<uint32_t>(short_ids[i]) == 0x80000000u) short_ids[i] = kNone;  // (the same bits: kNone is INT32_MIN)
   if (t == 0) {
@@ -2133,7 +2146,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->store.bind(mr, stream);
   v->d_slots   = v->store.allocate(v->slot_bytes);
   v->d_pool    = v->store.allocate(v->pool_bytes);
-  v->d_lens    = v->store.allocate(lens_size * sizeof(uint16_t));
+  v->d_lens    = v->store.allocate(lens_size * sizeof(uint32_t));
   v->d_short   = v->store.allocate(kShortIds * sizeof(int32_t));
   v->d_letters = v->store.allocate(kLetters3 * sizeof(uint16_t));
   Temp lens32(temp_mr, lens_size * sizeof(uint32_t));
@@ -2145,6 +2158,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   launch_fill_u32(static_cast<uint32_t*>(v->d_slots), 0u, static_cast<int64_t>(capacity) * 4, stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_pool), 0u, static_cast<int64_t>(v->pool_bytes / 4), stream);  // (the sizes are multiples of 8)
   launch_fill_u32(lens32.as<uint32_t>(), 0u, static_cast<int64_t>(lens_size), stream);
+  launch_fill_u32(static_cast<uint32_t*>(v->d_lens), 0u, static_cast<int64_t>(lens_size), stream);
   launch_fill_u32(bids.as<uint32_t>(), kNoBid, static_cast<int64_t>(capacity), stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_short), 0x80000000u, kShortIds, stream);
   launch_fill_u32(static_cast<uint32_t*>(v->d_letters), 0u, kLetters3 / 2, stream);
@@ -2156,7 +2170,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   v->table.unk_id      = -1;
   v->table.max_len[0]  = counts.max_len[0];
   v->table.max_len[1]  = counts.max_len[1];
-  v->table.lens        = static_cast<const uint16_t*>(v->d_lens);
+  v->table.lens        = static_cast<const uint32_t*>(v->d_lens);
   v->table.lens_mask   = static_cast<uint32_t>(lens_size - 1);
   v->table.short_ids   = static_cast<const int32_t*>(v->d_short);
   v->table.letters3    = static_cast<const uint16_t*>(v->d_letters);
@@ -2165,6 +2179,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   build.slots       = static_cast<uint32_t*>(v->d_slots);
   build.pool        = static_cast<uint8_t*>(v->d_pool);
   build.lens32      = lens32.as<uint32_t>();
+  build.lens_final  = static_cast<uint32_t*>(v->d_lens);
   build.short_ids   = static_cast<uint32_t*>(v->d_short);
   build.letters3    = static_cast<uint32_t*>(v->d_letters);
   build.bucket_mask = mask;
@@ -2176,7 +2191,7 @@ nvtext_amd_status nvtext_amd_wordpiece_vocabulary_create(const nvtext_amd_string
   hipLaunchKernelGGL(vocabulary_other_slots_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build, d_counts, bids.as<uint32_t>(),
                      bids.as<uint32_t>() + capacity / 2);
   hipLaunchKernelGGL(vocabulary_settle_kernel, dim3(key_grid), dim3(256), 0, stream, entries, build);
-  hipLaunchKernelGGL(vocabulary_finish_kernel, dim3(256), dim3(256), 0, stream, v->table, lens32.as<uint32_t>(), static_cast<uint16_t*>(v->d_lens),
+  hipLaunchKernelGGL(vocabulary_finish_kernel, dim3(256), dim3(256), 0, stream, v->table, lens32.as<uint32_t>(), static_cast<uint32_t*>(v->d_lens),
                      static_cast<uint32_t>(lens_size), static_cast<int32_t*>(v->d_short), d_counts);
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) e = hipMemcpyAsync(&counts, d_counts, sizeof(counts), hipMemcpyDeviceToHost, stream);
