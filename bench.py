@@ -27,25 +27,25 @@ HBM_PEAK_GBS = 8000.0
 #
 # HBM bytes per launch (fetched, written) of the tokenizer kernels on the full C2 workload: FETCH_SIZE / WRITE_SIZE
 # scaled by a copy kernel of known size.
-TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit bc76102)"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_pmc_all_workloads.md (library sources at commit 692bfef)"
 MEASURED_TRAFFIC_C2 = {
-    "range_first_row_kernel": (15969543, 248800),
-    "wordpiece_word_kernel": (1742939853, 1556629205),
-    "wordpiece_oov_kernel": (861196959, 858026467),
-    "wordpiece_emit_kernel": (1393672499, 905134125),
+    "range_first_row_kernel": (15968662, 248800),
+    "wordpiece_word_kernel": (1742880831, 1556229099),
+    "wordpiece_oov_kernel": (861252878, 857545519),
+    "wordpiece_emit_kernel": (1393668802, 905164798),
 }
 # (the fetch counter prices a read that misses L2 at a whole 128-byte line whatever was asked for, and counts the misses
 # that the Infinity Cache serves: most of what the tokenizer fetches on C5 is lines of its 8 MB table)
 MEASURED_TRAFFIC_C5_TOKENIZE = {
-    "range_first_row_kernel": (119511645, 995168),
-    "wordpiece_word_kernel": (24307722162, 5161941300),
-    "wordpiece_oov_kernel": (21480366513, 2093032708),
-    "wordpiece_emit_kernel": (4729677231, 3361254444),
+    "range_first_row_kernel": (119625264, 995168),
+    "wordpiece_word_kernel": (24310186114, 5163209271),
+    "wordpiece_oov_kernel": (21481440462, 2092868777),
+    "wordpiece_emit_kernel": (4729690208, 3361303065),
 }
 MEASURED_TRAFFIC_C5_NORMALIZE = {
-    "normalize_count_kernel": (4575177215, 63532923),
-    "normalize_tile_rows_kernel": (73449484, 7941631),
-    "normalize_write_kernel": (5469610964, 4672612955),
+    "normalize_count_kernel": (4575175068, 63532928),
+    "normalize_tile_rows_kernel": (73449328, 7941632),
+    "normalize_write_kernel": (5469615636, 4672395239),
 }
 # minhash: VALU wave-instructions executed per (window, parameter) of a wavefront (SQ_INSTS_VALU / (windows x P / 64)) and
 # the share of SIMD cycles that issued one (SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel cycles), capped at 1: adds and
@@ -54,11 +54,11 @@ MEASURED_TRAFFIC_C5_NORMALIZE = {
 # mod 2^64, a shift, a mask and one more v_mad_u64_u32 for the fold mod 2^61-1, one v_min_f64, one v_max3_u32 per two
 # products (8.5).  Every window of the input counts as one, also those whose hash the wavefront met lately and does not
 # fold again (windows of a row repeat, most in long rows: that is how C4 comes so near the floor).
-VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit bc76102)"
+VALU_SOURCE = "profiles/valu_issue_pmc_all_workloads.md (library sources at commit 692bfef)"
 MINHASH_VALU = {
-    "C3": {"floor": 1.5, "measured": 1.72, "issue": 0.96},
-    "C4": {"floor": 8.5, "measured": 8.92, "issue": 0.85},
-    "C5": {"floor": 8.5, "measured": 13.08, "issue": 1.04},
+    "C3": {"floor": 1.5, "measured": 1.72, "issue": 0.97},
+    "C4": {"floor": 8.5, "measured": 8.73, "issue": 0.88},
+    "C5": {"floor": 8.5, "measured": 13.08, "issue": 1.05},
 }
 
 
